@@ -1,0 +1,184 @@
+/*
+ * spcomm3d_hip.h - C ABI of the MI355X (gfx950) local SDDMM / SpMM library.
+ *
+ * The reference has no FFI layer: its local compute step is two C++ free
+ * functions with external linkage,
+ *     SpKernels::sddmm(denseMatrix& A, denseMatrix& B, cooMat& S, cooMat& C)
+ *     SpKernels::spmm (denseMatrix& X, cooMat& A, denseMatrix& Y)
+ * declared in src/core_ops.hpp:9-12 and defined in src/core_ops.cpp:5-35,
+ * called from src/distributed_comp.cpp:53,177,220,268,314,379 and
+ * miniapp/numCheckSeq.cpp:130.  A host shim with those two signatures
+ * (spcomm3d_amd/host) forwards to the entry points below; they are what a
+ * binding for this path binds.
+ *
+ * Conventions
+ *  - Plain pointers and sizes only.  Every function returns an spc3d_status;
+ *    spc3d_last_error() gives the message of the calling thread's last
+ *    failure.  No C++ exception crosses this boundary.  (The reference
+ *    returns void and fails by std::out_of_range from .at() -> terminate,
+ *    core_ops.cpp:16,18,32; the C++ shim turns a non-zero status back into
+ *    that exception.)
+ *  - Indices are uint32, 0-based, local (src/basic.hpp:16); dense panels are
+ *    row-major with K contiguous (src/basic.hpp:32,36); values are float or
+ *    double (the reference's real_t is double, src/basic.hpp:17; float is an
+ *    extension).
+ *  - COO entries may come in any order and may repeat.  SDDMM writes result e
+ *    at position e of the caller's order (core_ops.cpp:18); SpMM adds into Y
+ *    (core_ops.cpp:32), duplicates add.
+ *  - The reference computes panel offsets x*n+y in 32 bits
+ *    (src/basic.hpp:36), so its behaviour is defined only for m*n < 2^32.
+ *    This library uses 64-bit offsets; nnz must be < 2^32.
+ *  - A context is used by one host thread at a time and owns one HIP stream
+ *    (default priority).  Kernel-launching calls are asynchronous on that
+ *    stream; *_download and *_host calls return with host memory valid.
+ *  - Nothing here falls back to the CPU: without a usable GPU every device
+ *    call fails with SPC3D_ERR_NO_DEVICE.
+ */
+#ifndef SPCOMM3D_HIP_H
+#define SPCOMM3D_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#if defined(__GNUC__)
+#define SPC3D_API __attribute__((visibility("default")))
+#else
+#define SPC3D_API
+#endif
+
+typedef enum {
+    SPC3D_OK = 0,
+    SPC3D_ERR_INVALID_ARG = 1,   /* null pointer, unknown dtype, destroyed handle */
+    SPC3D_ERR_BAD_INDEX = 2,     /* ii[e] >= nrows or jj[e] >= ncols (reference: out_of_range) */
+    SPC3D_ERR_SIZE_MISMATCH = 3, /* panel / value-vector shape or dtype does not fit the plan */
+    SPC3D_ERR_TOO_LARGE = 4,     /* nnz >= 2^32 or a byte size overflows */
+    SPC3D_ERR_NO_DEVICE = 5,     /* no HIP device / device id out of range */
+    SPC3D_ERR_HIP = 6,           /* a HIP runtime call failed; see spc3d_last_error() */
+    SPC3D_ERR_ALLOC = 7          /* host or device allocation failed */
+} spc3d_status;
+
+typedef enum { SPC3D_F32 = 0, SPC3D_F64 = 1 } spc3d_dtype;
+
+typedef struct spc3d_ctx spc3d_ctx;     /* device + stream */
+typedef struct spc3d_panel spc3d_panel; /* device-resident denseMatrix::data (src/basic.hpp:30-36) */
+typedef struct spc3d_vals spc3d_vals;   /* device-resident cooMat::vv (src/SparseMatrix.hpp:36) */
+typedef struct spc3d_plan spc3d_plan;   /* device-resident cooMat pattern (ii, jj) in kernel order */
+
+typedef struct {
+    uint32_t nrows, ncols;
+    uint64_t nnz;
+    uint32_t rows_touched;   /* rows with at least one entry */
+    uint32_t cols_touched;   /* columns with at least one entry */
+    uint32_t nsegments;      /* row segments the kernels iterate over */
+    uint32_t nsplit_rows;    /* rows cut into several segments (SpMM combines partial sums) */
+    uint32_t npartial_slots; /* partial-sum rows kept for those */
+    uint32_t max_row_nnz;
+    uint32_t seg_max;        /* longest segment */
+    int32_t  order_is_identity; /* 1: caller's COO was already row-major grouped, no permutation read */
+} spc3d_plan_info;
+
+/* ---- library / errors ------------------------------------------------- */
+SPC3D_API const char *spc3d_version(void);
+SPC3D_API const char *spc3d_last_error(void);
+SPC3D_API const char *spc3d_status_name(int status);
+SPC3D_API int spc3d_device_count(int *count);
+
+/* ---- context ----------------------------------------------------------- */
+SPC3D_API int spc3d_ctx_create(int device, spc3d_ctx **out);
+SPC3D_API int spc3d_ctx_destroy(spc3d_ctx *ctx);
+SPC3D_API int spc3d_ctx_sync(spc3d_ctx *ctx);                 /* wait for the context's stream */
+SPC3D_API int spc3d_ctx_stream(spc3d_ctx *ctx, void **hip_stream); /* the hipStream_t, for callers that share it */
+
+/* Timing on the context's stream (the reference times the call with chrono in
+ * integer ms, src/distributed_comp.cpp:176-179; a kernel here lasts well under
+ * one).  spc3d_timer_mark records event `slot` (0..63) on the stream;
+ * spc3d_timer_elapsed_ms waits for `stop` and returns stop-start. */
+SPC3D_API int spc3d_timer_mark(spc3d_ctx *ctx, int slot);
+SPC3D_API int spc3d_timer_elapsed_ms(spc3d_ctx *ctx, int start, int stop, float *ms);
+
+/* ---- dense panels: denseMatrix (src/basic.hpp:30-44) ------------------- */
+SPC3D_API int spc3d_panel_create(spc3d_ctx *ctx, int dtype, uint32_t m, uint32_t n, spc3d_panel **out);
+SPC3D_API int spc3d_panel_destroy(spc3d_panel *p);
+SPC3D_API int spc3d_panel_upload(spc3d_panel *p, const void *host);   /* m*n reals, row-major */
+SPC3D_API int spc3d_panel_download(spc3d_panel *p, void *host);
+SPC3D_API int spc3d_panel_fill(spc3d_panel *p, double value);
+SPC3D_API int spc3d_panel_device_ptr(spc3d_panel *p, void **dev);
+SPC3D_API int spc3d_panel_shape(spc3d_panel *p, uint32_t *m, uint32_t *n, int *dtype);
+
+/* ---- value vectors: cooMat::vv (src/SparseMatrix.hpp:36) --------------- */
+SPC3D_API int spc3d_vals_create(spc3d_ctx *ctx, int dtype, uint64_t n, spc3d_vals **out);
+SPC3D_API int spc3d_vals_destroy(spc3d_vals *v);
+SPC3D_API int spc3d_vals_upload(spc3d_vals *v, const void *host);
+SPC3D_API int spc3d_vals_download(spc3d_vals *v, void *host);
+SPC3D_API int spc3d_vals_fill(spc3d_vals *v, double value);
+SPC3D_API int spc3d_vals_device_ptr(spc3d_vals *v, void **dev);
+
+/* ---- plan: the sparse operand ------------------------------------------ */
+/* Host-only check of a COO pattern; needs no GPU.  Mirrors the bounds checks
+ * of core_ops.cpp:16,32 (.at()): SPC3D_ERR_BAD_INDEX names the first bad entry
+ * in spc3d_last_error(). */
+SPC3D_API int spc3d_coo_validate(uint32_t nrows, uint32_t ncols, uint64_t nnz,
+                       const uint32_t *ii, const uint32_t *jj);
+
+/* Validates (as above), groups the entries by row keeping the caller's order
+ * within a row, cuts rows into segments, and uploads.  `vv` (nnz reals of
+ * `dtype`, caller's order) may be NULL and set later.  The pattern is copied:
+ * the caller's arrays are not referenced afterwards.  Replaces nothing in the
+ * reference (it walks the unsorted COO directly, core_ops.cpp:7-10); it is the
+ * amortised set-up for the five identical calls the benches make
+ * (miniapp/bench_both.cpp:202-203, bench_spmm.cpp:185-186). */
+SPC3D_API int spc3d_plan_create(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t ncols,
+                      uint64_t nnz, const uint32_t *ii, const uint32_t *jj,
+                      const void *vv, spc3d_plan **out);
+/* As above with the longest segment given explicitly (0 = library default). */
+SPC3D_API int spc3d_plan_create_ex(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t ncols,
+                         uint64_t nnz, const uint32_t *ii, const uint32_t *jj,
+                         const void *vv, uint32_t seg_max, spc3d_plan **out);
+/* Host-only: builds the same kernel-order form spc3d_plan_create uploads and
+ * hands it back, for inspection and for testing without a GPU.  `info` is
+ * always filled.  Each output may be NULL; otherwise col and perm hold nnz
+ * entries (perm[p] = caller's position of kernel-order entry p), segs holds
+ * 4 words per segment {row, start, len, slot} (slot 0xFFFFFFFF: the segment is
+ * the whole row) and needs seg_cap >= info->nsegments, splits holds 3 words per
+ * cut row {row, first_slot, nslots} and needs split_cap >= info->nsplit_rows;
+ * a capacity that is too small gives SPC3D_ERR_SIZE_MISMATCH. */
+SPC3D_API int spc3d_plan_build_host(uint32_t nrows, uint32_t ncols, uint64_t nnz,
+                          const uint32_t *ii, const uint32_t *jj, uint32_t seg_max,
+                          spc3d_plan_info *info, uint32_t *col, uint32_t *perm,
+                          uint32_t *segs, uint32_t seg_cap, uint32_t *splits,
+                          uint32_t split_cap);
+SPC3D_API int spc3d_plan_destroy(spc3d_plan *plan);
+SPC3D_API int spc3d_plan_set_values(spc3d_plan *plan, const void *vv_host);       /* caller's COO order */
+SPC3D_API int spc3d_plan_set_values_device(spc3d_plan *plan, const spc3d_vals *vv); /* caller's COO order */
+SPC3D_API int spc3d_plan_get_info(const spc3d_plan *plan, spc3d_plan_info *info);
+
+/* ---- the hot path -------------------------------------------------------
+ * spc3d_sddmm  = SpKernels::sddmm (src/core_ops.cpp:5-22):
+ *     C[e] = S.vv[e] * sum_j A[ii[e],j] * B[jj[e],j],  e in the caller's order.
+ *     K = A.n (core_ops.cpp:6); requires B.n == K, A.m >= nrows, B.m >= ncols,
+ *     C length >= nnz, all dtypes equal to the plan's.
+ * spc3d_spmm   = SpKernels::spmm  (src/core_ops.cpp:24-35):
+ *     Y[ii[e],:] += A.vv[e] * X[jj[e],:]   (accumulates; duplicates add).
+ *     K = X.n (core_ops.cpp:25); requires Y.n == K, X.m >= ncols, Y.m >= nrows.
+ * Both are asynchronous on the context's stream. */
+SPC3D_API int spc3d_sddmm(spc3d_ctx *ctx, spc3d_plan *S, const spc3d_panel *A,
+                const spc3d_panel *B, spc3d_vals *C);
+SPC3D_API int spc3d_spmm(spc3d_ctx *ctx, spc3d_plan *A, const spc3d_panel *X, spc3d_panel *Y);
+
+/* One-shot forms over host memory with exactly the reference's operands:
+ * plan, upload, run, download, free.  Synchronous. */
+SPC3D_API int spc3d_sddmm_host(spc3d_ctx *ctx, int dtype, uint32_t m, uint32_t n, uint32_t k,
+                     const void *A, const void *B, uint64_t nnz, const uint32_t *ii,
+                     const uint32_t *jj, const void *svv, void *cvv);
+SPC3D_API int spc3d_spmm_host(spc3d_ctx *ctx, int dtype, uint32_t ncols, uint32_t nrows, uint32_t k,
+                    const void *X, uint64_t nnz, const uint32_t *ii, const uint32_t *jj,
+                    const void *avv, void *Y);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SPCOMM3D_HIP_H */

@@ -1,0 +1,798 @@
+// C ABI of the local SDDMM / SpMM library (see include/spcomm3d_hip.h).
+// Owns device memory for panels, value vectors and plans; launches the
+// kernels of kernels.hip on the context's stream.  No CPU compute fallback:
+// without a device every device call fails.
+#include "../../include/spcomm3d_hip.h"
+
+#include <hip/hip_runtime_api.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <new>
+#include <string>
+
+#include "kernels.h"
+#include "plan_host.h"
+
+using namespace spc3d;
+
+namespace {
+
+thread_local std::string g_err;
+
+int fail(int status, const std::string &msg)
+{
+    g_err = msg;
+    return status;
+}
+
+int fail_hip(hipError_t e, const char *what)
+{
+    g_err = std::string(what) + ": " + hipGetErrorString(e);
+    if (e == hipErrorOutOfMemory)
+        return SPC3D_ERR_ALLOC;
+    if (e == hipErrorNoDevice || e == hipErrorInvalidDevice || e == hipErrorInsufficientDriver)
+        return SPC3D_ERR_NO_DEVICE;
+    return SPC3D_ERR_HIP;
+}
+
+#define HIP_TRY(expr)                                                                             \
+    do {                                                                                          \
+        hipError_t e_ = (expr);                                                                   \
+        if (e_ != hipSuccess)                                                                     \
+            return fail_hip(e_, #expr);                                                           \
+    } while (0)
+
+constexpr uint32_t kMagicCtx = 0x53433343;   // live handles carry a tag so that a
+constexpr uint32_t kMagicPanel = 0x53433350; // stale or foreign pointer is refused
+constexpr uint32_t kMagicVals = 0x53433356;  // instead of dereferenced further
+constexpr uint32_t kMagicPlan = 0x5343334c;
+constexpr int kTimerSlots = 64;
+
+inline size_t elem_size(int dtype) { return dtype == SPC3D_F64 ? 8 : 4; }
+inline bool dtype_ok(int dtype) { return dtype == SPC3D_F32 || dtype == SPC3D_F64; }
+
+} // namespace
+
+struct spc3d_ctx {
+    uint32_t magic;
+    int device;
+    hipStream_t stream;
+    hipEvent_t timers[kTimerSlots];
+    bool timer_set[kTimerSlots];
+};
+
+struct spc3d_panel {
+    uint32_t magic;
+    spc3d_ctx *ctx;
+    int dtype;
+    uint32_t m, n;
+    void *dev;
+};
+
+struct spc3d_vals {
+    uint32_t magic;
+    spc3d_ctx *ctx;
+    int dtype;
+    uint64_t n;
+    void *dev;
+};
+
+struct spc3d_plan {
+    uint32_t magic;
+    spc3d_ctx *ctx;
+    int dtype;
+    spc3d_plan_info info;
+    bool has_values;
+    // device arrays
+    Seg *segs;
+    uint32_t *col;
+    uint32_t *perm; // null when the caller's order is already the kernel order
+    void *sval;     // values in kernel order
+    SplitRow *splits;
+    void *partial; // [npartial_slots * partial_k] reals
+    uint32_t partial_k;
+};
+
+namespace {
+
+bool live(const spc3d_ctx *c) { return c && c->magic == kMagicCtx; }
+bool live(const spc3d_panel *p) { return p && p->magic == kMagicPanel && live(p->ctx); }
+bool live(const spc3d_vals *v) { return v && v->magic == kMagicVals && live(v->ctx); }
+bool live(const spc3d_plan *p) { return p && p->magic == kMagicPlan && live(p->ctx); }
+
+int use_device(const spc3d_ctx *ctx)
+{
+    HIP_TRY(hipSetDevice(ctx->device));
+    return SPC3D_OK;
+}
+
+template <typename T> int dev_alloc(T **out, size_t count)
+{
+    *out = nullptr;
+    if (count == 0)
+        return SPC3D_OK;
+    if (count > SIZE_MAX / sizeof(T))
+        return fail(SPC3D_ERR_TOO_LARGE, "allocation size overflows");
+    HIP_TRY(hipMalloc((void **)out, count * sizeof(T)));
+    return SPC3D_OK;
+}
+
+int dev_alloc_bytes(void **out, size_t bytes)
+{
+    *out = nullptr;
+    if (bytes == 0)
+        return SPC3D_OK;
+    HIP_TRY(hipMalloc(out, bytes));
+    return SPC3D_OK;
+}
+
+// Pageable-host <-> device copy ordered after everything queued on the
+// stream; returns when the host side may be reused / read.
+int copy_h2d(spc3d_ctx *ctx, void *dst, const void *src, size_t bytes)
+{
+    if (bytes == 0)
+        return SPC3D_OK;
+    HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx->stream));
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    return SPC3D_OK;
+}
+
+int copy_d2h(spc3d_ctx *ctx, void *dst, const void *src, size_t bytes)
+{
+    if (bytes == 0)
+        return SPC3D_OK;
+    HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    return SPC3D_OK;
+}
+
+void plan_free_device(spc3d_plan *p)
+{
+    if (p->segs) (void)hipFree(p->segs);
+    if (p->col) (void)hipFree(p->col);
+    if (p->perm) (void)hipFree(p->perm);
+    if (p->sval) (void)hipFree(p->sval);
+    if (p->splits) (void)hipFree(p->splits);
+    if (p->partial) (void)hipFree(p->partial);
+    p->segs = nullptr;
+    p->col = p->perm = nullptr;
+    p->sval = p->partial = nullptr;
+    p->splits = nullptr;
+}
+
+DevPlanView view_of(const spc3d_plan *p)
+{
+    DevPlanView v;
+    v.segs = p->segs;
+    v.nseg = p->info.nsegments;
+    v.col = p->col;
+    v.perm = p->perm;
+    v.sval = p->sval;
+    v.splits = p->splits;
+    v.nsplit = p->info.nsplit_rows;
+    v.partial = p->partial;
+    v.nnz = p->info.nnz;
+    return v;
+}
+
+} // namespace
+
+extern "C" {
+
+const char *spc3d_version(void) { return "spcomm3d_hip 0.1 (gfx950)"; }
+
+const char *spc3d_last_error(void) { return g_err.c_str(); }
+
+const char *spc3d_status_name(int status)
+{
+    switch (status) {
+    case SPC3D_OK: return "SPC3D_OK";
+    case SPC3D_ERR_INVALID_ARG: return "SPC3D_ERR_INVALID_ARG";
+    case SPC3D_ERR_BAD_INDEX: return "SPC3D_ERR_BAD_INDEX";
+    case SPC3D_ERR_SIZE_MISMATCH: return "SPC3D_ERR_SIZE_MISMATCH";
+    case SPC3D_ERR_TOO_LARGE: return "SPC3D_ERR_TOO_LARGE";
+    case SPC3D_ERR_NO_DEVICE: return "SPC3D_ERR_NO_DEVICE";
+    case SPC3D_ERR_HIP: return "SPC3D_ERR_HIP";
+    case SPC3D_ERR_ALLOC: return "SPC3D_ERR_ALLOC";
+    default: return "SPC3D_ERR_UNKNOWN";
+    }
+}
+
+int spc3d_device_count(int *count)
+{
+    if (!count)
+        return fail(SPC3D_ERR_INVALID_ARG, "count is NULL");
+    *count = 0;
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n <= 0) {
+        (void)hipGetLastError();
+        return fail(SPC3D_ERR_NO_DEVICE,
+                    std::string("no HIP device: ") +
+                        (e != hipSuccess ? hipGetErrorString(e) : "device count is 0"));
+    }
+    *count = n;
+    return SPC3D_OK;
+}
+
+/* ---- context ------------------------------------------------------------- */
+int spc3d_ctx_create(int device, spc3d_ctx **out)
+{
+    if (!out)
+        return fail(SPC3D_ERR_INVALID_ARG, "out is NULL");
+    *out = nullptr;
+    int n = 0;
+    int rc = spc3d_device_count(&n);
+    if (rc != SPC3D_OK)
+        return rc;
+    if (device < 0 || device >= n)
+        return fail(SPC3D_ERR_NO_DEVICE, "device id out of range");
+    HIP_TRY(hipSetDevice(device));
+    spc3d_ctx *c = new (std::nothrow) spc3d_ctx();
+    if (!c)
+        return fail(SPC3D_ERR_ALLOC, "host allocation failed");
+    c->device = device;
+    hipError_t e = hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking);
+    if (e != hipSuccess) {
+        delete c;
+        return fail_hip(e, "hipStreamCreateWithFlags");
+    }
+    for (int i = 0; i < kTimerSlots; ++i) {
+        c->timers[i] = nullptr;
+        c->timer_set[i] = false;
+    }
+    c->magic = kMagicCtx;
+    *out = c;
+    return SPC3D_OK;
+}
+
+int spc3d_ctx_destroy(spc3d_ctx *ctx)
+{
+    if (!live(ctx))
+        return fail(SPC3D_ERR_INVALID_ARG, "context is NULL or destroyed");
+    (void)hipSetDevice(ctx->device);
+    (void)hipStreamSynchronize(ctx->stream);
+    for (int i = 0; i < kTimerSlots; ++i)
+        if (ctx->timers[i])
+            (void)hipEventDestroy(ctx->timers[i]);
+    (void)hipStreamDestroy(ctx->stream);
+    ctx->magic = 0;
+    delete ctx;
+    return SPC3D_OK;
+}
+
+int spc3d_ctx_sync(spc3d_ctx *ctx)
+{
+    if (!live(ctx))
+        return fail(SPC3D_ERR_INVALID_ARG, "context is NULL or destroyed");
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    return SPC3D_OK;
+}
+
+int spc3d_ctx_stream(spc3d_ctx *ctx, void **hip_stream)
+{
+    if (!live(ctx) || !hip_stream)
+        return fail(SPC3D_ERR_INVALID_ARG, "context or out pointer is NULL");
+    *hip_stream = (void *)ctx->stream;
+    return SPC3D_OK;
+}
+
+int spc3d_timer_mark(spc3d_ctx *ctx, int slot)
+{
+    if (!live(ctx))
+        return fail(SPC3D_ERR_INVALID_ARG, "context is NULL or destroyed");
+    if (slot < 0 || slot >= kTimerSlots)
+        return fail(SPC3D_ERR_INVALID_ARG, "timer slot out of range");
+    if (!ctx->timers[slot])
+        HIP_TRY(hipEventCreate(&ctx->timers[slot]));
+    HIP_TRY(hipEventRecord(ctx->timers[slot], ctx->stream));
+    ctx->timer_set[slot] = true;
+    return SPC3D_OK;
+}
+
+int spc3d_timer_elapsed_ms(spc3d_ctx *ctx, int start, int stop, float *ms)
+{
+    if (!live(ctx) || !ms)
+        return fail(SPC3D_ERR_INVALID_ARG, "context or ms is NULL");
+    if (start < 0 || start >= kTimerSlots || stop < 0 || stop >= kTimerSlots ||
+        !ctx->timer_set[start] || !ctx->timer_set[stop])
+        return fail(SPC3D_ERR_INVALID_ARG, "timer slot not marked");
+    HIP_TRY(hipEventSynchronize(ctx->timers[stop]));
+    HIP_TRY(hipEventElapsedTime(ms, ctx->timers[start], ctx->timers[stop]));
+    return SPC3D_OK;
+}
+
+/* ---- panels -------------------------------------------------------------- */
+int spc3d_panel_create(spc3d_ctx *ctx, int dtype, uint32_t m, uint32_t n, spc3d_panel **out)
+{
+    if (!out)
+        return fail(SPC3D_ERR_INVALID_ARG, "out is NULL");
+    *out = nullptr;
+    if (!live(ctx))
+        return fail(SPC3D_ERR_INVALID_ARG, "context is NULL or destroyed");
+    if (!dtype_ok(dtype))
+        return fail(SPC3D_ERR_INVALID_ARG, "unknown dtype");
+    int rc = use_device(ctx);
+    if (rc)
+        return rc;
+    spc3d_panel *p = new (std::nothrow) spc3d_panel();
+    if (!p)
+        return fail(SPC3D_ERR_ALLOC, "host allocation failed");
+    p->ctx = ctx;
+    p->dtype = dtype;
+    p->m = m;
+    p->n = n;
+    rc = dev_alloc_bytes(&p->dev, (size_t)m * n * elem_size(dtype));
+    if (rc) {
+        delete p;
+        return rc;
+    }
+    p->magic = kMagicPanel;
+    *out = p;
+    return SPC3D_OK;
+}
+
+int spc3d_panel_destroy(spc3d_panel *p)
+{
+    if (!live(p))
+        return fail(SPC3D_ERR_INVALID_ARG, "panel is NULL or destroyed");
+    (void)hipSetDevice(p->ctx->device);
+    (void)hipStreamSynchronize(p->ctx->stream);
+    if (p->dev)
+        (void)hipFree(p->dev);
+    p->magic = 0;
+    delete p;
+    return SPC3D_OK;
+}
+
+int spc3d_panel_upload(spc3d_panel *p, const void *host)
+{
+    if (!live(p))
+        return fail(SPC3D_ERR_INVALID_ARG, "panel is NULL or destroyed");
+    const size_t bytes = (size_t)p->m * p->n * elem_size(p->dtype);
+    if (bytes && !host)
+        return fail(SPC3D_ERR_INVALID_ARG, "host pointer is NULL");
+    int rc = use_device(p->ctx);
+    return rc ? rc : copy_h2d(p->ctx, p->dev, host, bytes);
+}
+
+int spc3d_panel_download(spc3d_panel *p, void *host)
+{
+    if (!live(p))
+        return fail(SPC3D_ERR_INVALID_ARG, "panel is NULL or destroyed");
+    const size_t bytes = (size_t)p->m * p->n * elem_size(p->dtype);
+    if (bytes && !host)
+        return fail(SPC3D_ERR_INVALID_ARG, "host pointer is NULL");
+    int rc = use_device(p->ctx);
+    return rc ? rc : copy_d2h(p->ctx, host, p->dev, bytes);
+}
+
+int spc3d_panel_fill(spc3d_panel *p, double value)
+{
+    if (!live(p))
+        return fail(SPC3D_ERR_INVALID_ARG, "panel is NULL or destroyed");
+    int rc = use_device(p->ctx);
+    if (rc)
+        return rc;
+    HIP_TRY(launch_fill(p->dtype, p->dev, (uint64_t)p->m * p->n, value, p->ctx->stream));
+    return SPC3D_OK;
+}
+
+int spc3d_panel_device_ptr(spc3d_panel *p, void **dev)
+{
+    if (!live(p) || !dev)
+        return fail(SPC3D_ERR_INVALID_ARG, "panel or out pointer is NULL");
+    *dev = p->dev;
+    return SPC3D_OK;
+}
+
+int spc3d_panel_shape(spc3d_panel *p, uint32_t *m, uint32_t *n, int *dtype)
+{
+    if (!live(p))
+        return fail(SPC3D_ERR_INVALID_ARG, "panel is NULL or destroyed");
+    if (m) *m = p->m;
+    if (n) *n = p->n;
+    if (dtype) *dtype = p->dtype;
+    return SPC3D_OK;
+}
+
+/* ---- value vectors ------------------------------------------------------- */
+int spc3d_vals_create(spc3d_ctx *ctx, int dtype, uint64_t n, spc3d_vals **out)
+{
+    if (!out)
+        return fail(SPC3D_ERR_INVALID_ARG, "out is NULL");
+    *out = nullptr;
+    if (!live(ctx))
+        return fail(SPC3D_ERR_INVALID_ARG, "context is NULL or destroyed");
+    if (!dtype_ok(dtype))
+        return fail(SPC3D_ERR_INVALID_ARG, "unknown dtype");
+    if (n >= (1ull << 32))
+        return fail(SPC3D_ERR_TOO_LARGE, "value vector longer than 2^32 - 1");
+    int rc = use_device(ctx);
+    if (rc)
+        return rc;
+    spc3d_vals *v = new (std::nothrow) spc3d_vals();
+    if (!v)
+        return fail(SPC3D_ERR_ALLOC, "host allocation failed");
+    v->ctx = ctx;
+    v->dtype = dtype;
+    v->n = n;
+    rc = dev_alloc_bytes(&v->dev, (size_t)n * elem_size(dtype));
+    if (rc) {
+        delete v;
+        return rc;
+    }
+    v->magic = kMagicVals;
+    *out = v;
+    return SPC3D_OK;
+}
+
+int spc3d_vals_destroy(spc3d_vals *v)
+{
+    if (!live(v))
+        return fail(SPC3D_ERR_INVALID_ARG, "value vector is NULL or destroyed");
+    (void)hipSetDevice(v->ctx->device);
+    (void)hipStreamSynchronize(v->ctx->stream);
+    if (v->dev)
+        (void)hipFree(v->dev);
+    v->magic = 0;
+    delete v;
+    return SPC3D_OK;
+}
+
+int spc3d_vals_upload(spc3d_vals *v, const void *host)
+{
+    if (!live(v))
+        return fail(SPC3D_ERR_INVALID_ARG, "value vector is NULL or destroyed");
+    if (v->n && !host)
+        return fail(SPC3D_ERR_INVALID_ARG, "host pointer is NULL");
+    int rc = use_device(v->ctx);
+    return rc ? rc : copy_h2d(v->ctx, v->dev, host, (size_t)v->n * elem_size(v->dtype));
+}
+
+int spc3d_vals_download(spc3d_vals *v, void *host)
+{
+    if (!live(v))
+        return fail(SPC3D_ERR_INVALID_ARG, "value vector is NULL or destroyed");
+    if (v->n && !host)
+        return fail(SPC3D_ERR_INVALID_ARG, "host pointer is NULL");
+    int rc = use_device(v->ctx);
+    return rc ? rc : copy_d2h(v->ctx, host, v->dev, (size_t)v->n * elem_size(v->dtype));
+}
+
+int spc3d_vals_fill(spc3d_vals *v, double value)
+{
+    if (!live(v))
+        return fail(SPC3D_ERR_INVALID_ARG, "value vector is NULL or destroyed");
+    int rc = use_device(v->ctx);
+    if (rc)
+        return rc;
+    HIP_TRY(launch_fill(v->dtype, v->dev, v->n, value, v->ctx->stream));
+    return SPC3D_OK;
+}
+
+int spc3d_vals_device_ptr(spc3d_vals *v, void **dev)
+{
+    if (!live(v) || !dev)
+        return fail(SPC3D_ERR_INVALID_ARG, "value vector or out pointer is NULL");
+    *dev = v->dev;
+    return SPC3D_OK;
+}
+
+/* ---- plan ---------------------------------------------------------------- */
+int spc3d_coo_validate(uint32_t nrows, uint32_t ncols, uint64_t nnz, const uint32_t *ii,
+                       const uint32_t *jj)
+{
+    std::string err;
+    int rc = validate_coo(nrows, ncols, nnz, ii, jj, err);
+    return rc == SPC3D_OK ? rc : fail(rc, err);
+}
+
+static void fill_info(spc3d_plan_info &info, const HostPlan &H)
+{
+    info.nrows = H.nrows;
+    info.ncols = H.ncols;
+    info.nnz = H.nnz;
+    info.rows_touched = H.rows_touched;
+    info.cols_touched = H.cols_touched;
+    info.nsegments = (uint32_t)H.segs.size();
+    info.nsplit_rows = (uint32_t)H.splits.size();
+    info.npartial_slots = H.nslots;
+    info.max_row_nnz = H.max_row_nnz;
+    info.seg_max = H.seg_max;
+    info.order_is_identity = H.identity ? 1 : 0;
+}
+
+int spc3d_plan_build_host(uint32_t nrows, uint32_t ncols, uint64_t nnz, const uint32_t *ii,
+                          const uint32_t *jj, uint32_t seg_max, spc3d_plan_info *info,
+                          uint32_t *col, uint32_t *perm, uint32_t *segs, uint32_t seg_cap,
+                          uint32_t *splits, uint32_t split_cap)
+{
+    if (!info)
+        return fail(SPC3D_ERR_INVALID_ARG, "info is NULL");
+    HostPlan H;
+    std::string err;
+    int rc = build_host_plan(nrows, ncols, nnz, ii, jj, seg_max, H, err);
+    if (rc != SPC3D_OK)
+        return fail(rc, err);
+    fill_info(*info, H);
+    if ((segs && seg_cap < H.segs.size()) || (splits && split_cap < H.splits.size()))
+        return fail(SPC3D_ERR_SIZE_MISMATCH, "output capacity is smaller than the plan");
+    if (col && nnz)
+        std::memcpy(col, H.col.data(), (size_t)nnz * sizeof(uint32_t));
+    if (perm && nnz)
+        std::memcpy(perm, H.perm.data(), (size_t)nnz * sizeof(uint32_t));
+    if (segs && !H.segs.empty())
+        std::memcpy(segs, H.segs.data(), H.segs.size() * sizeof(Seg));
+    if (splits)
+        for (size_t i = 0; i < H.splits.size(); ++i) {
+            splits[3 * i + 0] = H.splits[i].row;
+            splits[3 * i + 1] = H.splits[i].first_slot;
+            splits[3 * i + 2] = H.splits[i].nslots;
+        }
+    return SPC3D_OK;
+}
+
+int spc3d_plan_create_ex(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t ncols, uint64_t nnz,
+                         const uint32_t *ii, const uint32_t *jj, const void *vv, uint32_t seg_max,
+                         spc3d_plan **out)
+{
+    if (!out)
+        return fail(SPC3D_ERR_INVALID_ARG, "out is NULL");
+    *out = nullptr;
+    if (!dtype_ok(dtype))
+        return fail(SPC3D_ERR_INVALID_ARG, "unknown dtype");
+    // The pattern is checked before the device is touched, so that a bad
+    // index is reported as such on a machine without a GPU as well.
+    HostPlan H;
+    std::string err;
+    int rc = build_host_plan(nrows, ncols, nnz, ii, jj, seg_max, H, err);
+    if (rc != SPC3D_OK)
+        return fail(rc, err);
+    if (!live(ctx))
+        return fail(SPC3D_ERR_INVALID_ARG, "context is NULL or destroyed");
+    rc = use_device(ctx);
+    if (rc)
+        return rc;
+
+    spc3d_plan *p = new (std::nothrow) spc3d_plan();
+    if (!p)
+        return fail(SPC3D_ERR_ALLOC, "host allocation failed");
+    p->ctx = ctx;
+    p->dtype = dtype;
+    fill_info(p->info, H);
+
+    rc = dev_alloc(&p->segs, H.segs.size());
+    if (!rc) rc = dev_alloc(&p->col, (size_t)nnz);
+    if (!rc && !H.identity) rc = dev_alloc(&p->perm, (size_t)nnz);
+    if (!rc) rc = dev_alloc_bytes(&p->sval, (size_t)nnz * elem_size(dtype));
+    if (!rc) rc = dev_alloc(&p->splits, H.splits.size());
+    if (!rc) rc = copy_h2d(ctx, p->segs, H.segs.data(), H.segs.size() * sizeof(Seg));
+    if (!rc) rc = copy_h2d(ctx, p->col, H.col.data(), (size_t)nnz * sizeof(uint32_t));
+    if (!rc && !H.identity)
+        rc = copy_h2d(ctx, p->perm, H.perm.data(), (size_t)nnz * sizeof(uint32_t));
+    if (!rc) rc = copy_h2d(ctx, p->splits, H.splits.data(), H.splits.size() * sizeof(SplitRow));
+    if (rc) {
+        plan_free_device(p);
+        delete p;
+        return rc;
+    }
+    p->magic = kMagicPlan;
+    if (vv) {
+        rc = spc3d_plan_set_values(p, vv);
+        if (rc) {
+            std::string keep = g_err;
+            spc3d_plan_destroy(p);
+            return fail(rc, keep);
+        }
+    }
+    *out = p;
+    return SPC3D_OK;
+}
+
+int spc3d_plan_create(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t ncols, uint64_t nnz,
+                      const uint32_t *ii, const uint32_t *jj, const void *vv, spc3d_plan **out)
+{
+    uint32_t seg_max = 0;
+    if (const char *s = std::getenv("SPC3D_SEG_MAX")) {
+        const long v = std::atol(s);
+        if (v > 0 && v <= 65536)
+            seg_max = (uint32_t)v;
+    }
+    return spc3d_plan_create_ex(ctx, dtype, nrows, ncols, nnz, ii, jj, vv, seg_max, out);
+}
+
+int spc3d_plan_destroy(spc3d_plan *plan)
+{
+    if (!live(plan))
+        return fail(SPC3D_ERR_INVALID_ARG, "plan is NULL or destroyed");
+    (void)hipSetDevice(plan->ctx->device);
+    (void)hipStreamSynchronize(plan->ctx->stream);
+    plan_free_device(plan);
+    plan->magic = 0;
+    delete plan;
+    return SPC3D_OK;
+}
+
+int spc3d_plan_set_values(spc3d_plan *plan, const void *vv_host)
+{
+    if (!live(plan))
+        return fail(SPC3D_ERR_INVALID_ARG, "plan is NULL or destroyed");
+    const uint64_t nnz = plan->info.nnz;
+    if (nnz && !vv_host)
+        return fail(SPC3D_ERR_INVALID_ARG, "vv is NULL");
+    int rc = use_device(plan->ctx);
+    if (rc)
+        return rc;
+    const size_t bytes = (size_t)nnz * elem_size(plan->dtype);
+    if (!plan->perm) {
+        rc = copy_h2d(plan->ctx, plan->sval, vv_host, bytes);
+    } else {
+        void *tmp = nullptr;
+        rc = dev_alloc_bytes(&tmp, bytes);
+        if (rc)
+            return rc;
+        rc = copy_h2d(plan->ctx, tmp, vv_host, bytes);
+        if (!rc) {
+            hipError_t e = launch_gather_vals(plan->dtype, tmp, plan->perm, plan->sval, nnz,
+                                              plan->ctx->stream);
+            if (e == hipSuccess)
+                e = hipStreamSynchronize(plan->ctx->stream);
+            if (e != hipSuccess)
+                rc = fail_hip(e, "gather of sparse values");
+        }
+        (void)hipFree(tmp);
+    }
+    if (!rc)
+        plan->has_values = true;
+    return rc;
+}
+
+int spc3d_plan_set_values_device(spc3d_plan *plan, const spc3d_vals *vv)
+{
+    if (!live(plan) || !live(vv))
+        return fail(SPC3D_ERR_INVALID_ARG, "plan or value vector is NULL or destroyed");
+    if (vv->dtype != plan->dtype || vv->n < plan->info.nnz || vv->ctx != plan->ctx)
+        return fail(SPC3D_ERR_SIZE_MISMATCH,
+                    "value vector dtype / length / context does not fit the plan");
+    int rc = use_device(plan->ctx);
+    if (rc)
+        return rc;
+    HIP_TRY(launch_gather_vals(plan->dtype, vv->dev, plan->perm, plan->sval, plan->info.nnz,
+                               plan->ctx->stream));
+    plan->has_values = true;
+    return SPC3D_OK;
+}
+
+int spc3d_plan_get_info(const spc3d_plan *plan, spc3d_plan_info *info)
+{
+    if (!live(plan) || !info)
+        return fail(SPC3D_ERR_INVALID_ARG, "plan or info is NULL");
+    *info = plan->info;
+    return SPC3D_OK;
+}
+
+/* ---- hot path ------------------------------------------------------------ */
+int spc3d_sddmm(spc3d_ctx *ctx, spc3d_plan *S, const spc3d_panel *A, const spc3d_panel *B,
+                spc3d_vals *C)
+{
+    if (!live(ctx) || !live(S) || !live(A) || !live(B) || !live(C))
+        return fail(SPC3D_ERR_INVALID_ARG, "a handle is NULL or destroyed");
+    if (S->ctx != ctx || A->ctx != ctx || B->ctx != ctx || C->ctx != ctx)
+        return fail(SPC3D_ERR_INVALID_ARG, "operands belong to different contexts");
+    if (A->dtype != S->dtype || B->dtype != S->dtype || C->dtype != S->dtype)
+        return fail(SPC3D_ERR_SIZE_MISMATCH, "operand dtypes differ from the plan's");
+    const uint32_t K = A->n; // core_ops.cpp:6
+    if (B->n != K)
+        return fail(SPC3D_ERR_SIZE_MISMATCH, "A.n != B.n");
+    if (S->info.nnz == 0)
+        return SPC3D_OK;
+    if (A->m < S->info.nrows || B->m < S->info.ncols)
+        return fail(SPC3D_ERR_SIZE_MISMATCH, "panel has fewer rows than the pattern addresses");
+    if (C->n < S->info.nnz)
+        return fail(SPC3D_ERR_SIZE_MISMATCH, "C.vv is shorter than nnz");
+    if (!S->has_values)
+        return fail(SPC3D_ERR_INVALID_ARG, "plan has no values (spc3d_plan_set_values)");
+    if (K == 0) { // empty dot product: every result is 0 * S.vv = 0
+        int rc = use_device(ctx);
+        if (rc)
+            return rc;
+        HIP_TRY(launch_fill(C->dtype, C->dev, S->info.nnz, 0.0, ctx->stream));
+        return SPC3D_OK;
+    }
+    int rc = use_device(ctx);
+    if (rc)
+        return rc;
+    HIP_TRY(launch_sddmm(S->dtype, view_of(S), A->dev, B->dev, C->dev, K, ctx->stream));
+    return SPC3D_OK;
+}
+
+int spc3d_spmm(spc3d_ctx *ctx, spc3d_plan *Ap, const spc3d_panel *X, spc3d_panel *Y)
+{
+    if (!live(ctx) || !live(Ap) || !live(X) || !live(Y))
+        return fail(SPC3D_ERR_INVALID_ARG, "a handle is NULL or destroyed");
+    if (Ap->ctx != ctx || X->ctx != ctx || Y->ctx != ctx)
+        return fail(SPC3D_ERR_INVALID_ARG, "operands belong to different contexts");
+    if (X->dtype != Ap->dtype || Y->dtype != Ap->dtype)
+        return fail(SPC3D_ERR_SIZE_MISMATCH, "operand dtypes differ from the plan's");
+    const uint32_t K = X->n; // core_ops.cpp:25
+    if (Y->n != K)
+        return fail(SPC3D_ERR_SIZE_MISMATCH, "X.n != Y.n");
+    if (Ap->info.nnz == 0 || K == 0)
+        return SPC3D_OK;
+    if (X->m < Ap->info.ncols || Y->m < Ap->info.nrows)
+        return fail(SPC3D_ERR_SIZE_MISMATCH, "panel has fewer rows than the pattern addresses");
+    if (X->dev == Y->dev)
+        return fail(SPC3D_ERR_INVALID_ARG, "X and Y must not alias");
+    if (!Ap->has_values)
+        return fail(SPC3D_ERR_INVALID_ARG, "plan has no values (spc3d_plan_set_values)");
+    int rc = use_device(ctx);
+    if (rc)
+        return rc;
+    if (Ap->info.npartial_slots && Ap->partial_k < K) {
+        // Partial-sum rows of cut rows; sized on first use for this K.
+        HIP_TRY(hipStreamSynchronize(ctx->stream));
+        if (Ap->partial)
+            (void)hipFree(Ap->partial);
+        Ap->partial = nullptr;
+        Ap->partial_k = 0;
+        rc = dev_alloc_bytes(&Ap->partial,
+                             (size_t)Ap->info.npartial_slots * K * elem_size(Ap->dtype));
+        if (rc)
+            return rc;
+        Ap->partial_k = K;
+    }
+    HIP_TRY(launch_spmm(Ap->dtype, view_of(Ap), X->dev, Y->dev, K, ctx->stream));
+    return SPC3D_OK;
+}
+
+int spc3d_sddmm_host(spc3d_ctx *ctx, int dtype, uint32_t m, uint32_t n, uint32_t k, const void *A,
+                     const void *B, uint64_t nnz, const uint32_t *ii, const uint32_t *jj,
+                     const void *svv, void *cvv)
+{
+    if (nnz && (!svv || !cvv))
+        return fail(SPC3D_ERR_INVALID_ARG, "svv or cvv is NULL");
+    spc3d_plan *S = nullptr;
+    spc3d_panel *a = nullptr, *b = nullptr;
+    spc3d_vals *c = nullptr;
+    int rc = spc3d_plan_create(ctx, dtype, m, n, nnz, ii, jj, svv, &S);
+    if (!rc) rc = spc3d_panel_create(ctx, dtype, m, k, &a);
+    if (!rc) rc = spc3d_panel_create(ctx, dtype, n, k, &b);
+    if (!rc) rc = spc3d_vals_create(ctx, dtype, nnz, &c);
+    if (!rc) rc = spc3d_panel_upload(a, A);
+    if (!rc) rc = spc3d_panel_upload(b, B);
+    if (!rc) rc = spc3d_sddmm(ctx, S, a, b, c);
+    if (!rc) rc = spc3d_vals_download(c, cvv);
+    const std::string keep = g_err;
+    if (c) spc3d_vals_destroy(c);
+    if (b) spc3d_panel_destroy(b);
+    if (a) spc3d_panel_destroy(a);
+    if (S) spc3d_plan_destroy(S);
+    return rc ? fail(rc, keep) : SPC3D_OK;
+}
+
+int spc3d_spmm_host(spc3d_ctx *ctx, int dtype, uint32_t ncols, uint32_t nrows, uint32_t k,
+                    const void *X, uint64_t nnz, const uint32_t *ii, const uint32_t *jj,
+                    const void *avv, void *Y)
+{
+    if (nnz && !avv)
+        return fail(SPC3D_ERR_INVALID_ARG, "avv is NULL");
+    spc3d_plan *S = nullptr;
+    spc3d_panel *x = nullptr, *y = nullptr;
+    int rc = spc3d_plan_create(ctx, dtype, nrows, ncols, nnz, ii, jj, avv, &S);
+    if (!rc) rc = spc3d_panel_create(ctx, dtype, ncols, k, &x);
+    if (!rc) rc = spc3d_panel_create(ctx, dtype, nrows, k, &y);
+    if (!rc) rc = spc3d_panel_upload(x, X);
+    if (!rc) rc = spc3d_panel_upload(y, Y);
+    if (!rc) rc = spc3d_spmm(ctx, S, x, y);
+    if (!rc) rc = spc3d_panel_download(y, Y);
+    const std::string keep = g_err;
+    if (y) spc3d_panel_destroy(y);
+    if (x) spc3d_panel_destroy(x);
+    if (S) spc3d_plan_destroy(S);
+    return rc ? fail(rc, keep) : SPC3D_OK;
+}
+
+} // extern "C"

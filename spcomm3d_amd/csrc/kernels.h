@@ -1,0 +1,38 @@
+// Launch interface between the C ABI (api.cpp) and the gfx950 kernels (kernels.hip).
+#pragma once
+#include <hip/hip_runtime_api.h>
+
+#include <cstdint>
+
+#include "plan_host.h"
+
+namespace spc3d {
+
+// Device-side view of a plan; all pointers are device pointers.
+struct DevPlanView {
+    const Seg *segs = nullptr;
+    uint32_t nseg = 0;
+    const uint32_t *col = nullptr;    // [nnz] kernel order
+    const uint32_t *perm = nullptr;   // [nnz] kernel order -> caller's position; null if identity
+    const void *sval = nullptr;       // [nnz] values in kernel order
+    const SplitRow *splits = nullptr;
+    uint32_t nsplit = 0;
+    void *partial = nullptr;          // [nslots * K] partial sums of cut rows (SpMM)
+    uint64_t nnz = 0;
+};
+
+// dtype: 0 = float, 1 = double.  All launches are asynchronous on `stream`.
+hipError_t launch_sddmm(int dtype, const DevPlanView &P, const void *A, const void *B, void *C,
+                        uint32_t K, hipStream_t stream);
+hipError_t launch_spmm(int dtype, const DevPlanView &P, const void *X, void *Y, uint32_t K,
+                       hipStream_t stream);
+// out[p] = in[perm[p]] (perm == null: copy)
+hipError_t launch_gather_vals(int dtype, const void *in, const uint32_t *perm, void *out,
+                              uint64_t n, hipStream_t stream);
+hipError_t launch_fill(int dtype, void *p, uint64_t n, double value, hipStream_t stream);
+
+// Name of the kernel variant launch_sddmm / launch_spmm picks for (dtype, K);
+// for logs and profiles.
+const char *kernel_variant(int dtype, uint32_t K);
+
+} // namespace spc3d

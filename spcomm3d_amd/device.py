@@ -1,0 +1,307 @@
+"""Thin object layer over the C ABI: device-resident panels, value vectors and
+plans.  Every method is one C-ABI call; nothing is computed in Python."""
+from __future__ import annotations
+
+import ctypes
+
+import numpy as np
+
+from . import _capi as capi
+from ._capi import PlanInfo, check
+
+_DT = {np.dtype(np.float32): capi.F32, np.dtype(np.float64): capi.F64}
+_NP = {capi.F32: np.dtype(np.float32), capi.F64: np.dtype(np.float64)}
+
+
+def dtype_code(dtype) -> int:
+    if isinstance(dtype, str):
+        dtype = {"f32": np.float32, "f64": np.float64}.get(dtype, dtype)
+    if isinstance(dtype, int) and dtype in _NP:
+        return dtype
+    try:
+        return _DT[np.dtype(dtype)]
+    except (KeyError, TypeError):
+        raise TypeError(f"unsupported real type {dtype!r}: float32 or float64") from None
+
+
+def _vp(a: np.ndarray | None):
+    return None if a is None else a.ctypes.data_as(ctypes.c_void_p)
+
+
+def _as_idx(a, name: str) -> np.ndarray:
+    a = np.asarray(a)
+    if a.dtype != np.uint32:
+        if a.size and (a.min() < 0 or a.max() > 0xFFFFFFFF):
+            raise capi.BadIndexError(capi.ERR_BAD_INDEX, f"{name} does not fit uint32", "as_idx")
+        a = a.astype(np.uint32)
+    return np.ascontiguousarray(a)
+
+
+class Context:
+    """One device and one stream (``spc3d_ctx``)."""
+
+    def __init__(self, device: int = 0):
+        self._lib = capi.load()
+        h = ctypes.c_void_p()
+        check(self._lib.spc3d_ctx_create(device, ctypes.byref(h)), "spc3d_ctx_create")
+        self._h = h
+        self.device = device
+
+    def close(self):
+        if getattr(self, "_h", None):
+            self._lib.spc3d_ctx_destroy(self._h)
+            self._h = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def sync(self):
+        check(self._lib.spc3d_ctx_sync(self._h), "spc3d_ctx_sync")
+
+    def mark(self, slot: int):
+        check(self._lib.spc3d_timer_mark(self._h, slot), "spc3d_timer_mark")
+
+    def elapsed_ms(self, start: int, stop: int) -> float:
+        ms = ctypes.c_float()
+        check(self._lib.spc3d_timer_elapsed_ms(self._h, start, stop, ctypes.byref(ms)),
+              "spc3d_timer_elapsed_ms")
+        return float(ms.value)
+
+    # -- factories ---------------------------------------------------------
+    def panel(self, m: int, n: int, dtype) -> "Panel":
+        return Panel(self, m, n, dtype)
+
+    def panel_from(self, host: np.ndarray) -> "Panel":
+        host = np.ascontiguousarray(host)
+        if host.ndim != 2:
+            raise ValueError("a panel is a 2-D row-major array")
+        p = Panel(self, host.shape[0], host.shape[1], host.dtype)
+        p.upload(host)
+        return p
+
+    def vals(self, n: int, dtype) -> "Vals":
+        return Vals(self, n, dtype)
+
+    def plan(self, nrows, ncols, ii, jj, vv=None, dtype=None, seg_max: int | None = None) -> "Plan":
+        return Plan(self, nrows, ncols, ii, jj, vv, dtype, seg_max)
+
+    # -- hot path ----------------------------------------------------------
+    def sddmm(self, S: "Plan", A: "Panel", B: "Panel", C: "Vals"):
+        """C.vv[e] = S.vv[e] * <A[ii[e]], B[jj[e]]>  (src/core_ops.cpp:5-22); asynchronous."""
+        check(self._lib.spc3d_sddmm(self._h, S._h, A._h, B._h, C._h), "spc3d_sddmm")
+
+    def spmm(self, A: "Plan", X: "Panel", Y: "Panel"):
+        """Y[ii[e]] += A.vv[e] * X[jj[e]]  (src/core_ops.cpp:24-35); asynchronous."""
+        check(self._lib.spc3d_spmm(self._h, A._h, X._h, Y._h), "spc3d_spmm")
+
+    def sddmm_host(self, A: np.ndarray, B: np.ndarray, ii, jj, svv: np.ndarray) -> np.ndarray:
+        """One-shot SDDMM over host arrays (``spc3d_sddmm_host``); returns C.vv."""
+        A, B, svv = (np.ascontiguousarray(x) for x in (A, B, svv))
+        if A.ndim != 2 or B.ndim != 2 or A.dtype != B.dtype or A.dtype != svv.dtype:
+            raise ValueError("A, B must be 2-D and share svv's dtype")
+        if A.shape[1] != B.shape[1]:
+            raise capi.Spc3dError(capi.ERR_SIZE_MISMATCH, "A.n != B.n", "sddmm_host")
+        ii, jj = _as_idx(ii, "ii"), _as_idx(jj, "jj")
+        out = np.empty(ii.size, dtype=A.dtype)
+        check(self._lib.spc3d_sddmm_host(self._h, dtype_code(A.dtype), A.shape[0], B.shape[0],
+                                         A.shape[1], _vp(A), _vp(B), ii.size, _vp(ii), _vp(jj),
+                                         _vp(svv), _vp(out)), "spc3d_sddmm_host")
+        return out
+
+    def spmm_host(self, X: np.ndarray, ii, jj, avv: np.ndarray, Y: np.ndarray) -> None:
+        """One-shot SpMM over host arrays (``spc3d_spmm_host``); adds into Y in place."""
+        X, avv = np.ascontiguousarray(X), np.ascontiguousarray(avv)
+        if not (Y.flags.c_contiguous and Y.flags.writeable):
+            raise ValueError("Y must be a writable C-contiguous array")
+        if X.ndim != 2 or Y.ndim != 2 or X.dtype != Y.dtype or X.dtype != avv.dtype:
+            raise ValueError("X, Y must be 2-D and share avv's dtype")
+        if X.shape[1] != Y.shape[1]:
+            raise capi.Spc3dError(capi.ERR_SIZE_MISMATCH, "X.n != Y.n", "spmm_host")
+        ii, jj = _as_idx(ii, "ii"), _as_idx(jj, "jj")
+        check(self._lib.spc3d_spmm_host(self._h, dtype_code(X.dtype), X.shape[0], Y.shape[0],
+                                        X.shape[1], _vp(X), ii.size, _vp(ii), _vp(jj), _vp(avv),
+                                        _vp(Y)), "spc3d_spmm_host")
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class Panel:
+    """Device-resident ``denseMatrix::data`` (``src/basic.hpp:30-36``)."""
+
+    def __init__(self, ctx: Context, m: int, n: int, dtype):
+        self.ctx, self.m, self.n = ctx, int(m), int(n)
+        self.code = dtype_code(dtype)
+        self.dtype = _NP[self.code]
+        h = ctypes.c_void_p()
+        check(ctx._lib.spc3d_panel_create(ctx._h, self.code, self.m, self.n, ctypes.byref(h)),
+              "spc3d_panel_create")
+        self._h = h
+
+    def upload(self, host: np.ndarray):
+        host = np.ascontiguousarray(host)
+        if host.dtype != self.dtype or host.size != self.m * self.n:
+            raise ValueError("host array does not match the panel's dtype / size")
+        check(self.ctx._lib.spc3d_panel_upload(self._h, _vp(host)), "spc3d_panel_upload")
+
+    def download(self) -> np.ndarray:
+        out = np.empty((self.m, self.n), dtype=self.dtype)
+        check(self.ctx._lib.spc3d_panel_download(self._h, _vp(out)), "spc3d_panel_download")
+        return out
+
+    def fill(self, value: float):
+        check(self.ctx._lib.spc3d_panel_fill(self._h, float(value)), "spc3d_panel_fill")
+
+    def device_ptr(self) -> int:
+        p = ctypes.c_void_p()
+        check(self.ctx._lib.spc3d_panel_device_ptr(self._h, ctypes.byref(p)),
+              "spc3d_panel_device_ptr")
+        return p.value or 0
+
+    def close(self):
+        if getattr(self, "_h", None) and getattr(self.ctx, "_h", None):
+            self.ctx._lib.spc3d_panel_destroy(self._h)
+        self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class Vals:
+    """Device-resident ``cooMat::vv`` (``src/SparseMatrix.hpp:36``)."""
+
+    def __init__(self, ctx: Context, n: int, dtype):
+        self.ctx, self.n = ctx, int(n)
+        self.code = dtype_code(dtype)
+        self.dtype = _NP[self.code]
+        h = ctypes.c_void_p()
+        check(ctx._lib.spc3d_vals_create(ctx._h, self.code, self.n, ctypes.byref(h)),
+              "spc3d_vals_create")
+        self._h = h
+
+    def upload(self, host: np.ndarray):
+        host = np.ascontiguousarray(host)
+        if host.dtype != self.dtype or host.size != self.n:
+            raise ValueError("host array does not match the vector's dtype / length")
+        check(self.ctx._lib.spc3d_vals_upload(self._h, _vp(host)), "spc3d_vals_upload")
+
+    def download(self) -> np.ndarray:
+        out = np.empty(self.n, dtype=self.dtype)
+        check(self.ctx._lib.spc3d_vals_download(self._h, _vp(out)), "spc3d_vals_download")
+        return out
+
+    def fill(self, value: float):
+        check(self.ctx._lib.spc3d_vals_fill(self._h, float(value)), "spc3d_vals_fill")
+
+    def close(self):
+        if getattr(self, "_h", None) and getattr(self.ctx, "_h", None):
+            self.ctx._lib.spc3d_vals_destroy(self._h)
+        self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class Plan:
+    """Device-resident sparse operand: the pattern of a ``cooMat`` in kernel
+    order plus its values (``spc3d_plan``)."""
+
+    def __init__(self, ctx: Context, nrows, ncols, ii, jj, vv=None, dtype=None,
+                 seg_max: int | None = None):
+        ii = _as_idx(ii, "ii")
+        jj = _as_idx(jj, "jj")
+        if ii.shape != jj.shape or ii.ndim != 1:
+            raise ValueError("ii and jj must be 1-D arrays of the same length")
+        if vv is not None:
+            vv = np.ascontiguousarray(vv)
+            if vv.shape != ii.shape:
+                raise ValueError("vv must have one value per entry")
+            dtype = vv.dtype if dtype is None else dtype
+        if dtype is None:
+            raise ValueError("dtype is required when vv is not given")
+        self.ctx = ctx
+        self.code = dtype_code(dtype)
+        self.dtype = _NP[self.code]
+        if vv is not None and vv.dtype != self.dtype:
+            raise ValueError("vv dtype differs from the plan dtype")
+        h = ctypes.c_void_p()
+        lib = ctx._lib
+        if seg_max is None:
+            rc = lib.spc3d_plan_create(ctx._h, self.code, int(nrows), int(ncols), ii.size, _vp(ii),
+                                       _vp(jj), _vp(vv), ctypes.byref(h))
+        else:
+            rc = lib.spc3d_plan_create_ex(ctx._h, self.code, int(nrows), int(ncols), ii.size,
+                                          _vp(ii), _vp(jj), _vp(vv), int(seg_max), ctypes.byref(h))
+        check(rc, "spc3d_plan_create")
+        self._h = h
+        self.nnz = int(ii.size)
+
+    def set_values(self, vv: np.ndarray):
+        vv = np.ascontiguousarray(vv)
+        if vv.dtype != self.dtype or vv.size != self.nnz:
+            raise ValueError("vv does not match the plan's dtype / nnz")
+        check(self.ctx._lib.spc3d_plan_set_values(self._h, _vp(vv)), "spc3d_plan_set_values")
+
+    def set_values_device(self, vv: Vals):
+        check(self.ctx._lib.spc3d_plan_set_values_device(self._h, vv._h),
+              "spc3d_plan_set_values_device")
+
+    @property
+    def info(self) -> PlanInfo:
+        info = PlanInfo()
+        check(self.ctx._lib.spc3d_plan_get_info(self._h, ctypes.byref(info)), "spc3d_plan_get_info")
+        return info
+
+    def close(self):
+        if getattr(self, "_h", None) and getattr(self.ctx, "_h", None):
+            self.ctx._lib.spc3d_plan_destroy(self._h)
+        self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def coo_validate(nrows: int, ncols: int, ii, jj) -> None:
+    """Host-only bounds check of a pattern; raises :class:`BadIndexError`."""
+    ii = _as_idx(ii, "ii")
+    jj = _as_idx(jj, "jj")
+    check(capi.load().spc3d_coo_validate(int(nrows), int(ncols), ii.size, _vp(ii), _vp(jj)),
+          "spc3d_coo_validate")
+
+
+def plan_build_host(nrows: int, ncols: int, ii, jj, seg_max: int = 0) -> dict:
+    """Host-only view of the kernel-order form of a pattern
+    (``spc3d_plan_build_host``): needs no GPU.  Returns ``info``, ``col``,
+    ``perm``, ``segs`` (``[nseg, 4]``: row, start, len, slot) and ``splits``
+    (``[nsplit, 3]``: row, first_slot, nslots)."""
+    lib = capi.load()
+    ii = _as_idx(ii, "ii")
+    jj = _as_idx(jj, "jj")
+    info = PlanInfo()
+    check(lib.spc3d_plan_build_host(int(nrows), int(ncols), ii.size, _vp(ii), _vp(jj),
+                                    int(seg_max), ctypes.byref(info), None, None, None, 0, None, 0),
+          "spc3d_plan_build_host")
+    col = np.empty(ii.size, dtype=np.uint32)
+    perm = np.empty(ii.size, dtype=np.uint32)
+    segs = np.empty((info.nsegments, 4), dtype=np.uint32)
+    splits = np.empty((info.nsplit_rows, 3), dtype=np.uint32)
+    check(lib.spc3d_plan_build_host(int(nrows), int(ncols), ii.size, _vp(ii), _vp(jj),
+                                    int(seg_max), ctypes.byref(info), _vp(col), _vp(perm),
+                                    _vp(segs), info.nsegments, _vp(splits), info.nsplit_rows),
+          "spc3d_plan_build_host")
+    return {"info": info, "col": col, "perm": perm, "segs": segs, "splits": splits}

@@ -1,0 +1,290 @@
+"""GPU parity: the HIP path, called through the C ABI, against the CPU oracle on
+the same seeded inputs.
+
+Bar: sparsity pattern / output position exact; values within 1e-12 (fp64) or
+1e-5 (fp32), relative to max(|reference value|, sum of |terms|) per output
+element (U[-1,1] dot products cancel towards zero, so the plain ratio to the
+value is meaningless there).  fp32 is additionally held to 1e-5 against the
+fp64 oracle on the same inputs.
+"""
+import numpy as np
+import pytest
+
+from spcomm3d_amd import _capi as capi
+from spcomm3d_amd import workloads as W
+from tests import _oracle as oracle
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = np.load(oracle.os.path.join(oracle.ROOT, "tests", "golden", "core_ops_golden.npz"),
+                 allow_pickle=False)
+DTYPES = [np.float32, np.float64]
+
+
+def tol_of(dtype):
+    return oracle.TOL[np.dtype(dtype)]
+
+
+def rand_case(seed, m, n, k, nnz, dtype, hub=None):
+    rng = np.random.default_rng(seed)
+    ii = rng.integers(0, m, nnz).astype(np.uint32)
+    jj = rng.integers(0, n, nnz).astype(np.uint32)
+    if hub:
+        ii[:hub] = m // 2
+    if nnz > 8:
+        ii[-3:], jj[-3:] = ii[:3], jj[:3]  # exact duplicates
+    o = rng.permutation(nnz)
+    ii, jj = np.ascontiguousarray(ii[o]), np.ascontiguousarray(jj[o])
+    vv = rng.random(nnz).astype(dtype)
+    A = rng.uniform(-1, 1, (m, k)).astype(dtype)
+    B = rng.uniform(-1, 1, (n, k)).astype(dtype)
+    Y0 = rng.uniform(-1, 1, (m, k)).astype(dtype)
+    return ii, jj, vv, A, B, Y0
+
+
+def gpu_sddmm(ctx, m, n, ii, jj, vv, A, B, seg_max=None, prefill=None):
+    S = ctx.plan(m, n, ii, jj, vv, seg_max=seg_max)
+    dA, dB = ctx.panel_from(A), ctx.panel_from(B)
+    dC = ctx.vals(ii.size, A.dtype)
+    if prefill is not None:
+        dC.fill(prefill)
+    ctx.sddmm(S, dA, dB, dC)
+    out = dC.download()
+    for h in (S, dA, dB, dC):
+        h.close()
+    return out
+
+
+def gpu_spmm(ctx, m, n, ii, jj, vv, X, Y0, seg_max=None, times=1):
+    S = ctx.plan(m, n, ii, jj, vv, seg_max=seg_max)
+    dX, dY = ctx.panel_from(X), ctx.panel_from(Y0)
+    for _ in range(times):
+        ctx.spmm(S, dX, dY)
+    out = dY.download()
+    for h in (S, dX, dY):
+        h.close()
+    return out
+
+
+def check_sddmm(A, B, ii, jj, vv, got):
+    assert got.dtype == A.dtype and got.shape == (ii.size,)
+    tol = tol_of(A.dtype)
+    err = oracle.sddmm_rel_err(A, B, ii, jj, vv, got)
+    assert err <= tol, f"sddmm rel err {err:.3e} > {tol}"
+    if A.dtype == np.float32:
+        assert oracle.sddmm_rel_err_exact(A, B, ii, jj, vv, got) <= tol
+
+
+def check_spmm(X, ii, jj, vv, Y0, got):
+    assert got.dtype == X.dtype and got.shape == Y0.shape
+    tol = tol_of(X.dtype)
+    err = oracle.spmm_rel_err(X, ii, jj, vv, Y0, got)
+    assert err <= tol, f"spmm rel err {err:.3e} > {tol}"
+    if X.dtype == np.float32:
+        assert oracle.spmm_rel_err_exact(X, ii, jj, vv, Y0, got) <= tol
+
+
+# ---- the reference's own outputs (golden vectors made from its compiled code) -
+@pytest.mark.parametrize("name", ["small", "k64", "hub", "k1"])
+def test_golden_reference_vectors_fp64(ctx, name):
+    g = {k: GOLDEN[f"{name}.{k}"] for k in ("ii", "jj", "vv", "A", "B", "Y0", "C", "Y")}
+    m, n = g["A"].shape[0], g["B"].shape[0]
+    C = gpu_sddmm(ctx, m, n, g["ii"], g["jj"], g["vv"], g["A"], g["B"], prefill=123.0)
+    scale = oracle.sddmm_scale(g["A"], g["B"], g["ii"], g["jj"], g["vv"])
+    assert oracle.rel_err(C, g["C"], scale) <= 1e-12
+    Y = gpu_spmm(ctx, m, n, g["ii"], g["jj"], g["vv"], g["B"], g["Y0"])
+    scale = oracle.spmm_scale(g["B"], g["ii"], g["jj"], g["vv"], g["Y0"])
+    assert oracle.rel_err(Y, g["Y"], scale) <= 1e-12
+
+
+def test_golden_numcheck_closed_form(ctx):
+    # miniapp/numCheckSeq.cpp:125-131
+    g = {k: GOLDEN[f"numcheck.{k}"] for k in ("ii", "jj", "vv", "A", "B", "C")}
+    C = gpu_sddmm(ctx, 6, 5, g["ii"], g["jj"], g["vv"], g["A"], g["B"])
+    np.testing.assert_allclose(C, g["C"], rtol=1e-13, atol=0)
+    assert abs(C.sum() - g["C"].sum()) < 1e-16
+
+
+# ---- K sweep: vector kernels (K*sizeof a multiple of 64 B) and the generic ones
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("k", [1, 3, 4, 8, 12, 16, 20, 32, 48, 64, 100, 128, 256, 512])
+def test_k_sweep_random_unsorted(ctx, dtype, k):
+    ii, jj, vv, A, B, Y0 = rand_case(100 + k, 300, 257, k, 6000, dtype, hub=700)
+    check_sddmm(A, B, ii, jj, vv, gpu_sddmm(ctx, 300, 257, ii, jj, vv, A, B, prefill=-5.0))
+    check_spmm(B, ii, jj, vv, Y0, gpu_spmm(ctx, 300, 257, ii, jj, vv, B, Y0))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("seg_max", [1, 3, 16, 17, 128, 1000])
+def test_segment_lengths_and_cut_rows(ctx, dtype, seg_max):
+    ii, jj, vv, A, B, Y0 = rand_case(7, 64, 500, 64, 5000, dtype, hub=2000)
+    check_sddmm(A, B, ii, jj, vv, gpu_sddmm(ctx, 64, 500, ii, jj, vv, A, B, seg_max=seg_max))
+    check_spmm(B, ii, jj, vv, Y0, gpu_spmm(ctx, 64, 500, ii, jj, vv, B, Y0, seg_max=seg_max))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nnz", [0, 1, 2, 15, 16, 17, 63, 65])
+def test_tiny_and_ragged(ctx, dtype, nnz):
+    ii, jj, vv, A, B, Y0 = rand_case(nnz, 5, 9, 64, nnz, dtype)
+    C = gpu_sddmm(ctx, 5, 9, ii, jj, vv, A, B)
+    Y = gpu_spmm(ctx, 5, 9, ii, jj, vv, B, Y0)
+    if nnz == 0:
+        assert C.size == 0 and np.array_equal(Y, Y0)
+        return
+    check_sddmm(A, B, ii, jj, vv, C)
+    check_spmm(B, ii, jj, vv, Y0, Y)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rectangular_empty_rows_untouched(ctx, dtype):
+    # only rows 3 and 40 of 100 have entries; every other Y row must come back bit-identical
+    rng = np.random.default_rng(5)
+    ii = np.concatenate([np.full(20, 3), np.full(300, 40)]).astype(np.uint32)
+    jj = rng.integers(0, 7, 320).astype(np.uint32)
+    vv = rng.random(320).astype(dtype)
+    X = rng.uniform(-1, 1, (7, 32)).astype(dtype)
+    Y0 = rng.uniform(-1, 1, (100, 32)).astype(dtype)
+    Y = gpu_spmm(ctx, 100, 7, ii, jj, vv, X, Y0)
+    untouched = np.setdiff1d(np.arange(100), [3, 40])
+    assert np.array_equal(Y[untouched], Y0[untouched])
+    check_spmm(X, ii, jj, vv, Y0, Y)
+
+
+# ---- semantics the reference fixes ----------------------------------------------
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_sddmm_overwrites_every_entry_in_callers_order(ctx, dtype):
+    ii, jj, vv, A, B, _ = rand_case(21, 40, 40, 16, 900, dtype)
+    C1 = gpu_sddmm(ctx, 40, 40, ii, jj, vv, A, B, prefill=np.nan)
+    assert np.all(np.isfinite(C1))
+    p = np.random.default_rng(2).permutation(ii.size)
+    C2 = gpu_sddmm(ctx, 40, 40, ii[p], jj[p], vv[p], A, B)
+    # per-entry results do not depend on where the entry sits in the stream
+    assert np.array_equal(C2, C1[p])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_spmm_accumulates_over_calls(ctx, dtype):
+    # miniapp/bench_spmm.cpp:185-186 never resets Y between its five calls
+    ii, jj, vv, _, X, Y0 = rand_case(22, 50, 60, 32, 2000, dtype, hub=300)
+    Y3 = gpu_spmm(ctx, 50, 60, ii, jj, vv, X, Y0, times=3)
+    ref = Y0
+    for _ in range(3):
+        ref = oracle.spmm(X, ii, jj, vv, ref)
+    scale = oracle.spmm_scale(X, ii, jj, 3 * vv.astype(np.float64), Y0)
+    assert oracle.rel_err(Y3, ref, scale) <= tol_of(dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_exact_cases(ctx, dtype):
+    # ones panels: C = K * S exactly (miniapp/bench_both.cpp:191-192); X = 1: row sums
+    ii, jj, vv, _, _, _ = rand_case(23, 30, 30, 64, 700, dtype)
+    one = np.ones((30, 64), dtype)
+    C = gpu_sddmm(ctx, 30, 30, ii, jj, vv, one, one)
+    assert np.array_equal(C, (64 * vv).astype(dtype))
+    eye = np.arange(30, dtype=np.uint32)
+    X = np.random.default_rng(3).uniform(-1, 1, (30, 64)).astype(dtype)
+    Y0 = np.random.default_rng(4).uniform(-1, 1, (30, 64)).astype(dtype)
+    Y = gpu_spmm(ctx, 30, 30, eye, eye, np.ones(30, dtype), X, Y0)
+    assert np.array_equal(Y, Y0 + X)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_runs_are_bitwise_reproducible(ctx, dtype):
+    ii, jj, vv, A, B, Y0 = rand_case(24, 64, 64, 64, 9000, dtype, hub=4000)
+    a = gpu_spmm(ctx, 64, 64, ii, jj, vv, B, Y0)
+    b = gpu_spmm(ctx, 64, 64, ii, jj, vv, B, Y0)
+    assert np.array_equal(a, b)
+    c = gpu_sddmm(ctx, 64, 64, ii, jj, vv, A, B)
+    d = gpu_sddmm(ctx, 64, 64, ii, jj, vv, A, B)
+    assert np.array_equal(c, d)
+
+
+# ---- the other entry points -------------------------------------------------------
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_one_shot_host_entry_points(ctx, dtype):
+    ii, jj, vv, A, B, Y0 = rand_case(31, 70, 90, 64, 3000, dtype, hub=500)
+    check_sddmm(A, B, ii, jj, vv, ctx.sddmm_host(A, B, ii, jj, vv))
+    Y = Y0.copy()
+    ctx.spmm_host(B, ii, jj, vv, Y)
+    check_spmm(B, ii, jj, vv, Y0, Y)
+
+
+def test_values_can_be_replaced_from_host_and_device(ctx):
+    ii, jj, vv, A, B, _ = rand_case(32, 40, 40, 32, 1500, np.float64)
+    S = ctx.plan(40, 40, ii, jj, dtype=np.float64)  # pattern only
+    dA, dB, dC = ctx.panel_from(A), ctx.panel_from(B), ctx.vals(1500, np.float64)
+    with pytest.raises(capi.Spc3dError):
+        ctx.sddmm(S, dA, dB, dC)  # no values yet
+    S.set_values(vv)
+    ctx.sddmm(S, dA, dB, dC)
+    check_sddmm(A, B, ii, jj, vv, dC.download())
+    v2 = (vv * 0.5 + 0.125)
+    dV = ctx.vals(1500, np.float64)
+    dV.upload(v2)
+    S.set_values_device(dV)
+    ctx.sddmm(S, dA, dB, dC)
+    check_sddmm(A, B, ii, jj, v2, dC.download())
+    # SDDMM output feeding the next SpMM as its values, all on the device
+    S.set_values_device(dC)
+    dY = ctx.panel_from(np.zeros((40, 32)))
+    ctx.spmm(S, dB, dY)
+    check_spmm(B, ii, jj, oracle.sddmm(A, B, ii, jj, v2), np.zeros((40, 32)), dY.download())
+
+
+def test_shape_and_dtype_mismatches_are_refused(ctx):
+    ii, jj, vv, A, B, Y0 = rand_case(33, 20, 30, 16, 200, np.float64)
+    S = ctx.plan(20, 30, ii, jj, vv)
+    dA, dB = ctx.panel_from(A), ctx.panel_from(B)
+    dC = ctx.vals(200, np.float64)
+    cases = [
+        lambda: ctx.sddmm(S, dA, ctx.panel_from(B[:, :8].copy()), dC),       # A.n != B.n
+        lambda: ctx.sddmm(S, ctx.panel_from(A[:10].copy()), dB, dC),         # A too short
+        lambda: ctx.sddmm(S, dA, dB, ctx.vals(199, np.float64)),             # C.vv too short
+        lambda: ctx.sddmm(S, dA, dB, ctx.vals(200, np.float32)),             # dtype
+        lambda: ctx.spmm(S, dB, ctx.panel_from(Y0[:, :8].copy())),           # X.n != Y.n
+        lambda: ctx.spmm(S, ctx.panel_from(B[:29].copy()), ctx.panel_from(Y0)),  # X too short
+        lambda: ctx.spmm(S, dB, dB),                                         # aliasing
+    ]
+    for c in cases:
+        with pytest.raises(capi.Spc3dError) as e:
+            c()
+        assert e.value.status in (capi.ERR_SIZE_MISMATCH, capi.ERR_INVALID_ARG)
+    with pytest.raises(IndexError):
+        ctx.plan(20, 29, ii, np.full_like(jj, 29), vv)
+
+
+# ---- the benchmark configurations at oracle-sized scale -----------------------------
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_config1_erdos_renyi_full(ctx, dtype):
+    w = W.erdos_renyi(16384, 16, 32)
+    A, B, vv = w.panel_A(dtype), w.panel_B(dtype), w.values(dtype)
+    C = gpu_sddmm(ctx, w.nrows, w.ncols, w.ii, w.jj, vv, A, B)
+    check_sddmm(A, B, w.ii, w.jj, vv, C)
+    Y0 = np.zeros_like(A)
+    Y = gpu_spmm(ctx, w.nrows, w.ncols, w.ii, w.jj, C, B, Y0)  # SDDMM then SpMM
+    check_spmm(B, w.ii, w.jj, C, Y0, Y)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("order", ["sorted", "shuffled"])
+def test_config2_rmat_scale16(ctx, dtype, order):
+    w = W.rmat(16, 16, 64)
+    if order == "shuffled":
+        w = w.shuffled()
+    A, B, Y0, vv = w.panel_A(dtype), w.panel_B(dtype), w.panel_Y0(dtype), w.values(dtype)
+    check_sddmm(A, B, w.ii, w.jj, vv, gpu_sddmm(ctx, w.nrows, w.ncols, w.ii, w.jj, vv, A, B))
+    check_spmm(B, w.ii, w.jj, vv, Y0, gpu_spmm(ctx, w.nrows, w.ncols, w.ii, w.jj, vv, B, Y0))
+
+
+def test_config4_stencil_256(ctx):
+    w = W.stencil5(256, 256, 32)
+    A, B, Y0, vv = (w.panel_A("f32"), w.panel_B("f32"), w.panel_Y0("f32"), w.values("f32"))
+    check_sddmm(A, B, w.ii, w.jj, vv, gpu_sddmm(ctx, w.nrows, w.ncols, w.ii, w.jj, vv, A, B))
+    check_spmm(B, w.ii, w.jj, vv, Y0, gpu_spmm(ctx, w.nrows, w.ncols, w.ii, w.jj, vv, B, Y0))
+
+
+def test_config5_hypergraph_small_k128(ctx):
+    w = W.hypergraph_zipf(20000, 5000, 128)
+    A, B, Y0, vv = (w.panel_A("f32"), w.panel_B("f32"), w.panel_Y0("f32"), w.values("f32"))
+    check_sddmm(A, B, w.ii, w.jj, vv, gpu_sddmm(ctx, w.nrows, w.ncols, w.ii, w.jj, vv, A, B))
+    check_spmm(B, w.ii, w.jj, vv, Y0, gpu_spmm(ctx, w.nrows, w.ncols, w.ii, w.jj, vv, B, Y0))
