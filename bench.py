@@ -1,0 +1,213 @@
+#!/usr/bin/env python3
+"""Benchmark of the local SDDMM + SpMM step on one MI355X.
+
+A step is one pass of the hot path over one resident workload: SDDMM
+(C = S .* (A B^T)) followed by SpMM (Y += S X), both through the C ABI, with
+every operand already in HBM when the timed region starts.  Default workload:
+R-MAT scale 20, edge factor 16, K = 64 (the configuration the metric is quoted
+on), in the reference's real type (fp64); the other real type is measured in
+the same run and reported under "also".
+
+Prints one JSON line.  `value` is (flops of both kernels) / (wall time per
+step).  `roofline` is the slower of the two kernels: strict-model bytes per
+launch over its mean launch time, measured with HIP events on the library's
+stream inside the timed region, against 8 TB/s.  `cpu_baseline` is the CPU
+oracle (a serial restatement of the reference's loops) timed on one host core
+on the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+METRIC = "SDDMM & SpMM GFLOP/s + % HBM roofline on 1 MI355X, RMAT-20 K=64"
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def ensure_built():
+    need = ["spcomm3d_amd/lib/libspcomm3d_hip.so", "spcomm3d_amd/gen/libspc3d_gen.so"]
+    if not all(os.path.exists(os.path.join(ROOT, p)) for p in need):
+        import __graft_entry__
+
+        __graft_entry__.build()
+
+
+def run_gpu(w, dtype, steps, warmup, seg_max=None, max_timed=1300):
+    """Times `steps` SDDMM+SpMM passes on resident operands; returns a dict."""
+    from spcomm3d_amd import device, roofline
+    from spcomm3d_amd import workloads as W
+
+    wbytes = np.dtype(W.np_dtype(dtype)).itemsize
+    A, B, Y0, vv = w.panel_A(dtype), w.panel_B(dtype), w.panel_Y0(dtype), w.values(dtype)
+    with device.Context(0) as ctx:
+        t0 = time.perf_counter()
+        S = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, vv, seg_max=seg_max)
+        ctx.sync()
+        plan_s = time.perf_counter() - t0
+        info = S.info
+        t0 = time.perf_counter()
+        dA, dB, dY = ctx.panel_from(A), ctx.panel_from(B), ctx.panel_from(Y0)
+        dC = ctx.vals(w.nnz, dtype)
+        ctx.sync()
+        upload_s = time.perf_counter() - t0
+        del A, B, Y0
+
+        for _ in range(warmup):
+            ctx.sddmm(S, dA, dB, dC)
+            ctx.spmm(S, dB, dY)
+        ctx.sync()
+        ntimed = min(steps, max_timed)
+        t0 = time.perf_counter()
+        for i in range(steps):
+            if i < ntimed:
+                ctx.mark(3 * i)
+                ctx.sddmm(S, dA, dB, dC)
+                ctx.mark(3 * i + 1)
+                ctx.spmm(S, dB, dY)
+                ctx.mark(3 * i + 2)
+            else:
+                ctx.sddmm(S, dA, dB, dC)
+                ctx.spmm(S, dB, dY)
+        ctx.sync()
+        wall = time.perf_counter() - t0
+        sd = np.array([ctx.elapsed_ms(3 * i, 3 * i + 1) for i in range(ntimed)])
+        sp = np.array([ctx.elapsed_ms(3 * i + 1, 3 * i + 2) for i in range(ntimed)])
+        for h in (S, dA, dB, dY, dC):
+            h.close()
+
+    m_t, n_t = info.rows_touched, info.cols_touched
+    with_perm = not info.order_is_identity
+    fl = roofline.flops(w.nnz, w.k)
+    out = {"dtype": dtype, "ms_per_step": wall / steps * 1e3, "plan_build_s": plan_s,
+           "upload_s": upload_s, "nsegments": info.nsegments, "nsplit_rows": info.nsplit_rows,
+           "seg_max": info.seg_max, "rows_touched": m_t, "cols_touched": n_t,
+           "gflops": 2 * fl / (wall / steps) / 1e9, "kernels": {}}
+    for name, ms, strict, gather in (
+            ("sddmm", sd,
+             roofline.sddmm_bytes(w.nrows, w.nnz, w.k, wbytes, m_t, n_t, with_perm),
+             roofline.sddmm_bytes(w.nrows, w.nnz, w.k, wbytes, m_t, n_t, with_perm, gather=True)),
+            ("spmm", sp,
+             roofline.spmm_bytes(w.nrows, w.nnz, w.k, wbytes, m_t, n_t),
+             roofline.spmm_bytes(w.nrows, w.nnz, w.k, wbytes, m_t, n_t, gather=True))):
+        avg = float(ms.mean())
+        out["kernels"][name] = {
+            "ms_avg": avg, "ms_min": float(ms.min()), "ms_median": float(np.median(ms)),
+            "gflops": fl / avg / 1e6, "strict_bytes": int(strict), "gather_bytes": int(gather),
+            "strict_gbs": strict / avg / 1e6, "gather_gbs": gather / avg / 1e6,
+            "strict_frac": strict / avg / 1e6 / roofline.HBM_PEAK_GBS,
+            "gather_frac": gather / avg / 1e6 / roofline.HBM_PEAK_GBS}
+    return out
+
+
+def run_cpu_baseline(w, dtype):
+    """The CPU oracle (serial, one core, as the reference's per-rank path is:
+    no threads anywhere in it) on the same workload, one SDDMM + SpMM pass."""
+    import subprocess
+
+    from tests import _oracle as oracle
+
+    native = os.path.join(oracle.ORACLE_DIR, "liboracle_native.so")
+    try:
+        subprocess.run(["make", "-C", oracle.ORACLE_DIR, "liboracle_native.so"], check=True,
+                       capture_output=True)
+        lib = oracle.load(native)
+        flags = "-O3 -march=native -ffp-contract=off"
+    except Exception:  # noqa: BLE001 - any build problem: time the portable build instead
+        lib = oracle.load()
+        flags = "-O3 -ffp-contract=off"
+    try:
+        os.sched_setaffinity(0, {sorted(os.sched_getaffinity(0))[0]})
+        pinned = True
+    except OSError:
+        pinned = False
+    A, B, Y0, vv = w.panel_A(dtype), w.panel_B(dtype), w.panel_Y0(dtype), w.values(dtype)
+    t0 = time.perf_counter()
+    oracle.sddmm(A, B, w.ii, w.jj, vv, lib=lib)
+    t1 = time.perf_counter()
+    oracle.spmm(B, w.ii, w.jj, vv, Y0, lib=lib)
+    t2 = time.perf_counter()
+    fl = 2 * w.nnz * w.k
+    return {"value": 2 * fl / (t2 - t0) / 1e9, "unit": "GFLOP/s", "cores": 1, "kind": "port",
+            "sample": f"one full SDDMM+SpMM pass over {w.name} K={w.k} {dtype} "
+                      f"({w.order} COO, nnz={w.nnz})",
+            "sddmm_s": t1 - t0, "spmm_s": t2 - t1,
+            "sddmm_gflops": fl / (t1 - t0) / 1e9, "spmm_gflops": fl / (t2 - t1) / 1e9,
+            "host_cores": os.cpu_count(), "pinned": pinned, "flags": flags,
+            "note": "spmm time includes one copy of Y (the oracle leaves its input intact)"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--config", default="rmat20", help="workload name (spcomm3d_amd.workloads)")
+    ap.add_argument("--dtype", default="f64", choices=["f32", "f64"],
+                    help="real type of the headline value (the reference's is f64)")
+    ap.add_argument("--order", default="sorted", choices=["sorted", "shuffled"],
+                    help="order in which the COO entries are handed to the library")
+    ap.add_argument("--seg-max", type=int, default=None)
+    ap.add_argument("--only", action="store_true", help="skip the other real type")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path; run with --gpus 1")
+
+    ensure_built()
+    from spcomm3d_amd import workloads as W
+
+    t0 = time.perf_counter()
+    w = W.make(args.config)
+    if args.order == "shuffled":
+        w = w.shuffled()
+    log(f"workload {w.name}: {w.nrows}x{w.ncols} nnz={w.nnz} K={w.k} order={w.order} "
+        f"(generated in {time.perf_counter() - t0:.1f}s)")
+
+    main_r = run_gpu(w, args.dtype, args.steps, args.warmup, args.seg_max)
+    log(json.dumps(main_r))
+    also = {}
+    if not args.only:
+        other = "f32" if args.dtype == "f64" else "f64"
+        also[other] = run_gpu(w, other, args.steps, args.warmup, args.seg_max)
+        log(json.dumps(also[other]))
+    cpu = None if args.no_cpu else run_cpu_baseline(w, args.dtype)
+
+    dom = max(main_r["kernels"], key=lambda k: main_r["kernels"][k]["ms_avg"])
+    kd = main_r["kernels"][dom]
+    from spcomm3d_amd import roofline
+
+    line = {
+        "metric": METRIC, "value": main_r["gflops"], "unit": "GFLOP/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": main_r["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": args.dtype,
+        "data": "synthetic",
+        "config": {"workload": f"{w.name} K={w.k} ({w.order} COO)", "nrows": w.nrows,
+                   "ncols": w.ncols, "nnz": w.nnz, "k": w.k, "step": "SDDMM then SpMM",
+                   "rows_touched": main_r["rows_touched"], "cols_touched": main_r["cols_touched"]},
+        "roofline": {"bound": "hbm", "kernel": dom, "achieved": kd["strict_gbs"],
+                     "peak": roofline.HBM_PEAK_GBS, "unit": "GB/s", "frac": kd["strict_frac"],
+                     "traffic": None, "bytes_per_launch": kd["strict_bytes"],
+                     "ms_per_launch": kd["ms_avg"], "model": "strict (each operand once)"},
+        "cpu_baseline": cpu,
+        "kernels": main_r["kernels"],
+        "plan": {k: main_r[k] for k in ("plan_build_s", "upload_s", "nsegments", "nsplit_rows",
+                                        "seg_max")},
+        "also": also,
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -95,7 +95,7 @@ SPC3D_API int spc3d_ctx_stream(spc3d_ctx *ctx, void **hip_stream); /* the hipStr
 
 /* Timing on the context's stream (the reference times the call with chrono in
  * integer ms, src/distributed_comp.cpp:176-179; a kernel here lasts well under
- * one).  spc3d_timer_mark records event `slot` (0..63) on the stream;
+ * one).  spc3d_timer_mark records event `slot` (0..4095) on the stream;
  * spc3d_timer_elapsed_ms waits for `stop` and returns stop-start. */
 SPC3D_API int spc3d_timer_mark(spc3d_ctx *ctx, int slot);
 SPC3D_API int spc3d_timer_elapsed_ms(spc3d_ctx *ctx, int start, int stop, float *ms);

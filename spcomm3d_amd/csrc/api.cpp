@@ -48,7 +48,7 @@ constexpr uint32_t kMagicCtx = 0x53433343;   // live handles carry a tag so that
 constexpr uint32_t kMagicPanel = 0x53433350; // stale or foreign pointer is refused
 constexpr uint32_t kMagicVals = 0x53433356;  // instead of dereferenced further
 constexpr uint32_t kMagicPlan = 0x5343334c;
-constexpr int kTimerSlots = 64;
+constexpr int kTimerSlots = 4096;
 
 inline size_t elem_size(int dtype) { return dtype == SPC3D_F64 ? 8 : 4; }
 inline bool dtype_ok(int dtype) { return dtype == SPC3D_F32 || dtype == SPC3D_F64; }
