@@ -44,7 +44,7 @@ def ensure_built():
         __graft_entry__.build()
 
 
-def run_gpu(w, dtype, steps, warmup, seg_max=None, max_timed=1300):
+def run_gpu(w, dtype, steps, warmup, seg_max=None, max_timed=1300, copies=0):
     """Times `steps` SDDMM+SpMM passes on resident operands; returns a dict."""
     from spcomm3d_amd import device, roofline
     from spcomm3d_amd import workloads as W
@@ -64,6 +64,16 @@ def run_gpu(w, dtype, steps, warmup, seg_max=None, max_timed=1300):
         upload_s = time.perf_counter() - t0
         del A, B, Y0
 
+        if copies:
+            # Plain device copies of known size, so that a counter run of this same
+            # command has a dispatch (copy_kernel) to calibrate FETCH_SIZE/WRITE_SIZE on.
+            dT = ctx.panel(w.nrows, w.k, dtype)
+            for _ in range(copies):
+                dT.copy_from(dA)
+            ctx.sync()
+            dT.close()
+            log(f"calibration: {copies} x copy_kernel, {w.nrows * w.k * wbytes} bytes read and "
+                f"as many written per launch")
         for _ in range(warmup):
             ctx.sddmm(S, dA, dB, dC)
             ctx.spmm(S, dB, dY)
@@ -159,6 +169,9 @@ def main():
     ap.add_argument("--order", default="sorted", choices=["sorted", "shuffled"],
                     help="order in which the COO entries are handed to the library")
     ap.add_argument("--seg-max", type=int, default=None)
+    ap.add_argument("--calibration-copies", type=int, default=0,
+                    help="also launch this many plain device copies of an m x K panel "
+                         "(a known-size dispatch for counter calibration)")
     ap.add_argument("--only", action="store_true", help="skip the other real type")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     args = ap.parse_args()
@@ -175,7 +188,8 @@ def main():
     log(f"workload {w.name}: {w.nrows}x{w.ncols} nnz={w.nnz} K={w.k} order={w.order} "
         f"(generated in {time.perf_counter() - t0:.1f}s)")
 
-    main_r = run_gpu(w, args.dtype, args.steps, args.warmup, args.seg_max)
+    main_r = run_gpu(w, args.dtype, args.steps, args.warmup, args.seg_max,
+                     copies=args.calibration_copies)
     log(json.dumps(main_r))
     also = {}
     if not args.only:

@@ -106,6 +106,8 @@ SPC3D_API int spc3d_panel_destroy(spc3d_panel *p);
 SPC3D_API int spc3d_panel_upload(spc3d_panel *p, const void *host);   /* m*n reals, row-major */
 SPC3D_API int spc3d_panel_download(spc3d_panel *p, void *host);
 SPC3D_API int spc3d_panel_fill(spc3d_panel *p, double value);
+/* dst = src on the device (same shape and dtype); e.g. resetting Y to Y0 between runs. */
+SPC3D_API int spc3d_panel_copy(spc3d_panel *dst, const spc3d_panel *src);
 SPC3D_API int spc3d_panel_device_ptr(spc3d_panel *p, void **dev);
 SPC3D_API int spc3d_panel_shape(spc3d_panel *p, uint32_t *m, uint32_t *n, int *dtype);
 

@@ -47,6 +47,7 @@ SIGNATURES = {
     "spc3d_panel_upload": (c_int, [c_vp, c_vp]),
     "spc3d_panel_download": (c_int, [c_vp, c_vp]),
     "spc3d_panel_fill": (c_int, [c_vp, c_double]),
+    "spc3d_panel_copy": (c_int, [c_vp, c_vp]),
     "spc3d_panel_device_ptr": (c_int, [c_vp, P(c_vp)]),
     "spc3d_panel_shape": (c_int, [c_vp, P(c_u32), P(c_u32), P(c_int)]),
     "spc3d_vals_create": (c_int, [c_vp, c_int, c_u64, P(c_vp)]),

@@ -380,6 +380,24 @@ int spc3d_panel_fill(spc3d_panel *p, double value)
     return SPC3D_OK;
 }
 
+int spc3d_panel_copy(spc3d_panel *dst, const spc3d_panel *src)
+{
+    if (!live(dst) || !live(src))
+        return fail(SPC3D_ERR_INVALID_ARG, "panel is NULL or destroyed");
+    if (dst->ctx != src->ctx)
+        return fail(SPC3D_ERR_INVALID_ARG, "panels belong to different contexts");
+    if (dst->dtype != src->dtype || dst->m != src->m || dst->n != src->n)
+        return fail(SPC3D_ERR_SIZE_MISMATCH, "panels differ in shape or dtype");
+    if (dst->dev == src->dev)
+        return SPC3D_OK;
+    int rc = use_device(dst->ctx);
+    if (rc)
+        return rc;
+    HIP_TRY(launch_copy(dst->dev, src->dev, (uint64_t)dst->m * dst->n * elem_size(dst->dtype),
+                        dst->ctx->stream));
+    return SPC3D_OK;
+}
+
 int spc3d_panel_device_ptr(spc3d_panel *p, void **dev)
 {
     if (!live(p) || !dev)

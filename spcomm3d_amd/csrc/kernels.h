@@ -29,6 +29,8 @@ hipError_t launch_spmm(int dtype, const DevPlanView &P, const void *X, void *Y, 
 // out[p] = in[perm[p]] (perm == null: copy)
 hipError_t launch_gather_vals(int dtype, const void *in, const uint32_t *perm, void *out,
                               uint64_t n, hipStream_t stream);
+// dst[0..bytes) = src[0..bytes); both 16-byte aligned, non-overlapping
+hipError_t launch_copy(void *dst, const void *src, uint64_t bytes, hipStream_t stream);
 hipError_t launch_fill(int dtype, void *p, uint64_t n, double value, hipStream_t stream);
 
 // Name of the kernel variant launch_sddmm / launch_spmm picks for (dtype, K);

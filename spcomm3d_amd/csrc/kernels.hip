@@ -6,22 +6,33 @@
 // Both are gather-bound (about 0.25 flop per byte): no MFMA.  The unit of work
 // is a row segment (plan_host.h): at most seg_max consecutive entries of one
 // row.  A dense row of K reals is covered by LPR lanes holding VPL 16-byte
-// vectors each (K * sizeof(T) = LPR * VPL * 16), so one wavefront works on
-// 64 / LPR segments at once and every global load instruction moves
-// 64 x 16 B.  Segments arrive sorted longest first, so the lane groups of a
-// wavefront run the same trip count.
+// vectors each (K * sizeof(T) = LPR * VPL * 16, so K is a compile-time
+// constant of each instantiation), one wavefront works on 64 / LPR segments at
+// once and every global load instruction moves 64 x 16 B.  Segments arrive
+// sorted longest first, so the lane groups of a wavefront run the same trip
+// count.
 //
-//   sddmm: the group keeps its A row slice in registers, gathers B row slices
-//          for UB entries at a time, and reduces the UB per-lane partial dot
-//          products across the group with a halving exchange (UB-1 shuffles
-//          for UB entries instead of UB*log2(LPR)), leaving entry u's dot
-//          product in lane u*(LPR/UB); that lane scales by S.vv and stores to
-//          the caller's position.
+// A segment is walked in batches of UB entries, then one batch each of
+// UB/2, ..., 2, 1 entries as the remaining length requires: every batch size
+// is its own straight-line code with no per-entry predicates.  Within a batch
+// all gathers are issued before any arithmetic (a scheduling barrier keeps the
+// compiler from serialising them).
+//
+//   sddmm: the group keeps its A row slice in registers, gathers the B row
+//          slices of a batch, and reduces the per-lane partial dot products
+//          across the group with a halving exchange (NB-1 exchanges for NB
+//          entries instead of NB*log2(LPR)); exchanges inside a 16-lane row
+//          are DPP moves.  The lane that ends up with entry u's dot product
+//          scales it by S.vv and stores it at the caller's position.
 //   spmm : lane = slice of K, no cross-lane reduction; the group accumulates
 //          a * X[c,:] in registers and does one read-modify-write of the Y
 //          row slice.  Rows cut into several segments write partial sums that
 //          spmm_fixup adds into Y in a fixed order (no atomics, results are
 //          reproducible run to run).
+//
+// Streams that are read once (indices, sparse values, segment descriptors, A
+// rows, Y rows) use non-temporal accesses so that the per-XCD L2 is left to
+// the gathered B / X rows, the only operand with reuse.
 #include <hip/hip_runtime.h>
 
 #include "kernels.h"
@@ -39,94 +50,175 @@ template <> struct Vec<double> {
     static constexpr int N = 2;
 };
 
-template <typename T>
-__device__ __forceinline__ T vdot(const typename Vec<T>::type &a, const typename Vec<T>::type &b,
-                                  T acc)
-{
-#pragma unroll
-    for (int i = 0; i < Vec<T>::N; ++i)
-        acc += a[i] * b[i];
-    return acc;
-}
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kBlock = 256; // 4 wavefronts
 
+template <typename P> __device__ __forceinline__ P nt_load(const P *p)
+{
+    return __builtin_nontemporal_load(p);
+}
+template <typename P> __device__ __forceinline__ void nt_store(P v, P *p)
+{
+    __builtin_nontemporal_store(v, p);
+}
+
+__device__ __forceinline__ constexpr int ilog2(int x) { return x <= 1 ? 0 : 1 + ilog2(x >> 1); }
+
+// ---- lane exchange ----------------------------------------------------------
+// xchg<S>(v): the value lane (id ^ S) holds.  S < 16 stays inside a 16-lane DPP
+// row: xor 1 and 2 are quad permutes, xor 8 is a rotation by 8, xor 4 is
+// half-row mirror (i -> 7 - i = i ^ 7) after quad reverse (i ^ 3).
+template <int CTRL> __device__ __forceinline__ int dpp_mov(int v)
+{
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, false);
+}
+template <int S> __device__ __forceinline__ int xchg_i32(int v)
+{
+    if constexpr (S == 1)
+        return dpp_mov<0xB1>(v); // quad_perm [1,0,3,2]
+    else if constexpr (S == 2)
+        return dpp_mov<0x4E>(v); // quad_perm [2,3,0,1]
+    else if constexpr (S == 4)
+        return dpp_mov<0x141>(dpp_mov<0x1B>(v)); // row_half_mirror o quad_perm [3,2,1,0]
+    else if constexpr (S == 8)
+        return dpp_mov<0x128>(v); // row_ror:8
+    else
+        return __shfl_xor(v, S, 64);
+}
+template <int S> __device__ __forceinline__ float xchg(float v)
+{
+    return __int_as_float(xchg_i32<S>(__float_as_int(v)));
+}
+template <int S> __device__ __forceinline__ double xchg(double v)
+{
+    const int lo = xchg_i32<S>(__double2loint(v));
+    const int hi = xchg_i32<S>(__double2hiint(v));
+    return __hiloint2double(hi, lo);
+}
+
+// Order in which the xor strides of an LPR-lane group are used: the steps that
+// move the most values come first and get the single-instruction exchanges;
+// strides 16 and 32 (LDS-crossbar permutes) come last.
+template <int LPR> struct Strides;
+template <> struct Strides<4> { static constexpr int s[2] = {2, 1}; };
+template <> struct Strides<8> { static constexpr int s[3] = {2, 1, 4}; };
+template <> struct Strides<16> { static constexpr int s[4] = {8, 2, 1, 4}; };
+template <> struct Strides<32> { static constexpr int s[5] = {8, 2, 1, 4, 16}; };
+template <> struct Strides<64> { static constexpr int s[6] = {8, 2, 1, 4, 16, 32}; };
+
+// Halving exchange + finishing all-reduce over an LPR-lane group.
+// In: part[u] = this lane's partial sum for entry u, u < NB.  Out: part[0] =
+// the full sum of entry entry_of<LPR, NB>(sub), identical in every lane that
+// maps to that entry.
+template <typename T, int LPR, int NB, int STEP = 0, int N = NB>
+__device__ __forceinline__ void group_reduce(T (&part)[NB], uint32_t sub)
+{
+    if constexpr (STEP < ilog2(LPR)) {
+        constexpr int S = Strides<LPR>::s[STEP];
+        if constexpr (N > 1) {
+            const bool upper = (sub & S) != 0;
+#pragma unroll
+            for (int i = 0; i < N / 2; ++i) {
+                const T keep = upper ? part[i + N / 2] : part[i];
+                const T send = upper ? part[i] : part[i + N / 2];
+                part[i] = keep + xchg<S>(send);
+            }
+            group_reduce<T, LPR, NB, STEP + 1, N / 2>(part, sub);
+        } else {
+            part[0] += xchg<S>(part[0]);
+            group_reduce<T, LPR, NB, STEP + 1, 1>(part, sub);
+        }
+    }
+}
+
+// Entry (0 .. NB-1) whose sum lane `sub` holds after group_reduce<LPR, NB>.
+template <int LPR, int NB> __device__ __forceinline__ uint32_t entry_of(uint32_t sub)
+{
+    uint32_t u = 0;
+#pragma unroll
+    for (int t = 0; t < ilog2(NB); ++t)
+        u |= ((sub & Strides<LPR>::s[t]) ? 1u : 0u) << (ilog2(NB) - 1 - t);
+    return u;
+}
+
+// One lane per entry stores: the lane whose bits for the finishing strides are 0.
+template <int LPR, int NB> __device__ __forceinline__ bool is_writer(uint32_t sub)
+{
+    uint32_t mask = 0;
+#pragma unroll
+    for (int t = ilog2(NB); t < ilog2(LPR); ++t)
+        mask |= Strides<LPR>::s[t];
+    return (sub & mask) == 0;
+}
+
+template <typename T, int LPR, int VPL>
+__device__ __forceinline__ const typename Vec<T>::type *row_ptr(const T *base, uint32_t row,
+                                                                uint32_t sub)
+{
+    constexpr uint64_t kRowBytes = (uint64_t)LPR * VPL * 16;
+    return reinterpret_cast<const typename Vec<T>::type *>(
+               reinterpret_cast<const char *>(base) + (uint64_t)row * kRowBytes) +
+           sub;
+}
+
 // ---------------------------------------------------------------- SDDMM ----
-template <typename T, int LPR, int VPL, int UB, bool TAIL>
+template <typename T, int LPR, int VPL, int NB>
 __device__ __forceinline__ void
 sddmm_batch(const typename Vec<T>::type (&a)[VPL], const uint32_t *__restrict__ col,
             const uint32_t *__restrict__ perm, const T *__restrict__ sval,
-            const T *__restrict__ B, T *__restrict__ C, uint32_t K, uint32_t p0, uint32_t nb,
-            uint32_t sub)
+            const T *__restrict__ B, T *__restrict__ C, uint32_t p0, uint32_t sub)
 {
     using V = typename Vec<T>::type;
-    constexpr int RED = LPR / UB;
-    const uint32_t ul = sub & (UB - 1);
-    const uint32_t uo = sub / RED;
+    static_assert(NB <= LPR, "batch must fit the lane group");
 
-    // Indices and the output lane's operands first: they head the dependency chain.
-    const uint32_t cme = col[p0 + (TAIL ? (ul < nb ? ul : nb - 1) : ul)];
+    // Lane u of the group fetches the column of entry u; the writer lanes fetch
+    // what they need for the store.  These head the dependency chain.
+    const uint32_t cme = nt_load(col + p0 + (sub & (NB - 1)));
+    const bool writer = is_writer<LPR, NB>(sub);
+    const uint32_t uo = entry_of<LPR, NB>(sub);
     T sv = (T)0;
-    uint32_t dst = 0;
-    const bool writer = (sub % RED) == 0 && (!TAIL || uo < nb);
+    uint32_t dst = p0 + uo;
     if (writer) {
-        sv = sval[p0 + uo];
-        dst = perm ? perm[p0 + uo] : p0 + uo;
+        sv = nt_load(sval + p0 + uo);
+        if (perm)
+            dst = nt_load(perm + p0 + uo);
     }
 
-    V b[UB][VPL];
+    V b[NB][VPL];
 #pragma unroll
-    for (int u = 0; u < UB; ++u) {
+    for (int u = 0; u < NB; ++u) {
         const uint32_t c = __shfl(cme, u, LPR);
-        const V *brow = reinterpret_cast<const V *>(B + (size_t)c * K);
-        if (!TAIL || (uint32_t)u < nb) {
+        const V *brow = row_ptr<T, LPR, VPL>(B, c, sub);
 #pragma unroll
-            for (int v = 0; v < VPL; ++v)
-                b[u][v] = brow[sub + v * LPR];
-        } else {
-#pragma unroll
-            for (int v = 0; v < VPL; ++v)
-                b[u][v] = V{};
-        }
+        for (int v = 0; v < VPL; ++v)
+            b[u][v] = brow[v * LPR];
     }
-    T part[UB];
+    __builtin_amdgcn_sched_barrier(0); // all gathers in flight before the first use
+
+    T part[NB];
 #pragma unroll
-    for (int u = 0; u < UB; ++u) {
+    for (int u = 0; u < NB; ++u) {
         T acc = (T)0;
 #pragma unroll
         for (int v = 0; v < VPL; ++v)
-            acc = vdot<T>(a[v], b[u][v], acc);
+#pragma unroll
+            for (int i = 0; i < Vec<T>::N; ++i)
+                acc += a[v][i] * b[u][v][i];
         part[u] = acc;
     }
-    // Halving exchange: after the step with stride s a lane keeps the half of
-    // its values selected by (sub & s); UB values shrink to 1 in log2(UB) steps
-    // and lane `sub` ends with the sum, over its RED-aligned partners so far
-    // excluded, of entry sub / RED.
-#pragma unroll
-    for (int s = LPR / 2, n = UB; n > 1; s >>= 1, n >>= 1) {
-        const bool upper = (sub & s) != 0;
-#pragma unroll
-        for (int i = 0; i < n / 2; ++i) {
-            const T keep = upper ? part[i + n / 2] : part[i];
-            const T send = upper ? part[i] : part[i + n / 2];
-            part[i] = keep + __shfl_xor(send, s, LPR);
-        }
-    }
-#pragma unroll
-    for (int s = RED / 2; s >= 1; s >>= 1)
-        part[0] += __shfl_xor(part[0], s, LPR);
-
+    group_reduce<T, LPR, NB>(part, sub);
     if (writer)
-        C[dst] = part[0] * sv;
+        nt_store(part[0] * sv, C + dst);
 }
 
 template <typename T, int LPR, int VPL, int UB>
 __global__ void __launch_bounds__(kBlock)
 sddmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, const uint32_t *__restrict__ col,
                  const uint32_t *__restrict__ perm, const T *__restrict__ sval,
-                 const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C, uint32_t K)
+                 const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C)
 {
-    static_assert(UB <= LPR && LPR <= 64, "batch must fit the lane group");
+    static_assert(UB <= LPR && UB <= 16 && LPR <= 64, "batch must fit the lane group");
     using V = typename Vec<T>::type;
     constexpr int G = 64 / LPR;
     const uint32_t lane = threadIdx.x & 63u;
@@ -135,21 +227,36 @@ sddmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, const uint32_t *__
     const uint64_t sid = wave * G + lane / LPR;
     if (sid >= nseg)
         return;
-    const Seg sg = segs[sid];
+    const u32x4 sg = nt_load(reinterpret_cast<const u32x4 *>(segs) + sid); // row, start, len, slot
 
     V a[VPL];
     {
-        const V *arow = reinterpret_cast<const V *>(A + (size_t)sg.row * K);
+        const V *arow = row_ptr<T, LPR, VPL>(A, sg[0], sub);
 #pragma unroll
         for (int v = 0; v < VPL; ++v)
-            a[v] = arow[sub + v * LPR];
+            a[v] = nt_load(arow + v * LPR);
     }
-    uint32_t base = 0;
-    for (; base + UB <= sg.len; base += UB)
-        sddmm_batch<T, LPR, VPL, UB, false>(a, col, perm, sval, B, C, K, sg.start + base, UB, sub);
-    if (base < sg.len)
-        sddmm_batch<T, LPR, VPL, UB, true>(a, col, perm, sval, B, C, K, sg.start + base,
-                                           sg.len - base, sub);
+    uint32_t p = sg[1], rem = sg[2];
+    for (; rem >= UB; rem -= UB, p += UB)
+        sddmm_batch<T, LPR, VPL, UB>(a, col, perm, sval, B, C, p, sub);
+    if constexpr (UB > 8)
+        if (rem & 8) {
+            sddmm_batch<T, LPR, VPL, 8>(a, col, perm, sval, B, C, p, sub);
+            p += 8;
+        }
+    if constexpr (UB > 4)
+        if (rem & 4) {
+            sddmm_batch<T, LPR, VPL, 4>(a, col, perm, sval, B, C, p, sub);
+            p += 4;
+        }
+    if constexpr (UB > 2)
+        if (rem & 2) {
+            sddmm_batch<T, LPR, VPL, 2>(a, col, perm, sval, B, C, p, sub);
+            p += 2;
+        }
+    if constexpr (UB > 1)
+        if (rem & 1)
+            sddmm_batch<T, LPR, VPL, 1>(a, col, perm, sval, B, C, p, sub);
 }
 
 // Any K: one wavefront per segment, lanes stride over K, scalar loads.
@@ -181,39 +288,32 @@ sddmm_generic_kernel(const Seg *__restrict__ segs, uint32_t nseg, const uint32_t
 }
 
 // ----------------------------------------------------------------- SpMM ----
-template <typename T, int LPR, int VPL, int UB, bool TAIL>
+template <typename T, int LPR, int VPL, int NB>
 __device__ __forceinline__ void
 spmm_batch(typename Vec<T>::type (&acc)[VPL], const uint32_t *__restrict__ col,
-           const T *__restrict__ sval, const T *__restrict__ X, uint32_t K, uint32_t p0,
-           uint32_t nb, uint32_t sub)
+           const T *__restrict__ sval, const T *__restrict__ X, uint32_t p0, uint32_t sub)
 {
     using V = typename Vec<T>::type;
-    const uint32_t ul = sub & (UB - 1);
-    const uint32_t pl = p0 + (TAIL ? (ul < nb ? ul : nb - 1) : ul);
-    const uint32_t cme = col[pl];
-    const T vme = sval[pl];
+    static_assert(NB <= LPR, "batch must fit the lane group");
+    const uint32_t pl = p0 + (sub & (NB - 1));
+    const uint32_t cme = nt_load(col + pl);
+    const T vme = nt_load(sval + pl);
 
-    V x[UB][VPL];
-    T av[UB];
+    V x[NB][VPL];
+    T av[NB];
 #pragma unroll
-    for (int u = 0; u < UB; ++u) {
+    for (int u = 0; u < NB; ++u) {
         const uint32_t c = __shfl(cme, u, LPR);
         av[u] = __shfl(vme, u, LPR);
-        const V *xrow = reinterpret_cast<const V *>(X + (size_t)c * K);
-        if (!TAIL || (uint32_t)u < nb) {
+        const V *xrow = row_ptr<T, LPR, VPL>(X, c, sub);
 #pragma unroll
-            for (int v = 0; v < VPL; ++v)
-                x[u][v] = xrow[sub + v * LPR];
-        } else {
-            av[u] = (T)0;
-#pragma unroll
-            for (int v = 0; v < VPL; ++v)
-                x[u][v] = V{};
-        }
+        for (int v = 0; v < VPL; ++v)
+            x[u][v] = xrow[v * LPR];
     }
+    __builtin_amdgcn_sched_barrier(0); // all gathers in flight before the first use
     // Entries are added in kernel order, which within a row is the caller's order.
 #pragma unroll
-    for (int u = 0; u < UB; ++u)
+    for (int u = 0; u < NB; ++u)
 #pragma unroll
         for (int v = 0; v < VPL; ++v)
             acc[v] += x[u][v] * av[u];
@@ -223,9 +323,9 @@ template <typename T, int LPR, int VPL, int UB>
 __global__ void __launch_bounds__(kBlock)
 spmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, const uint32_t *__restrict__ col,
                 const T *__restrict__ sval, const T *__restrict__ X, T *__restrict__ Y,
-                T *__restrict__ partial, uint32_t K)
+                T *__restrict__ partial)
 {
-    static_assert(UB <= LPR && LPR <= 64, "batch must fit the lane group");
+    static_assert(UB <= LPR && UB <= 16 && LPR <= 64, "batch must fit the lane group");
     using V = typename Vec<T>::type;
     constexpr int G = 64 / LPR;
     const uint32_t lane = threadIdx.x & 63u;
@@ -234,9 +334,10 @@ spmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, const uint32_t *__r
     const uint64_t sid = wave * G + lane / LPR;
     if (sid >= nseg)
         return;
-    const Seg sg = segs[sid];
-    const bool whole = sg.slot == kWholeRow;
-    V *dst = reinterpret_cast<V *>(whole ? Y + (size_t)sg.row * K : partial + (size_t)sg.slot * K);
+    const u32x4 sg = nt_load(reinterpret_cast<const u32x4 *>(segs) + sid); // row, start, len, slot
+    const bool whole = sg[3] == kWholeRow;
+    V *dst = const_cast<V *>(whole ? row_ptr<T, LPR, VPL>(Y, sg[0], sub)
+                                   : row_ptr<T, LPR, VPL>(partial, sg[3], sub));
 
     V acc[VPL], y0[VPL];
 #pragma unroll
@@ -247,17 +348,38 @@ spmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, const uint32_t *__r
     if (whole) {
 #pragma unroll
         for (int v = 0; v < VPL; ++v)
-            y0[v] = dst[sub + v * LPR];
+            y0[v] = nt_load(dst + v * LPR);
     }
-    uint32_t base = 0;
-    for (; base + UB <= sg.len; base += UB)
-        spmm_batch<T, LPR, VPL, UB, false>(acc, col, sval, X, K, sg.start + base, UB, sub);
-    if (base < sg.len)
-        spmm_batch<T, LPR, VPL, UB, true>(acc, col, sval, X, K, sg.start + base, sg.len - base,
-                                          sub);
+    uint32_t p = sg[1], rem = sg[2];
+    for (; rem >= UB; rem -= UB, p += UB)
+        spmm_batch<T, LPR, VPL, UB>(acc, col, sval, X, p, sub);
+    if constexpr (UB > 8)
+        if (rem & 8) {
+            spmm_batch<T, LPR, VPL, 8>(acc, col, sval, X, p, sub);
+            p += 8;
+        }
+    if constexpr (UB > 4)
+        if (rem & 4) {
+            spmm_batch<T, LPR, VPL, 4>(acc, col, sval, X, p, sub);
+            p += 4;
+        }
+    if constexpr (UB > 2)
+        if (rem & 2) {
+            spmm_batch<T, LPR, VPL, 2>(acc, col, sval, X, p, sub);
+            p += 2;
+        }
+    if constexpr (UB > 1)
+        if (rem & 1)
+            spmm_batch<T, LPR, VPL, 1>(acc, col, sval, X, p, sub);
+    if (whole) {
 #pragma unroll
-    for (int v = 0; v < VPL; ++v)
-        dst[sub + v * LPR] = y0[v] + acc[v];
+        for (int v = 0; v < VPL; ++v)
+            nt_store(y0[v] + acc[v], dst + v * LPR);
+    } else {
+#pragma unroll
+        for (int v = 0; v < VPL; ++v)
+            dst[v * LPR] = acc[v]; // read back by spmm_fixup right after
+    }
 }
 
 template <typename T>
@@ -317,6 +439,21 @@ __global__ void __launch_bounds__(kBlock) fill_kernel(T *__restrict__ p, uint64_
         p[i] = value;
 }
 
+// Plain streaming copy, 16 bytes per lane per iteration; the tail (< 16 bytes)
+// is moved bytewise by the first lanes.
+__global__ void __launch_bounds__(kBlock)
+copy_kernel(uint4 *__restrict__ dst, const uint4 *__restrict__ src, uint64_t nvec,
+            uint32_t tail_bytes)
+{
+    const uint64_t stride = (uint64_t)gridDim.x * kBlock;
+    const uint64_t tid = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    for (uint64_t i = tid; i < nvec; i += stride)
+        dst[i] = src[i];
+    if (tid < tail_bytes)
+        reinterpret_cast<unsigned char *>(dst + nvec)[tid] =
+            reinterpret_cast<const unsigned char *>(src + nvec)[tid];
+}
+
 // ------------------------------------------------------------- dispatch ----
 struct Shape {
     int lpr, vpl, ub; // lpr == 0: generic kernel
@@ -352,21 +489,22 @@ inline uint32_t blocks_for_groups(uint32_t nseg, int groups_per_wave)
 }
 
 template <typename T, int LPR, int VPL, int UB>
-void run_sddmm(const DevPlanView &P, const T *A, const T *B, T *C, uint32_t K, hipStream_t st)
+void run_sddmm(const DevPlanView &P, const T *A, const T *B, T *C, hipStream_t st)
 {
     const uint32_t grid = blocks_for_groups(P.nseg, 64 / LPR);
     hipLaunchKernelGGL((sddmm_seg_kernel<T, LPR, VPL, UB>), dim3(grid), dim3(kBlock), 0, st, P.segs,
-                       P.nseg, P.col, P.perm, (const T *)P.sval, A, B, C, K);
+                       P.nseg, P.col, P.perm, (const T *)P.sval, A, B, C);
 }
 
 template <typename T, int LPR, int VPL, int UB>
-void run_spmm(const DevPlanView &P, const T *X, T *Y, uint32_t K, hipStream_t st)
+void run_spmm(const DevPlanView &P, const T *X, T *Y, hipStream_t st)
 {
     const uint32_t grid = blocks_for_groups(P.nseg, 64 / LPR);
     hipLaunchKernelGGL((spmm_seg_kernel<T, LPR, VPL, UB>), dim3(grid), dim3(kBlock), 0, st, P.segs,
-                       P.nseg, P.col, (const T *)P.sval, X, Y, (T *)P.partial, K);
+                       P.nseg, P.col, (const T *)P.sval, X, Y, (T *)P.partial);
 }
 
+// (LPR, VPL, UB): UB * VPL 16-byte gathers are in flight per lane.
 #define SPC3D_FOR_SHAPES(X)                                                                       \
     X(4, 1, 4) X(8, 1, 8) X(16, 1, 16) X(32, 1, 16) X(64, 1, 16)                                  \
     X(4, 2, 4) X(8, 2, 8) X(16, 2, 8) X(32, 2, 8) X(64, 2, 8)                                     \
@@ -382,7 +520,7 @@ hipError_t sddmm_typed(const DevPlanView &P, const void *A, const void *B, void 
     bool done = false;
 #define X(L, V, U)                                                                                \
     if (!done && sh.lpr == L && sh.vpl == V) {                                                    \
-        run_sddmm<T, L, V, U>(P, (const T *)A, (const T *)B, (T *)C, K, st);                      \
+        run_sddmm<T, L, V, U>(P, (const T *)A, (const T *)B, (T *)C, st);                         \
         done = true;                                                                              \
     }
     SPC3D_FOR_SHAPES(X)
@@ -405,7 +543,7 @@ hipError_t spmm_typed(const DevPlanView &P, const void *X_, void *Y, uint32_t K,
     bool done = false;
 #define X(L, V, U)                                                                                \
     if (!done && sh.lpr == L && sh.vpl == V) {                                                    \
-        run_spmm<T, L, V, U>(P, (const T *)X_, (T *)Y, K, st);                                    \
+        run_spmm<T, L, V, U>(P, (const T *)X_, (T *)Y, st);                                       \
         done = true;                                                                              \
     }
     SPC3D_FOR_SHAPES(X)
@@ -461,6 +599,16 @@ hipError_t launch_gather_vals(int dtype, const void *in, const uint32_t *perm, v
     else
         hipLaunchKernelGGL((gather_kernel<float>), dim3(stream_grid(n)), dim3(kBlock), 0, stream,
                            (const float *)in, perm, (float *)out, n);
+    return hipGetLastError();
+}
+
+hipError_t launch_copy(void *dst, const void *src, uint64_t bytes, hipStream_t stream)
+{
+    if (bytes == 0)
+        return hipSuccess;
+    const uint64_t nvec = bytes / 16;
+    hipLaunchKernelGGL(copy_kernel, dim3(stream_grid(nvec ? nvec : 1)), dim3(kBlock), 0, stream,
+                       (uint4 *)dst, (const uint4 *)src, nvec, (uint32_t)(bytes % 16));
     return hipGetLastError();
 }
 

@@ -158,6 +158,10 @@ class Panel:
     def fill(self, value: float):
         check(self.ctx._lib.spc3d_panel_fill(self._h, float(value)), "spc3d_panel_fill")
 
+    def copy_from(self, src: "Panel"):
+        """self = src on the device (``spc3d_panel_copy``); asynchronous."""
+        check(self.ctx._lib.spc3d_panel_copy(self._h, src._h), "spc3d_panel_copy")
+
     def device_ptr(self) -> int:
         p = ctypes.c_void_p()
         check(self.ctx._lib.spc3d_panel_device_ptr(self._h, ctypes.byref(p)),
