@@ -71,15 +71,35 @@ typedef struct spc3d_plan spc3d_plan;   /* device-resident cooMat pattern (ii, j
 typedef struct {
     uint32_t nrows, ncols;
     uint64_t nnz;
-    uint32_t rows_touched;   /* rows with at least one entry */
-    uint32_t cols_touched;   /* columns with at least one entry */
-    uint32_t nsegments;      /* row segments the kernels iterate over */
-    uint32_t nsplit_rows;    /* rows cut into several segments (SpMM combines partial sums) */
-    uint32_t npartial_slots; /* partial-sum rows kept for those */
+    uint32_t rows_touched;     /* rows with at least one entry */
+    uint32_t cols_touched;     /* columns with at least one entry */
+    uint32_t nsegments;        /* row segments the kernels work on */
+    uint32_t nsegments_padded; /* stored segments: the above plus padding of short XCD queues */
+    uint32_t nsplit_rows;      /* rows cut into several segments (SpMM combines partial sums) */
+    uint32_t npartial_slots;   /* partial-sum rows kept for those */
     uint32_t max_row_nnz;
-    uint32_t seg_max;        /* longest segment */
-    int32_t  order_is_identity; /* 1: caller's COO was already row-major grouped, no permutation read */
+    uint32_t seg_max;          /* longest segment allowed */
+    int32_t  order_is_identity; /* 1: the caller's order is the kernel order, no permutation read */
+    uint32_t nqueues;          /* 1, or 8: segments are dealt to the 8 XCDs by column slice */
+    uint32_t hot_cols;         /* XCD slicing: columns planned to stay in some L2 (0: slicing off) */
+    uint32_t hub_rows;         /* XCD slicing: rows cut by column slice */
+    uint64_t hot_entries;      /* XCD slicing: entries in those columns */
 } spc3d_plan_info;
+
+/* Plan tuning; a zero field selects the default.  Only speed depends on these. */
+typedef struct {
+    uint32_t seg_max;      /* longest segment in entries (default: nnz / 2048 rounded down to
+                              a power of two, within 64 .. 2048) */
+    uint32_t k_hint;       /* XCD slicing: K the plan will mostly run with (default 64) */
+    uint32_t l2_hot_bytes; /* XCD slicing: share of one XCD's 4 MiB L2 planned for dense rows
+                              (default 3 MiB) */
+    uint32_t hub_min;      /* XCD slicing: rows with at least this many entries are cut by
+                              column slice (default 128) */
+    uint32_t xcd_slices;   /* 8: the entries of long rows are dealt to the 8 XCDs by column, so
+                              that each L2 caches its own eighth of the hot dense rows;
+                              0 or 1 (default): off */
+    uint32_t reserved[3];  /* must be 0 */
+} spc3d_plan_opts;
 
 /* ---- library / errors ------------------------------------------------- */
 SPC3D_API const char *spc3d_version(void);
@@ -92,6 +112,11 @@ SPC3D_API int spc3d_ctx_create(int device, spc3d_ctx **out);
 SPC3D_API int spc3d_ctx_destroy(spc3d_ctx *ctx);
 SPC3D_API int spc3d_ctx_sync(spc3d_ctx *ctx);                 /* wait for the context's stream */
 SPC3D_API int spc3d_ctx_stream(spc3d_ctx *ctx, void **hip_stream); /* the hipStream_t, for callers that share it */
+/* xcd[b] = id of the XCD that workgroup b of an nblocks-wide grid ran on.  The
+ * kernels assume workgroups are dealt to the 8 XCDs round-robin (xcd = b % 8)
+ * when they place work next to the L2 that caches its dense rows; this lets a
+ * caller check that on its machine.  Synchronous. */
+SPC3D_API int spc3d_ctx_probe_xcd(spc3d_ctx *ctx, uint32_t nblocks, uint32_t *xcd);
 
 /* Timing on the context's stream (the reference times the call with chrono in
  * integer ms, src/distributed_comp.cpp:176-179; a kernel here lasts well under
@@ -127,7 +152,7 @@ SPC3D_API int spc3d_coo_validate(uint32_t nrows, uint32_t ncols, uint64_t nnz,
                        const uint32_t *ii, const uint32_t *jj);
 
 /* Validates (as above), groups the entries by row keeping the caller's order
- * within a row, cuts rows into segments, and uploads.  `vv` (nnz reals of
+ * within a row, cuts long rows into segments, and uploads.  `vv` (nnz reals of
  * `dtype`, caller's order) may be NULL and set later.  The pattern is copied:
  * the caller's arrays are not referenced afterwards.  Replaces nothing in the
  * reference (it walks the unsorted COO directly, core_ops.cpp:7-10); it is the
@@ -136,23 +161,24 @@ SPC3D_API int spc3d_coo_validate(uint32_t nrows, uint32_t ncols, uint64_t nnz,
 SPC3D_API int spc3d_plan_create(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t ncols,
                       uint64_t nnz, const uint32_t *ii, const uint32_t *jj,
                       const void *vv, spc3d_plan **out);
-/* As above with the longest segment given explicitly (0 = library default). */
+/* As above with explicit tuning (NULL = defaults). */
 SPC3D_API int spc3d_plan_create_ex(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t ncols,
                          uint64_t nnz, const uint32_t *ii, const uint32_t *jj,
-                         const void *vv, uint32_t seg_max, spc3d_plan **out);
-/* Host-only: builds the same kernel-order form spc3d_plan_create uploads and
+                         const void *vv, const spc3d_plan_opts *opts, spc3d_plan **out);
+/* Host-only: builds the same kernel-order form spc3d_plan_create_ex uploads and
  * hands it back, for inspection and for testing without a GPU.  `info` is
  * always filled.  Each output may be NULL; otherwise col and perm hold nnz
  * entries (perm[p] = caller's position of kernel-order entry p), segs holds
- * 4 words per segment {row, start, len, slot} (slot 0xFFFFFFFF: the segment is
- * the whole row) and needs seg_cap >= info->nsegments, splits holds 3 words per
- * cut row {row, first_slot, nslots} and needs split_cap >= info->nsplit_rows;
- * a capacity that is too small gives SPC3D_ERR_SIZE_MISMATCH. */
-SPC3D_API int spc3d_plan_build_host(uint32_t nrows, uint32_t ncols, uint64_t nnz,
-                          const uint32_t *ii, const uint32_t *jj, uint32_t seg_max,
-                          spc3d_plan_info *info, uint32_t *col, uint32_t *perm,
-                          uint32_t *segs, uint32_t seg_cap, uint32_t *splits,
-                          uint32_t split_cap);
+ * 4 words per stored segment {row, start, len, slot} (slot 0xFFFFFFFF: the
+ * segment is the whole row; len 0: padding) and needs
+ * seg_cap >= info->nsegments_padded, splits holds 3 words per cut row
+ * {row, first_slot, nslots} and needs split_cap >= info->nsplit_rows; a
+ * capacity that is too small gives SPC3D_ERR_SIZE_MISMATCH. */
+SPC3D_API int spc3d_plan_build_host(int dtype, uint32_t nrows, uint32_t ncols, uint64_t nnz,
+                          const uint32_t *ii, const uint32_t *jj,
+                          const spc3d_plan_opts *opts, spc3d_plan_info *info,
+                          uint32_t *col, uint32_t *perm, uint32_t *segs, uint32_t seg_cap,
+                          uint32_t *splits, uint32_t split_cap);
 SPC3D_API int spc3d_plan_destroy(spc3d_plan *plan);
 SPC3D_API int spc3d_plan_set_values(spc3d_plan *plan, const void *vv_host);       /* caller's COO order */
 SPC3D_API int spc3d_plan_set_values_device(spc3d_plan *plan, const spc3d_vals *vv); /* caller's COO order */

@@ -25,9 +25,16 @@ P = ctypes.POINTER
 class PlanInfo(ctypes.Structure):
     _fields_ = [("nrows", c_u32), ("ncols", c_u32), ("nnz", c_u64),
                 ("rows_touched", c_u32), ("cols_touched", c_u32),
-                ("nsegments", c_u32), ("nsplit_rows", c_u32),
-                ("npartial_slots", c_u32), ("max_row_nnz", c_u32),
-                ("seg_max", c_u32), ("order_is_identity", ctypes.c_int32)]
+                ("nsegments", c_u32), ("nsegments_padded", c_u32),
+                ("nsplit_rows", c_u32), ("npartial_slots", c_u32),
+                ("max_row_nnz", c_u32), ("seg_max", c_u32),
+                ("order_is_identity", ctypes.c_int32), ("nqueues", c_u32),
+                ("hot_cols", c_u32), ("hub_rows", c_u32), ("hot_entries", c_u64)]
+
+
+class PlanOpts(ctypes.Structure):
+    _fields_ = [("seg_max", c_u32), ("k_hint", c_u32), ("l2_hot_bytes", c_u32),
+                ("hub_min", c_u32), ("xcd_slices", c_u32), ("reserved", c_u32 * 3)]
 
 
 # name -> (restype, argtypes); one entry for every function the header declares.
@@ -40,6 +47,7 @@ SIGNATURES = {
     "spc3d_ctx_destroy": (c_int, [c_vp]),
     "spc3d_ctx_sync": (c_int, [c_vp]),
     "spc3d_ctx_stream": (c_int, [c_vp, P(c_vp)]),
+    "spc3d_ctx_probe_xcd": (c_int, [c_vp, c_u32, c_vp]),
     "spc3d_timer_mark": (c_int, [c_vp, c_int]),
     "spc3d_timer_elapsed_ms": (c_int, [c_vp, c_int, c_int, P(c_float)]),
     "spc3d_panel_create": (c_int, [c_vp, c_int, c_u32, c_u32, P(c_vp)]),
@@ -58,10 +66,10 @@ SIGNATURES = {
     "spc3d_vals_device_ptr": (c_int, [c_vp, P(c_vp)]),
     "spc3d_coo_validate": (c_int, [c_u32, c_u32, c_u64, c_vp, c_vp]),
     "spc3d_plan_create": (c_int, [c_vp, c_int, c_u32, c_u32, c_u64, c_vp, c_vp, c_vp, P(c_vp)]),
-    "spc3d_plan_create_ex": (c_int, [c_vp, c_int, c_u32, c_u32, c_u64, c_vp, c_vp, c_vp, c_u32,
-                                     P(c_vp)]),
-    "spc3d_plan_build_host": (c_int, [c_u32, c_u32, c_u64, c_vp, c_vp, c_u32, P(PlanInfo), c_vp,
-                                      c_vp, c_vp, c_u32, c_vp, c_u32]),
+    "spc3d_plan_create_ex": (c_int, [c_vp, c_int, c_u32, c_u32, c_u64, c_vp, c_vp, c_vp,
+                                     P(PlanOpts), P(c_vp)]),
+    "spc3d_plan_build_host": (c_int, [c_int, c_u32, c_u32, c_u64, c_vp, c_vp, P(PlanOpts),
+                                      P(PlanInfo), c_vp, c_vp, c_vp, c_u32, c_vp, c_u32]),
     "spc3d_plan_destroy": (c_int, [c_vp]),
     "spc3d_plan_set_values": (c_int, [c_vp, c_vp]),
     "spc3d_plan_set_values_device": (c_int, [c_vp, c_vp]),

@@ -166,7 +166,8 @@ DevPlanView view_of(const spc3d_plan *p)
 {
     DevPlanView v;
     v.segs = p->segs;
-    v.nseg = p->info.nsegments;
+    v.nseg = p->info.nsegments_padded;
+    v.nqueues = p->info.nqueues;
     v.col = p->col;
     v.perm = p->perm;
     v.sval = p->sval;
@@ -277,6 +278,29 @@ int spc3d_ctx_stream(spc3d_ctx *ctx, void **hip_stream)
         return fail(SPC3D_ERR_INVALID_ARG, "context or out pointer is NULL");
     *hip_stream = (void *)ctx->stream;
     return SPC3D_OK;
+}
+
+int spc3d_ctx_probe_xcd(spc3d_ctx *ctx, uint32_t nblocks, uint32_t *xcd)
+{
+    if (!live(ctx) || (nblocks && !xcd))
+        return fail(SPC3D_ERR_INVALID_ARG, "context or output is NULL");
+    if (nblocks == 0)
+        return SPC3D_OK;
+    int rc = use_device(ctx);
+    if (rc)
+        return rc;
+    uint32_t *dev = nullptr;
+    rc = dev_alloc(&dev, (size_t)nblocks);
+    if (rc)
+        return rc;
+    hipError_t e = launch_xcc_probe(dev, nblocks, ctx->stream);
+    if (e != hipSuccess) {
+        (void)hipFree(dev);
+        return fail_hip(e, "xcc probe");
+    }
+    rc = copy_d2h(ctx, xcd, dev, (size_t)nblocks * sizeof(uint32_t));
+    (void)hipFree(dev);
+    return rc;
 }
 
 int spc3d_timer_mark(spc3d_ctx *ctx, int slot)
@@ -515,24 +539,56 @@ static void fill_info(spc3d_plan_info &info, const HostPlan &H)
     info.nnz = H.nnz;
     info.rows_touched = H.rows_touched;
     info.cols_touched = H.cols_touched;
-    info.nsegments = (uint32_t)H.segs.size();
+    info.nsegments = H.nseg_real;
+    info.nsegments_padded = (uint32_t)H.segs.size();
     info.nsplit_rows = (uint32_t)H.splits.size();
     info.npartial_slots = H.nslots;
     info.max_row_nnz = H.max_row_nnz;
     info.seg_max = H.seg_max;
     info.order_is_identity = H.identity ? 1 : 0;
+    info.nqueues = H.nqueues;
+    info.hot_cols = H.hot_cols;
+    info.hub_rows = H.hub_rows;
+    info.hot_entries = H.hot_entries;
 }
 
-int spc3d_plan_build_host(uint32_t nrows, uint32_t ncols, uint64_t nnz, const uint32_t *ii,
-                          const uint32_t *jj, uint32_t seg_max, spc3d_plan_info *info,
-                          uint32_t *col, uint32_t *perm, uint32_t *segs, uint32_t seg_cap,
-                          uint32_t *splits, uint32_t split_cap)
+// Library defaults, overridable field by field.  With XCD slicing, 3 MiB of
+// each 4 MiB L2 is planned for dense rows, the rest is left to the streams.
+static int resolve_opts(int dtype, const spc3d_plan_opts *o, PlanOpts &out)
+{
+    spc3d_plan_opts z;
+    std::memset(&z, 0, sizeof z);
+    if (o)
+        z = *o;
+    if (z.reserved[0] || z.reserved[1] || z.reserved[2])
+        return fail(SPC3D_ERR_INVALID_ARG, "spc3d_plan_opts.reserved must be 0");
+    if (z.xcd_slices != 0 && z.xcd_slices != 1 && z.xcd_slices != 8)
+        return fail(SPC3D_ERR_INVALID_ARG, "xcd_slices must be 0, 1 or 8");
+    out.seg_max = z.seg_max;
+    out.hub_min = z.hub_min;
+    out.xcd_slices = z.xcd_slices;
+    const uint64_t k = z.k_hint ? z.k_hint : 64;
+    const uint64_t bytes = z.l2_hot_bytes ? z.l2_hot_bytes : 3u << 20;
+    out.hot_cols = (uint32_t)(bytes / (k * elem_size(dtype)));
+    return SPC3D_OK;
+}
+
+int spc3d_plan_build_host(int dtype, uint32_t nrows, uint32_t ncols, uint64_t nnz,
+                          const uint32_t *ii, const uint32_t *jj, const spc3d_plan_opts *opts,
+                          spc3d_plan_info *info, uint32_t *col, uint32_t *perm, uint32_t *segs,
+                          uint32_t seg_cap, uint32_t *splits, uint32_t split_cap)
 {
     if (!info)
         return fail(SPC3D_ERR_INVALID_ARG, "info is NULL");
+    if (!dtype_ok(dtype))
+        return fail(SPC3D_ERR_INVALID_ARG, "unknown dtype");
+    PlanOpts po;
+    int rc = resolve_opts(dtype, opts, po);
+    if (rc)
+        return rc;
     HostPlan H;
     std::string err;
-    int rc = build_host_plan(nrows, ncols, nnz, ii, jj, seg_max, H, err);
+    rc = build_host_plan(nrows, ncols, nnz, ii, jj, po, H, err);
     if (rc != SPC3D_OK)
         return fail(rc, err);
     fill_info(*info, H);
@@ -554,8 +610,8 @@ int spc3d_plan_build_host(uint32_t nrows, uint32_t ncols, uint64_t nnz, const ui
 }
 
 int spc3d_plan_create_ex(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t ncols, uint64_t nnz,
-                         const uint32_t *ii, const uint32_t *jj, const void *vv, uint32_t seg_max,
-                         spc3d_plan **out)
+                         const uint32_t *ii, const uint32_t *jj, const void *vv,
+                         const spc3d_plan_opts *opts, spc3d_plan **out)
 {
     if (!out)
         return fail(SPC3D_ERR_INVALID_ARG, "out is NULL");
@@ -564,9 +620,13 @@ int spc3d_plan_create_ex(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t nco
         return fail(SPC3D_ERR_INVALID_ARG, "unknown dtype");
     // The pattern is checked before the device is touched, so that a bad
     // index is reported as such on a machine without a GPU as well.
+    PlanOpts po;
+    int rc = resolve_opts(dtype, opts, po);
+    if (rc)
+        return rc;
     HostPlan H;
     std::string err;
-    int rc = build_host_plan(nrows, ncols, nnz, ii, jj, seg_max, H, err);
+    rc = build_host_plan(nrows, ncols, nnz, ii, jj, po, H, err);
     if (rc != SPC3D_OK)
         return fail(rc, err);
     if (!live(ctx))
@@ -613,13 +673,24 @@ int spc3d_plan_create_ex(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t nco
 int spc3d_plan_create(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t ncols, uint64_t nnz,
                       const uint32_t *ii, const uint32_t *jj, const void *vv, spc3d_plan **out)
 {
-    uint32_t seg_max = 0;
-    if (const char *s = std::getenv("SPC3D_SEG_MAX")) {
-        const long v = std::atol(s);
-        if (v > 0 && v <= 65536)
-            seg_max = (uint32_t)v;
-    }
-    return spc3d_plan_create_ex(ctx, dtype, nrows, ncols, nnz, ii, jj, vv, seg_max, out);
+    // Defaults, each overridable from the environment for tuning runs.
+    spc3d_plan_opts o;
+    std::memset(&o, 0, sizeof o);
+    struct {
+        const char *name;
+        uint32_t *field;
+    } env[] = {{"SPC3D_SEG_MAX", &o.seg_max},
+               {"SPC3D_K_HINT", &o.k_hint},
+               {"SPC3D_L2_HOT_BYTES", &o.l2_hot_bytes},
+               {"SPC3D_HUB_MIN", &o.hub_min},
+               {"SPC3D_XCD_SLICES", &o.xcd_slices}};
+    for (auto &e : env)
+        if (const char *s = std::getenv(e.name)) {
+            const long long v = std::atoll(s);
+            if (v > 0 && v <= 0xFFFFFFFFll)
+                *e.field = (uint32_t)v;
+        }
+    return spc3d_plan_create_ex(ctx, dtype, nrows, ncols, nnz, ii, jj, vv, &o, out);
 }
 
 int spc3d_plan_destroy(spc3d_plan *plan)

@@ -11,7 +11,8 @@ namespace spc3d {
 // Device-side view of a plan; all pointers are device pointers.
 struct DevPlanView {
     const Seg *segs = nullptr;
-    uint32_t nseg = 0;
+    uint32_t nseg = 0;                // including padding segments
+    uint32_t nqueues = 1;             // 1, or 8: chunk v of the segments belongs to XCD v % 8
     const uint32_t *col = nullptr;    // [nnz] kernel order
     const uint32_t *perm = nullptr;   // [nnz] kernel order -> caller's position; null if identity
     const void *sval = nullptr;       // [nnz] values in kernel order
@@ -29,6 +30,8 @@ hipError_t launch_spmm(int dtype, const DevPlanView &P, const void *X, void *Y, 
 // out[p] = in[perm[p]] (perm == null: copy)
 hipError_t launch_gather_vals(int dtype, const void *in, const uint32_t *perm, void *out,
                               uint64_t n, hipStream_t stream);
+// out[b] = id of the XCD workgroup b of an nblocks-wide grid ran on
+hipError_t launch_xcc_probe(uint32_t *out, uint32_t nblocks, hipStream_t stream);
 // dst[0..bytes) = src[0..bytes); both 16-byte aligned, non-overlapping
 hipError_t launch_copy(void *dst, const void *src, uint64_t bytes, hipStream_t stream);
 hipError_t launch_fill(int dtype, void *p, uint64_t n, double value, hipStream_t stream);

@@ -32,7 +32,9 @@
 //
 // Streams that are read once (indices, sparse values, segment descriptors, A
 // rows, Y rows) use non-temporal accesses so that the per-XCD L2 is left to
-// the gathered B / X rows, the only operand with reuse.
+// the gathered B / X rows, the only operand with reuse.  The gathers themselves
+// are plain loads: a non-temporal hint on the gathers of low-degree columns
+// was measured to slow both kernels down by 15 to 40 %.
 #include <hip/hip_runtime.h>
 
 #include "kernels.h"
@@ -152,6 +154,32 @@ template <int LPR, int NB> __device__ __forceinline__ bool is_writer(uint32_t su
     return (sub & mask) == 0;
 }
 
+// Segment this lane group works on.  Segments are stored in chunks of kChunk;
+// with nq == 8, chunk v belongs to XCD v % 8.  Workgroups are dispatched to
+// the XCDs round-robin by workgroup id, so workgroup b runs on XCD b % 8 and
+// takes its segments from that XCD's chunks: the dense rows of one column
+// slice are then only ever gathered through one L2.  (If the hardware dealt
+// workgroups differently the result would be the same, only slower.)
+template <int G> __device__ __forceinline__ uint64_t seg_index(uint32_t nq)
+{
+    constexpr uint32_t kSegPerBlock = (kBlock / 64) * G;
+    constexpr uint32_t kBlocksPerChunk = kChunk / kSegPerBlock;
+    static_assert(kChunk % kSegPerBlock == 0, "a chunk is a whole number of workgroups");
+    const uint32_t b = blockIdx.x;
+    uint64_t chunk;
+    uint32_t inner;
+    if (nq == 8) {
+        const uint32_t j = b >> 3;
+        chunk = (uint64_t)(j / kBlocksPerChunk) * 8 + (b & 7u);
+        inner = j % kBlocksPerChunk;
+    } else {
+        chunk = b / kBlocksPerChunk;
+        inner = b % kBlocksPerChunk;
+    }
+    return chunk * kChunk + inner * kSegPerBlock + (threadIdx.x >> 6) * G +
+           (threadIdx.x & 63u) / (64 / G);
+}
+
 template <typename T, int LPR, int VPL>
 __device__ __forceinline__ const typename Vec<T>::type *row_ptr(const T *base, uint32_t row,
                                                                 uint32_t sub)
@@ -212,22 +240,51 @@ sddmm_batch(const typename Vec<T>::type (&a)[VPL], const uint32_t *__restrict__ 
         nt_store(part[0] * sv, C + dst);
 }
 
+// n consecutive entries from p: batches of UB, then UB/2, ..., 1 as n requires.
+template <typename T, int LPR, int VPL, int UB>
+__device__ __forceinline__ void
+sddmm_walk(const typename Vec<T>::type (&a)[VPL], const uint32_t *__restrict__ col,
+           const uint32_t *__restrict__ perm, const T *__restrict__ sval,
+           const T *__restrict__ B, T *__restrict__ C, uint32_t p, uint32_t n, uint32_t sub)
+{
+    for (; n >= UB; n -= UB, p += UB)
+        sddmm_batch<T, LPR, VPL, UB>(a, col, perm, sval, B, C, p, sub);
+    if constexpr (UB > 8)
+        if (n & 8) {
+            sddmm_batch<T, LPR, VPL, 8>(a, col, perm, sval, B, C, p, sub);
+            p += 8;
+        }
+    if constexpr (UB > 4)
+        if (n & 4) {
+            sddmm_batch<T, LPR, VPL, 4>(a, col, perm, sval, B, C, p, sub);
+            p += 4;
+        }
+    if constexpr (UB > 2)
+        if (n & 2) {
+            sddmm_batch<T, LPR, VPL, 2>(a, col, perm, sval, B, C, p, sub);
+            p += 2;
+        }
+    if constexpr (UB > 1)
+        if (n & 1)
+            sddmm_batch<T, LPR, VPL, 1>(a, col, perm, sval, B, C, p, sub);
+}
+
 template <typename T, int LPR, int VPL, int UB>
 __global__ void __launch_bounds__(kBlock)
-sddmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, const uint32_t *__restrict__ col,
-                 const uint32_t *__restrict__ perm, const T *__restrict__ sval,
-                 const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C)
+sddmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq,
+                 const uint32_t *__restrict__ col, const uint32_t *__restrict__ perm,
+                 const T *__restrict__ sval, const T *__restrict__ A, const T *__restrict__ B,
+                 T *__restrict__ C)
 {
     static_assert(UB <= LPR && UB <= 16 && LPR <= 64, "batch must fit the lane group");
     using V = typename Vec<T>::type;
-    constexpr int G = 64 / LPR;
-    const uint32_t lane = threadIdx.x & 63u;
-    const uint32_t sub = lane & (LPR - 1);
-    const uint64_t wave = (uint64_t)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
-    const uint64_t sid = wave * G + lane / LPR;
+    const uint32_t sub = threadIdx.x & (LPR - 1);
+    const uint64_t sid = seg_index<64 / LPR>(nq);
     if (sid >= nseg)
         return;
     const u32x4 sg = nt_load(reinterpret_cast<const u32x4 *>(segs) + sid); // row, start, len, slot
+    if (sg[2] == 0)
+        return;
 
     V a[VPL];
     {
@@ -236,44 +293,25 @@ sddmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, const uint32_t *__
         for (int v = 0; v < VPL; ++v)
             a[v] = nt_load(arow + v * LPR);
     }
-    uint32_t p = sg[1], rem = sg[2];
-    for (; rem >= UB; rem -= UB, p += UB)
-        sddmm_batch<T, LPR, VPL, UB>(a, col, perm, sval, B, C, p, sub);
-    if constexpr (UB > 8)
-        if (rem & 8) {
-            sddmm_batch<T, LPR, VPL, 8>(a, col, perm, sval, B, C, p, sub);
-            p += 8;
-        }
-    if constexpr (UB > 4)
-        if (rem & 4) {
-            sddmm_batch<T, LPR, VPL, 4>(a, col, perm, sval, B, C, p, sub);
-            p += 4;
-        }
-    if constexpr (UB > 2)
-        if (rem & 2) {
-            sddmm_batch<T, LPR, VPL, 2>(a, col, perm, sval, B, C, p, sub);
-            p += 2;
-        }
-    if constexpr (UB > 1)
-        if (rem & 1)
-            sddmm_batch<T, LPR, VPL, 1>(a, col, perm, sval, B, C, p, sub);
+    sddmm_walk<T, LPR, VPL, UB>(a, col, perm, sval, B, C, sg[1], sg[2], sub);
 }
 
 // Any K: one wavefront per segment, lanes stride over K, scalar loads.
 template <typename T>
 __global__ void __launch_bounds__(kBlock)
-sddmm_generic_kernel(const Seg *__restrict__ segs, uint32_t nseg, const uint32_t *__restrict__ col,
-                     const uint32_t *__restrict__ perm, const T *__restrict__ sval,
-                     const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C,
-                     uint32_t K)
+sddmm_generic_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq,
+                     const uint32_t *__restrict__ col, const uint32_t *__restrict__ perm,
+                     const T *__restrict__ sval, const T *__restrict__ A,
+                     const T *__restrict__ B, T *__restrict__ C, uint32_t K)
 {
     const uint32_t lane = threadIdx.x & 63u;
-    const uint64_t sid = (uint64_t)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
+    const uint64_t sid = seg_index<1>(nq);
     if (sid >= nseg)
         return;
     const Seg sg = segs[sid];
+    const uint32_t len = sg.len;
     const T *arow = A + (size_t)sg.row * K;
-    for (uint32_t i = 0; i < sg.len; ++i) {
+    for (uint32_t i = 0; i < len; ++i) {
         const uint32_t p = sg.start + i;
         const T *brow = B + (size_t)col[p] * K;
         T acc = (T)0;
@@ -311,7 +349,7 @@ spmm_batch(typename Vec<T>::type (&acc)[VPL], const uint32_t *__restrict__ col,
             x[u][v] = xrow[v * LPR];
     }
     __builtin_amdgcn_sched_barrier(0); // all gathers in flight before the first use
-    // Entries are added in kernel order, which within a row is the caller's order.
+    // Entries are added in kernel order.
 #pragma unroll
     for (int u = 0; u < NB; ++u)
 #pragma unroll
@@ -320,21 +358,48 @@ spmm_batch(typename Vec<T>::type (&acc)[VPL], const uint32_t *__restrict__ col,
 }
 
 template <typename T, int LPR, int VPL, int UB>
+__device__ __forceinline__ void
+spmm_walk(typename Vec<T>::type (&acc)[VPL], const uint32_t *__restrict__ col,
+          const T *__restrict__ sval, const T *__restrict__ X, uint32_t p, uint32_t n,
+          uint32_t sub)
+{
+    for (; n >= UB; n -= UB, p += UB)
+        spmm_batch<T, LPR, VPL, UB>(acc, col, sval, X, p, sub);
+    if constexpr (UB > 8)
+        if (n & 8) {
+            spmm_batch<T, LPR, VPL, 8>(acc, col, sval, X, p, sub);
+            p += 8;
+        }
+    if constexpr (UB > 4)
+        if (n & 4) {
+            spmm_batch<T, LPR, VPL, 4>(acc, col, sval, X, p, sub);
+            p += 4;
+        }
+    if constexpr (UB > 2)
+        if (n & 2) {
+            spmm_batch<T, LPR, VPL, 2>(acc, col, sval, X, p, sub);
+            p += 2;
+        }
+    if constexpr (UB > 1)
+        if (n & 1)
+            spmm_batch<T, LPR, VPL, 1>(acc, col, sval, X, p, sub);
+}
+
+template <typename T, int LPR, int VPL, int UB>
 __global__ void __launch_bounds__(kBlock)
-spmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, const uint32_t *__restrict__ col,
-                const T *__restrict__ sval, const T *__restrict__ X, T *__restrict__ Y,
-                T *__restrict__ partial)
+spmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq,
+                const uint32_t *__restrict__ col, const T *__restrict__ sval,
+                const T *__restrict__ X, T *__restrict__ Y, T *__restrict__ partial)
 {
     static_assert(UB <= LPR && UB <= 16 && LPR <= 64, "batch must fit the lane group");
     using V = typename Vec<T>::type;
-    constexpr int G = 64 / LPR;
-    const uint32_t lane = threadIdx.x & 63u;
-    const uint32_t sub = lane & (LPR - 1);
-    const uint64_t wave = (uint64_t)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
-    const uint64_t sid = wave * G + lane / LPR;
+    const uint32_t sub = threadIdx.x & (LPR - 1);
+    const uint64_t sid = seg_index<64 / LPR>(nq);
     if (sid >= nseg)
         return;
     const u32x4 sg = nt_load(reinterpret_cast<const u32x4 *>(segs) + sid); // row, start, len, slot
+    if (sg[2] == 0)
+        return;
     const bool whole = sg[3] == kWholeRow;
     V *dst = const_cast<V *>(whole ? row_ptr<T, LPR, VPL>(Y, sg[0], sub)
                                    : row_ptr<T, LPR, VPL>(partial, sg[3], sub));
@@ -350,27 +415,7 @@ spmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, const uint32_t *__r
         for (int v = 0; v < VPL; ++v)
             y0[v] = nt_load(dst + v * LPR);
     }
-    uint32_t p = sg[1], rem = sg[2];
-    for (; rem >= UB; rem -= UB, p += UB)
-        spmm_batch<T, LPR, VPL, UB>(acc, col, sval, X, p, sub);
-    if constexpr (UB > 8)
-        if (rem & 8) {
-            spmm_batch<T, LPR, VPL, 8>(acc, col, sval, X, p, sub);
-            p += 8;
-        }
-    if constexpr (UB > 4)
-        if (rem & 4) {
-            spmm_batch<T, LPR, VPL, 4>(acc, col, sval, X, p, sub);
-            p += 4;
-        }
-    if constexpr (UB > 2)
-        if (rem & 2) {
-            spmm_batch<T, LPR, VPL, 2>(acc, col, sval, X, p, sub);
-            p += 2;
-        }
-    if constexpr (UB > 1)
-        if (rem & 1)
-            spmm_batch<T, LPR, VPL, 1>(acc, col, sval, X, p, sub);
+    spmm_walk<T, LPR, VPL, UB>(acc, col, sval, X, sg[1], sg[2], sub);
     if (whole) {
 #pragma unroll
         for (int v = 0; v < VPL; ++v)
@@ -384,20 +429,24 @@ spmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, const uint32_t *__r
 
 template <typename T>
 __global__ void __launch_bounds__(kBlock)
-spmm_generic_kernel(const Seg *__restrict__ segs, uint32_t nseg, const uint32_t *__restrict__ col,
-                    const T *__restrict__ sval, const T *__restrict__ X, T *__restrict__ Y,
-                    T *__restrict__ partial, uint32_t K)
+spmm_generic_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq,
+                    const uint32_t *__restrict__ col, const T *__restrict__ sval,
+                    const T *__restrict__ X, T *__restrict__ Y, T *__restrict__ partial,
+                    uint32_t K)
 {
     const uint32_t lane = threadIdx.x & 63u;
-    const uint64_t sid = (uint64_t)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
+    const uint64_t sid = seg_index<1>(nq);
     if (sid >= nseg)
         return;
     const Seg sg = segs[sid];
+    const uint32_t len = sg.len;
+    if (len == 0)
+        return;
     const bool whole = sg.slot == kWholeRow;
     T *dst = whole ? Y + (size_t)sg.row * K : partial + (size_t)sg.slot * K;
     for (uint32_t j = lane; j < K; j += 64) {
         T acc = (T)0;
-        for (uint32_t i = 0; i < sg.len; ++i) {
+        for (uint32_t i = 0; i < len; ++i) {
             const uint32_t p = sg.start + i;
             acc += sval[p] * X[(size_t)col[p] * K + j];
         }
@@ -418,6 +467,15 @@ spmm_fixup_kernel(const SplitRow *__restrict__ splits, const T *__restrict__ par
             s += partial[(size_t)(sr.first_slot + q) * K + j];
         Y[(size_t)sr.row * K + j] += s;
     }
+}
+
+// XCD on which each workgroup of a 1-D grid runs (hardware register XCC_ID).
+__global__ void __launch_bounds__(64) xcc_probe_kernel(uint32_t *__restrict__ out)
+{
+    // s_getreg_b32 hwreg(HW_REG_XCC_ID = 20, offset 0, width 4)
+    const uint32_t id = __builtin_amdgcn_s_getreg(20 | (0 << 6) | ((4 - 1) << 11));
+    if (threadIdx.x == 0)
+        out[blockIdx.x] = id;
 }
 
 // ------------------------------------------------------------- utilities ----
@@ -482,26 +540,31 @@ Shape pick_shape(size_t elem, uint32_t K)
     return {0, 0, 0};
 }
 
-inline uint32_t blocks_for_groups(uint32_t nseg, int groups_per_wave)
+// Workgroups needed to cover nseg segments (a whole number of chunks, and of
+// rounds of 8 chunks when they are dealt to XCDs) with `groups_per_wave` segments
+// per wavefront.
+inline uint32_t blocks_for_groups(uint32_t nseg, uint32_t nq, int groups_per_wave)
 {
-    const uint64_t waves = ((uint64_t)nseg + groups_per_wave - 1) / groups_per_wave;
-    return (uint32_t)((waves + kBlock / 64 - 1) / (kBlock / 64));
+    uint64_t chunks = ((uint64_t)nseg + kChunk - 1) / kChunk;
+    if (nq == 8)
+        chunks = (chunks + 7) / 8 * 8;
+    return (uint32_t)(chunks * (kChunk / ((kBlock / 64) * groups_per_wave)));
 }
 
 template <typename T, int LPR, int VPL, int UB>
 void run_sddmm(const DevPlanView &P, const T *A, const T *B, T *C, hipStream_t st)
 {
-    const uint32_t grid = blocks_for_groups(P.nseg, 64 / LPR);
+    const uint32_t grid = blocks_for_groups(P.nseg, P.nqueues, 64 / LPR);
     hipLaunchKernelGGL((sddmm_seg_kernel<T, LPR, VPL, UB>), dim3(grid), dim3(kBlock), 0, st, P.segs,
-                       P.nseg, P.col, P.perm, (const T *)P.sval, A, B, C);
+                       P.nseg, P.nqueues, P.col, P.perm, (const T *)P.sval, A, B, C);
 }
 
 template <typename T, int LPR, int VPL, int UB>
 void run_spmm(const DevPlanView &P, const T *X, T *Y, hipStream_t st)
 {
-    const uint32_t grid = blocks_for_groups(P.nseg, 64 / LPR);
+    const uint32_t grid = blocks_for_groups(P.nseg, P.nqueues, 64 / LPR);
     hipLaunchKernelGGL((spmm_seg_kernel<T, LPR, VPL, UB>), dim3(grid), dim3(kBlock), 0, st, P.segs,
-                       P.nseg, P.col, (const T *)P.sval, X, Y, (T *)P.partial);
+                       P.nseg, P.nqueues, P.col, (const T *)P.sval, X, Y, (T *)P.partial);
 }
 
 // (LPR, VPL, UB): UB * VPL 16-byte gathers are in flight per lane.
@@ -526,9 +589,9 @@ hipError_t sddmm_typed(const DevPlanView &P, const void *A, const void *B, void 
     SPC3D_FOR_SHAPES(X)
 #undef X
     if (!done) {
-        const uint32_t grid = blocks_for_groups(P.nseg, 1);
+        const uint32_t grid = blocks_for_groups(P.nseg, P.nqueues, 1);
         hipLaunchKernelGGL((sddmm_generic_kernel<T>), dim3(grid), dim3(kBlock), 0, st, P.segs,
-                           P.nseg, P.col, P.perm, (const T *)P.sval, (const T *)A, (const T *)B,
+                           P.nseg, P.nqueues, P.col, P.perm, (const T *)P.sval, (const T *)A, (const T *)B,
                            (T *)C, K);
     }
     return hipGetLastError();
@@ -549,9 +612,9 @@ hipError_t spmm_typed(const DevPlanView &P, const void *X_, void *Y, uint32_t K,
     SPC3D_FOR_SHAPES(X)
 #undef X
     if (!done) {
-        const uint32_t grid = blocks_for_groups(P.nseg, 1);
+        const uint32_t grid = blocks_for_groups(P.nseg, P.nqueues, 1);
         hipLaunchKernelGGL((spmm_generic_kernel<T>), dim3(grid), dim3(kBlock), 0, st, P.segs,
-                           P.nseg, P.col, (const T *)P.sval, (const T *)X_, (T *)Y,
+                           P.nseg, P.nqueues, P.col, (const T *)P.sval, (const T *)X_, (T *)Y,
                            (T *)P.partial, K);
     }
     hipError_t e = hipGetLastError();
@@ -599,6 +662,14 @@ hipError_t launch_gather_vals(int dtype, const void *in, const uint32_t *perm, v
     else
         hipLaunchKernelGGL((gather_kernel<float>), dim3(stream_grid(n)), dim3(kBlock), 0, stream,
                            (const float *)in, perm, (float *)out, n);
+    return hipGetLastError();
+}
+
+hipError_t launch_xcc_probe(uint32_t *out, uint32_t nblocks, hipStream_t stream)
+{
+    if (nblocks == 0)
+        return hipSuccess;
+    hipLaunchKernelGGL(xcc_probe_kernel, dim3(nblocks), dim3(64), 0, stream, out);
     return hipGetLastError();
 }
 

@@ -1,8 +1,10 @@
-// Host-side plan construction: validation, row grouping, segmentation.
+// Host-side plan construction: validation, column classification, row
+// grouping, segmentation and the dealing of segments to XCD queues.
 #include "plan_host.h"
 
 #include <algorithm>
 #include <cstdio>
+#include <new>
 
 #include "../../include/spcomm3d_hip.h"
 
@@ -38,14 +40,70 @@ int validate_coo(uint32_t nrows, uint32_t ncols, uint64_t nnz, const uint32_t *i
     return SPC3D_ERR_BAD_INDEX;
 }
 
+namespace {
+
+// Column classes (XCD slicing).  A "replicated" column is hot enough that every
+// L2 keeps its dense row; a "slice s" column is meant to be kept by the L2 of
+// XCD s, so the entries of hub rows in it are queued to XCD s; "cold" columns
+// are not expected to stay in any L2.
+constexpr uint8_t kRep = 8, kCold = 9;
+constexpr uint8_t kAnyQueue = 0xFF;
+constexpr uint32_t kSlices = 8;
+
+struct Piece {
+    Seg seg;
+    uint8_t queue;
+};
+
+// Columns are dealt to slices in degree order, back and forth (0..7, 7..0, ...),
+// so that no slice collects the larger column of every round.
+inline uint8_t slice_of_rank(uint64_t i)
+{
+    const uint32_t pos = (uint32_t)(i % kSlices);
+    return (uint8_t)(((i / kSlices) & 1) ? kSlices - 1 - pos : pos);
+}
+
+// Replicated-hot entries of a hub row ride with one of its slices; a hash of
+// the row id picks it (low row-id bits correlate with degree in R-MAT-like
+// graphs, so they would not spread the rows evenly).
+inline uint32_t rep_slice(uint32_t row) { return (row * 2654435761u) >> 29; }
+
+inline uint32_t seg_len(const Seg &s) { return s.len; }
+
+// Stable counting sort of `v` by segment length, longest first.
+void sort_longest_first(std::vector<Piece> &v, uint32_t seg_max)
+{
+    std::vector<uint32_t> bucket((size_t)seg_max + 2, 0);
+    for (const Piece &p : v)
+        ++bucket[seg_max - seg_len(p.seg) + 1];
+    for (uint32_t i = 0; i <= seg_max; ++i)
+        bucket[i + 1] += bucket[i];
+    std::vector<Piece> out(v.size());
+    for (const Piece &p : v)
+        out[bucket[seg_max - seg_len(p.seg)]++] = p;
+    v.swap(out);
+}
+
+} // namespace
+
+uint32_t default_seg_max(uint64_t nnz)
+{
+    uint32_t s = 64;
+    while (s < 2048 && (uint64_t)s * 2 * 2048 <= nnz)
+        s *= 2;
+    return s;
+}
+
 int build_host_plan(uint32_t nrows, uint32_t ncols, uint64_t nnz, const uint32_t *ii,
-                    const uint32_t *jj, uint32_t seg_max, HostPlan &out, std::string &err)
+                    const uint32_t *jj, const PlanOpts &opts, HostPlan &out, std::string &err)
 {
     int rc = validate_coo(nrows, ncols, nnz, ii, jj, err);
     if (rc != SPC3D_OK)
         return rc;
-    if (seg_max == 0)
-        seg_max = kDefaultSegMax;
+    const uint32_t seg_max =
+        std::min<uint32_t>(opts.seg_max ? opts.seg_max : default_seg_max(nnz), 1u << 30);
+    const uint32_t hub_min = opts.hub_min ? opts.hub_min : kDefaultHubMin;
+    const bool want_slices = opts.xcd_slices == kSlices;
 
     HostPlan P;
     P.nrows = nrows;
@@ -53,10 +111,12 @@ int build_host_plan(uint32_t nrows, uint32_t ncols, uint64_t nnz, const uint32_t
     P.nnz = nnz;
     P.seg_max = seg_max;
     try {
-        // Row histogram -> exclusive prefix.
-        std::vector<uint32_t> rowptr((size_t)nrows + 1, 0);
-        for (uint64_t e = 0; e < nnz; ++e)
+        // ---- histograms -------------------------------------------------
+        std::vector<uint32_t> rowptr((size_t)nrows + 1, 0), coldeg((size_t)ncols, 0);
+        for (uint64_t e = 0; e < nnz; ++e) {
             ++rowptr[(size_t)ii[e] + 1];
+            ++coldeg[jj[e]];
+        }
         uint32_t touched = 0, maxlen = 0;
         for (uint32_t r = 0; r < nrows; ++r) {
             const uint32_t len = rowptr[(size_t)r + 1];
@@ -64,65 +124,193 @@ int build_host_plan(uint32_t nrows, uint32_t ncols, uint64_t nnz, const uint32_t
             maxlen = std::max(maxlen, len);
             rowptr[(size_t)r + 1] += rowptr[r];
         }
+        uint32_t ctouched = 0, maxcdeg = 0;
+        for (uint32_t c = 0; c < ncols; ++c) {
+            ctouched += coldeg[c] != 0;
+            maxcdeg = std::max(maxcdeg, coldeg[c]);
+        }
         P.rows_touched = touched;
+        P.cols_touched = ctouched;
         P.max_row_nnz = maxlen;
 
-        // Stable scatter into row groups.
+        // ---- column classes (XCD slicing only) -----------------------------
+        // One L2 is expected to keep hot_cols dense rows.  A sixth of that goes to
+        // the columns replicated in every L2, the rest to this XCD's slice of
+        // the next 8 * (5/6) hot_cols columns.  Slicing is used only when the
+        // column degrees are skewed enough for that hot set to cover well more
+        // than its share of the entries.
+        std::vector<uint8_t> cls;
+        bool slices = false;
+        if (want_slices && opts.hot_cols > 0 && ctouched > opts.hot_cols && nnz > 0) {
+            const uint32_t h1 = opts.hot_cols;
+            const uint32_t hrep = std::max<uint32_t>(h1 / 6, 1);
+            const uint64_t htot =
+                std::min<uint64_t>((uint64_t)hrep + (uint64_t)(h1 - hrep) * kSlices, ctouched);
+            // columns by degree, highest first (counting sort, stable in column id)
+            std::vector<uint32_t> bucket((size_t)maxcdeg + 2, 0);
+            for (uint32_t c = 0; c < ncols; ++c)
+                if (coldeg[c])
+                    ++bucket[maxcdeg - coldeg[c] + 1];
+            for (uint32_t d = 0; d <= maxcdeg; ++d)
+                bucket[d + 1] += bucket[d];
+            std::vector<uint32_t> order(ctouched);
+            for (uint32_t c = 0; c < ncols; ++c)
+                if (coldeg[c])
+                    order[bucket[maxcdeg - coldeg[c]]++] = c;
+            uint64_t covered = 0;
+            for (uint64_t i = 0; i < htot; ++i)
+                covered += coldeg[order[i]];
+            const double coverage = (double)covered / (double)nnz;
+            const double share = (double)htot / (double)ctouched;
+            if (coverage >= 0.2 && coverage >= 2.0 * share) {
+                slices = true;
+                cls.assign((size_t)ncols, kCold);
+                for (uint64_t i = 0; i < htot; ++i)
+                    cls[order[i]] = i < hrep ? kRep : slice_of_rank(i - hrep);
+                P.hot_cols = (uint32_t)htot;
+                P.hot_entries = covered;
+            }
+        }
+
+        // ---- hub rows: group counts -------------------------------------------
+        // A hub row's entries are grouped [slice 0 | ... | slice 7 | cold], its
+        // replicated-hot entries riding with slice rep_slice(row).  Other rows
+        // keep the caller's order.
+        std::vector<int32_t> hubidx;
+        std::vector<uint32_t> hubcnt; // 9 group counts per hub row
+        auto group_of = [&](uint32_t r, uint32_t c) -> uint32_t {
+            const uint8_t k = cls[c];
+            return k == kRep ? rep_slice(r) : (k == kCold ? 8u : k);
+        };
+        if (slices) {
+            hubidx.assign((size_t)nrows, -1);
+            uint32_t nh = 0;
+            for (uint32_t r = 0; r < nrows; ++r)
+                if (rowptr[(size_t)r + 1] - rowptr[r] >= hub_min)
+                    hubidx[r] = (int32_t)nh++;
+            P.hub_rows = nh;
+            hubcnt.assign((size_t)nh * 9, 0);
+            for (uint64_t e = 0; e < nnz; ++e)
+                if (hubidx[ii[e]] >= 0)
+                    ++hubcnt[(size_t)hubidx[ii[e]] * 9 + group_of(ii[e], jj[e])];
+        }
+
+        // ---- stable scatter into kernel order ------------------------------
         P.col.resize(nnz);
         P.perm.resize(nnz);
         {
-            std::vector<uint32_t> cursor(rowptr.begin(), rowptr.end() - 1);
-            std::vector<uint8_t> seen((size_t)ncols, 0);
+            std::vector<uint32_t> cur(rowptr.begin(), rowptr.end() - 1);
+            std::vector<uint32_t> cur_h(hubcnt.size()); // hub rows: 9 cursors
+            for (uint32_t r = 0; slices && r < nrows; ++r) {
+                if (hubidx[r] < 0)
+                    continue;
+                uint32_t at = rowptr[r];
+                for (uint32_t k = 0; k < 9; ++k) {
+                    cur_h[(size_t)hubidx[r] * 9 + k] = at;
+                    at += hubcnt[(size_t)hubidx[r] * 9 + k];
+                }
+            }
             uint32_t notid = 0;
             for (uint64_t e = 0; e < nnz; ++e) {
-                const uint32_t p = cursor[ii[e]]++;
+                const uint32_t r = ii[e];
+                const uint32_t p = (slices && hubidx[r] >= 0)
+                                       ? cur_h[(size_t)hubidx[r] * 9 + group_of(r, jj[e])]++
+                                       : cur[r]++;
                 P.perm[p] = (uint32_t)e;
                 P.col[p] = jj[e];
                 notid |= (uint32_t)(p != (uint32_t)e);
-                seen[jj[e]] = 1;
             }
             P.identity = notid == 0;
-            uint32_t ct = 0;
-            for (uint32_t c = 0; c < ncols; ++c)
-                ct += seen[c];
-            P.cols_touched = ct;
         }
 
-        // Segments in row order.
-        std::vector<Seg> segs;
-        segs.reserve((size_t)touched + nnz / seg_max + 1);
+        // ---- segments --------------------------------------------------------
+        std::vector<Piece> pieces;
+        pieces.reserve((size_t)touched + nnz / seg_max + (size_t)P.hub_rows * 4 + 1);
         uint32_t nslots = 0;
+        std::vector<Piece> rowp;
+        // Cuts [start, start+len) into balanced parts of at most seg_max entries.
+        auto add_range = [&](uint32_t row, uint32_t start, uint32_t len, uint8_t queue) {
+            if (len == 0)
+                return;
+            const uint32_t parts = (len + seg_max - 1) / seg_max;
+            const uint32_t base = len / parts, rem = len % parts;
+            uint32_t at = 0;
+            for (uint32_t q = 0; q < parts; ++q) {
+                const uint32_t l = base + (q < rem ? 1u : 0u);
+                rowp.push_back(Piece{Seg{row, start + at, l, kWholeRow}, queue});
+                at += l;
+            }
+        };
         for (uint32_t r = 0; r < nrows; ++r) {
             const uint32_t s = rowptr[r], len = rowptr[(size_t)r + 1] - s;
             if (len == 0)
                 continue;
-            if (len <= seg_max) {
-                segs.push_back(Seg{r, s, len, kWholeRow});
-                continue;
+            rowp.clear();
+            if (slices && hubidx[r] >= 0) {
+                uint32_t at = s;
+                for (uint32_t k = 0; k < 9; ++k) {
+                    const uint32_t n = hubcnt[(size_t)hubidx[r] * 9 + k];
+                    add_range(r, at, n, k < 8 ? (uint8_t)k : kAnyQueue);
+                    at += n;
+                }
+            } else {
+                add_range(r, s, len, kAnyQueue);
             }
-            const uint32_t parts = (len + seg_max - 1) / seg_max;
-            const uint32_t base = len / parts, rem = len % parts;
-            P.splits.push_back(SplitRow{r, nslots, parts, 0});
-            uint32_t at = s;
-            for (uint32_t q = 0; q < parts; ++q) {
-                const uint32_t l = base + (q < rem ? 1u : 0u);
-                segs.push_back(Seg{r, at, l, nslots++});
-                at += l;
+            if (rowp.size() > 1) {
+                P.splits.push_back(SplitRow{r, nslots, (uint32_t)rowp.size(), 0});
+                for (Piece &p : rowp)
+                    p.seg.slot = nslots++;
             }
+            pieces.insert(pieces.end(), rowp.begin(), rowp.end());
         }
         P.nslots = nslots;
+        P.nseg_real = (uint32_t)pieces.size();
 
-        // Longest first (lane groups of one wavefront then run the same trip
-        // count); equal lengths keep row order (neighbouring rows of banded
-        // patterns share dense rows).  Counting sort on len in [1, seg_max].
-        std::vector<uint32_t> bucket((size_t)seg_max + 2, 0);
-        for (const Seg &g : segs)
-            ++bucket[seg_max - g.len + 1];
-        for (uint32_t i = 0; i <= seg_max; ++i)
-            bucket[i + 1] += bucket[i];
-        P.segs.resize(segs.size());
-        for (const Seg &g : segs)
-            P.segs[bucket[seg_max - g.len]++] = g;
+        // ---- order and deal ----------------------------------------------------
+        // Longest first, so that the lane groups of one wavefront run the same
+        // trip count; equal lengths keep row order (neighbouring rows of banded
+        // patterns share dense rows).
+        if (!slices) {
+            sort_longest_first(pieces, seg_max);
+            P.nqueues = 1;
+            P.segs.resize(pieces.size());
+            for (size_t i = 0; i < pieces.size(); ++i)
+                P.segs[i] = pieces[i].seg;
+        } else {
+            // Hub pieces go to the queue of their column slice.  The rest go,
+            // longest first, to whichever queue has the least work so far.
+            P.nqueues = kSlices;
+            std::vector<Piece> queue[kSlices], any;
+            uint64_t load[kSlices] = {0};
+            for (const Piece &p : pieces) {
+                if (p.queue == kAnyQueue) {
+                    any.push_back(p);
+                } else {
+                    queue[p.queue].push_back(p);
+                    load[p.queue] += seg_len(p.seg) + 4; // + a per-segment overhead
+                }
+            }
+            sort_longest_first(any, seg_max);
+            for (const Piece &p : any) {
+                uint32_t best = 0;
+                for (uint32_t q = 1; q < kSlices; ++q)
+                    if (load[q] < load[best])
+                        best = q;
+                queue[best].push_back(p);
+                load[best] += seg_len(p.seg) + 4;
+            }
+            size_t nchunks = 0;
+            for (uint32_t q = 0; q < kSlices; ++q) {
+                sort_longest_first(queue[q], seg_max);
+                nchunks = std::max(nchunks, (queue[q].size() + kChunk - 1) / kChunk);
+            }
+            // Chunk i of queue q is global chunk i * 8 + q; short queues are padded
+            // with empty segments.
+            P.segs.assign(nchunks * kSlices * kChunk, Seg{0, 0, 0, kWholeRow});
+            for (uint32_t q = 0; q < kSlices; ++q)
+                for (size_t i = 0; i < queue[q].size(); ++i)
+                    P.segs[((i / kChunk) * kSlices + q) * kChunk + i % kChunk] = queue[q][i].seg;
+        }
     } catch (const std::bad_alloc &) {
         err = "host allocation failed while building the plan";
         return SPC3D_ERR_ALLOC;

@@ -8,9 +8,9 @@
 namespace spc3d {
 
 // One unit of work for a lane group: `len` consecutive entries of one row in
-// kernel order.  slot == kWholeRow: the segment is the whole row (SpMM adds
-// its sum straight into Y); otherwise the row was cut and the segment's sum
-// goes to partial-sum row `slot`.
+// kernel order.  slot == kWholeRow: the segment is the whole row (SpMM adds its
+// sum straight into Y); otherwise the row was cut and the segment's sum goes to
+// partial-sum row `slot`.  len == 0 is padding.
 struct Seg {
     uint32_t row;
     uint32_t start;
@@ -18,6 +18,7 @@ struct Seg {
     uint32_t slot;
 };
 constexpr uint32_t kWholeRow = 0xFFFFFFFFu;
+constexpr uint32_t kChunk = 64; // segments per chunk; one chunk is dealt to one XCD
 
 // A row cut into several segments: its partial sums are slots
 // [first_slot, first_slot + nslots).
@@ -28,6 +29,14 @@ struct SplitRow {
     uint32_t pad;
 };
 
+// Zero in any field selects the default.
+struct PlanOpts {
+    uint32_t seg_max = 0;    // longest segment (default: by nnz, 64 .. 2048)
+    uint32_t xcd_slices = 0; // 8: hot columns are dealt to the 8 XCD L2s; 0 / 1: off (default)
+    uint32_t hot_cols = 0;   // slicing: dense rows one L2 is expected to keep
+    uint32_t hub_min = 0;    // slicing: rows with at least this many entries are cut by slice (default 128)
+};
+
 struct HostPlan {
     uint32_t nrows = 0, ncols = 0;
     uint64_t nnz = 0;
@@ -35,23 +44,35 @@ struct HostPlan {
     uint32_t max_row_nnz = 0;
     uint32_t seg_max = 0;
     uint32_t nslots = 0;
+    uint32_t nseg_real = 0;        // segments with entries (segs.size() includes padding)
+    uint32_t nqueues = 1;          // 1, or 8 when chunks are dealt round-robin to XCDs
+    uint32_t hot_cols = 0;         // columns dealt to slices or replicated (0: slicing off)
+    uint64_t hot_entries = 0;      // entries in those columns
+    uint32_t hub_rows = 0;         // rows cut by column slice
     bool identity = true;          // perm[p] == p for all p
     std::vector<uint32_t> col;     // [nnz] column of kernel-order entry p
     std::vector<uint32_t> perm;    // [nnz] caller's position of kernel-order entry p
-    std::vector<Seg> segs;         // longest first; equal lengths keep row order
+    std::vector<Seg> segs;         // chunked: chunk v (64 segments) belongs to queue v % nqueues
     std::vector<SplitRow> splits;
 };
 
-constexpr uint32_t kDefaultSegMax = 128;
+constexpr uint32_t kDefaultHubMin = 128;
+
+// Default longest segment: long enough that few rows are cut (each cut costs a
+// partial-sum row in SpMM), short enough that the longest segments do not
+// outlast the rest of the grid: nnz / 2048 rounded down to a power of two,
+// within [64, 2048].
+uint32_t default_seg_max(uint64_t nnz);
 
 // Returns 0, or an spc3d_status value with `err` filled.
 int validate_coo(uint32_t nrows, uint32_t ncols, uint64_t nnz, const uint32_t *ii,
                  const uint32_t *jj, std::string &err);
 
-// Validates, then builds.  Entries are grouped by row with a stable counting
-// sort, so within a row the caller's order (the order the reference
-// accumulates in, core_ops.cpp:26-34) is kept.
+// Validates, then builds.  Entries are grouped by row, the caller's order kept
+// inside a row (the order the reference accumulates in, core_ops.cpp:26-34).
+// With XCD slicing, the entries of a hub row are further grouped by the slice
+// of their column, the caller's order kept inside each group.
 int build_host_plan(uint32_t nrows, uint32_t ncols, uint64_t nnz, const uint32_t *ii,
-                    const uint32_t *jj, uint32_t seg_max, HostPlan &out, std::string &err);
+                    const uint32_t *jj, const PlanOpts &opts, HostPlan &out, std::string &err);
 
 } // namespace spc3d

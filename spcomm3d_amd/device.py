@@ -7,7 +7,7 @@ import ctypes
 import numpy as np
 
 from . import _capi as capi
-from ._capi import PlanInfo, check
+from ._capi import PlanInfo, PlanOpts, check
 
 _DT = {np.dtype(np.float32): capi.F32, np.dtype(np.float64): capi.F64}
 _NP = {capi.F32: np.dtype(np.float32), capi.F64: np.dtype(np.float64)}
@@ -26,6 +26,18 @@ def dtype_code(dtype) -> int:
 
 def _vp(a: np.ndarray | None):
     return None if a is None else a.ctypes.data_as(ctypes.c_void_p)
+
+
+def make_opts(seg_max=None, k_hint=None, l2_hot_bytes=None, hub_min=None,
+              xcd_slices=None) -> PlanOpts:
+    """``spc3d_plan_opts``; ``None`` keeps the library default."""
+    o = PlanOpts()
+    o.seg_max = int(seg_max or 0)
+    o.k_hint = int(k_hint or 0)
+    o.l2_hot_bytes = int(l2_hot_bytes or 0)
+    o.hub_min = int(hub_min or 0)
+    o.xcd_slices = int(xcd_slices or 0)
+    return o
 
 
 def _as_idx(a, name: str) -> np.ndarray:
@@ -85,8 +97,18 @@ class Context:
     def vals(self, n: int, dtype) -> "Vals":
         return Vals(self, n, dtype)
 
-    def plan(self, nrows, ncols, ii, jj, vv=None, dtype=None, seg_max: int | None = None) -> "Plan":
-        return Plan(self, nrows, ncols, ii, jj, vv, dtype, seg_max)
+    def plan(self, nrows, ncols, ii, jj, vv=None, dtype=None, seg_max: int | None = None,
+             **opts) -> "Plan":
+        """``opts``: fields of :func:`make_opts`; none given = ``spc3d_plan_create`` defaults."""
+        if seg_max is not None:
+            opts["seg_max"] = seg_max
+        return Plan(self, nrows, ncols, ii, jj, vv, dtype, opts or None)
+
+    def probe_xcd(self, nblocks: int) -> np.ndarray:
+        """XCD id each workgroup of an ``nblocks``-wide grid ran on (``spc3d_ctx_probe_xcd``)."""
+        out = np.zeros(nblocks, dtype=np.uint32)
+        check(self._lib.spc3d_ctx_probe_xcd(self._h, nblocks, _vp(out)), "spc3d_ctx_probe_xcd")
+        return out
 
     # -- hot path ----------------------------------------------------------
     def sddmm(self, S: "Plan", A: "Panel", B: "Panel", C: "Vals"):
@@ -223,7 +245,7 @@ class Plan:
     order plus its values (``spc3d_plan``)."""
 
     def __init__(self, ctx: Context, nrows, ncols, ii, jj, vv=None, dtype=None,
-                 seg_max: int | None = None):
+                 opts: dict | None = None):
         ii = _as_idx(ii, "ii")
         jj = _as_idx(jj, "jj")
         if ii.shape != jj.shape or ii.ndim != 1:
@@ -242,12 +264,13 @@ class Plan:
             raise ValueError("vv dtype differs from the plan dtype")
         h = ctypes.c_void_p()
         lib = ctx._lib
-        if seg_max is None:
+        if opts is None:
             rc = lib.spc3d_plan_create(ctx._h, self.code, int(nrows), int(ncols), ii.size, _vp(ii),
                                        _vp(jj), _vp(vv), ctypes.byref(h))
         else:
             rc = lib.spc3d_plan_create_ex(ctx._h, self.code, int(nrows), int(ncols), ii.size,
-                                          _vp(ii), _vp(jj), _vp(vv), int(seg_max), ctypes.byref(h))
+                                          _vp(ii), _vp(jj), _vp(vv),
+                                          ctypes.byref(make_opts(**opts)), ctypes.byref(h))
         check(rc, "spc3d_plan_create")
         self._h = h
         self.nnz = int(ii.size)
@@ -288,24 +311,29 @@ def coo_validate(nrows: int, ncols: int, ii, jj) -> None:
           "spc3d_coo_validate")
 
 
-def plan_build_host(nrows: int, ncols: int, ii, jj, seg_max: int = 0) -> dict:
+def plan_build_host(nrows: int, ncols: int, ii, jj, dtype="f32", **opts) -> dict:
     """Host-only view of the kernel-order form of a pattern
-    (``spc3d_plan_build_host``): needs no GPU.  Returns ``info``, ``col``,
-    ``perm``, ``segs`` (``[nseg, 4]``: row, start, len, slot) and ``splits``
-    (``[nsplit, 3]``: row, first_slot, nslots)."""
+    (``spc3d_plan_build_host``): needs no GPU.  ``opts`` as :func:`make_opts`.
+    Returns ``info``, ``col``, ``perm``, ``segs`` (``[nseg_padded, 4]``: row,
+    start, len, slot) and ``splits`` (``[nsplit, 3]``: row,
+    first_slot, nslots)."""
     lib = capi.load()
     ii = _as_idx(ii, "ii")
     jj = _as_idx(jj, "jj")
+    code = dtype_code(dtype)
+    o = make_opts(**opts)
     info = PlanInfo()
-    check(lib.spc3d_plan_build_host(int(nrows), int(ncols), ii.size, _vp(ii), _vp(jj),
-                                    int(seg_max), ctypes.byref(info), None, None, None, 0, None, 0),
+    check(lib.spc3d_plan_build_host(code, int(nrows), int(ncols), ii.size, _vp(ii), _vp(jj),
+                                    ctypes.byref(o), ctypes.byref(info), None, None, None, 0,
+                                    None, 0),
           "spc3d_plan_build_host")
     col = np.empty(ii.size, dtype=np.uint32)
     perm = np.empty(ii.size, dtype=np.uint32)
-    segs = np.empty((info.nsegments, 4), dtype=np.uint32)
+    segs = np.empty((info.nsegments_padded, 4), dtype=np.uint32)
     splits = np.empty((info.nsplit_rows, 3), dtype=np.uint32)
-    check(lib.spc3d_plan_build_host(int(nrows), int(ncols), ii.size, _vp(ii), _vp(jj),
-                                    int(seg_max), ctypes.byref(info), _vp(col), _vp(perm),
-                                    _vp(segs), info.nsegments, _vp(splits), info.nsplit_rows),
+    check(lib.spc3d_plan_build_host(code, int(nrows), int(ncols), ii.size, _vp(ii), _vp(jj),
+                                    ctypes.byref(o), ctypes.byref(info), _vp(col), _vp(perm),
+                                    _vp(segs), info.nsegments_padded, _vp(splits),
+                                    info.nsplit_rows),
           "spc3d_plan_build_host")
     return {"info": info, "col": col, "perm": perm, "segs": segs, "splits": splits}

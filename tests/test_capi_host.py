@@ -8,6 +8,7 @@ import pytest
 
 from spcomm3d_amd import _capi as capi
 from spcomm3d_amd import device
+from spcomm3d_amd import workloads as W
 
 WHOLE = 0xFFFFFFFF
 
@@ -80,65 +81,96 @@ def test_no_device_fails_loudly_without_fallback():
 
 
 # ---- host plan builder --------------------------------------------------------
-def _check_plan(nrows, ncols, ii, jj, seg_max):
-    P = device.plan_build_host(nrows, ncols, ii, jj, seg_max)
+def _check_plan(nrows, ncols, ii, jj, **opts):
+    P = device.plan_build_host(nrows, ncols, ii, jj, "f32", **opts)
     info, col, perm, segs, splits = P["info"], P["col"], P["perm"], P["segs"], P["splits"]
     nnz = ii.size
-    assert info.nnz == nnz and info.seg_max == (seg_max or 128)
-    # perm is a permutation; kernel order is grouped by row, stable within a row
+    assert info.nnz == nnz
+    if opts.get("seg_max"):
+        assert info.seg_max == opts["seg_max"]
+    # perm is a permutation; kernel order is grouped by row
     assert np.array_equal(np.sort(perm), np.arange(nnz, dtype=np.uint32))
     assert np.array_equal(col, jj[perm])
     rows_k = ii[perm]
     assert np.all(np.diff(rows_k.astype(np.int64)) >= 0)
-    same = rows_k[1:] == rows_k[:-1]
-    assert np.all(perm[1:][same] > perm[:-1][same]), "caller's order must survive inside a row"
+    if info.nqueues == 1:  # no slicing: the caller's order survives inside every row
+        same = rows_k[1:] == rows_k[:-1]
+        assert np.all(perm[1:][same] > perm[:-1][same])
     assert bool(info.order_is_identity) == bool(np.array_equal(perm, np.arange(nnz)))
     assert info.rows_touched == np.unique(ii).size and info.cols_touched == np.unique(jj).size
     assert info.max_row_nnz == (np.bincount(ii).max() if nnz else 0)
-    # segments tile [0, nnz) exactly once and stay inside one row
-    assert segs.shape[0] == info.nsegments
+    # real segments tile [0, nnz) exactly once and stay inside one row; the rest is padding
+    assert segs.shape[0] == info.nsegments_padded
+    real = segs[segs[:, 2] > 0]
+    assert real.shape[0] == info.nsegments
+    assert np.all(segs[segs[:, 2] == 0][:, 3] == WHOLE)
     cover = np.zeros(nnz, dtype=np.int32)
-    for row, start, ln, slot in segs:
+    for row, start, ln, slot in real:
         assert 1 <= ln <= info.seg_max
         cover[start:start + ln] += 1
         assert np.all(rows_k[start:start + ln] == row)
+        if info.nqueues == 1:
+            continue
     assert np.all(cover == 1)
-    # longest first; ties keep row order
-    lens = segs[:, 2].astype(np.int64)
-    assert np.all(np.diff(lens) <= 0)
-    tie = lens[1:] == lens[:-1]
-    assert np.all((segs[1:, 1] > segs[:-1, 1])[tie])
+    # inside each queue: longest first; ties keep position order
+    chunk = np.arange(segs.shape[0]) // 64
+    for q in range(info.nqueues):
+        mine = segs[(chunk % info.nqueues) == q]
+        mine = mine[mine[:, 2] > 0]
+        lens = mine[:, 2].astype(np.int64)
+        assert np.all(np.diff(lens) <= 0)
+        if info.nqueues == 1:
+            tie = lens[1:] == lens[:-1]
+            assert np.all((mine[1:, 1] > mine[:-1, 1])[tie])
+    if info.nqueues == 8:
+        assert segs.shape[0] % (8 * 64) == 0
     # cut rows: slots are a partition of [0, npartial_slots), whole rows carry the marker
-    counts = np.bincount(ii, minlength=nrows) if nnz else np.zeros(nrows, dtype=np.int64)
-    cut_rows = np.flatnonzero(counts > info.seg_max)
+    nseg_of_row = np.bincount(real[:, 0], minlength=nrows)
+    cut_rows = np.flatnonzero(nseg_of_row > 1)
     assert np.array_equal(np.sort(splits[:, 0]), cut_rows)
     used = np.zeros(info.npartial_slots, dtype=np.int32)
     for row, first, n in splits:
-        mine = segs[(segs[:, 0] == row)]
-        assert mine.shape[0] == n and n == -(-counts[row] // info.seg_max)
+        mine = real[real[:, 0] == row]
+        assert mine.shape[0] == n
         assert np.array_equal(np.sort(mine[:, 3]), np.arange(first, first + n))
-        assert mine[:, 2].max() - mine[:, 2].min() <= 1  # balanced pieces
         used[first:first + n] += 1
     assert np.all(used == 1)
-    whole = segs[~np.isin(segs[:, 0], cut_rows)]
+    whole = real[~np.isin(real[:, 0], cut_rows)]
     assert np.all(whole[:, 3] == WHOLE)
+    if info.nqueues == 1:  # rows are cut only when longer than seg_max, into balanced pieces
+        counts = np.bincount(ii, minlength=nrows) if nnz else np.zeros(nrows, dtype=np.int64)
+        assert np.array_equal(cut_rows, np.flatnonzero(counts > info.seg_max))
+        for row in cut_rows:
+            mine = real[real[:, 0] == row]
+            assert mine.shape[0] == -(-counts[row] // info.seg_max)
+            assert mine[:, 2].max() - mine[:, 2].min() <= 1
     return P
 
 
-@pytest.mark.parametrize("seg_max", [0, 4, 7, 64])
+@pytest.mark.parametrize("seg_max", [None, 4, 7, 64])
 def test_plan_random_unsorted_with_duplicates(seg_max):
     rng = np.random.default_rng(3)
     ii = rng.integers(0, 50, 900).astype(np.uint32)
     jj = rng.integers(0, 70, 900).astype(np.uint32)
     ii[:300] = 7  # a hub row
     o = rng.permutation(900)
-    _check_plan(50, 70, ii[o], jj[o], seg_max)
+    _check_plan(50, 70, ii[o], jj[o], seg_max=seg_max)
+
+
+def test_plan_default_seg_max_follows_nnz():
+    e = np.zeros(0, dtype=np.uint32)
+    assert device.plan_build_host(5, 5, e, e)["info"].seg_max == 64
+    w = W.rmat(14, 16, 64)
+    assert device.plan_build_host(w.nrows, w.ncols, w.ii, w.jj)["info"].seg_max == 64
+    w = W.rmat(17, 16, 64)
+    s = device.plan_build_host(w.nrows, w.ncols, w.ii, w.jj)["info"].seg_max
+    assert s == 1 << int(np.log2(w.nnz / 2048)) and 64 <= s <= 2048
 
 
 def test_plan_sorted_input_is_identity_and_empty_rows_are_skipped():
     ii = np.array([1, 1, 4, 4, 4, 9], dtype=np.uint32)
     jj = np.array([5, 2, 0, 0, 3, 1], dtype=np.uint32)
-    P = _check_plan(12, 6, ii, jj, 0)
+    P = _check_plan(12, 6, ii, jj)
     assert P["info"].order_is_identity == 1
     assert P["info"].nsegments == 3 and P["info"].nsplit_rows == 0
     assert sorted(P["segs"][:, 0]) == [1, 4, 9]
@@ -148,11 +180,48 @@ def test_plan_empty_and_single():
     e = np.zeros(0, dtype=np.uint32)
     P = device.plan_build_host(5, 5, e, e)
     assert P["info"].nsegments == 0 and P["info"].nnz == 0 and P["info"].order_is_identity == 1
-    P = _check_plan(1, 1, np.zeros(1, np.uint32), np.zeros(1, np.uint32), 0)
+    P = _check_plan(1, 1, np.zeros(1, np.uint32), np.zeros(1, np.uint32))
     assert P["info"].nsegments == 1
 
 
-def test_plan_build_host_rejects_bad_index_and_small_capacity():
+def test_plan_xcd_slicing_on_skewed_pattern():
+    w = W.rmat(15, 16, 64).shuffled()
+    # a small L2 share so that the 2^15-column panel does not fit and slicing engages
+    P = _check_plan(w.nrows, w.ncols, w.ii, w.jj, xcd_slices=8, l2_hot_bytes=64 * 1024,
+                    hub_min=32, seg_max=256)
+    info, segs = P["info"], P["segs"]
+    assert info.nqueues == 8 and info.hub_rows > 0 and 0 < info.hot_cols < info.cols_touched
+    assert 0.2 * info.nnz < info.hot_entries <= info.nnz
+    # the eight queues carry nearly the same number of entries
+    chunk = np.arange(segs.shape[0]) // 64
+    load = np.array([segs[(chunk % 8) == q][:, 2].sum() for q in range(8)], dtype=np.int64)
+    assert load.max() - load.min() <= 0.02 * load.mean() + 256
+    # inside a hub row the caller's order survives within each piece
+    perm, rows_k = P["perm"], w.ii[P["perm"]]
+    for row, start, ln, slot in segs[segs[:, 2] > 1][:200]:
+        assert np.all(np.diff(perm[start:start + ln].astype(np.int64)) > 0)
+    # every entry of one hub piece with a slice column sits in that slice's queue:
+    # same column -> same queue, wherever it appears in hub rows
+    counts = np.bincount(w.ii, minlength=w.nrows)
+    qcol = {}
+    for idx in np.flatnonzero(segs[:, 2] > 0):
+        row, start, ln, slot = segs[idx]
+        if counts[row] < 32 or slot == WHOLE:
+            continue
+        q = (idx // 64) % 8
+        for c in P["col"][start:start + ln][:4]:
+            qcol.setdefault(int(c), set()).add(int(q))
+    sliced = [c for c, qs in qcol.items() if len(qs) == 1]
+    assert len(sliced) > 0.3 * len(qcol)
+
+
+def test_plan_slicing_stays_off_for_uniform_columns():
+    w = W.erdos_renyi(4096, 16, 32)
+    P = _check_plan(w.nrows, w.ncols, w.ii, w.jj, xcd_slices=8, l2_hot_bytes=16 * 1024)
+    assert P["info"].nqueues == 1 and P["info"].hot_cols == 0 and P["info"].order_is_identity == 1
+
+
+def test_plan_build_host_rejects_bad_arguments():
     lib = capi.load()
     ii = np.array([0, 1, 1], dtype=np.uint32)
     jj = np.array([0, 1, 5], dtype=np.uint32)
@@ -161,6 +230,13 @@ def test_plan_build_host_rejects_bad_index_and_small_capacity():
     info = capi.PlanInfo()
     segs = np.zeros(4, dtype=np.uint32)
     vp = lambda a: a.ctypes.data_as(ctypes.c_void_p)  # noqa: E731
-    rc = lib.spc3d_plan_build_host(2, 6, 3, vp(ii), vp(jj), 0, ctypes.byref(info), None, None,
-                                   vp(segs), 1, None, 0)
+    rc = lib.spc3d_plan_build_host(capi.F32, 2, 6, 3, vp(ii), vp(jj), None, ctypes.byref(info),
+                                   None, None, vp(segs), 1, None, 0)
     assert rc == capi.ERR_SIZE_MISMATCH and info.nsegments == 2
+    with pytest.raises(capi.Spc3dError):
+        device.plan_build_host(2, 6, ii, jj, xcd_slices=4)
+    o = capi.PlanOpts()
+    o.reserved[1] = 7
+    rc = lib.spc3d_plan_build_host(capi.F32, 2, 6, 3, vp(ii), vp(jj), ctypes.byref(o),
+                                   ctypes.byref(info), None, None, None, 0, None, 0)
+    assert rc == capi.ERR_INVALID_ARG

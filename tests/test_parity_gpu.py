@@ -288,3 +288,34 @@ def test_config5_hypergraph_small_k128(ctx):
     A, B, Y0, vv = (w.panel_A("f32"), w.panel_B("f32"), w.panel_Y0("f32"), w.values("f32"))
     check_sddmm(A, B, w.ii, w.jj, vv, gpu_sddmm(ctx, w.nrows, w.ncols, w.ii, w.jj, vv, A, B))
     check_spmm(B, w.ii, w.jj, vv, Y0, gpu_spmm(ctx, w.nrows, w.ncols, w.ii, w.jj, vv, B, Y0))
+
+
+# ---- optional plan layouts ------------------------------------------------------------
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_xcd_sliced_plan_matches_oracle(ctx, dtype):
+    # a small planned L2 share so that slicing engages on this 2^15-column panel
+    w = W.rmat(15, 16, 64).shuffled()
+    A, B, Y0, vv = w.panel_A(dtype), w.panel_B(dtype), w.panel_Y0(dtype), w.values(dtype)
+    S = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, vv, xcd_slices=8, l2_hot_bytes=64 * 1024,
+                 hub_min=32, seg_max=256)
+    assert S.info.nqueues == 8 and S.info.hub_rows > 0
+    dA, dB, dY, dC = ctx.panel_from(A), ctx.panel_from(B), ctx.panel_from(Y0), ctx.vals(w.nnz, dtype)
+    ctx.sddmm(S, dA, dB, dC)
+    ctx.spmm(S, dB, dY)
+    check_sddmm(A, B, w.ii, w.jj, vv, dC.download())
+    check_spmm(B, w.ii, w.jj, vv, Y0, dY.download())
+
+
+def test_workgroups_are_dealt_to_xcds_round_robin(ctx):
+    # what the XCD-sliced plan layout relies on for its speed (not for its results)
+    x = ctx.probe_xcd(1024)
+    assert np.array_equal(x, np.arange(1024) % 8)
+
+
+def test_panel_copy_on_device(ctx):
+    a = np.random.default_rng(0).uniform(-1, 1, (1000, 33)).astype(np.float32)
+    src, dst = ctx.panel_from(a), ctx.panel(1000, 33, np.float32)
+    dst.copy_from(src)
+    assert np.array_equal(dst.download(), a)
+    with pytest.raises(capi.Spc3dError):
+        ctx.panel(1000, 32, np.float32).copy_from(src)
