@@ -92,12 +92,12 @@ typedef struct {
                               a power of two, within 64 .. 2048) */
     uint32_t k_hint;       /* XCD slicing: K the plan will mostly run with (default 64) */
     uint32_t l2_hot_bytes; /* XCD slicing: share of one XCD's 4 MiB L2 planned for dense rows
-                              (default 3 MiB) */
+                              (default 2 MiB) */
     uint32_t hub_min;      /* XCD slicing: rows with at least this many entries are cut by
                               column slice (default 128) */
-    uint32_t xcd_slices;   /* 8: the entries of long rows are dealt to the 8 XCDs by column, so
-                              that each L2 caches its own eighth of the hot dense rows;
-                              0 or 1 (default): off */
+    uint32_t xcd_slices;   /* 8 (default): when the column degrees are skewed, the entries of
+                              long rows are dealt to the 8 XCDs by column, so that each L2
+                              caches its own eighth of the hot dense rows; 1: never */
     uint32_t reserved[3];  /* must be 0 */
 } spc3d_plan_opts;
 

@@ -552,8 +552,8 @@ static void fill_info(spc3d_plan_info &info, const HostPlan &H)
     info.hot_entries = H.hot_entries;
 }
 
-// Library defaults, overridable field by field.  With XCD slicing, 3 MiB of
-// each 4 MiB L2 is planned for dense rows, the rest is left to the streams.
+// Library defaults, overridable field by field.  With XCD slicing, 2 MiB of
+// each 4 MiB L2 is planned for dense rows, the rest is left to everything else.
 static int resolve_opts(int dtype, const spc3d_plan_opts *o, PlanOpts &out)
 {
     spc3d_plan_opts z;
@@ -568,7 +568,7 @@ static int resolve_opts(int dtype, const spc3d_plan_opts *o, PlanOpts &out)
     out.hub_min = z.hub_min;
     out.xcd_slices = z.xcd_slices;
     const uint64_t k = z.k_hint ? z.k_hint : 64;
-    const uint64_t bytes = z.l2_hot_bytes ? z.l2_hot_bytes : 3u << 20;
+    const uint64_t bytes = z.l2_hot_bytes ? z.l2_hot_bytes : 2u << 20;
     out.hot_cols = (uint32_t)(bytes / (k * elem_size(dtype)));
     return SPC3D_OK;
 }

@@ -236,8 +236,15 @@ sddmm_batch(const typename Vec<T>::type (&a)[VPL], const uint32_t *__restrict__ 
         part[u] = acc;
     }
     group_reduce<T, LPR, NB>(part, sub);
-    if (writer)
-        nt_store(part[0] * sv, C + dst);
+    // Results in the caller's order: when that is the kernel order the stores of a
+    // batch fill whole lines and stream out; when it is not they are scattered, and
+    // plain stores let the L2 merge neighbours into lines before writing back.
+    if (writer) {
+        if (perm)
+            C[dst] = part[0] * sv;
+        else
+            nt_store(part[0] * sv, C + dst);
+    }
 }
 
 // n consecutive entries from p: batches of UB, then UB/2, ..., 1 as n requires.

@@ -103,7 +103,7 @@ int build_host_plan(uint32_t nrows, uint32_t ncols, uint64_t nnz, const uint32_t
     const uint32_t seg_max =
         std::min<uint32_t>(opts.seg_max ? opts.seg_max : default_seg_max(nnz), 1u << 30);
     const uint32_t hub_min = opts.hub_min ? opts.hub_min : kDefaultHubMin;
-    const bool want_slices = opts.xcd_slices == kSlices;
+    const bool want_slices = opts.xcd_slices == 0 || opts.xcd_slices == kSlices;
 
     HostPlan P;
     P.nrows = nrows;

@@ -32,7 +32,7 @@ struct SplitRow {
 // Zero in any field selects the default.
 struct PlanOpts {
     uint32_t seg_max = 0;    // longest segment (default: by nnz, 64 .. 2048)
-    uint32_t xcd_slices = 0; // 8: hot columns are dealt to the 8 XCD L2s; 0 / 1: off (default)
+    uint32_t xcd_slices = 0; // 8 (default): hot columns are dealt to the 8 XCD L2s; 1: off
     uint32_t hot_cols = 0;   // slicing: dense rows one L2 is expected to keep
     uint32_t hub_min = 0;    // slicing: rows with at least this many entries are cut by slice (default 128)
 };
