@@ -31,6 +31,16 @@ if ROOT not in sys.path:
 
 METRIC = "SDDMM & SpMM GFLOP/s + % HBM roofline on 1 MI355X, RMAT-20 K=64"
 
+# HBM-side bytes per launch (L2 fills + write-backs) measured with rocprofv3
+# --pmc FETCH_SIZE / WRITE_SIZE, calibrated on a plain copy; they cannot be
+# collected from inside this process, so they are quoted from
+# profiles/sddmm_spmm_rmat20_k64_hbm_traffic.md for the workload they were taken
+# on (default plan options) and left null for any other.  spmm includes its fix-up.
+MEASURED_TRAFFIC = {
+    ("rmat20_ef16", 64, "sorted", "f64"): {"sddmm": 5907.7e6, "spmm": 5434.4e6 + 125.1e6},
+    ("rmat20_ef16", 64, "sorted", "f32"): {"sddmm": 3100.6e6, "spmm": 2582.5e6 + 63.9e6},
+}
+
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
@@ -202,6 +212,10 @@ def main():
     kd = main_r["kernels"][dom]
     from spcomm3d_amd import roofline
 
+    traffic = None
+    if args.seg_max is None and not any(k.startswith("SPC3D_") for k in os.environ):
+        traffic = MEASURED_TRAFFIC.get((w.name, w.k, w.order, args.dtype), {}).get(dom)
+
     line = {
         "metric": METRIC, "value": main_r["gflops"], "unit": "GFLOP/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": main_r["ms_per_step"],
@@ -212,7 +226,7 @@ def main():
                    "rows_touched": main_r["rows_touched"], "cols_touched": main_r["cols_touched"]},
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": kd["strict_gbs"],
                      "peak": roofline.HBM_PEAK_GBS, "unit": "GB/s", "frac": kd["strict_frac"],
-                     "traffic": None, "bytes_per_launch": kd["strict_bytes"],
+                     "traffic": traffic, "bytes_per_launch": kd["strict_bytes"],
                      "ms_per_launch": kd["ms_avg"], "model": "strict (each operand once)"},
         "cpu_baseline": cpu,
         "kernels": main_r["kernels"],
