@@ -461,17 +461,28 @@ spmm_generic_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq,
     }
 }
 
-// One block per cut row: Y[row,:] += partial sums in slot order.
+// Y[row,:] += the partial sums of a cut row, in slot order.  `lanes` (a power of
+// two, <= kBlock) threads share one cut row, kBlock / lanes rows per block.
 template <typename T>
 __global__ void __launch_bounds__(kBlock)
-spmm_fixup_kernel(const SplitRow *__restrict__ splits, const T *__restrict__ partial,
-                  T *__restrict__ Y, uint32_t K)
+spmm_fixup_kernel(const SplitRow *__restrict__ splits, uint32_t nsplit,
+                  const T *__restrict__ partial, T *__restrict__ Y, uint32_t K, uint32_t lanes)
 {
-    const SplitRow sr = splits[blockIdx.x];
-    for (uint32_t j = threadIdx.x; j < K; j += kBlock) {
+    const uint32_t idx = blockIdx.x * (kBlock / lanes) + threadIdx.x / lanes;
+    if (idx >= nsplit)
+        return;
+    const SplitRow sr = splits[idx];
+    for (uint32_t j = threadIdx.x % lanes; j < K; j += lanes) {
+        const T *p = partial + (size_t)sr.first_slot * K + j;
         T s = (T)0;
-        for (uint32_t q = 0; q < sr.nslots; ++q)
-            s += partial[(size_t)(sr.first_slot + q) * K + j];
+        uint32_t q = 0;
+        for (; q + 4 <= sr.nslots; q += 4) { // four loads in flight, added in slot order
+            const T v0 = p[(size_t)(q + 0) * K], v1 = p[(size_t)(q + 1) * K];
+            const T v2 = p[(size_t)(q + 2) * K], v3 = p[(size_t)(q + 3) * K];
+            s = (((s + v0) + v1) + v2) + v3;
+        }
+        for (; q < sr.nslots; ++q)
+            s += p[(size_t)q * K];
         Y[(size_t)sr.row * K + j] += s;
     }
 }
@@ -628,8 +639,13 @@ hipError_t spmm_typed(const DevPlanView &P, const void *X_, void *Y, uint32_t K,
     if (e != hipSuccess)
         return e;
     if (P.nsplit) {
-        hipLaunchKernelGGL((spmm_fixup_kernel<T>), dim3(P.nsplit), dim3(kBlock), 0, st, P.splits,
-                           (const T *)P.partial, (T *)Y, K);
+        uint32_t lanes = 4;
+        while (lanes < (uint32_t)kBlock && lanes < K)
+            lanes *= 2;
+        const uint32_t rows_per_block = kBlock / lanes;
+        hipLaunchKernelGGL((spmm_fixup_kernel<T>),
+                           dim3((P.nsplit + rows_per_block - 1) / rows_per_block), dim3(kBlock), 0,
+                           st, P.splits, P.nsplit, (const T *)P.partial, (T *)Y, K, lanes);
         e = hipGetLastError();
     }
     return e;
