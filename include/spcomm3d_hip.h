@@ -197,6 +197,30 @@ SPC3D_API int spc3d_sddmm(spc3d_ctx *ctx, spc3d_plan *S, const spc3d_panel *A,
                 const spc3d_panel *B, spc3d_vals *C);
 SPC3D_API int spc3d_spmm(spc3d_ctx *ctx, spc3d_plan *A, const spc3d_panel *X, spc3d_panel *Y);
 
+/* ---- the copies either side of a sparse exchange ---------------------------
+ * A row map ties buffer slot i to dense row rows[i] of a panel: the device form
+ * of SparseComm::sendptr / recvptr (src/comm.hpp:41,49; one pointer per row of
+ * dataUnitSize = K reals).  Rows may repeat (several peers can return partial
+ * sums of one row).  rows[i] < panel_rows is checked on the host
+ * (SPC3D_ERR_BAD_INDEX).  The buffer is an spc3d_vals of at least n * K reals,
+ * slot after slot, as sendBuff / recvBuff are.
+ *   spc3d_rows_pack       = copy_to_sendbuff   (src/comm.hpp:90-103):  buf[i,:]  = P[rows[i],:]
+ *   spc3d_rows_unpack     = copy_from_recvbuff (src/comm.hpp:166-177): P[rows[i],:]  = buf[i,:]
+ *   spc3d_rows_unpack_sum = SUM_from_recvbuff  (src/comm.hpp:178-189): P[rows[i],:] += buf[i,:]
+ * For a repeated row the results are those of the reference's sequential loop:
+ * the last slot wins (unpack), slots are added in ascending order (unpack_sum,
+ * no atomics).  Asynchronous on the context's stream. */
+typedef struct spc3d_rowmap spc3d_rowmap;
+SPC3D_API int spc3d_rowmap_create(spc3d_ctx *ctx, uint32_t panel_rows, uint64_t n,
+                        const uint32_t *rows, spc3d_rowmap **out);
+SPC3D_API int spc3d_rowmap_destroy(spc3d_rowmap *map);
+SPC3D_API int spc3d_rows_pack(spc3d_ctx *ctx, const spc3d_panel *P, const spc3d_rowmap *map,
+                    spc3d_vals *buf);
+SPC3D_API int spc3d_rows_unpack(spc3d_ctx *ctx, spc3d_panel *P, const spc3d_rowmap *map,
+                      const spc3d_vals *buf);
+SPC3D_API int spc3d_rows_unpack_sum(spc3d_ctx *ctx, spc3d_panel *P, const spc3d_rowmap *map,
+                          const spc3d_vals *buf);
+
 /* One-shot forms over host memory with exactly the reference's operands:
  * plan, upload, run, download, free.  Synchronous. */
 SPC3D_API int spc3d_sddmm_host(spc3d_ctx *ctx, int dtype, uint32_t m, uint32_t n, uint32_t k,

@@ -139,3 +139,41 @@ ORACLE_API int oracle_spmm_scale_f64(uint32_t ncols, uint32_t nrows, uint32_t k,
     }
     return 0;
 }
+
+/*
+ * The copies either side of the reference's sparse exchanges, restated from
+ * SparseComm (src/comm.hpp): slot i of the buffer holds `unit` reals that
+ * belong to dense row rows[i] of a row-major panel with `unit` columns
+ * (sendptr[i] / recvptr[i] point at the start of that row, comm_setup.cpp:121,131).
+ *   op 0  copy_to_sendbuff   (:90-103)   buf[i,:]  = panel[rows[i],:]
+ *   op 1  copy_from_recvbuff (:166-177)  panel[rows[i],:]  = buf[i,:]
+ *   op 2  SUM_from_recvbuff  (:178-189)  panel[rows[i],:] += buf[i,:]
+ * Slots are visited in ascending order, so for a repeated row the last slot
+ * wins (op 1) and the slots add up in order (op 2).
+ * Pinned in tests/test_rows.py by numpy fancy indexing / np.add.at, by
+ * unpack(pack(P)) == P on distinct rows, and by the slot-order rule on repeats.
+ */
+#define DEFINE_ROWS(NAME, REAL)                                                \
+    ORACLE_API int NAME(int op, uint32_t panel_rows, uint32_t unit,            \
+                        REAL *panel, uint64_t n, const uint32_t *rows,         \
+                        REAL *buf)                                             \
+    {                                                                          \
+        for (uint64_t i = 0; i < n; ++i) {                                     \
+            if (rows[i] >= panel_rows)                                         \
+                return -1;                                                     \
+            REAL *p = panel + (size_t)rows[i] * unit;                          \
+            REAL *b = buf + (size_t)i * unit;                                  \
+            for (uint32_t j = 0; j < unit; ++j) {                              \
+                if (op == 0)                                                   \
+                    b[j] = p[j];                                               \
+                else if (op == 1)                                              \
+                    p[j] = b[j];                                               \
+                else                                                           \
+                    p[j] += b[j];                                              \
+            }                                                                  \
+        }                                                                      \
+        return 0;                                                              \
+    }
+
+DEFINE_ROWS(oracle_rows_f64, double)
+DEFINE_ROWS(oracle_rows_f32, float)

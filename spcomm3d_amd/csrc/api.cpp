@@ -11,6 +11,7 @@
 #include <cstring>
 #include <new>
 #include <string>
+#include <vector>
 
 #include "kernels.h"
 #include "plan_host.h"
@@ -48,6 +49,7 @@ constexpr uint32_t kMagicCtx = 0x53433343;   // live handles carry a tag so that
 constexpr uint32_t kMagicPanel = 0x53433350; // stale or foreign pointer is refused
 constexpr uint32_t kMagicVals = 0x53433356;  // instead of dereferenced further
 constexpr uint32_t kMagicPlan = 0x5343334c;
+constexpr uint32_t kMagicRowMap = 0x5343334d;
 constexpr int kTimerSlots = 4096;
 
 inline size_t elem_size(int dtype) { return dtype == SPC3D_F64 ? 8 : 4; }
@@ -79,6 +81,14 @@ struct spc3d_vals {
     void *dev;
 };
 
+struct spc3d_rowmap {
+    uint32_t magic;
+    spc3d_ctx *ctx;
+    uint32_t panel_rows;
+    uint32_t nslots, nuniq;
+    uint32_t *rows, *urows, *ptr, *slots; // device
+};
+
 struct spc3d_plan {
     uint32_t magic;
     spc3d_ctx *ctx;
@@ -101,6 +111,7 @@ bool live(const spc3d_ctx *c) { return c && c->magic == kMagicCtx; }
 bool live(const spc3d_panel *p) { return p && p->magic == kMagicPanel && live(p->ctx); }
 bool live(const spc3d_vals *v) { return v && v->magic == kMagicVals && live(v->ctx); }
 bool live(const spc3d_plan *p) { return p && p->magic == kMagicPlan && live(p->ctx); }
+bool live(const spc3d_rowmap *p) { return p && p->magic == kMagicRowMap && live(p->ctx); }
 
 int use_device(const spc3d_ctx *ctx)
 {
@@ -835,6 +846,139 @@ int spc3d_spmm(spc3d_ctx *ctx, spc3d_plan *Ap, const spc3d_panel *X, spc3d_panel
     }
     HIP_TRY(launch_spmm(Ap->dtype, view_of(Ap), X->dev, Y->dev, K, ctx->stream));
     return SPC3D_OK;
+}
+
+/* ---- row maps and the pack / unpack copies ------------------------------------ */
+int spc3d_rowmap_create(spc3d_ctx *ctx, uint32_t panel_rows, uint64_t n, const uint32_t *rows,
+                        spc3d_rowmap **out)
+{
+    if (!out)
+        return fail(SPC3D_ERR_INVALID_ARG, "out is NULL");
+    *out = nullptr;
+    if (n && !rows)
+        return fail(SPC3D_ERR_INVALID_ARG, "rows is NULL");
+    if (n >= (1ull << 32))
+        return fail(SPC3D_ERR_TOO_LARGE, "more than 2^32 - 1 slots");
+    for (uint64_t i = 0; i < n; ++i)
+        if (rows[i] >= panel_rows) {
+            char buf[128];
+            std::snprintf(buf, sizeof buf, "slot %llu names row %u of a panel with %u rows",
+                          (unsigned long long)i, rows[i], panel_rows);
+            return fail(SPC3D_ERR_BAD_INDEX, buf);
+        }
+    if (!live(ctx))
+        return fail(SPC3D_ERR_INVALID_ARG, "context is NULL or destroyed");
+    // Group the slots by row, ascending inside a row (stable counting sort).
+    std::vector<uint32_t> cnt, urows, ptr, slots;
+    try {
+        cnt.assign((size_t)panel_rows + 1, 0);
+        for (uint64_t i = 0; i < n; ++i)
+            ++cnt[(size_t)rows[i] + 1];
+        std::vector<uint32_t> start((size_t)panel_rows, 0);
+        ptr.push_back(0);
+        uint32_t at = 0;
+        for (uint32_t r = 0; r < panel_rows; ++r) {
+            start[r] = at;
+            if (cnt[(size_t)r + 1]) {
+                urows.push_back(r);
+                at += cnt[(size_t)r + 1];
+                ptr.push_back(at);
+            }
+        }
+        slots.resize(n);
+        for (uint64_t i = 0; i < n; ++i)
+            slots[start[rows[i]]++] = (uint32_t)i;
+    } catch (const std::bad_alloc &) {
+        return fail(SPC3D_ERR_ALLOC, "host allocation failed");
+    }
+    int rc = use_device(ctx);
+    if (rc)
+        return rc;
+    spc3d_rowmap *m = new (std::nothrow) spc3d_rowmap();
+    if (!m)
+        return fail(SPC3D_ERR_ALLOC, "host allocation failed");
+    m->ctx = ctx;
+    m->panel_rows = panel_rows;
+    m->nslots = (uint32_t)n;
+    m->nuniq = (uint32_t)urows.size();
+    rc = dev_alloc(&m->rows, (size_t)n);
+    if (!rc) rc = dev_alloc(&m->urows, urows.size());
+    if (!rc) rc = dev_alloc(&m->ptr, n ? ptr.size() : 0);
+    if (!rc) rc = dev_alloc(&m->slots, (size_t)n);
+    if (!rc) rc = copy_h2d(ctx, m->rows, rows, (size_t)n * 4);
+    if (!rc) rc = copy_h2d(ctx, m->urows, urows.data(), urows.size() * 4);
+    if (!rc && n) rc = copy_h2d(ctx, m->ptr, ptr.data(), ptr.size() * 4);
+    if (!rc) rc = copy_h2d(ctx, m->slots, slots.data(), (size_t)n * 4);
+    if (rc) {
+        if (m->rows) (void)hipFree(m->rows);
+        if (m->urows) (void)hipFree(m->urows);
+        if (m->ptr) (void)hipFree(m->ptr);
+        if (m->slots) (void)hipFree(m->slots);
+        delete m;
+        return rc;
+    }
+    m->magic = kMagicRowMap;
+    *out = m;
+    return SPC3D_OK;
+}
+
+int spc3d_rowmap_destroy(spc3d_rowmap *m)
+{
+    if (!live(m))
+        return fail(SPC3D_ERR_INVALID_ARG, "row map is NULL or destroyed");
+    (void)hipSetDevice(m->ctx->device);
+    (void)hipStreamSynchronize(m->ctx->stream);
+    if (m->rows) (void)hipFree(m->rows);
+    if (m->urows) (void)hipFree(m->urows);
+    if (m->ptr) (void)hipFree(m->ptr);
+    if (m->slots) (void)hipFree(m->slots);
+    m->magic = 0;
+    delete m;
+    return SPC3D_OK;
+}
+
+static int rows_op(int op, spc3d_ctx *ctx, const spc3d_panel *P, const spc3d_rowmap *map,
+                   const spc3d_vals *buf)
+{
+    if (!live(ctx) || !live(P) || !live(map) || !live(buf))
+        return fail(SPC3D_ERR_INVALID_ARG, "a handle is NULL or destroyed");
+    if (P->ctx != ctx || map->ctx != ctx || buf->ctx != ctx)
+        return fail(SPC3D_ERR_INVALID_ARG, "operands belong to different contexts");
+    if (buf->dtype != P->dtype)
+        return fail(SPC3D_ERR_SIZE_MISMATCH, "buffer dtype differs from the panel's");
+    if (P->m < map->panel_rows)
+        return fail(SPC3D_ERR_SIZE_MISMATCH, "panel has fewer rows than the row map was made for");
+    if (buf->n < (uint64_t)map->nslots * P->n)
+        return fail(SPC3D_ERR_SIZE_MISMATCH, "buffer holds fewer than n * K reals");
+    int rc = use_device(ctx);
+    if (rc)
+        return rc;
+    RowMapView v;
+    v.rows = map->rows;
+    v.urows = map->urows;
+    v.ptr = map->ptr;
+    v.slots = map->slots;
+    v.nslots = map->nslots;
+    v.nuniq = map->nuniq;
+    HIP_TRY(launch_rows(op, P->dtype, P->dev, v, P->n, buf->dev, ctx->stream));
+    return SPC3D_OK;
+}
+
+int spc3d_rows_pack(spc3d_ctx *ctx, const spc3d_panel *P, const spc3d_rowmap *map, spc3d_vals *buf)
+{
+    return rows_op(0, ctx, P, map, buf);
+}
+
+int spc3d_rows_unpack(spc3d_ctx *ctx, spc3d_panel *P, const spc3d_rowmap *map,
+                      const spc3d_vals *buf)
+{
+    return rows_op(1, ctx, P, map, buf);
+}
+
+int spc3d_rows_unpack_sum(spc3d_ctx *ctx, spc3d_panel *P, const spc3d_rowmap *map,
+                          const spc3d_vals *buf)
+{
+    return rows_op(2, ctx, P, map, buf);
 }
 
 int spc3d_sddmm_host(spc3d_ctx *ctx, int dtype, uint32_t m, uint32_t n, uint32_t k, const void *A,

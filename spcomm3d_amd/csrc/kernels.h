@@ -30,6 +30,18 @@ hipError_t launch_spmm(int dtype, const DevPlanView &P, const void *X, void *Y, 
 // out[p] = in[perm[p]] (perm == null: copy)
 hipError_t launch_gather_vals(int dtype, const void *in, const uint32_t *perm, void *out,
                               uint64_t n, hipStream_t stream);
+// Device-side view of a row map (buffer slot i <-> dense row rows[i]).
+struct RowMapView {
+    const uint32_t *rows = nullptr;  // [nslots]
+    const uint32_t *urows = nullptr; // [nuniq] distinct rows
+    const uint32_t *ptr = nullptr;   // [nuniq + 1] into slots
+    const uint32_t *slots = nullptr; // [nslots] slots grouped by row, ascending inside a row
+    uint32_t nslots = 0, nuniq = 0;
+};
+// op 0: buf[i,:] = panel[rows[i],:]; op 1: panel[rows[i],:] = buf[i,:] (last slot of a row
+// wins); op 2: panel[rows[i],:] += buf[i,:] in slot order.  K reals per row.
+hipError_t launch_rows(int op, int dtype, void *panel, const RowMapView &M, uint32_t K, void *buf,
+                       hipStream_t stream);
 // out[b] = id of the XCD workgroup b of an nblocks-wide grid ran on
 hipError_t launch_xcc_probe(uint32_t *out, uint32_t nblocks, hipStream_t stream);
 // dst[0..bytes) = src[0..bytes); both 16-byte aligned, non-overlapping

@@ -487,6 +487,54 @@ spmm_fixup_kernel(const SplitRow *__restrict__ splits, uint32_t nsplit,
     }
 }
 
+// ---------------------------------------------- row pack / unpack (comm buffers) ----
+// The copies either side of the reference's sparse exchanges
+// (SparseComm::copy_to_sendbuff / copy_from_recvbuff / SUM_from_recvbuff,
+// src/comm.hpp:90-103,166-189): buffer slot i holds the dense row rows[i].
+// W = what one lane moves (a 16-byte vector of reals when the row size allows,
+// else one real); upr = units of W per row.
+
+// buf[i, :] = panel[rows[i], :]
+template <typename W>
+__global__ void __launch_bounds__(kBlock)
+rows_pack_kernel(const W *__restrict__ panel, const uint32_t *__restrict__ rows, uint64_t total,
+                 uint32_t upr, W *__restrict__ buf)
+{
+    const uint64_t stride = (uint64_t)gridDim.x * kBlock;
+    for (uint64_t t = (uint64_t)blockIdx.x * kBlock + threadIdx.x; t < total; t += stride) {
+        const uint64_t slot = t / upr;
+        const uint32_t v = (uint32_t)(t - slot * upr);
+        nt_store(panel[(uint64_t)rows[slot] * upr + v], buf + t);
+    }
+}
+
+// For every distinct destination row u (urows[u], buffer slots slots[ptr[u] ..
+// ptr[u+1]) in ascending slot order): ADD = false: panel row = its last slot
+// (what the reference's sequential copy leaves); ADD = true: panel row += each
+// slot in order (the reference's sequential sum, bit for bit).
+template <typename W, bool ADD>
+__global__ void __launch_bounds__(kBlock)
+rows_unpack_kernel(W *__restrict__ panel, const uint32_t *__restrict__ urows,
+                   const uint32_t *__restrict__ ptr, const uint32_t *__restrict__ slots,
+                   uint64_t total, uint32_t upr, const W *__restrict__ buf)
+{
+    const uint64_t stride = (uint64_t)gridDim.x * kBlock;
+    for (uint64_t t = (uint64_t)blockIdx.x * kBlock + threadIdx.x; t < total; t += stride) {
+        const uint64_t u = t / upr;
+        const uint32_t v = (uint32_t)(t - u * upr);
+        W *dst = panel + (uint64_t)urows[u] * upr + v;
+        const uint32_t lo = ptr[u], hi = ptr[u + 1];
+        if (!ADD) {
+            *dst = nt_load(buf + (uint64_t)slots[hi - 1] * upr + v);
+        } else {
+            W acc = *dst;
+            for (uint32_t s = lo; s < hi; ++s)
+                acc += nt_load(buf + (uint64_t)slots[s] * upr + v);
+            *dst = acc;
+        }
+    }
+}
+
 // XCD on which each workgroup of a 1-D grid runs (hardware register XCC_ID).
 __global__ void __launch_bounds__(64) xcc_probe_kernel(uint32_t *__restrict__ out)
 {
@@ -686,6 +734,45 @@ hipError_t launch_gather_vals(int dtype, const void *in, const uint32_t *perm, v
         hipLaunchKernelGGL((gather_kernel<float>), dim3(stream_grid(n)), dim3(kBlock), 0, stream,
                            (const float *)in, perm, (float *)out, n);
     return hipGetLastError();
+}
+
+namespace {
+template <typename W>
+hipError_t rows_typed(int op, void *panel, const RowMapView &M, uint32_t upr, void *buf,
+                      hipStream_t st)
+{
+    if (op == 0) {
+        const uint64_t total = (uint64_t)M.nslots * upr;
+        hipLaunchKernelGGL((rows_pack_kernel<W>), dim3(stream_grid(total)), dim3(kBlock), 0, st,
+                           (const W *)panel, M.rows, total, upr, (W *)buf);
+    } else {
+        const uint64_t total = (uint64_t)M.nuniq * upr;
+        if (op == 1)
+            hipLaunchKernelGGL((rows_unpack_kernel<W, false>), dim3(stream_grid(total)),
+                               dim3(kBlock), 0, st, (W *)panel, M.urows, M.ptr, M.slots, total, upr,
+                               (const W *)buf);
+        else
+            hipLaunchKernelGGL((rows_unpack_kernel<W, true>), dim3(stream_grid(total)),
+                               dim3(kBlock), 0, st, (W *)panel, M.urows, M.ptr, M.slots, total, upr,
+                               (const W *)buf);
+    }
+    return hipGetLastError();
+}
+} // namespace
+
+hipError_t launch_rows(int op, int dtype, void *panel, const RowMapView &M, uint32_t K, void *buf,
+                       hipStream_t stream)
+{
+    if (M.nslots == 0 || K == 0)
+        return hipSuccess;
+    const size_t row_bytes = (size_t)K * (dtype == 1 ? 8 : 4);
+    if (row_bytes % 16 == 0) {
+        const uint32_t upr = (uint32_t)(row_bytes / 16);
+        return dtype == 1 ? rows_typed<Vec<double>::type>(op, panel, M, upr, buf, stream)
+                          : rows_typed<Vec<float>::type>(op, panel, M, upr, buf, stream);
+    }
+    return dtype == 1 ? rows_typed<double>(op, panel, M, K, buf, stream)
+                      : rows_typed<float>(op, panel, M, K, buf, stream);
 }
 
 hipError_t launch_xcc_probe(uint32_t *out, uint32_t nblocks, hipStream_t stream)

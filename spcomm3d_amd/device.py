@@ -303,6 +303,45 @@ class Plan:
             pass
 
 
+class RowMap:
+    """Buffer slot i <-> dense row ``rows[i]`` of a panel (``spc3d_rowmap``): the
+    device form of ``SparseComm::sendptr`` / ``recvptr`` (``src/comm.hpp:41,49``)."""
+
+    def __init__(self, ctx: Context, panel_rows: int, rows):
+        rows = _as_idx(rows, "rows")
+        self.ctx, self.n = ctx, int(rows.size)
+        h = ctypes.c_void_p()
+        check(ctx._lib.spc3d_rowmap_create(ctx._h, int(panel_rows), rows.size, _vp(rows),
+                                           ctypes.byref(h)), "spc3d_rowmap_create")
+        self._h = h
+
+    def pack(self, panel: Panel, buf: Vals):
+        """buf[i,:] = panel[rows[i],:]  (``copy_to_sendbuff``, ``src/comm.hpp:90-103``)."""
+        check(self.ctx._lib.spc3d_rows_pack(self.ctx._h, panel._h, self._h, buf._h),
+              "spc3d_rows_pack")
+
+    def unpack(self, panel: Panel, buf: Vals):
+        """panel[rows[i],:] = buf[i,:]  (``copy_from_recvbuff``, ``src/comm.hpp:166-177``)."""
+        check(self.ctx._lib.spc3d_rows_unpack(self.ctx._h, panel._h, self._h, buf._h),
+              "spc3d_rows_unpack")
+
+    def unpack_sum(self, panel: Panel, buf: Vals):
+        """panel[rows[i],:] += buf[i,:]  (``SUM_from_recvbuff``, ``src/comm.hpp:178-189``)."""
+        check(self.ctx._lib.spc3d_rows_unpack_sum(self.ctx._h, panel._h, self._h, buf._h),
+              "spc3d_rows_unpack_sum")
+
+    def close(self):
+        if getattr(self, "_h", None) and getattr(self.ctx, "_h", None):
+            self.ctx._lib.spc3d_rowmap_destroy(self._h)
+        self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
 def coo_validate(nrows: int, ncols: int, ii, jj) -> None:
     """Host-only bounds check of a pattern; raises :class:`BadIndexError`."""
     ii = _as_idx(ii, "ii")
