@@ -1,0 +1,169 @@
+// The two on-disk formats the reference's drivers read, with the reference's
+// names: the MatrixMarket reader `SpKernels::mm` (src/mm.hpp:13-80) and the
+// binary triplet file of tools/read_convert_mm.cpp.
+//
+// Binary layout (tools/read_convert_mm.cpp:81-94, read side :96-115 and
+// src/parallel_io.hpp:61-63,91-94): little-endian, no padding,
+//     uint32 rows, uint32 cols, uint64 nnz,
+//     nnz x { uint32 row, uint32 col, float64 value }      (16 bytes each)
+// indices 0-based.  Values are float64 on disk whatever real_t is in memory.
+#pragma once
+
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <fstream>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "SparseMatrix.hpp"
+#include "basic.hpp"
+
+namespace SpKernels {
+
+// MatrixMarket coordinate reader.  What it does with the file is what the
+// reference does, quirks included:
+//   - "pattern", "symmetric", "complex" are recognised anywhere in the banner;
+//   - entries become 0-based; a pattern entry gets value 1; the imaginary part
+//     of a complex entry is dropped;
+//   - a symmetric file yields 2 x (stored entries): entry i is mirrored into
+//     position i + stored, diagonal entries included (so a diagonal entry
+//     appears twice, src/mm.hpp:53-57);
+//   - nnz = gnnz, nrows = gnrows, ncols = gncols are set from the size line.
+// Unlike the reference it reports a file that cannot be opened or that ends
+// early (std::runtime_error) instead of returning garbage.
+class mm {
+  public:
+    explicit mm(std::string FN) : _FN(std::move(FN)) {}
+    virtual ~mm() = default;
+
+    void read_mm(std::string FN, cooMat &M)
+    {
+        std::ifstream f(FN.c_str());
+        if (!f)
+            throw std::runtime_error("read_mm: cannot open " + FN);
+        std::string banner;
+        std::getline(f, banner);
+        const bool pattern = banner.find("pattern") != std::string::npos;
+        const bool symm = banner.find("symmetric") != std::string::npos;
+        const bool cplx = banner.find("complex") != std::string::npos;
+        while (f.peek() == '%')
+            f.ignore(1 << 20, '\n');
+        idx_t rows = 0, cols = 0;
+        idx_large_t stored = 0;
+        if (!(f >> rows >> cols >> stored))
+            throw std::runtime_error("read_mm: no size line in " + FN);
+        const idx_large_t total = symm ? 2 * stored : stored;
+        M.ii.assign(total, 0);
+        M.jj.assign(total, 0);
+        M.vv.assign(total, (real_t)0);
+        M.gnnz = M.nnz = total;
+        M.gnrows = M.nrows = rows;
+        M.gncols = M.ncols = cols;
+        for (idx_large_t i = 0; i < stored; ++i) {
+            idx_t r = 0, c = 0;
+            double v = 1.0, im = 0.0;
+            f >> r >> c;
+            if (!pattern) {
+                f >> v;
+                if (cplx)
+                    f >> im;
+            }
+            if (!f)
+                throw std::runtime_error("read_mm: " + FN + " ends before its last entry");
+            M.ii[i] = r - 1;
+            M.jj[i] = c - 1;
+            M.vv[i] = (real_t)v;
+            if (symm) {
+                M.ii[i + stored] = c - 1;
+                M.jj[i + stored] = r - 1;
+                M.vv[i + stored] = (real_t)v;
+            }
+        }
+    }
+
+  private:
+    std::string _FN;
+};
+
+// tools/read_convert_mm.cpp:81-94: header from gnrows / gncols / gnnz, then the
+// first gnnz triplets.
+inline void convert_to_binary(const cooMat &C, const std::string &outputFN)
+{
+    if (C.ii.size() < C.gnnz || C.jj.size() < C.gnnz || C.vv.size() < C.gnnz)
+        throw std::out_of_range("convert_to_binary: fewer than gnnz entries");
+    std::ofstream o(outputFN, std::ios::binary | std::ios::trunc);
+    if (!o)
+        throw std::runtime_error("convert_to_binary: cannot open " + outputFN);
+    const std::uint32_t r = C.gnrows, c = C.gncols;
+    const std::uint64_t n = C.gnnz;
+    o.write(reinterpret_cast<const char *>(&r), 4);
+    o.write(reinterpret_cast<const char *>(&c), 4);
+    o.write(reinterpret_cast<const char *>(&n), 8);
+    std::vector<char> block;
+    const idx_large_t kChunk = 1 << 16;
+    for (idx_large_t at = 0; at < n; at += kChunk) {
+        const idx_large_t m = std::min<idx_large_t>(kChunk, n - at);
+        block.resize(m * 16);
+        for (idx_large_t i = 0; i < m; ++i) {
+            const std::uint32_t ri = C.ii[at + i], ci = C.jj[at + i];
+            const double v = (double)C.vv[at + i];
+            std::memcpy(&block[i * 16], &ri, 4);
+            std::memcpy(&block[i * 16 + 4], &ci, 4);
+            std::memcpy(&block[i * 16 + 8], &v, 8);
+        }
+        o.write(block.data(), (std::streamsize)block.size());
+    }
+    if (!o)
+        throw std::runtime_error("convert_to_binary: write to " + outputFN + " failed");
+}
+
+// The serial reader (tools/read_convert_mm.cpp:96-115): fills gnrows, gncols,
+// gnnz and the three arrays.  With single_rank = true it also sets nnz, nrows,
+// ncols to the global sizes, which is what one rank ends up holding after
+// read_bin_parallel_distribute_coo (src/parallel_io.hpp:132-190) before
+// localizeIndices.
+inline void read_binary(const std::string &inFN, cooMat &C, bool single_rank = true)
+{
+    std::ifstream f(inFN, std::ios::binary);
+    if (!f)
+        throw std::runtime_error("read_binary: cannot open " + inFN);
+    std::uint32_t r = 0, c = 0;
+    std::uint64_t n = 0;
+    f.read(reinterpret_cast<char *>(&r), 4);
+    f.read(reinterpret_cast<char *>(&c), 4);
+    f.read(reinterpret_cast<char *>(&n), 8);
+    if (!f)
+        throw std::runtime_error("read_binary: " + inFN + " has no header");
+    C.gnrows = r;
+    C.gncols = c;
+    C.gnnz = n;
+    C.ii.resize(n);
+    C.jj.resize(n);
+    C.vv.resize(n);
+    std::vector<char> block;
+    const idx_large_t kChunk = 1 << 16;
+    for (idx_large_t at = 0; at < n; at += kChunk) {
+        const idx_large_t m = std::min<idx_large_t>(kChunk, n - at);
+        block.resize(m * 16);
+        f.read(block.data(), (std::streamsize)block.size());
+        if (!f)
+            throw std::runtime_error("read_binary: " + inFN + " ends before its last entry");
+        for (idx_large_t i = 0; i < m; ++i) {
+            double v;
+            std::memcpy(&C.ii[at + i], &block[i * 16], 4);
+            std::memcpy(&C.jj[at + i], &block[i * 16 + 4], 4);
+            std::memcpy(&v, &block[i * 16 + 8], 8);
+            C.vv[at + i] = (real_t)v;
+        }
+    }
+    if (single_rank) {
+        C.nnz = n;
+        C.nrows = r;
+        C.ncols = c;
+        C.ownedNnz = (idx_t)n;
+    }
+}
+
+} // namespace SpKernels

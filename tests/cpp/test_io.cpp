@@ -1,0 +1,109 @@
+// Host-only test of spc3d/io.hpp against golden files written by the reference's
+// own converter (tests/golden/io/*.bin, made by tests/golden/make_golden_io.py
+// from the .mtx files beside them): reading a .mtx and converting it must give
+// the reference's bytes; reading the reference's .bin must give the same matrix.
+//
+//   test_io <dir with the golden files>
+#include <cstdio>
+#include <fstream>
+#include <iterator>
+#include <string>
+#include <vector>
+
+#include "spc3d/io.hpp"
+
+using namespace SpKernels;
+
+static int g_fail = 0;
+#define CHECK(cond)                                                                               \
+    do {                                                                                          \
+        if (!(cond)) {                                                                            \
+            std::printf("FAIL %s:%d: %s\n", __FILE__, __LINE__, #cond);                           \
+            ++g_fail;                                                                             \
+        }                                                                                         \
+    } while (0)
+
+static std::vector<char> slurp(const std::string &fn)
+{
+    std::ifstream f(fn, std::ios::binary);
+    return std::vector<char>((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
+}
+
+static void check_file(const std::string &dir, const char *stem, idx_large_t want_nnz)
+{
+    const std::string mtx = dir + "/" + stem + ".mtx", bin = dir + "/" + stem + ".bin";
+    cooMat M;
+    mm reader(mtx);
+    reader.read_mm(mtx, M);
+    CHECK(M.nnz == want_nnz && M.gnnz == want_nnz);
+    const std::string tmp = std::string("/tmp/spc3d_test_io_") + stem + ".bin";
+    convert_to_binary(M, tmp);
+    const std::vector<char> mine = slurp(tmp), ref = slurp(bin);
+    CHECK(!ref.empty());
+    if (sizeof(real_t) == 8)
+        CHECK(mine == ref); // byte for byte what the reference's converter wrote
+    else
+        CHECK(mine.size() == ref.size());
+    cooMat R;
+    read_binary(bin, R);
+    CHECK(R.gnrows == M.gnrows && R.gncols == M.gncols && R.gnnz == M.gnnz && R.nnz == M.nnz);
+    CHECK(R.ii == M.ii && R.jj == M.jj && R.vv == M.vv);
+    std::remove(tmp.c_str());
+}
+
+int main(int argc, char **argv)
+{
+    if (argc < 2) {
+        std::printf("usage: test_io <golden dir>\n");
+        return 2;
+    }
+    const std::string dir = argv[1];
+    check_file(dir, "general", 9);
+    check_file(dir, "symmetric", 12);        // mirrored, the two diagonal entries twice
+    check_file(dir, "pattern_symmetric", 8); // values 1
+    check_file(dir, "complex", 3);           // imaginary parts dropped
+    check_file(dir, "integer", 2);
+
+    // content of one file, spelled out (src/mm.hpp:45-57 semantics)
+    {
+        cooMat M;
+        mm reader(dir + "/symmetric.mtx");
+        reader.read_mm(dir + "/symmetric.mtx", M);
+        CHECK(M.gnrows == 5 && M.gncols == 5);
+        const idx_t wi[] = {0, 1, 2, 3, 4, 4, 0, 0, 1, 3, 0, 3};
+        const idx_t wj[] = {0, 0, 1, 3, 0, 3, 0, 1, 2, 3, 4, 4};
+        const double wv[] = {2, -1, .5, 3, 1e10, -.125, 2, -1, .5, 3, 1e10, -.125};
+        for (int i = 0; i < 12; ++i)
+            CHECK(M.ii[i] == wi[i] && M.jj[i] == wj[i] && M.vv[i] == (real_t)wv[i]);
+        cooMat P;
+        mm r2(dir + "/pattern_symmetric.mtx");
+        r2.read_mm(dir + "/pattern_symmetric.mtx", P);
+        for (idx_large_t i = 0; i < P.nnz; ++i)
+            CHECK(P.vv[i] == (real_t)1);
+        CHECK(P.ii[3] == 3 && P.jj[3] == 3 && P.ii[7] == 3 && P.jj[7] == 3); // diagonal twice
+    }
+    // failures are reported, not swallowed
+    bool threw = false;
+    try {
+        cooMat M;
+        mm r(dir + "/does_not_exist.mtx");
+        r.read_mm(dir + "/does_not_exist.mtx", M);
+    } catch (const std::runtime_error &) {
+        threw = true;
+    }
+    CHECK(threw);
+    threw = false;
+    try {
+        cooMat R;
+        const std::string cut = "/tmp/spc3d_test_io_cut.bin";
+        std::vector<char> ref = slurp(dir + "/general.bin");
+        std::ofstream(cut, std::ios::binary).write(ref.data(), 100);
+        read_binary(cut, R);
+    } catch (const std::runtime_error &) {
+        threw = true;
+    }
+    CHECK(threw);
+    std::printf("%s (%d failures, real_t = %s)\n", g_fail ? "FAILED" : "PASSED", g_fail,
+                sizeof(real_t) == 8 ? "double" : "float");
+    return g_fail ? 1 : 0;
+}

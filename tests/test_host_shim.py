@@ -29,6 +29,27 @@ def test_host_types_index_transforms_and_errors(name):
     _run(name, "--host")
 
 
+@pytest.mark.parametrize("name", ["test_io_f64", "test_io_f32"])
+def test_matrixmarket_and_binary_io_against_reference_files(name):
+    # tests/golden/io/*.bin were written by the reference's own converter
+    _run(name, os.path.join(ROOT, "tests", "golden", "io"))
+
+
+def test_binary_file_layout_with_numpy():
+    # uint32 rows, uint32 cols, uint64 nnz, then nnz x {uint32, uint32, float64}
+    # (tools/read_convert_mm.cpp:81-94): checked on the reference-written file
+    import numpy as np
+
+    raw = open(os.path.join(ROOT, "tests", "golden", "io", "general.bin"), "rb").read()
+    rows, cols = np.frombuffer(raw, dtype="<u4", count=2)
+    nnz = int(np.frombuffer(raw, dtype="<u8", count=1, offset=8)[0])
+    assert (rows, cols, nnz) == (6, 5, 9) and len(raw) == 16 + 16 * nnz
+    t = np.frombuffer(raw, dtype=np.dtype([("r", "<u4"), ("c", "<u4"), ("v", "<f8")]), offset=16)
+    assert t["r"].tolist() == [0, 1, 1, 2, 3, 4, 5, 5, 2]
+    assert t["c"].tolist() == [1, 0, 4, 2, 3, 1, 0, 4, 2]
+    assert t["v"].tolist() == [1.5, -2.25, 3.0, 4.125, 5e-3, 6.0, 7.0, -8.5, 9.0]
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("name", ["test_shim_f64", "test_shim_f32"])
 def test_shim_on_gpu(name):
