@@ -84,6 +84,9 @@ typedef struct {
     uint32_t hot_cols;         /* XCD slicing: columns planned to stay in some L2 (0: slicing off) */
     uint32_t hub_rows;         /* XCD slicing: rows cut by column slice */
     uint64_t hot_entries;      /* XCD slicing: entries in those columns */
+    uint32_t nsegments_long;   /* leading stored segments (all of >= 16 entries) that run in the
+                                  wide-batch launch; the rest run in the high-occupancy one */
+    uint32_t reserved;
 } spc3d_plan_info;
 
 /* Plan tuning; a zero field selects the default.  Only speed depends on these. */

@@ -29,7 +29,8 @@ class PlanInfo(ctypes.Structure):
                 ("nsplit_rows", c_u32), ("npartial_slots", c_u32),
                 ("max_row_nnz", c_u32), ("seg_max", c_u32),
                 ("order_is_identity", ctypes.c_int32), ("nqueues", c_u32),
-                ("hot_cols", c_u32), ("hub_rows", c_u32), ("hot_entries", c_u64)]
+                ("hot_cols", c_u32), ("hub_rows", c_u32), ("hot_entries", c_u64),
+                ("nsegments_long", c_u32), ("reserved", c_u32)]
 
 
 class PlanOpts(ctypes.Structure):

@@ -61,6 +61,9 @@ struct spc3d_ctx {
     uint32_t magic;
     int device;
     hipStream_t stream;
+    hipStream_t aux_stream; // short-segment launches run here, beside the long-segment ones
+    hipEvent_t fork_event, join_event;
+    uint32_t aux_rot; // (XCD of workgroup 0 on aux - XCD of workgroup 0 on main) mod 8
     hipEvent_t timers[kTimerSlots];
     bool timer_set[kTimerSlots];
 };
@@ -173,11 +176,23 @@ void plan_free_device(spc3d_plan *p)
     p->splits = nullptr;
 }
 
+Streams streams_of(const spc3d_ctx *c)
+{
+    Streams s;
+    s.main = c->stream;
+    s.aux = c->aux_stream;
+    s.fork = c->fork_event;
+    s.join = c->join_event;
+    s.aux_rot = c->aux_rot;
+    return s;
+}
+
 DevPlanView view_of(const spc3d_plan *p)
 {
     DevPlanView v;
     v.segs = p->segs;
     v.nseg = p->info.nsegments_padded;
+    v.nseg_long = p->info.nsegments_long;
     v.nqueues = p->info.nqueues;
     v.col = p->col;
     v.perm = p->perm;
@@ -251,6 +266,49 @@ int spc3d_ctx_create(int device, spc3d_ctx **out)
         delete c;
         return fail_hip(e, "hipStreamCreateWithFlags");
     }
+    // Same (default) priority as the main stream.  SPC3D_AUX_STREAM=0 keeps every
+    // launch on the main stream.
+    c->aux_stream = nullptr;
+    c->fork_event = c->join_event = nullptr;
+    const char *aux = std::getenv("SPC3D_AUX_STREAM");
+    if (!aux || std::atoi(aux) != 0) {
+        e = hipStreamCreateWithFlags(&c->aux_stream, hipStreamNonBlocking);
+        if (e == hipSuccess)
+            e = hipEventCreateWithFlags(&c->fork_event, hipEventDisableTiming);
+        if (e == hipSuccess)
+            e = hipEventCreateWithFlags(&c->join_event, hipEventDisableTiming);
+        if (e != hipSuccess) {
+            if (c->join_event) (void)hipEventDestroy(c->join_event);
+            if (c->fork_event) (void)hipEventDestroy(c->fork_event);
+            if (c->aux_stream) (void)hipStreamDestroy(c->aux_stream);
+            (void)hipStreamDestroy(c->stream);
+            delete c;
+            return fail_hip(e, "auxiliary stream");
+        }
+    }
+    // Each hardware queue starts its round-robin over the XCDs at its own XCD:
+    // measure where workgroup 0 lands on either stream.
+    c->aux_rot = 0;
+    if (c->aux_stream) {
+        uint32_t *probe = nullptr, host[2] = {0, 0};
+        e = hipMalloc((void **)&probe, 2 * sizeof(uint32_t));
+        if (e == hipSuccess)
+            e = launch_xcc_probe(probe, 1, c->stream);
+        if (e == hipSuccess)
+            e = launch_xcc_probe(probe + 1, 1, c->aux_stream);
+        if (e == hipSuccess)
+            e = hipStreamSynchronize(c->stream);
+        if (e == hipSuccess)
+            e = hipStreamSynchronize(c->aux_stream);
+        if (e == hipSuccess)
+            e = hipMemcpy(host, probe, sizeof host, hipMemcpyDeviceToHost);
+        if (probe)
+            (void)hipFree(probe);
+        if (e == hipSuccess)
+            c->aux_rot = (host[1] - host[0]) & 7u;
+        else
+            (void)hipGetLastError(); // the rotation only affects speed
+    }
     for (int i = 0; i < kTimerSlots; ++i) {
         c->timers[i] = nullptr;
         c->timer_set[i] = false;
@@ -269,6 +327,12 @@ int spc3d_ctx_destroy(spc3d_ctx *ctx)
     for (int i = 0; i < kTimerSlots; ++i)
         if (ctx->timers[i])
             (void)hipEventDestroy(ctx->timers[i]);
+    if (ctx->aux_stream) {
+        (void)hipStreamSynchronize(ctx->aux_stream);
+        (void)hipEventDestroy(ctx->fork_event);
+        (void)hipEventDestroy(ctx->join_event);
+        (void)hipStreamDestroy(ctx->aux_stream);
+    }
     (void)hipStreamDestroy(ctx->stream);
     ctx->magic = 0;
     delete ctx;
@@ -561,6 +625,8 @@ static void fill_info(spc3d_plan_info &info, const HostPlan &H)
     info.hot_cols = H.hot_cols;
     info.hub_rows = H.hub_rows;
     info.hot_entries = H.hot_entries;
+    info.nsegments_long = H.nseg_long;
+    info.reserved = 0;
 }
 
 // Library defaults, overridable field by field.  With XCD slicing, 2 MiB of
@@ -805,7 +871,7 @@ int spc3d_sddmm(spc3d_ctx *ctx, spc3d_plan *S, const spc3d_panel *A, const spc3d
     int rc = use_device(ctx);
     if (rc)
         return rc;
-    HIP_TRY(launch_sddmm(S->dtype, view_of(S), A->dev, B->dev, C->dev, K, ctx->stream));
+    HIP_TRY(launch_sddmm(S->dtype, view_of(S), A->dev, B->dev, C->dev, K, streams_of(ctx)));
     return SPC3D_OK;
 }
 
@@ -844,7 +910,7 @@ int spc3d_spmm(spc3d_ctx *ctx, spc3d_plan *Ap, const spc3d_panel *X, spc3d_panel
             return rc;
         Ap->partial_k = K;
     }
-    HIP_TRY(launch_spmm(Ap->dtype, view_of(Ap), X->dev, Y->dev, K, ctx->stream));
+    HIP_TRY(launch_spmm(Ap->dtype, view_of(Ap), X->dev, Y->dev, K, streams_of(ctx)));
     return SPC3D_OK;
 }
 

@@ -12,6 +12,7 @@ namespace spc3d {
 struct DevPlanView {
     const Seg *segs = nullptr;
     uint32_t nseg = 0;                // including padding segments
+    uint32_t nseg_long = 0;           // leading segments that are all long (whole chunk rounds)
     uint32_t nqueues = 1;             // 1, or 8: chunk v of the segments belongs to XCD v % 8
     const uint32_t *col = nullptr;    // [nnz] kernel order
     const uint32_t *perm = nullptr;   // [nnz] kernel order -> caller's position; null if identity
@@ -22,11 +23,22 @@ struct DevPlanView {
     uint64_t nnz = 0;
 };
 
-// dtype: 0 = float, 1 = double.  All launches are asynchronous on `stream`.
+// The context's stream, plus an auxiliary stream of the same (default) priority
+// and two timing-free events with which a call can run two launches side by
+// side and rejoin the main stream.  aux == null: everything goes to `main`.
+struct Streams {
+    hipStream_t main = nullptr;
+    hipStream_t aux = nullptr;
+    hipEvent_t fork = nullptr, join = nullptr;
+    uint32_t aux_rot = 0; // workgroup b of an aux launch runs on the XCD of main's b + aux_rot
+};
+
+// dtype: 0 = float, 1 = double.  Asynchronous; everything launched is ordered
+// before whatever is queued on streams.main afterwards.
 hipError_t launch_sddmm(int dtype, const DevPlanView &P, const void *A, const void *B, void *C,
-                        uint32_t K, hipStream_t stream);
+                        uint32_t K, const Streams &streams);
 hipError_t launch_spmm(int dtype, const DevPlanView &P, const void *X, void *Y, uint32_t K,
-                       hipStream_t stream);
+                       const Streams &streams);
 // out[p] = in[perm[p]] (perm == null: copy)
 hipError_t launch_gather_vals(int dtype, const void *in, const uint32_t *perm, void *out,
                               uint64_t n, hipStream_t stream);

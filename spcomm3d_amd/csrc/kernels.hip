@@ -155,12 +155,16 @@ template <int LPR, int NB> __device__ __forceinline__ bool is_writer(uint32_t su
 }
 
 // Segment this lane group works on.  Segments are stored in chunks of kChunk;
-// with nq == 8, chunk v belongs to XCD v % 8.  Workgroups are dispatched to
-// the XCDs round-robin by workgroup id, so workgroup b runs on XCD b % 8 and
-// takes its segments from that XCD's chunks: the dense rows of one column
-// slice are then only ever gathered through one L2.  (If the hardware dealt
-// workgroups differently the result would be the same, only slower.)
-template <int G> __device__ __forceinline__ uint64_t seg_index(uint32_t nq)
+// with nq == 8, chunk v belongs to queue v % 8.  The hardware deals the
+// workgroups of a dispatch to the 8 XCDs round-robin by workgroup id, starting
+// from an XCD that is fixed per hardware queue, so the workgroups b with equal
+// (b + rot) % 8 all run on one XCD; they take the chunks of queue (b + rot) % 8
+// and the dense rows of one column slice are then only ever gathered through
+// one L2.  `rot` lines the queues of the auxiliary stream up with those of the
+// main stream.  Any rot gives each segment to exactly one workgroup: if the
+// hardware dealt workgroups differently the result would be the same, only
+// slower.
+template <int G> __device__ __forceinline__ uint64_t seg_index(uint32_t nq, uint32_t rot)
 {
     constexpr uint32_t kSegPerBlock = (kBlock / 64) * G;
     constexpr uint32_t kBlocksPerChunk = kChunk / kSegPerBlock;
@@ -170,7 +174,7 @@ template <int G> __device__ __forceinline__ uint64_t seg_index(uint32_t nq)
     uint32_t inner;
     if (nq == 8) {
         const uint32_t j = b >> 3;
-        chunk = (uint64_t)(j / kBlocksPerChunk) * 8 + (b & 7u);
+        chunk = (uint64_t)(j / kBlocksPerChunk) * 8 + ((b + rot) & 7u);
         inner = j % kBlocksPerChunk;
     } else {
         chunk = b / kBlocksPerChunk;
@@ -278,7 +282,7 @@ sddmm_walk(const typename Vec<T>::type (&a)[VPL], const uint32_t *__restrict__ c
 
 template <typename T, int LPR, int VPL, int UB>
 __global__ void __launch_bounds__(kBlock)
-sddmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq,
+sddmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint32_t rot,
                  const uint32_t *__restrict__ col, const uint32_t *__restrict__ perm,
                  const T *__restrict__ sval, const T *__restrict__ A, const T *__restrict__ B,
                  T *__restrict__ C)
@@ -286,7 +290,7 @@ sddmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq,
     static_assert(UB <= LPR && UB <= 16 && LPR <= 64, "batch must fit the lane group");
     using V = typename Vec<T>::type;
     const uint32_t sub = threadIdx.x & (LPR - 1);
-    const uint64_t sid = seg_index<64 / LPR>(nq);
+    const uint64_t sid = seg_index<64 / LPR>(nq, rot);
     if (sid >= nseg)
         return;
     const u32x4 sg = nt_load(reinterpret_cast<const u32x4 *>(segs) + sid); // row, start, len, slot
@@ -306,13 +310,13 @@ sddmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq,
 // Any K: one wavefront per segment, lanes stride over K, scalar loads.
 template <typename T>
 __global__ void __launch_bounds__(kBlock)
-sddmm_generic_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq,
+sddmm_generic_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint32_t rot,
                      const uint32_t *__restrict__ col, const uint32_t *__restrict__ perm,
                      const T *__restrict__ sval, const T *__restrict__ A,
                      const T *__restrict__ B, T *__restrict__ C, uint32_t K)
 {
     const uint32_t lane = threadIdx.x & 63u;
-    const uint64_t sid = seg_index<1>(nq);
+    const uint64_t sid = seg_index<1>(nq, rot);
     if (sid >= nseg)
         return;
     const Seg sg = segs[sid];
@@ -394,14 +398,14 @@ spmm_walk(typename Vec<T>::type (&acc)[VPL], const uint32_t *__restrict__ col,
 
 template <typename T, int LPR, int VPL, int UB>
 __global__ void __launch_bounds__(kBlock)
-spmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq,
+spmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint32_t rot,
                 const uint32_t *__restrict__ col, const T *__restrict__ sval,
                 const T *__restrict__ X, T *__restrict__ Y, T *__restrict__ partial)
 {
     static_assert(UB <= LPR && UB <= 16 && LPR <= 64, "batch must fit the lane group");
     using V = typename Vec<T>::type;
     const uint32_t sub = threadIdx.x & (LPR - 1);
-    const uint64_t sid = seg_index<64 / LPR>(nq);
+    const uint64_t sid = seg_index<64 / LPR>(nq, rot);
     if (sid >= nseg)
         return;
     const u32x4 sg = nt_load(reinterpret_cast<const u32x4 *>(segs) + sid); // row, start, len, slot
@@ -436,13 +440,13 @@ spmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq,
 
 template <typename T>
 __global__ void __launch_bounds__(kBlock)
-spmm_generic_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq,
+spmm_generic_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint32_t rot,
                     const uint32_t *__restrict__ col, const T *__restrict__ sval,
                     const T *__restrict__ X, T *__restrict__ Y, T *__restrict__ partial,
                     uint32_t K)
 {
     const uint32_t lane = threadIdx.x & 63u;
-    const uint64_t sid = seg_index<1>(nq);
+    const uint64_t sid = seg_index<1>(nq, rot);
     if (sid >= nseg)
         return;
     const Seg sg = segs[sid];
@@ -617,39 +621,87 @@ inline uint32_t blocks_for_groups(uint32_t nseg, uint32_t nq, int groups_per_wav
     return (uint32_t)(chunks * (kChunk / ((kBlock / 64) * groups_per_wave)));
 }
 
-template <typename T, int LPR, int VPL, int UB>
-void run_sddmm(const DevPlanView &P, const T *A, const T *B, T *C, hipStream_t st)
+// Two launches per call: the leading nseg_long segments (all at least
+// kLongSegment entries long) run with UB gathers in flight per lane and
+// 4 wavefronts per SIMD; the rest run the US-wide variant, whose register
+// budget lets 8 wavefronts per SIMD hide the three dependent memory latencies
+// of a short segment (descriptor -> indices -> gathers).  Measured: 5-entry
+// rows of a stencil 1.6x faster with US = 4 than with 16, R-MAT hub segments
+// 1.5x slower.
+// Starts `second` on the auxiliary stream so that it runs alongside what is
+// queued on the main stream after `fork`; the main stream waits for it at `join`.
+inline void fork_aux(const Streams &S)
 {
-    const uint32_t grid = blocks_for_groups(P.nseg, P.nqueues, 64 / LPR);
-    hipLaunchKernelGGL((sddmm_seg_kernel<T, LPR, VPL, UB>), dim3(grid), dim3(kBlock), 0, st, P.segs,
-                       P.nseg, P.nqueues, P.col, P.perm, (const T *)P.sval, A, B, C);
+    (void)hipEventRecord(S.fork, S.main);
+    (void)hipStreamWaitEvent(S.aux, S.fork, 0);
+}
+inline void join_aux(const Streams &S)
+{
+    (void)hipEventRecord(S.join, S.aux);
+    (void)hipStreamWaitEvent(S.main, S.join, 0);
 }
 
-template <typename T, int LPR, int VPL, int UB>
-void run_spmm(const DevPlanView &P, const T *X, T *Y, hipStream_t st)
+template <typename T, int LPR, int VPL, int UB, int US>
+void run_sddmm(const DevPlanView &P, const T *A, const T *B, T *C, const Streams &S)
 {
-    const uint32_t grid = blocks_for_groups(P.nseg, P.nqueues, 64 / LPR);
-    hipLaunchKernelGGL((spmm_seg_kernel<T, LPR, VPL, UB>), dim3(grid), dim3(kBlock), 0, st, P.segs,
-                       P.nseg, P.nqueues, P.col, (const T *)P.sval, X, Y, (T *)P.partial);
+    const uint32_t nl = P.nseg_long, ns = P.nseg - P.nseg_long;
+    const bool both = nl && ns && S.aux;
+    if (both)
+        fork_aux(S);
+    if (nl)
+        hipLaunchKernelGGL((sddmm_seg_kernel<T, LPR, VPL, UB>),
+                           dim3(blocks_for_groups(nl, P.nqueues, 64 / LPR)), dim3(kBlock), 0,
+                           S.main, P.segs, nl, P.nqueues, 0u, P.col, P.perm, (const T *)P.sval,
+                           A, B, C);
+    if (ns)
+        hipLaunchKernelGGL((sddmm_seg_kernel<T, LPR, VPL, US>),
+                           dim3(blocks_for_groups(ns, P.nqueues, 64 / LPR)), dim3(kBlock), 0,
+                           both ? S.aux : S.main, P.segs + nl, ns, P.nqueues,
+                           both ? S.aux_rot : 0u, P.col, P.perm, (const T *)P.sval, A, B, C);
+    if (both)
+        join_aux(S);
 }
 
-// (LPR, VPL, UB): UB * VPL 16-byte gathers are in flight per lane.
+template <typename T, int LPR, int VPL, int UB, int US>
+void run_spmm(const DevPlanView &P, const T *X, T *Y, const Streams &S)
+{
+    const uint32_t nl = P.nseg_long, ns = P.nseg - P.nseg_long;
+    const bool both = nl && ns && S.aux;
+    if (both)
+        fork_aux(S);
+    if (nl)
+        hipLaunchKernelGGL((spmm_seg_kernel<T, LPR, VPL, UB>),
+                           dim3(blocks_for_groups(nl, P.nqueues, 64 / LPR)), dim3(kBlock), 0,
+                           S.main, P.segs, nl, P.nqueues, 0u, P.col, (const T *)P.sval, X, Y,
+                           (T *)P.partial);
+    if (ns)
+        hipLaunchKernelGGL((spmm_seg_kernel<T, LPR, VPL, US>),
+                           dim3(blocks_for_groups(ns, P.nqueues, 64 / LPR)), dim3(kBlock), 0,
+                           both ? S.aux : S.main, P.segs + nl, ns, P.nqueues,
+                           both ? S.aux_rot : 0u, P.col, (const T *)P.sval, X, Y, (T *)P.partial);
+    if (both)
+        join_aux(S);
+}
+
+// (LPR, VPL, UB, US): UB * VPL 16-byte gathers are in flight per lane in the
+// long-segment launch, US * VPL in the short-segment one.
 #define SPC3D_FOR_SHAPES(X)                                                                       \
-    X(4, 1, 4) X(8, 1, 8) X(16, 1, 16) X(32, 1, 16) X(64, 1, 16)                                  \
-    X(4, 2, 4) X(8, 2, 8) X(16, 2, 8) X(32, 2, 8) X(64, 2, 8)                                     \
-    X(4, 4, 4) X(8, 4, 4) X(16, 4, 4) X(32, 4, 4) X(64, 4, 4)
+    X(4, 1, 4, 4) X(8, 1, 8, 4) X(16, 1, 16, 4) X(32, 1, 16, 4) X(64, 1, 16, 4)                   \
+    X(4, 2, 4, 2) X(8, 2, 8, 2) X(16, 2, 8, 2) X(32, 2, 8, 2) X(64, 2, 8, 2)                      \
+    X(4, 4, 4, 1) X(8, 4, 4, 1) X(16, 4, 4, 1) X(32, 4, 4, 1) X(64, 4, 4, 1)
 
 template <typename T>
 hipError_t sddmm_typed(const DevPlanView &P, const void *A, const void *B, void *C, uint32_t K,
-                       hipStream_t st)
+                       const Streams &SS)
 {
+    const hipStream_t st = SS.main;
     if (P.nseg == 0)
         return hipSuccess;
     const Shape sh = pick_shape(sizeof(T), K);
     bool done = false;
-#define X(L, V, U)                                                                                \
+#define X(L, V, U, S)                                                                             \
     if (!done && sh.lpr == L && sh.vpl == V) {                                                    \
-        run_sddmm<T, L, V, U>(P, (const T *)A, (const T *)B, (T *)C, st);                         \
+        run_sddmm<T, L, V, U, S>(P, (const T *)A, (const T *)B, (T *)C, SS);                      \
         done = true;                                                                              \
     }
     SPC3D_FOR_SHAPES(X)
@@ -657,22 +709,24 @@ hipError_t sddmm_typed(const DevPlanView &P, const void *A, const void *B, void 
     if (!done) {
         const uint32_t grid = blocks_for_groups(P.nseg, P.nqueues, 1);
         hipLaunchKernelGGL((sddmm_generic_kernel<T>), dim3(grid), dim3(kBlock), 0, st, P.segs,
-                           P.nseg, P.nqueues, P.col, P.perm, (const T *)P.sval, (const T *)A, (const T *)B,
+                           P.nseg, P.nqueues, 0u, P.col, P.perm, (const T *)P.sval, (const T *)A, (const T *)B,
                            (T *)C, K);
     }
     return hipGetLastError();
 }
 
 template <typename T>
-hipError_t spmm_typed(const DevPlanView &P, const void *X_, void *Y, uint32_t K, hipStream_t st)
+hipError_t spmm_typed(const DevPlanView &P, const void *X_, void *Y, uint32_t K,
+                      const Streams &SS)
 {
+    const hipStream_t st = SS.main;
     if (P.nseg == 0)
         return hipSuccess;
     const Shape sh = pick_shape(sizeof(T), K);
     bool done = false;
-#define X(L, V, U)                                                                                \
+#define X(L, V, U, S)                                                                             \
     if (!done && sh.lpr == L && sh.vpl == V) {                                                    \
-        run_spmm<T, L, V, U>(P, (const T *)X_, (T *)Y, st);                                       \
+        run_spmm<T, L, V, U, S>(P, (const T *)X_, (T *)Y, SS);                                    \
         done = true;                                                                              \
     }
     SPC3D_FOR_SHAPES(X)
@@ -680,7 +734,7 @@ hipError_t spmm_typed(const DevPlanView &P, const void *X_, void *Y, uint32_t K,
     if (!done) {
         const uint32_t grid = blocks_for_groups(P.nseg, P.nqueues, 1);
         hipLaunchKernelGGL((spmm_generic_kernel<T>), dim3(grid), dim3(kBlock), 0, st, P.segs,
-                           P.nseg, P.nqueues, P.col, (const T *)P.sval, (const T *)X_, (T *)Y,
+                           P.nseg, P.nqueues, 0u, P.col, (const T *)P.sval, (const T *)X_, (T *)Y,
                            (T *)P.partial, K);
     }
     hipError_t e = hipGetLastError();
@@ -709,14 +763,14 @@ inline uint32_t stream_grid(uint64_t n)
 } // namespace
 
 hipError_t launch_sddmm(int dtype, const DevPlanView &P, const void *A, const void *B, void *C,
-                        uint32_t K, hipStream_t stream)
+                        uint32_t K, const Streams &stream)
 {
     return dtype == 1 ? sddmm_typed<double>(P, A, B, C, K, stream)
                       : sddmm_typed<float>(P, A, B, C, K, stream);
 }
 
 hipError_t launch_spmm(int dtype, const DevPlanView &P, const void *X, void *Y, uint32_t K,
-                       hipStream_t stream)
+                       const Streams &stream)
 {
     return dtype == 1 ? spmm_typed<double>(P, X, Y, K, stream)
                       : spmm_typed<float>(P, X, Y, K, stream);

@@ -311,6 +311,22 @@ int build_host_plan(uint32_t nrows, uint32_t ncols, uint64_t nnz, const uint32_t
                 for (size_t i = 0; i < queue[q].size(); ++i)
                     P.segs[((i / kChunk) * kSlices + q) * kChunk + i % kChunk] = queue[q][i].seg;
         }
+        // Leading whole rounds of chunks (one chunk per queue) made of long
+        // segments only; every queue is sorted longest first.
+        {
+            const size_t round = (size_t)P.nqueues * kChunk;
+            size_t rounds = 0;
+            while ((rounds + 1) * round <= P.segs.size()) {
+                bool all_long = true;
+                for (uint32_t q = 0; q < P.nqueues && all_long; ++q)
+                    all_long = P.segs[rounds * round + (size_t)q * kChunk + kChunk - 1].len >=
+                               kLongSegment;
+                if (!all_long)
+                    break;
+                ++rounds;
+            }
+            P.nseg_long = (uint32_t)(rounds * round);
+        }
     } catch (const std::bad_alloc &) {
         err = "host allocation failed while building the plan";
         return SPC3D_ERR_ALLOC;

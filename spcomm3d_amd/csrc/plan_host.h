@@ -19,6 +19,7 @@ struct Seg {
 };
 constexpr uint32_t kWholeRow = 0xFFFFFFFFu;
 constexpr uint32_t kChunk = 64; // segments per chunk; one chunk is dealt to one XCD
+constexpr uint32_t kLongSegment = 16; // segments this long fill the wide kernel's batches
 
 // A row cut into several segments: its partial sums are slots
 // [first_slot, first_slot + nslots).
@@ -45,6 +46,8 @@ struct HostPlan {
     uint32_t seg_max = 0;
     uint32_t nslots = 0;
     uint32_t nseg_real = 0;        // segments with entries (segs.size() includes padding)
+    uint32_t nseg_long = 0;        // leading stored segments, a whole number of chunk rounds, all
+                                   // of at least kLongSegment entries
     uint32_t nqueues = 1;          // 1, or 8 when chunks are dealt round-robin to XCDs
     uint32_t hot_cols = 0;         // columns dealt to slices or replicated (0: slicing off)
     uint64_t hot_entries = 0;      // entries in those columns
