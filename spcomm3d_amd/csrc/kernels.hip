@@ -567,15 +567,29 @@ __global__ void __launch_bounds__(kBlock) fill_kernel(T *__restrict__ p, uint64_
         p[i] = value;
 }
 
-// Plain streaming copy, 16 bytes per lane per iteration; the tail (< 16 bytes)
-// is moved bytewise by the first lanes.
+// Plain streaming copy: four 16-byte non-temporal loads in flight per lane, then
+// four non-temporal stores (5.8 TB/s read + written on this GPU; one load per
+// iteration with plain accesses gives 4.6).  The last (< 4 * block) vectors go
+// one by one, the tail (< 16 bytes) bytewise by the first lanes.
 __global__ void __launch_bounds__(kBlock)
-copy_kernel(uint4 *__restrict__ dst, const uint4 *__restrict__ src, uint64_t nvec,
+copy_kernel(u32x4 *__restrict__ dst, const u32x4 *__restrict__ src, uint64_t nvec,
             uint32_t tail_bytes)
 {
-    const uint64_t stride = (uint64_t)gridDim.x * kBlock;
+    constexpr uint64_t U = 4;
     const uint64_t tid = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
-    for (uint64_t i = tid; i < nvec; i += stride)
+    const uint64_t span = (uint64_t)kBlock * U; // vectors one block moves per iteration
+    const uint64_t nfull = nvec / span * span;
+    for (uint64_t i = (uint64_t)blockIdx.x * span + threadIdx.x; i < nfull;
+         i += (uint64_t)gridDim.x * span) {
+        u32x4 v[U];
+#pragma unroll
+        for (uint64_t u = 0; u < U; ++u)
+            v[u] = nt_load(src + i + u * kBlock);
+#pragma unroll
+        for (uint64_t u = 0; u < U; ++u)
+            nt_store(v[u], dst + i + u * kBlock);
+    }
+    for (uint64_t i = nfull + tid; i < nvec; i += (uint64_t)gridDim.x * kBlock)
         dst[i] = src[i];
     if (tid < tail_bytes)
         reinterpret_cast<unsigned char *>(dst + nvec)[tid] =
@@ -627,27 +641,32 @@ inline uint32_t blocks_for_groups(uint32_t nseg, uint32_t nq, int groups_per_wav
 // budget lets 8 wavefronts per SIMD hide the three dependent memory latencies
 // of a short segment (descriptor -> indices -> gathers).  Measured: 5-entry
 // rows of a stencil 1.6x faster with US = 4 than with 16, R-MAT hub segments
-// 1.5x slower.
-// Starts `second` on the auxiliary stream so that it runs alongside what is
-// queued on the main stream after `fork`; the main stream waits for it at `join`.
-inline void fork_aux(const Streams &S)
+// 1.5x slower.  With an auxiliary stream the two run side by side.
+
+// Makes the auxiliary stream wait for everything queued on the main stream so
+// far.  On failure nothing was queued on aux and the caller stays on main.
+inline bool fork_aux(const Streams &S)
 {
-    (void)hipEventRecord(S.fork, S.main);
-    (void)hipStreamWaitEvent(S.aux, S.fork, 0);
+    return S.aux && hipEventRecord(S.fork, S.main) == hipSuccess &&
+           hipStreamWaitEvent(S.aux, S.fork, 0) == hipSuccess;
 }
-inline void join_aux(const Streams &S)
+
+// Makes the main stream wait for what was queued on the auxiliary stream; if the
+// events fail, waits on the host instead, so the ordering holds either way.
+inline hipError_t join_aux(const Streams &S)
 {
-    (void)hipEventRecord(S.join, S.aux);
-    (void)hipStreamWaitEvent(S.main, S.join, 0);
+    if (hipEventRecord(S.join, S.aux) == hipSuccess &&
+        hipStreamWaitEvent(S.main, S.join, 0) == hipSuccess)
+        return hipSuccess;
+    (void)hipGetLastError();
+    return hipStreamSynchronize(S.aux);
 }
 
 template <typename T, int LPR, int VPL, int UB, int US>
-void run_sddmm(const DevPlanView &P, const T *A, const T *B, T *C, const Streams &S)
+hipError_t run_sddmm(const DevPlanView &P, const T *A, const T *B, T *C, const Streams &S)
 {
     const uint32_t nl = P.nseg_long, ns = P.nseg - P.nseg_long;
-    const bool both = nl && ns && S.aux;
-    if (both)
-        fork_aux(S);
+    const bool both = nl && ns && fork_aux(S);
     if (nl)
         hipLaunchKernelGGL((sddmm_seg_kernel<T, LPR, VPL, UB>),
                            dim3(blocks_for_groups(nl, P.nqueues, 64 / LPR)), dim3(kBlock), 0,
@@ -658,17 +677,16 @@ void run_sddmm(const DevPlanView &P, const T *A, const T *B, T *C, const Streams
                            dim3(blocks_for_groups(ns, P.nqueues, 64 / LPR)), dim3(kBlock), 0,
                            both ? S.aux : S.main, P.segs + nl, ns, P.nqueues,
                            both ? S.aux_rot : 0u, P.col, P.perm, (const T *)P.sval, A, B, C);
-    if (both)
-        join_aux(S);
+    const hipError_t launched = hipGetLastError();
+    const hipError_t joined = both ? join_aux(S) : hipSuccess;
+    return launched != hipSuccess ? launched : joined;
 }
 
 template <typename T, int LPR, int VPL, int UB, int US>
-void run_spmm(const DevPlanView &P, const T *X, T *Y, const Streams &S)
+hipError_t run_spmm(const DevPlanView &P, const T *X, T *Y, const Streams &S)
 {
     const uint32_t nl = P.nseg_long, ns = P.nseg - P.nseg_long;
-    const bool both = nl && ns && S.aux;
-    if (both)
-        fork_aux(S);
+    const bool both = nl && ns && fork_aux(S);
     if (nl)
         hipLaunchKernelGGL((spmm_seg_kernel<T, LPR, VPL, UB>),
                            dim3(blocks_for_groups(nl, P.nqueues, 64 / LPR)), dim3(kBlock), 0,
@@ -679,8 +697,9 @@ void run_spmm(const DevPlanView &P, const T *X, T *Y, const Streams &S)
                            dim3(blocks_for_groups(ns, P.nqueues, 64 / LPR)), dim3(kBlock), 0,
                            both ? S.aux : S.main, P.segs + nl, ns, P.nqueues,
                            both ? S.aux_rot : 0u, P.col, (const T *)P.sval, X, Y, (T *)P.partial);
-    if (both)
-        join_aux(S);
+    const hipError_t launched = hipGetLastError();
+    const hipError_t joined = both ? join_aux(S) : hipSuccess;
+    return launched != hipSuccess ? launched : joined;
 }
 
 // (LPR, VPL, UB, US): UB * VPL 16-byte gathers are in flight per lane in the
@@ -699,9 +718,10 @@ hipError_t sddmm_typed(const DevPlanView &P, const void *A, const void *B, void 
         return hipSuccess;
     const Shape sh = pick_shape(sizeof(T), K);
     bool done = false;
+    hipError_t e = hipSuccess;
 #define X(L, V, U, S)                                                                             \
     if (!done && sh.lpr == L && sh.vpl == V) {                                                    \
-        run_sddmm<T, L, V, U, S>(P, (const T *)A, (const T *)B, (T *)C, SS);                      \
+        e = run_sddmm<T, L, V, U, S>(P, (const T *)A, (const T *)B, (T *)C, SS);                  \
         done = true;                                                                              \
     }
     SPC3D_FOR_SHAPES(X)
@@ -712,7 +732,8 @@ hipError_t sddmm_typed(const DevPlanView &P, const void *A, const void *B, void 
                            P.nseg, P.nqueues, 0u, P.col, P.perm, (const T *)P.sval, (const T *)A, (const T *)B,
                            (T *)C, K);
     }
-    return hipGetLastError();
+    const hipError_t last = hipGetLastError();
+    return e != hipSuccess ? e : last;
 }
 
 template <typename T>
@@ -724,9 +745,10 @@ hipError_t spmm_typed(const DevPlanView &P, const void *X_, void *Y, uint32_t K,
         return hipSuccess;
     const Shape sh = pick_shape(sizeof(T), K);
     bool done = false;
+    hipError_t e = hipSuccess;
 #define X(L, V, U, S)                                                                             \
     if (!done && sh.lpr == L && sh.vpl == V) {                                                    \
-        run_spmm<T, L, V, U, S>(P, (const T *)X_, (T *)Y, SS);                                    \
+        e = run_spmm<T, L, V, U, S>(P, (const T *)X_, (T *)Y, SS);                                \
         done = true;                                                                              \
     }
     SPC3D_FOR_SHAPES(X)
@@ -737,7 +759,8 @@ hipError_t spmm_typed(const DevPlanView &P, const void *X_, void *Y, uint32_t K,
                            P.nseg, P.nqueues, 0u, P.col, (const T *)P.sval, (const T *)X_, (T *)Y,
                            (T *)P.partial, K);
     }
-    hipError_t e = hipGetLastError();
+    if (e == hipSuccess)
+        e = hipGetLastError();
     if (e != hipSuccess)
         return e;
     if (P.nsplit) {
@@ -842,8 +865,8 @@ hipError_t launch_copy(void *dst, const void *src, uint64_t bytes, hipStream_t s
     if (bytes == 0)
         return hipSuccess;
     const uint64_t nvec = bytes / 16;
-    hipLaunchKernelGGL(copy_kernel, dim3(stream_grid(nvec ? nvec : 1)), dim3(kBlock), 0, stream,
-                       (uint4 *)dst, (const uint4 *)src, nvec, (uint32_t)(bytes % 16));
+    hipLaunchKernelGGL(copy_kernel, dim3(stream_grid((nvec + 3) / 4 + 1)), dim3(kBlock), 0, stream,
+                       (u32x4 *)dst, (const u32x4 *)src, nvec, (uint32_t)(bytes % 16));
     return hipGetLastError();
 }
 

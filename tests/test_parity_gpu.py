@@ -314,10 +314,13 @@ def test_workgroups_are_dealt_to_xcds_round_robin(ctx):
     assert np.array_equal(ctx.probe_xcd(13).astype(np.int64)[:8], x[:8])  # same start every time
 
 
-def test_panel_copy_on_device(ctx):
-    a = np.random.default_rng(0).uniform(-1, 1, (1000, 33)).astype(np.float32)
-    src, dst = ctx.panel_from(a), ctx.panel(1000, 33, np.float32)
+@pytest.mark.parametrize("shape", [(1000, 33), (1001, 33), (3, 1), (70000, 64)])
+def test_panel_copy_on_device(ctx, shape):
+    # sizes with and without a 16-byte tail, below and above one block's span
+    a = np.random.default_rng(0).uniform(-1, 1, shape).astype(np.float32)
+    src, dst = ctx.panel_from(a), ctx.panel(shape[0], shape[1], np.float32)
+    dst.fill(7.0)
     dst.copy_from(src)
     assert np.array_equal(dst.download(), a)
     with pytest.raises(capi.Spc3dError):
-        ctx.panel(1000, 32, np.float32).copy_from(src)
+        ctx.panel(shape[0], shape[1] + 1, np.float32).copy_from(src)
