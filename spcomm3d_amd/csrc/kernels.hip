@@ -184,22 +184,32 @@ template <int G> __device__ __forceinline__ uint64_t seg_index(uint32_t nq, uint
            (threadIdx.x & 63u) / (64 / G);
 }
 
-template <typename T, int LPR, int VPL>
+// RG ("ragged"): a dense row is nvec 16-byte vectors with nvec < LPR * VPL, given at
+// run time; lanes whose vector index is >= nvec idle.  !RG: nvec == LPR * VPL
+// exactly and the row stride is a compile-time constant.
+template <typename T, int LPR, int VPL, bool RG>
 __device__ __forceinline__ const typename Vec<T>::type *row_ptr(const T *base, uint32_t row,
-                                                                uint32_t sub)
+                                                                uint32_t sub, uint32_t nvec)
 {
-    constexpr uint64_t kRowBytes = (uint64_t)LPR * VPL * 16;
+    const uint64_t row_bytes = RG ? (uint64_t)nvec * 16 : (uint64_t)LPR * VPL * 16;
     return reinterpret_cast<const typename Vec<T>::type *>(
-               reinterpret_cast<const char *>(base) + (uint64_t)row * kRowBytes) +
+               reinterpret_cast<const char *>(base) + (uint64_t)row * row_bytes) +
            sub;
 }
 
+template <int LPR, bool RG>
+__device__ __forceinline__ bool lane_on(uint32_t sub, int v, uint32_t nvec)
+{
+    return !RG || sub + (uint32_t)v * LPR < nvec;
+}
+
 // ---------------------------------------------------------------- SDDMM ----
-template <typename T, int LPR, int VPL, int NB>
+template <typename T, int LPR, int VPL, int NB, bool RG>
 __device__ __forceinline__ void
 sddmm_batch(const typename Vec<T>::type (&a)[VPL], const uint32_t *__restrict__ col,
             const uint32_t *__restrict__ perm, const T *__restrict__ sval,
-            const T *__restrict__ B, T *__restrict__ C, uint32_t p0, uint32_t sub)
+            const T *__restrict__ B, T *__restrict__ C, uint32_t p0, uint32_t sub,
+            uint32_t nvec)
 {
     using V = typename Vec<T>::type;
     static_assert(NB <= LPR, "batch must fit the lane group");
@@ -221,10 +231,10 @@ sddmm_batch(const typename Vec<T>::type (&a)[VPL], const uint32_t *__restrict__ 
 #pragma unroll
     for (int u = 0; u < NB; ++u) {
         const uint32_t c = __shfl(cme, u, LPR);
-        const V *brow = row_ptr<T, LPR, VPL>(B, c, sub);
+        const V *brow = row_ptr<T, LPR, VPL, RG>(B, c, sub, nvec);
 #pragma unroll
         for (int v = 0; v < VPL; ++v)
-            b[u][v] = brow[v * LPR];
+            b[u][v] = lane_on<LPR, RG>(sub, v, nvec) ? brow[v * LPR] : V{};
     }
     __builtin_amdgcn_sched_barrier(0); // all gathers in flight before the first use
 
@@ -252,40 +262,41 @@ sddmm_batch(const typename Vec<T>::type (&a)[VPL], const uint32_t *__restrict__ 
 }
 
 // n consecutive entries from p: batches of UB, then UB/2, ..., 1 as n requires.
-template <typename T, int LPR, int VPL, int UB>
+template <typename T, int LPR, int VPL, int UB, bool RG>
 __device__ __forceinline__ void
 sddmm_walk(const typename Vec<T>::type (&a)[VPL], const uint32_t *__restrict__ col,
            const uint32_t *__restrict__ perm, const T *__restrict__ sval,
-           const T *__restrict__ B, T *__restrict__ C, uint32_t p, uint32_t n, uint32_t sub)
+           const T *__restrict__ B, T *__restrict__ C, uint32_t p, uint32_t n, uint32_t sub,
+           uint32_t nvec)
 {
     for (; n >= UB; n -= UB, p += UB)
-        sddmm_batch<T, LPR, VPL, UB>(a, col, perm, sval, B, C, p, sub);
+        sddmm_batch<T, LPR, VPL, UB, RG>(a, col, perm, sval, B, C, p, sub, nvec);
     if constexpr (UB > 8)
         if (n & 8) {
-            sddmm_batch<T, LPR, VPL, 8>(a, col, perm, sval, B, C, p, sub);
+            sddmm_batch<T, LPR, VPL, 8, RG>(a, col, perm, sval, B, C, p, sub, nvec);
             p += 8;
         }
     if constexpr (UB > 4)
         if (n & 4) {
-            sddmm_batch<T, LPR, VPL, 4>(a, col, perm, sval, B, C, p, sub);
+            sddmm_batch<T, LPR, VPL, 4, RG>(a, col, perm, sval, B, C, p, sub, nvec);
             p += 4;
         }
     if constexpr (UB > 2)
         if (n & 2) {
-            sddmm_batch<T, LPR, VPL, 2>(a, col, perm, sval, B, C, p, sub);
+            sddmm_batch<T, LPR, VPL, 2, RG>(a, col, perm, sval, B, C, p, sub, nvec);
             p += 2;
         }
     if constexpr (UB > 1)
         if (n & 1)
-            sddmm_batch<T, LPR, VPL, 1>(a, col, perm, sval, B, C, p, sub);
+            sddmm_batch<T, LPR, VPL, 1, RG>(a, col, perm, sval, B, C, p, sub, nvec);
 }
 
-template <typename T, int LPR, int VPL, int UB>
+template <typename T, int LPR, int VPL, int UB, bool RG>
 __global__ void __launch_bounds__(kBlock)
 sddmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint32_t rot,
                  const uint32_t *__restrict__ col, const uint32_t *__restrict__ perm,
                  const T *__restrict__ sval, const T *__restrict__ A, const T *__restrict__ B,
-                 T *__restrict__ C)
+                 T *__restrict__ C, uint32_t nvec)
 {
     static_assert(UB <= LPR && UB <= 16 && LPR <= 64, "batch must fit the lane group");
     using V = typename Vec<T>::type;
@@ -299,12 +310,12 @@ sddmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint3
 
     V a[VPL];
     {
-        const V *arow = row_ptr<T, LPR, VPL>(A, sg[0], sub);
+        const V *arow = row_ptr<T, LPR, VPL, RG>(A, sg[0], sub, nvec);
 #pragma unroll
         for (int v = 0; v < VPL; ++v)
-            a[v] = nt_load(arow + v * LPR);
+            a[v] = lane_on<LPR, RG>(sub, v, nvec) ? nt_load(arow + v * LPR) : V{};
     }
-    sddmm_walk<T, LPR, VPL, UB>(a, col, perm, sval, B, C, sg[1], sg[2], sub);
+    sddmm_walk<T, LPR, VPL, UB, RG>(a, col, perm, sval, B, C, sg[1], sg[2], sub, nvec);
 }
 
 // Any K: one wavefront per segment, lanes stride over K, scalar loads.
@@ -337,10 +348,11 @@ sddmm_generic_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, u
 }
 
 // ----------------------------------------------------------------- SpMM ----
-template <typename T, int LPR, int VPL, int NB>
+template <typename T, int LPR, int VPL, int NB, bool RG>
 __device__ __forceinline__ void
 spmm_batch(typename Vec<T>::type (&acc)[VPL], const uint32_t *__restrict__ col,
-           const T *__restrict__ sval, const T *__restrict__ X, uint32_t p0, uint32_t sub)
+           const T *__restrict__ sval, const T *__restrict__ X, uint32_t p0, uint32_t sub,
+           uint32_t nvec)
 {
     using V = typename Vec<T>::type;
     static_assert(NB <= LPR, "batch must fit the lane group");
@@ -354,10 +366,10 @@ spmm_batch(typename Vec<T>::type (&acc)[VPL], const uint32_t *__restrict__ col,
     for (int u = 0; u < NB; ++u) {
         const uint32_t c = __shfl(cme, u, LPR);
         av[u] = __shfl(vme, u, LPR);
-        const V *xrow = row_ptr<T, LPR, VPL>(X, c, sub);
+        const V *xrow = row_ptr<T, LPR, VPL, RG>(X, c, sub, nvec);
 #pragma unroll
         for (int v = 0; v < VPL; ++v)
-            x[u][v] = xrow[v * LPR];
+            x[u][v] = lane_on<LPR, RG>(sub, v, nvec) ? xrow[v * LPR] : V{};
     }
     __builtin_amdgcn_sched_barrier(0); // all gathers in flight before the first use
     // Entries are added in kernel order.
@@ -368,39 +380,40 @@ spmm_batch(typename Vec<T>::type (&acc)[VPL], const uint32_t *__restrict__ col,
             acc[v] += x[u][v] * av[u];
 }
 
-template <typename T, int LPR, int VPL, int UB>
+template <typename T, int LPR, int VPL, int UB, bool RG>
 __device__ __forceinline__ void
 spmm_walk(typename Vec<T>::type (&acc)[VPL], const uint32_t *__restrict__ col,
           const T *__restrict__ sval, const T *__restrict__ X, uint32_t p, uint32_t n,
-          uint32_t sub)
+          uint32_t sub, uint32_t nvec)
 {
     for (; n >= UB; n -= UB, p += UB)
-        spmm_batch<T, LPR, VPL, UB>(acc, col, sval, X, p, sub);
+        spmm_batch<T, LPR, VPL, UB, RG>(acc, col, sval, X, p, sub, nvec);
     if constexpr (UB > 8)
         if (n & 8) {
-            spmm_batch<T, LPR, VPL, 8>(acc, col, sval, X, p, sub);
+            spmm_batch<T, LPR, VPL, 8, RG>(acc, col, sval, X, p, sub, nvec);
             p += 8;
         }
     if constexpr (UB > 4)
         if (n & 4) {
-            spmm_batch<T, LPR, VPL, 4>(acc, col, sval, X, p, sub);
+            spmm_batch<T, LPR, VPL, 4, RG>(acc, col, sval, X, p, sub, nvec);
             p += 4;
         }
     if constexpr (UB > 2)
         if (n & 2) {
-            spmm_batch<T, LPR, VPL, 2>(acc, col, sval, X, p, sub);
+            spmm_batch<T, LPR, VPL, 2, RG>(acc, col, sval, X, p, sub, nvec);
             p += 2;
         }
     if constexpr (UB > 1)
         if (n & 1)
-            spmm_batch<T, LPR, VPL, 1>(acc, col, sval, X, p, sub);
+            spmm_batch<T, LPR, VPL, 1, RG>(acc, col, sval, X, p, sub, nvec);
 }
 
-template <typename T, int LPR, int VPL, int UB>
+template <typename T, int LPR, int VPL, int UB, bool RG>
 __global__ void __launch_bounds__(kBlock)
 spmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint32_t rot,
                 const uint32_t *__restrict__ col, const T *__restrict__ sval,
-                const T *__restrict__ X, T *__restrict__ Y, T *__restrict__ partial)
+                const T *__restrict__ X, T *__restrict__ Y, T *__restrict__ partial,
+                uint32_t nvec)
 {
     static_assert(UB <= LPR && UB <= 16 && LPR <= 64, "batch must fit the lane group");
     using V = typename Vec<T>::type;
@@ -412,8 +425,8 @@ spmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint32
     if (sg[2] == 0)
         return;
     const bool whole = sg[3] == kWholeRow;
-    V *dst = const_cast<V *>(whole ? row_ptr<T, LPR, VPL>(Y, sg[0], sub)
-                                   : row_ptr<T, LPR, VPL>(partial, sg[3], sub));
+    V *dst = const_cast<V *>(whole ? row_ptr<T, LPR, VPL, RG>(Y, sg[0], sub, nvec)
+                                   : row_ptr<T, LPR, VPL, RG>(partial, sg[3], sub, nvec));
 
     V acc[VPL], y0[VPL];
 #pragma unroll
@@ -424,16 +437,17 @@ spmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint32
     if (whole) {
 #pragma unroll
         for (int v = 0; v < VPL; ++v)
-            y0[v] = nt_load(dst + v * LPR);
+            if (lane_on<LPR, RG>(sub, v, nvec))
+                y0[v] = nt_load(dst + v * LPR);
     }
-    spmm_walk<T, LPR, VPL, UB>(acc, col, sval, X, sg[1], sg[2], sub);
-    if (whole) {
+    spmm_walk<T, LPR, VPL, UB, RG>(acc, col, sval, X, sg[1], sg[2], sub, nvec);
 #pragma unroll
-        for (int v = 0; v < VPL; ++v)
+    for (int v = 0; v < VPL; ++v) {
+        if (!lane_on<LPR, RG>(sub, v, nvec))
+            continue;
+        if (whole)
             nt_store(y0[v] + acc[v], dst + v * LPR);
-    } else {
-#pragma unroll
-        for (int v = 0; v < VPL; ++v)
+        else
             dst[v * LPR] = acc[v]; // read back by spmm_fixup right after
     }
 }
@@ -598,30 +612,38 @@ copy_kernel(u32x4 *__restrict__ dst, const u32x4 *__restrict__ src, uint64_t nve
 
 // ------------------------------------------------------------- dispatch ----
 struct Shape {
-    int lpr, vpl, ub; // lpr == 0: generic kernel
+    int lpr, vpl;  // lpr == 0: generic kernel
+    bool ragged;   // fewer vectors per row than lpr * vpl
+    uint32_t nvec; // 16-byte vectors per dense row
 };
 
-// K * sizeof(T) must be LPR * VPL * 16 bytes with LPR a power of two in
-// [4, 64] and VPL in {1, 2, 4}; anything else takes the generic kernels.
+// A dense row of K reals must be a whole number nvec <= 256 of 16-byte vectors;
+// anything else takes the generic kernels.  nvec == LPR * VPL with LPR a power of
+// two in [4, 64] and VPL in {1, 2, 4} runs a kernel with the row stride compiled
+// in; other nvec run the "ragged" variant of the smallest shape that covers a row,
+// in which the lanes past the row's end idle.
 Shape pick_shape(size_t elem, uint32_t K)
 {
     const size_t bytes = (size_t)K * elem;
-    if (K == 0 || bytes % 16)
-        return {0, 0, 0};
-    const size_t nvec = bytes / 16;
+    if (K == 0 || bytes % 16 || bytes / 16 > 256)
+        return {0, 0, false, 0};
+    const uint32_t nvec = (uint32_t)(bytes / 16);
     for (int lpr = 64; lpr >= 4; lpr >>= 1) {
         if (nvec % lpr)
             continue;
-        const size_t vpl = nvec / lpr;
-        if (vpl == 1)
-            return {lpr, 1, lpr < 16 ? lpr : 16};
-        if (vpl == 2)
-            return {lpr, 2, lpr < 8 ? lpr : 8};
-        if (vpl == 4)
-            return {lpr, 4, 4};
-        return {0, 0, 0};
+        const uint32_t vpl = nvec / lpr;
+        if (vpl == 1 || vpl == 2 || vpl == 4)
+            return {lpr, (int)vpl, false, nvec};
+        break;
     }
-    return {0, 0, 0};
+    if (nvec > 128)
+        return {64, 4, true, nvec};
+    if (nvec > 64)
+        return {64, 2, true, nvec};
+    int lpr = 4;
+    while ((uint32_t)lpr < nvec)
+        lpr *= 2;
+    return {lpr, 1, true, nvec};
 }
 
 // Workgroups needed to cover nseg segments (a whole number of chunks, and of
@@ -662,41 +684,44 @@ inline hipError_t join_aux(const Streams &S)
     return hipStreamSynchronize(S.aux);
 }
 
-template <typename T, int LPR, int VPL, int UB, int US>
-hipError_t run_sddmm(const DevPlanView &P, const T *A, const T *B, T *C, const Streams &S)
+template <typename T, int LPR, int VPL, int UB, int US, bool RG>
+hipError_t run_sddmm(const DevPlanView &P, const T *A, const T *B, T *C, const Streams &S,
+                     uint32_t nvec)
 {
     const uint32_t nl = P.nseg_long, ns = P.nseg - P.nseg_long;
     const bool both = nl && ns && fork_aux(S);
     if (nl)
-        hipLaunchKernelGGL((sddmm_seg_kernel<T, LPR, VPL, UB>),
+        hipLaunchKernelGGL((sddmm_seg_kernel<T, LPR, VPL, UB, RG>),
                            dim3(blocks_for_groups(nl, P.nqueues, 64 / LPR)), dim3(kBlock), 0,
                            S.main, P.segs, nl, P.nqueues, 0u, P.col, P.perm, (const T *)P.sval,
-                           A, B, C);
+                           A, B, C, nvec);
     if (ns)
-        hipLaunchKernelGGL((sddmm_seg_kernel<T, LPR, VPL, US>),
+        hipLaunchKernelGGL((sddmm_seg_kernel<T, LPR, VPL, US, RG>),
                            dim3(blocks_for_groups(ns, P.nqueues, 64 / LPR)), dim3(kBlock), 0,
                            both ? S.aux : S.main, P.segs + nl, ns, P.nqueues,
-                           both ? S.aux_rot : 0u, P.col, P.perm, (const T *)P.sval, A, B, C);
+                           both ? S.aux_rot : 0u, P.col, P.perm, (const T *)P.sval, A, B, C,
+                           nvec);
     const hipError_t launched = hipGetLastError();
     const hipError_t joined = both ? join_aux(S) : hipSuccess;
     return launched != hipSuccess ? launched : joined;
 }
 
-template <typename T, int LPR, int VPL, int UB, int US>
-hipError_t run_spmm(const DevPlanView &P, const T *X, T *Y, const Streams &S)
+template <typename T, int LPR, int VPL, int UB, int US, bool RG>
+hipError_t run_spmm(const DevPlanView &P, const T *X, T *Y, const Streams &S, uint32_t nvec)
 {
     const uint32_t nl = P.nseg_long, ns = P.nseg - P.nseg_long;
     const bool both = nl && ns && fork_aux(S);
     if (nl)
-        hipLaunchKernelGGL((spmm_seg_kernel<T, LPR, VPL, UB>),
+        hipLaunchKernelGGL((spmm_seg_kernel<T, LPR, VPL, UB, RG>),
                            dim3(blocks_for_groups(nl, P.nqueues, 64 / LPR)), dim3(kBlock), 0,
                            S.main, P.segs, nl, P.nqueues, 0u, P.col, (const T *)P.sval, X, Y,
-                           (T *)P.partial);
+                           (T *)P.partial, nvec);
     if (ns)
-        hipLaunchKernelGGL((spmm_seg_kernel<T, LPR, VPL, US>),
+        hipLaunchKernelGGL((spmm_seg_kernel<T, LPR, VPL, US, RG>),
                            dim3(blocks_for_groups(ns, P.nqueues, 64 / LPR)), dim3(kBlock), 0,
                            both ? S.aux : S.main, P.segs + nl, ns, P.nqueues,
-                           both ? S.aux_rot : 0u, P.col, (const T *)P.sval, X, Y, (T *)P.partial);
+                           both ? S.aux_rot : 0u, P.col, (const T *)P.sval, X, Y, (T *)P.partial,
+                           nvec);
     const hipError_t launched = hipGetLastError();
     const hipError_t joined = both ? join_aux(S) : hipSuccess;
     return launched != hipSuccess ? launched : joined;
@@ -708,6 +733,11 @@ hipError_t run_spmm(const DevPlanView &P, const T *X, T *Y, const Streams &S)
     X(4, 1, 4, 4) X(8, 1, 8, 4) X(16, 1, 16, 4) X(32, 1, 16, 4) X(64, 1, 16, 4)                   \
     X(4, 2, 4, 2) X(8, 2, 8, 2) X(16, 2, 8, 2) X(32, 2, 8, 2) X(64, 2, 8, 2)                      \
     X(4, 4, 4, 1) X(8, 4, 4, 1) X(16, 4, 4, 1) X(32, 4, 4, 1) X(64, 4, 4, 1)
+// Rows that do not fill a shape: the smallest power-of-two LPR covering the row,
+// then 64 lanes with 2 or 4 vectors each.
+#define SPC3D_FOR_RAGGED_SHAPES(X)                                                                \
+    X(4, 1, 4, 4) X(8, 1, 8, 4) X(16, 1, 16, 4) X(32, 1, 16, 4) X(64, 1, 16, 4) X(64, 2, 8, 2)    \
+    X(64, 4, 4, 1)
 
 template <typename T>
 hipError_t sddmm_typed(const DevPlanView &P, const void *A, const void *B, void *C, uint32_t K,
@@ -720,11 +750,18 @@ hipError_t sddmm_typed(const DevPlanView &P, const void *A, const void *B, void 
     bool done = false;
     hipError_t e = hipSuccess;
 #define X(L, V, U, S)                                                                             \
-    if (!done && sh.lpr == L && sh.vpl == V) {                                                    \
-        e = run_sddmm<T, L, V, U, S>(P, (const T *)A, (const T *)B, (T *)C, SS);                  \
+    if (!done && !sh.ragged && sh.lpr == L && sh.vpl == V) {                                      \
+        e = run_sddmm<T, L, V, U, S, false>(P, (const T *)A, (const T *)B, (T *)C, SS, sh.nvec);  \
         done = true;                                                                              \
     }
     SPC3D_FOR_SHAPES(X)
+#undef X
+#define X(L, V, U, S)                                                                             \
+    if (!done && sh.ragged && sh.lpr == L && sh.vpl == V) {                                       \
+        e = run_sddmm<T, L, V, U, S, true>(P, (const T *)A, (const T *)B, (T *)C, SS, sh.nvec);   \
+        done = true;                                                                              \
+    }
+    SPC3D_FOR_RAGGED_SHAPES(X)
 #undef X
     if (!done) {
         const uint32_t grid = blocks_for_groups(P.nseg, P.nqueues, 1);
@@ -747,11 +784,18 @@ hipError_t spmm_typed(const DevPlanView &P, const void *X_, void *Y, uint32_t K,
     bool done = false;
     hipError_t e = hipSuccess;
 #define X(L, V, U, S)                                                                             \
-    if (!done && sh.lpr == L && sh.vpl == V) {                                                    \
-        e = run_spmm<T, L, V, U, S>(P, (const T *)X_, (T *)Y, SS);                                \
+    if (!done && !sh.ragged && sh.lpr == L && sh.vpl == V) {                                      \
+        e = run_spmm<T, L, V, U, S, false>(P, (const T *)X_, (T *)Y, SS, sh.nvec);                \
         done = true;                                                                              \
     }
     SPC3D_FOR_SHAPES(X)
+#undef X
+#define X(L, V, U, S)                                                                             \
+    if (!done && sh.ragged && sh.lpr == L && sh.vpl == V) {                                       \
+        e = run_spmm<T, L, V, U, S, true>(P, (const T *)X_, (T *)Y, SS, sh.nvec);                 \
+        done = true;                                                                              \
+    }
+    SPC3D_FOR_RAGGED_SHAPES(X)
 #undef X
     if (!done) {
         const uint32_t grid = blocks_for_groups(P.nseg, P.nqueues, 1);
@@ -890,8 +934,8 @@ const char *kernel_variant(int dtype, uint32_t K)
     if (sh.lpr == 0)
         snprintf(buf, sizeof buf, "generic<%s>", dtype == 1 ? "f64" : "f32");
     else
-        snprintf(buf, sizeof buf, "seg<%s,LPR=%d,VPL=%d,UB=%d>", dtype == 1 ? "f64" : "f32",
-                 sh.lpr, sh.vpl, sh.ub);
+        snprintf(buf, sizeof buf, "seg<%s,LPR=%d,VPL=%d%s>", dtype == 1 ? "f64" : "f32", sh.lpr,
+                 sh.vpl, sh.ragged ? ",ragged" : "");
     return buf;
 }
 

@@ -105,9 +105,12 @@ def test_golden_numcheck_closed_form(ctx):
     assert abs(C.sum() - g["C"].sum()) < 1e-16
 
 
-# ---- K sweep: vector kernels (K*sizeof a multiple of 64 B) and the generic ones
+# ---- K sweep: rows that fill a kernel shape exactly (a power of two of 16-byte
+# vectors), rows that do not (the "ragged" variants: 12, 20, 48, 100, 300 ...), rows
+# that are no whole number of vectors or longer than 4 KiB (the generic kernels)
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("k", [1, 3, 4, 8, 12, 16, 20, 32, 48, 64, 100, 128, 256, 512])
+@pytest.mark.parametrize("k", [1, 2, 3, 4, 6, 8, 10, 12, 16, 20, 24, 32, 36, 48, 64, 72, 96, 100,
+                               128, 130, 200, 256, 300, 384, 512, 1024, 1028])
 def test_k_sweep_random_unsorted(ctx, dtype, k):
     ii, jj, vv, A, B, Y0 = rand_case(100 + k, 300, 257, k, 6000, dtype, hub=700)
     check_sddmm(A, B, ii, jj, vv, gpu_sddmm(ctx, 300, 257, ii, jj, vv, A, B, prefill=-5.0))
@@ -120,6 +123,15 @@ def test_segment_lengths_and_cut_rows(ctx, dtype, seg_max):
     ii, jj, vv, A, B, Y0 = rand_case(7, 64, 500, 64, 5000, dtype, hub=2000)
     check_sddmm(A, B, ii, jj, vv, gpu_sddmm(ctx, 64, 500, ii, jj, vv, A, B, seg_max=seg_max))
     check_spmm(B, ii, jj, vv, Y0, gpu_spmm(ctx, 64, 500, ii, jj, vv, B, Y0, seg_max=seg_max))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("k", [12, 48, 100, 136, 264])
+def test_cut_rows_with_ragged_k(ctx, dtype, k):
+    # partial rows of cut segments and the fix-up pass at row widths that leave lanes idle
+    ii, jj, vv, A, B, Y0 = rand_case(11 + k, 40, 300, k, 4000, dtype, hub=1500)
+    check_sddmm(A, B, ii, jj, vv, gpu_sddmm(ctx, 40, 300, ii, jj, vv, A, B, seg_max=64))
+    check_spmm(B, ii, jj, vv, Y0, gpu_spmm(ctx, 40, 300, ii, jj, vv, B, Y0, seg_max=64))
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
