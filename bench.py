@@ -35,10 +35,13 @@ METRIC = "SDDMM & SpMM GFLOP/s + % HBM roofline on 1 MI355X, RMAT-20 K=64"
 # --pmc FETCH_SIZE / WRITE_SIZE, calibrated on a plain copy; they cannot be
 # collected from inside this process, so they are quoted from
 # profiles/sddmm_spmm_rmat20_k64_hbm_traffic.md for the workload they were taken
-# on (default plan options) and left null for any other.  spmm includes its fix-up.
+# on (default plan options) and left null for any other: long-segment launch +
+# short-segment launch (+ fix-up for spmm).
 MEASURED_TRAFFIC = {
-    ("rmat20_ef16", 64, "sorted", "f64"): {"sddmm": 5907.7e6, "spmm": 5434.4e6 + 125.1e6},
-    ("rmat20_ef16", 64, "sorted", "f32"): {"sddmm": 3100.6e6, "spmm": 2582.5e6 + 63.9e6},
+    ("rmat20_ef16", 64, "sorted", "f64"): {"sddmm": 4675.3e6 + 1289.8e6,
+                                           "spmm": 4143.0e6 + 1328.7e6 + 123.1e6},
+    ("rmat20_ef16", 64, "sorted", "f32"): {"sddmm": 2358.9e6 + 796.0e6,
+                                           "spmm": 1885.2e6 + 724.9e6 + 61.8e6},
 }
 
 
