@@ -204,11 +204,15 @@ __device__ __forceinline__ bool lane_on(uint32_t sub, int v, uint32_t nvec)
 }
 
 // ---------------------------------------------------------------- SDDMM ----
-template <typename T, int LPR, int VPL, int NB, bool RG>
+// One batch of NB entries from p0.  MK ("masked"): only the first n (1 <= n <= NB)
+// exist; the others repeat entry n - 1 (loads without branches, from addresses
+// that are being read anyway) and store nothing, so that a tail of any length
+// costs one round of gathers.
+template <typename T, int LPR, int VPL, int NB, bool RG, bool MK>
 __device__ __forceinline__ void
 sddmm_batch(const typename Vec<T>::type (&a)[VPL], const uint32_t *__restrict__ col,
             const uint32_t *__restrict__ perm, const T *__restrict__ sval,
-            const T *__restrict__ B, T *__restrict__ C, uint32_t p0, uint32_t sub,
+            const T *__restrict__ B, T *__restrict__ C, uint32_t p0, uint32_t n, uint32_t sub,
             uint32_t nvec)
 {
     using V = typename Vec<T>::type;
@@ -216,9 +220,12 @@ sddmm_batch(const typename Vec<T>::type (&a)[VPL], const uint32_t *__restrict__ 
 
     // Lane u of the group fetches the column of entry u; the writer lanes fetch
     // what they need for the store.  These head the dependency chain.
-    const uint32_t cme = nt_load(col + p0 + (sub & (NB - 1)));
-    const bool writer = is_writer<LPR, NB>(sub);
+    uint32_t e = sub & (NB - 1);
+    if (MK)
+        e = e < n ? e : n - 1;
+    const uint32_t cme = nt_load(col + p0 + e);
     const uint32_t uo = entry_of<LPR, NB>(sub);
+    const bool writer = is_writer<LPR, NB>(sub) && (!MK || uo < n);
     T sv = (T)0;
     uint32_t dst = p0 + uo;
     if (writer) {
@@ -261,37 +268,47 @@ sddmm_batch(const typename Vec<T>::type (&a)[VPL], const uint32_t *__restrict__ 
     }
 }
 
-// n consecutive entries from p: batches of UB, then UB/2, ..., 1 as n requires.
-template <typename T, int LPR, int VPL, int UB, bool RG>
+// n consecutive entries from p.  WIDE: full batches of UB, then one masked batch
+// of the smallest size in {4, 8, 16} that holds the rest.  !WIDE (segments known
+// to be short, run at twice the occupancy): masked batches of UB throughout.
+template <typename T, int LPR, int VPL, int UB, bool RG, bool WIDE>
 __device__ __forceinline__ void
 sddmm_walk(const typename Vec<T>::type (&a)[VPL], const uint32_t *__restrict__ col,
            const uint32_t *__restrict__ perm, const T *__restrict__ sval,
            const T *__restrict__ B, T *__restrict__ C, uint32_t p, uint32_t n, uint32_t sub,
            uint32_t nvec)
 {
-    for (; n >= UB; n -= UB, p += UB)
-        sddmm_batch<T, LPR, VPL, UB, RG>(a, col, perm, sval, B, C, p, sub, nvec);
-    if constexpr (UB > 8)
-        if (n & 8) {
-            sddmm_batch<T, LPR, VPL, 8, RG>(a, col, perm, sval, B, C, p, sub, nvec);
-            p += 8;
+    if constexpr (WIDE) {
+        for (; n >= UB; n -= UB, p += UB)
+            sddmm_batch<T, LPR, VPL, UB, RG, false>(a, col, perm, sval, B, C, p, UB, sub, nvec);
+        if (n == 0)
+            return;
+        if constexpr (UB > 8) {
+            if (n > 8) {
+                sddmm_batch<T, LPR, VPL, UB, RG, true>(a, col, perm, sval, B, C, p, n, sub, nvec);
+                return;
+            }
         }
-    if constexpr (UB > 4)
-        if (n & 4) {
-            sddmm_batch<T, LPR, VPL, 4, RG>(a, col, perm, sval, B, C, p, sub, nvec);
-            p += 4;
+        if constexpr (UB > 4) {
+            if (n > 4) {
+                sddmm_batch<T, LPR, VPL, 8, RG, true>(a, col, perm, sval, B, C, p, n, sub, nvec);
+                return;
+            }
         }
-    if constexpr (UB > 2)
-        if (n & 2) {
-            sddmm_batch<T, LPR, VPL, 2, RG>(a, col, perm, sval, B, C, p, sub, nvec);
-            p += 2;
+        sddmm_batch<T, LPR, VPL, (UB < 4 ? UB : 4), RG, true>(a, col, perm, sval, B, C, p, n, sub,
+                                                              nvec);
+    } else {
+#pragma nounroll
+        while (n > 0) {
+            const uint32_t m = n < (uint32_t)UB ? n : (uint32_t)UB;
+            sddmm_batch<T, LPR, VPL, UB, RG, true>(a, col, perm, sval, B, C, p, m, sub, nvec);
+            n -= m;
+            p += m;
         }
-    if constexpr (UB > 1)
-        if (n & 1)
-            sddmm_batch<T, LPR, VPL, 1, RG>(a, col, perm, sval, B, C, p, sub, nvec);
+    }
 }
 
-template <typename T, int LPR, int VPL, int UB, bool RG>
+template <typename T, int LPR, int VPL, int UB, bool RG, bool WIDE>
 __global__ void __launch_bounds__(kBlock)
 sddmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint32_t rot,
                  const uint32_t *__restrict__ col, const uint32_t *__restrict__ perm,
@@ -315,7 +332,7 @@ sddmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint3
         for (int v = 0; v < VPL; ++v)
             a[v] = lane_on<LPR, RG>(sub, v, nvec) ? nt_load(arow + v * LPR) : V{};
     }
-    sddmm_walk<T, LPR, VPL, UB, RG>(a, col, perm, sval, B, C, sg[1], sg[2], sub, nvec);
+    sddmm_walk<T, LPR, VPL, UB, RG, WIDE>(a, col, perm, sval, B, C, sg[1], sg[2], sub, nvec);
 }
 
 // Any K: one wavefront per segment, lanes stride over K, scalar loads.
@@ -348,17 +365,21 @@ sddmm_generic_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, u
 }
 
 // ----------------------------------------------------------------- SpMM ----
-template <typename T, int LPR, int VPL, int NB, bool RG>
+// MK: only the first n of the NB entries exist; the others repeat the loads of
+// entry n - 1 and add zero times zero.
+template <typename T, int LPR, int VPL, int NB, bool RG, bool MK>
 __device__ __forceinline__ void
 spmm_batch(typename Vec<T>::type (&acc)[VPL], const uint32_t *__restrict__ col,
-           const T *__restrict__ sval, const T *__restrict__ X, uint32_t p0, uint32_t sub,
-           uint32_t nvec)
+           const T *__restrict__ sval, const T *__restrict__ X, uint32_t p0, uint32_t n,
+           uint32_t sub, uint32_t nvec)
 {
     using V = typename Vec<T>::type;
     static_assert(NB <= LPR, "batch must fit the lane group");
-    const uint32_t pl = p0 + (sub & (NB - 1));
-    const uint32_t cme = nt_load(col + pl);
-    const T vme = nt_load(sval + pl);
+    uint32_t e = sub & (NB - 1);
+    if (MK)
+        e = e < n ? e : n - 1;
+    const uint32_t cme = nt_load(col + p0 + e);
+    const T vme = nt_load(sval + p0 + e);
 
     V x[NB][VPL];
     T av[NB];
@@ -374,41 +395,68 @@ spmm_batch(typename Vec<T>::type (&acc)[VPL], const uint32_t *__restrict__ col,
     __builtin_amdgcn_sched_barrier(0); // all gathers in flight before the first use
     // Entries are added in kernel order.
 #pragma unroll
-    for (int u = 0; u < NB; ++u)
+    for (int u = 0; u < NB; ++u) {
+        const bool on = !MK || (uint32_t)u < n;
+        const T a = on ? av[u] : (T)0;
 #pragma unroll
         for (int v = 0; v < VPL; ++v)
-            acc[v] += x[u][v] * av[u];
+            acc[v] += (on ? x[u][v] : V{}) * a;
+    }
 }
 
-template <typename T, int LPR, int VPL, int UB, bool RG>
+template <typename T, int LPR, int VPL, int UB, bool RG, bool WIDE>
 __device__ __forceinline__ void
 spmm_walk(typename Vec<T>::type (&acc)[VPL], const uint32_t *__restrict__ col,
           const T *__restrict__ sval, const T *__restrict__ X, uint32_t p, uint32_t n,
           uint32_t sub, uint32_t nvec)
 {
-    for (; n >= UB; n -= UB, p += UB)
-        spmm_batch<T, LPR, VPL, UB, RG>(acc, col, sval, X, p, sub, nvec);
-    if constexpr (UB > 8)
-        if (n & 8) {
-            spmm_batch<T, LPR, VPL, 8, RG>(acc, col, sval, X, p, sub, nvec);
-            p += 8;
+    // Short segments: exact batches of UB, then UB/2 ... 1 as n requires.  Measured
+    // against masked batches here (which cost registers, hence occupancy): 3 % faster
+    // on 5-entry rows, level elsewhere.  SpMM's short rows are bound by the Y
+    // read-modify-write stream, not by rounds of gathers.
+    if constexpr (!WIDE) {
+        for (; n >= UB; n -= UB, p += UB)
+            spmm_batch<T, LPR, VPL, UB, RG, false>(acc, col, sval, X, p, UB, sub, nvec);
+        if constexpr (UB > 8)
+            if (n & 8) {
+                spmm_batch<T, LPR, VPL, 8, RG, false>(acc, col, sval, X, p, 8, sub, nvec);
+                p += 8;
+            }
+        if constexpr (UB > 4)
+            if (n & 4) {
+                spmm_batch<T, LPR, VPL, 4, RG, false>(acc, col, sval, X, p, 4, sub, nvec);
+                p += 4;
+            }
+        if constexpr (UB > 2)
+            if (n & 2) {
+                spmm_batch<T, LPR, VPL, 2, RG, false>(acc, col, sval, X, p, 2, sub, nvec);
+                p += 2;
+            }
+        if constexpr (UB > 1)
+            if (n & 1)
+                spmm_batch<T, LPR, VPL, 1, RG, false>(acc, col, sval, X, p, 1, sub, nvec);
+    } else {
+        for (; n >= UB; n -= UB, p += UB)
+            spmm_batch<T, LPR, VPL, UB, RG, false>(acc, col, sval, X, p, UB, sub, nvec);
+        if (n == 0)
+            return;
+        if constexpr (UB > 8) {
+            if (n > 8) {
+                spmm_batch<T, LPR, VPL, UB, RG, true>(acc, col, sval, X, p, n, sub, nvec);
+                return;
+            }
         }
-    if constexpr (UB > 4)
-        if (n & 4) {
-            spmm_batch<T, LPR, VPL, 4, RG>(acc, col, sval, X, p, sub, nvec);
-            p += 4;
+        if constexpr (UB > 4) {
+            if (n > 4) {
+                spmm_batch<T, LPR, VPL, 8, RG, true>(acc, col, sval, X, p, n, sub, nvec);
+                return;
+            }
         }
-    if constexpr (UB > 2)
-        if (n & 2) {
-            spmm_batch<T, LPR, VPL, 2, RG>(acc, col, sval, X, p, sub, nvec);
-            p += 2;
-        }
-    if constexpr (UB > 1)
-        if (n & 1)
-            spmm_batch<T, LPR, VPL, 1, RG>(acc, col, sval, X, p, sub, nvec);
+        spmm_batch<T, LPR, VPL, (UB < 4 ? UB : 4), RG, true>(acc, col, sval, X, p, n, sub, nvec);
+    }
 }
 
-template <typename T, int LPR, int VPL, int UB, bool RG>
+template <typename T, int LPR, int VPL, int UB, bool RG, bool WIDE>
 __global__ void __launch_bounds__(kBlock)
 spmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint32_t rot,
                 const uint32_t *__restrict__ col, const T *__restrict__ sval,
@@ -440,7 +488,7 @@ spmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint32
             if (lane_on<LPR, RG>(sub, v, nvec))
                 y0[v] = nt_load(dst + v * LPR);
     }
-    spmm_walk<T, LPR, VPL, UB, RG>(acc, col, sval, X, sg[1], sg[2], sub, nvec);
+    spmm_walk<T, LPR, VPL, UB, RG, WIDE>(acc, col, sval, X, sg[1], sg[2], sub, nvec);
 #pragma unroll
     for (int v = 0; v < VPL; ++v) {
         if (!lane_on<LPR, RG>(sub, v, nvec))
@@ -691,12 +739,12 @@ hipError_t run_sddmm(const DevPlanView &P, const T *A, const T *B, T *C, const S
     const uint32_t nl = P.nseg_long, ns = P.nseg - P.nseg_long;
     const bool both = nl && ns && fork_aux(S);
     if (nl)
-        hipLaunchKernelGGL((sddmm_seg_kernel<T, LPR, VPL, UB, RG>),
+        hipLaunchKernelGGL((sddmm_seg_kernel<T, LPR, VPL, UB, RG, true>),
                            dim3(blocks_for_groups(nl, P.nqueues, 64 / LPR)), dim3(kBlock), 0,
                            S.main, P.segs, nl, P.nqueues, 0u, P.col, P.perm, (const T *)P.sval,
                            A, B, C, nvec);
     if (ns)
-        hipLaunchKernelGGL((sddmm_seg_kernel<T, LPR, VPL, US, RG>),
+        hipLaunchKernelGGL((sddmm_seg_kernel<T, LPR, VPL, US, RG, false>),
                            dim3(blocks_for_groups(ns, P.nqueues, 64 / LPR)), dim3(kBlock), 0,
                            both ? S.aux : S.main, P.segs + nl, ns, P.nqueues,
                            both ? S.aux_rot : 0u, P.col, P.perm, (const T *)P.sval, A, B, C,
@@ -712,12 +760,12 @@ hipError_t run_spmm(const DevPlanView &P, const T *X, T *Y, const Streams &S, ui
     const uint32_t nl = P.nseg_long, ns = P.nseg - P.nseg_long;
     const bool both = nl && ns && fork_aux(S);
     if (nl)
-        hipLaunchKernelGGL((spmm_seg_kernel<T, LPR, VPL, UB, RG>),
+        hipLaunchKernelGGL((spmm_seg_kernel<T, LPR, VPL, UB, RG, true>),
                            dim3(blocks_for_groups(nl, P.nqueues, 64 / LPR)), dim3(kBlock), 0,
                            S.main, P.segs, nl, P.nqueues, 0u, P.col, (const T *)P.sval, X, Y,
                            (T *)P.partial, nvec);
     if (ns)
-        hipLaunchKernelGGL((spmm_seg_kernel<T, LPR, VPL, US, RG>),
+        hipLaunchKernelGGL((spmm_seg_kernel<T, LPR, VPL, US, RG, false>),
                            dim3(blocks_for_groups(ns, P.nqueues, 64 / LPR)), dim3(kBlock), 0,
                            both ? S.aux : S.main, P.segs + nl, ns, P.nqueues,
                            both ? S.aux_rot : 0u, P.col, (const T *)P.sval, X, Y, (T *)P.partial,
@@ -727,17 +775,17 @@ hipError_t run_spmm(const DevPlanView &P, const T *X, T *Y, const Streams &S, ui
     return launched != hipSuccess ? launched : joined;
 }
 
-// (LPR, VPL, UB, US): UB * VPL 16-byte gathers are in flight per lane in the
-// long-segment launch, US * VPL in the short-segment one.
+// (LPR, VPL, UB, US_SDDMM, US_SPMM): UB * VPL 16-byte gathers are in flight per
+// lane in the long-segment launch, US * VPL in the short-segment one.
 #define SPC3D_FOR_SHAPES(X)                                                                       \
-    X(4, 1, 4, 4) X(8, 1, 8, 4) X(16, 1, 16, 4) X(32, 1, 16, 4) X(64, 1, 16, 4)                   \
-    X(4, 2, 4, 2) X(8, 2, 8, 2) X(16, 2, 8, 2) X(32, 2, 8, 2) X(64, 2, 8, 2)                      \
-    X(4, 4, 4, 1) X(8, 4, 4, 1) X(16, 4, 4, 1) X(32, 4, 4, 1) X(64, 4, 4, 1)
+    X(4, 1, 4, 4, 4) X(8, 1, 8, 8, 4) X(16, 1, 16, 8, 4) X(32, 1, 16, 8, 4) X(64, 1, 16, 8, 4)    \
+    X(4, 2, 4, 4, 2) X(8, 2, 8, 4, 2) X(16, 2, 8, 4, 2) X(32, 2, 8, 4, 2) X(64, 2, 8, 4, 2)       \
+    X(4, 4, 4, 2, 1) X(8, 4, 4, 2, 1) X(16, 4, 4, 2, 1) X(32, 4, 4, 2, 1) X(64, 4, 4, 2, 1)
 // Rows that do not fill a shape: the smallest power-of-two LPR covering the row,
 // then 64 lanes with 2 or 4 vectors each.
 #define SPC3D_FOR_RAGGED_SHAPES(X)                                                                \
-    X(4, 1, 4, 4) X(8, 1, 8, 4) X(16, 1, 16, 4) X(32, 1, 16, 4) X(64, 1, 16, 4) X(64, 2, 8, 2)    \
-    X(64, 4, 4, 1)
+    X(4, 1, 4, 4, 4) X(8, 1, 8, 8, 4) X(16, 1, 16, 8, 4) X(32, 1, 16, 8, 4) X(64, 1, 16, 8, 4)    \
+    X(64, 2, 8, 4, 2) X(64, 4, 4, 2, 1)
 
 template <typename T>
 hipError_t sddmm_typed(const DevPlanView &P, const void *A, const void *B, void *C, uint32_t K,
@@ -749,14 +797,14 @@ hipError_t sddmm_typed(const DevPlanView &P, const void *A, const void *B, void 
     const Shape sh = pick_shape(sizeof(T), K);
     bool done = false;
     hipError_t e = hipSuccess;
-#define X(L, V, U, S)                                                                             \
+#define X(L, V, U, S, S2)                                                                         \
     if (!done && !sh.ragged && sh.lpr == L && sh.vpl == V) {                                      \
         e = run_sddmm<T, L, V, U, S, false>(P, (const T *)A, (const T *)B, (T *)C, SS, sh.nvec);  \
         done = true;                                                                              \
     }
     SPC3D_FOR_SHAPES(X)
 #undef X
-#define X(L, V, U, S)                                                                             \
+#define X(L, V, U, S, S2)                                                                         \
     if (!done && sh.ragged && sh.lpr == L && sh.vpl == V) {                                       \
         e = run_sddmm<T, L, V, U, S, true>(P, (const T *)A, (const T *)B, (T *)C, SS, sh.nvec);   \
         done = true;                                                                              \
@@ -783,16 +831,16 @@ hipError_t spmm_typed(const DevPlanView &P, const void *X_, void *Y, uint32_t K,
     const Shape sh = pick_shape(sizeof(T), K);
     bool done = false;
     hipError_t e = hipSuccess;
-#define X(L, V, U, S)                                                                             \
+#define X(L, V, U, S, S2)                                                                         \
     if (!done && !sh.ragged && sh.lpr == L && sh.vpl == V) {                                      \
-        e = run_spmm<T, L, V, U, S, false>(P, (const T *)X_, (T *)Y, SS, sh.nvec);                \
+        e = run_spmm<T, L, V, U, S2, false>(P, (const T *)X_, (T *)Y, SS, sh.nvec);               \
         done = true;                                                                              \
     }
     SPC3D_FOR_SHAPES(X)
 #undef X
-#define X(L, V, U, S)                                                                             \
+#define X(L, V, U, S, S2)                                                                         \
     if (!done && sh.ragged && sh.lpr == L && sh.vpl == V) {                                       \
-        e = run_spmm<T, L, V, U, S, true>(P, (const T *)X_, (T *)Y, SS, sh.nvec);                 \
+        e = run_spmm<T, L, V, U, S2, true>(P, (const T *)X_, (T *)Y, SS, sh.nvec);                \
         done = true;                                                                              \
     }
     SPC3D_FOR_RAGGED_SHAPES(X)
