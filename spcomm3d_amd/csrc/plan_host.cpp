@@ -277,28 +277,31 @@ int build_host_plan(uint32_t nrows, uint32_t ncols, uint64_t nnz, const uint32_t
             for (size_t i = 0; i < pieces.size(); ++i)
                 P.segs[i] = pieces[i].seg;
         } else {
-            // Hub pieces go to the queue of their column slice.  The rest go,
-            // longest first, to whichever queue has the least work so far.
+            // Hub pieces go to the queue of their column slice.  The rest, longest
+            // first, fill every queue up to the same total: piece i of that order
+            // goes to the queue whose share of the unit interval holds the i-th
+            // point of a low-discrepancy sequence, shares being proportional to
+            // what each queue still lacks.  Any window of consecutive (hence
+            // similar) pieces is thereby split among the queues in those
+            // proportions, and the rule needs nothing but i, so that a parallel
+            // builder deals identically.
             P.nqueues = kSlices;
             std::vector<Piece> queue[kSlices], any;
-            uint64_t load[kSlices] = {0};
+            uint64_t load[kSlices] = {0}, any_load = 0;
             for (const Piece &p : pieces) {
                 if (p.queue == kAnyQueue) {
                     any.push_back(p);
+                    any_load += seg_len(p.seg) + kSegCost;
                 } else {
                     queue[p.queue].push_back(p);
-                    load[p.queue] += seg_len(p.seg) + 4; // + a per-segment overhead
+                    load[p.queue] += seg_len(p.seg) + kSegCost;
                 }
             }
             sort_longest_first(any, seg_max);
-            for (const Piece &p : any) {
-                uint32_t best = 0;
-                for (uint32_t q = 1; q < kSlices; ++q)
-                    if (load[q] < load[best])
-                        best = q;
-                queue[best].push_back(p);
-                load[best] += seg_len(p.seg) + 4;
-            }
+            uint32_t upto[kSlices];
+            deal_thresholds(load, any_load, upto);
+            for (size_t i = 0; i < any.size(); ++i)
+                queue[deal_queue((uint32_t)i, upto)].push_back(any[i]);
             size_t nchunks = 0;
             for (uint32_t q = 0; q < kSlices; ++q) {
                 sort_longest_first(queue[q], seg_max);

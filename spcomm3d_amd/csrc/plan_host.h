@@ -61,6 +61,63 @@ struct HostPlan {
 
 constexpr uint32_t kDefaultHubMin = 128;
 
+// ---- dealing of free segments to the 8 XCD queues -------------------------
+// A segment weighs its length plus kSegCost (descriptor, dense row, write-back).
+constexpr uint32_t kSegCost = 4;
+constexpr uint32_t kDealQueues = 8;
+
+// upto[q] = end of queue q's share of [0, 2^32), shares proportional to what
+// queue q lacks to reach the mean of (load[] + free_load / 8); upto[7] = 2^32 - 1.
+inline void deal_thresholds(const uint64_t (&load)[kDealQueues], uint64_t free_load,
+                            uint32_t (&upto)[kDealQueues])
+{
+    // Water level: queues above it get nothing, the others are filled up to it.
+    uint64_t lack[kDealQueues];
+    uint64_t level_num = free_load; // level = level_num / active over the active queues
+    bool active[kDealQueues];
+    uint32_t nact = kDealQueues;
+    for (uint32_t q = 0; q < kDealQueues; ++q) {
+        active[q] = true;
+        level_num += load[q];
+    }
+    for (bool again = true; again;) {
+        again = false;
+        for (uint32_t q = 0; q < kDealQueues; ++q)
+            if (active[q] && nact > 1 && load[q] * nact > level_num) {
+                active[q] = false;
+                level_num -= load[q];
+                --nact;
+                again = true;
+            }
+    }
+    uint64_t total = 0;
+    for (uint32_t q = 0; q < kDealQueues; ++q) {
+        lack[q] = active[q] ? (level_num / nact > load[q] ? level_num / nact - load[q] : 0) : 0;
+        total += lack[q];
+    }
+    uint64_t acc = 0;
+    for (uint32_t q = 0; q < kDealQueues; ++q) {
+        acc += total ? lack[q] : 1;
+        const uint64_t den = total ? total : kDealQueues;
+        // acc / den of 2^32, without overflow: loads are < 2^40 (nnz < 2^32, cost 4)
+        const uint64_t hi = (acc << 20) / den; // 20 fractional bits, then 12 more
+        const uint64_t t = hi >= (1ull << 20) ? 0xFFFFFFFFull : (hi << 12);
+        upto[q] = (uint32_t)(t > 0xFFFFFFFFull ? 0xFFFFFFFFull : t);
+    }
+    upto[kDealQueues - 1] = 0xFFFFFFFFu;
+}
+
+// Queue of the i-th free segment (longest first): the share that holds the i-th
+// point of the golden-ratio sequence i * 0x9E3779B9 mod 2^32.
+inline uint32_t deal_queue(uint32_t i, const uint32_t (&upto)[kDealQueues])
+{
+    const uint32_t x = i * 0x9E3779B9u;
+    uint32_t q = 0;
+    while (q + 1 < kDealQueues && x > upto[q])
+        ++q;
+    return q;
+}
+
 // Default longest segment: long enough that few rows are cut (each cut costs a
 // partial-sum row in SpMM), short enough that the longest segments do not
 // outlast the rest of the grid: nnz / 2048 rounded down to a power of two,
