@@ -101,7 +101,10 @@ typedef struct {
     uint32_t xcd_slices;   /* 8 (default): when the column degrees are skewed, the entries of
                               long rows are dealt to the 8 XCDs by column, so that each L2
                               caches its own eighth of the hot dense rows; 1: never */
-    uint32_t reserved[3];  /* must be 0 */
+    uint32_t builder;      /* where spc3d_plan_create[_ex] builds the plan: 0 (default) or 2:
+                              on the GPU; 1: on the host, then uploaded.  Both give the same
+                              arrays bit for bit. */
+    uint32_t reserved[2];  /* must be 0 */
 } spc3d_plan_opts;
 
 /* ---- library / errors ------------------------------------------------- */
@@ -155,7 +158,11 @@ SPC3D_API int spc3d_coo_validate(uint32_t nrows, uint32_t ncols, uint64_t nnz,
                        const uint32_t *ii, const uint32_t *jj);
 
 /* Validates (as above), groups the entries by row keeping the caller's order
- * within a row, cuts long rows into segments, and uploads.  `vv` (nnz reals of
+ * within a row, and cuts long rows into segments.  By default the pattern is
+ * uploaded as it is and all of this happens on the GPU (histograms, scans and
+ * stable radix sorts; milliseconds for 16 M entries); spc3d_plan_opts.builder or
+ * SPC3D_PLAN_BUILDER=host in the environment (spc3d_plan_create only) selects
+ * the single-threaded host builder instead.  `vv` (nnz reals of
  * `dtype`, caller's order) may be NULL and set later.  The pattern is copied:
  * the caller's arrays are not referenced afterwards.  Replaces nothing in the
  * reference (it walks the unsorted COO directly, core_ops.cpp:7-10); it is the
@@ -182,6 +189,21 @@ SPC3D_API int spc3d_plan_build_host(int dtype, uint32_t nrows, uint32_t ncols, u
                           const spc3d_plan_opts *opts, spc3d_plan_info *info,
                           uint32_t *col, uint32_t *perm, uint32_t *segs, uint32_t seg_cap,
                           uint32_t *splits, uint32_t split_cap);
+/* As spc3d_plan_create_ex for a pattern that already lives on the GPU: dev_ii and
+ * dev_jj are device pointers to nnz uint32 each (memory of the context's
+ * device, e.g. from spc3d_vals_device_ptr or the caller's own hipMalloc), read
+ * on the context's stream.  The plan has no values until spc3d_plan_set_values[_device].
+ * Has no counterpart in the reference, whose COO lives in host vectors
+ * (src/SparseMatrix.hpp:35). */
+SPC3D_API int spc3d_plan_create_from_device(spc3d_ctx *ctx, int dtype, uint32_t nrows,
+                                  uint32_t ncols, uint64_t nnz, const void *dev_ii,
+                                  const void *dev_jj, const spc3d_plan_opts *opts,
+                                  spc3d_plan **out);
+/* Copies a plan's arrays back from the device, in the layout of
+ * spc3d_plan_build_host (each output may be NULL; perm is the identity when the
+ * plan stores none).  For inspection and tests.  Synchronous. */
+SPC3D_API int spc3d_plan_download(spc3d_plan *plan, uint32_t *col, uint32_t *perm, uint32_t *segs,
+                        uint32_t seg_cap, uint32_t *splits, uint32_t split_cap);
 SPC3D_API int spc3d_plan_destroy(spc3d_plan *plan);
 SPC3D_API int spc3d_plan_set_values(spc3d_plan *plan, const void *vv_host);       /* caller's COO order */
 SPC3D_API int spc3d_plan_set_values_device(spc3d_plan *plan, const spc3d_vals *vv); /* caller's COO order */

@@ -35,7 +35,8 @@ class PlanInfo(ctypes.Structure):
 
 class PlanOpts(ctypes.Structure):
     _fields_ = [("seg_max", c_u32), ("k_hint", c_u32), ("l2_hot_bytes", c_u32),
-                ("hub_min", c_u32), ("xcd_slices", c_u32), ("reserved", c_u32 * 3)]
+                ("hub_min", c_u32), ("xcd_slices", c_u32), ("builder", c_u32),
+                ("reserved", c_u32 * 2)]
 
 
 # name -> (restype, argtypes); one entry for every function the header declares.
@@ -71,6 +72,9 @@ SIGNATURES = {
                                      P(PlanOpts), P(c_vp)]),
     "spc3d_plan_build_host": (c_int, [c_int, c_u32, c_u32, c_u64, c_vp, c_vp, P(PlanOpts),
                                       P(PlanInfo), c_vp, c_vp, c_vp, c_u32, c_vp, c_u32]),
+    "spc3d_plan_create_from_device": (c_int, [c_vp, c_int, c_u32, c_u32, c_u64, c_vp, c_vp,
+                                              P(PlanOpts), P(c_vp)]),
+    "spc3d_plan_download": (c_int, [c_vp, c_vp, c_vp, c_vp, c_u32, c_vp, c_u32]),
     "spc3d_plan_destroy": (c_int, [c_vp]),
     "spc3d_plan_set_values": (c_int, [c_vp, c_vp]),
     "spc3d_plan_set_values_device": (c_int, [c_vp, c_vp]),

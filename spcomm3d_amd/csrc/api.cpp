@@ -14,6 +14,7 @@
 #include <vector>
 
 #include "kernels.h"
+#include "plan_device.h"
 #include "plan_host.h"
 
 using namespace spc3d;
@@ -637,8 +638,10 @@ static int resolve_opts(int dtype, const spc3d_plan_opts *o, PlanOpts &out)
     std::memset(&z, 0, sizeof z);
     if (o)
         z = *o;
-    if (z.reserved[0] || z.reserved[1] || z.reserved[2])
+    if (z.reserved[0] || z.reserved[1])
         return fail(SPC3D_ERR_INVALID_ARG, "spc3d_plan_opts.reserved must be 0");
+    if (z.builder > 2)
+        return fail(SPC3D_ERR_INVALID_ARG, "spc3d_plan_opts.builder must be 0, 1 or 2");
     if (z.xcd_slices != 0 && z.xcd_slices != 1 && z.xcd_slices != 8)
         return fail(SPC3D_ERR_INVALID_ARG, "xcd_slices must be 0, 1 or 8");
     out.seg_max = z.seg_max;
@@ -686,6 +689,68 @@ int spc3d_plan_build_host(int dtype, uint32_t nrows, uint32_t ncols, uint64_t nn
     return SPC3D_OK;
 }
 
+// Plan over arrays that build_device_plan left on the device.
+static int adopt_device_plan(spc3d_ctx *ctx, int dtype, const HostPlan &meta, DevPlanArrays &arr,
+                             spc3d_plan **out)
+{
+    spc3d_plan *p = new (std::nothrow) spc3d_plan();
+    int rc = SPC3D_OK;
+    if (!p)
+        rc = fail(SPC3D_ERR_ALLOC, "host allocation failed");
+    if (!rc) {
+        p->ctx = ctx;
+        p->dtype = dtype;
+        fill_info(p->info, meta);
+        p->info.nsegments_padded = arr.nseg_padded;
+        p->info.nsplit_rows = arr.nsplit;
+        rc = dev_alloc_bytes(&p->sval, (size_t)meta.nnz * elem_size(dtype));
+    }
+    if (rc) {
+        if (arr.segs) (void)hipFree(arr.segs);
+        if (arr.col) (void)hipFree(arr.col);
+        if (arr.perm) (void)hipFree(arr.perm);
+        if (arr.splits) (void)hipFree(arr.splits);
+        delete p;
+        return rc;
+    }
+    p->segs = arr.segs;
+    p->col = arr.col;
+    p->perm = arr.perm;
+    p->splits = arr.splits;
+    arr = DevPlanArrays{};
+    p->magic = kMagicPlan;
+    *out = p;
+    return SPC3D_OK;
+}
+
+int spc3d_plan_create_from_device(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t ncols,
+                                  uint64_t nnz, const void *dev_ii, const void *dev_jj,
+                                  const spc3d_plan_opts *opts, spc3d_plan **out)
+{
+    if (!out)
+        return fail(SPC3D_ERR_INVALID_ARG, "out is NULL");
+    *out = nullptr;
+    if (!dtype_ok(dtype))
+        return fail(SPC3D_ERR_INVALID_ARG, "unknown dtype");
+    PlanOpts po;
+    int rc = resolve_opts(dtype, opts, po);
+    if (rc)
+        return rc;
+    if (!live(ctx))
+        return fail(SPC3D_ERR_INVALID_ARG, "context is NULL or destroyed");
+    rc = use_device(ctx);
+    if (rc)
+        return rc;
+    HostPlan meta;
+    DevPlanArrays arr;
+    std::string err;
+    rc = build_device_plan(ctx->stream, nrows, ncols, nnz, (const uint32_t *)dev_ii,
+                           (const uint32_t *)dev_jj, po, meta, arr, err);
+    if (rc != SPC3D_OK)
+        return fail(rc, err);
+    return adopt_device_plan(ctx, dtype, meta, arr, out);
+}
+
 int spc3d_plan_create_ex(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t ncols, uint64_t nnz,
                          const uint32_t *ii, const uint32_t *jj, const void *vv,
                          const spc3d_plan_opts *opts, spc3d_plan **out)
@@ -695,46 +760,80 @@ int spc3d_plan_create_ex(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t nco
     *out = nullptr;
     if (!dtype_ok(dtype))
         return fail(SPC3D_ERR_INVALID_ARG, "unknown dtype");
-    // The pattern is checked before the device is touched, so that a bad
-    // index is reported as such on a machine without a GPU as well.
     PlanOpts po;
     int rc = resolve_opts(dtype, opts, po);
     if (rc)
         return rc;
-    HostPlan H;
-    std::string err;
-    rc = build_host_plan(nrows, ncols, nnz, ii, jj, po, H, err);
-    if (rc != SPC3D_OK)
-        return fail(rc, err);
-    if (!live(ctx))
-        return fail(SPC3D_ERR_INVALID_ARG, "context is NULL or destroyed");
-    rc = use_device(ctx);
-    if (rc)
-        return rc;
+    const bool on_host = opts && opts->builder == 1;
+    spc3d_plan *p = nullptr;
+    if (!on_host && live(ctx)) {
+        if (nnz > 0 && (ii == nullptr || jj == nullptr))
+            return fail(SPC3D_ERR_INVALID_ARG, "ii/jj is NULL with nnz > 0");
+        if (nnz >= (1ull << 32))
+            return fail(SPC3D_ERR_TOO_LARGE, "nnz >= 2^32 is not supported");
+        rc = use_device(ctx);
+        if (rc)
+            return rc;
+        // The pattern goes up as it is; validation and everything else happens there.
+        uint32_t *d_ii = nullptr, *d_jj = nullptr;
+        rc = dev_alloc(&d_ii, (size_t)nnz);
+        if (!rc) rc = dev_alloc(&d_jj, (size_t)nnz);
+        if (!rc) rc = copy_h2d(ctx, d_ii, ii, (size_t)nnz * sizeof(uint32_t));
+        if (!rc) rc = copy_h2d(ctx, d_jj, jj, (size_t)nnz * sizeof(uint32_t));
+        HostPlan meta;
+        DevPlanArrays arr;
+        if (!rc) {
+            std::string err;
+            rc = build_device_plan(ctx->stream, nrows, ncols, nnz, d_ii, d_jj, po, meta, arr, err);
+            if (rc != SPC3D_OK)
+                fail(rc, err);
+        }
+        if (d_ii) (void)hipFree(d_ii);
+        if (d_jj) (void)hipFree(d_jj);
+        if (rc)
+            return rc;
+        rc = adopt_device_plan(ctx, dtype, meta, arr, &p);
+        if (rc)
+            return rc;
+    } else {
+        // The pattern is checked before the device is touched, so that a bad
+        // index is reported as such on a machine without a GPU as well.
+        HostPlan H;
+        std::string err;
+        rc = build_host_plan(nrows, ncols, nnz, ii, jj, po, H, err);
+        if (rc != SPC3D_OK)
+            return fail(rc, err);
+        if (!live(ctx))
+            return fail(SPC3D_ERR_INVALID_ARG, "context is NULL or destroyed");
+        rc = use_device(ctx);
+        if (rc)
+            return rc;
 
-    spc3d_plan *p = new (std::nothrow) spc3d_plan();
-    if (!p)
-        return fail(SPC3D_ERR_ALLOC, "host allocation failed");
-    p->ctx = ctx;
-    p->dtype = dtype;
-    fill_info(p->info, H);
+        p = new (std::nothrow) spc3d_plan();
+        if (!p)
+            return fail(SPC3D_ERR_ALLOC, "host allocation failed");
+        p->ctx = ctx;
+        p->dtype = dtype;
+        fill_info(p->info, H);
 
-    rc = dev_alloc(&p->segs, H.segs.size());
-    if (!rc) rc = dev_alloc(&p->col, (size_t)nnz);
-    if (!rc && !H.identity) rc = dev_alloc(&p->perm, (size_t)nnz);
-    if (!rc) rc = dev_alloc_bytes(&p->sval, (size_t)nnz * elem_size(dtype));
-    if (!rc) rc = dev_alloc(&p->splits, H.splits.size());
-    if (!rc) rc = copy_h2d(ctx, p->segs, H.segs.data(), H.segs.size() * sizeof(Seg));
-    if (!rc) rc = copy_h2d(ctx, p->col, H.col.data(), (size_t)nnz * sizeof(uint32_t));
-    if (!rc && !H.identity)
-        rc = copy_h2d(ctx, p->perm, H.perm.data(), (size_t)nnz * sizeof(uint32_t));
-    if (!rc) rc = copy_h2d(ctx, p->splits, H.splits.data(), H.splits.size() * sizeof(SplitRow));
-    if (rc) {
-        plan_free_device(p);
-        delete p;
-        return rc;
+        rc = dev_alloc(&p->segs, H.segs.size());
+        if (!rc) rc = dev_alloc(&p->col, (size_t)nnz);
+        if (!rc && !H.identity) rc = dev_alloc(&p->perm, (size_t)nnz);
+        if (!rc) rc = dev_alloc_bytes(&p->sval, (size_t)nnz * elem_size(dtype));
+        if (!rc) rc = dev_alloc(&p->splits, H.splits.size());
+        if (!rc) rc = copy_h2d(ctx, p->segs, H.segs.data(), H.segs.size() * sizeof(Seg));
+        if (!rc) rc = copy_h2d(ctx, p->col, H.col.data(), (size_t)nnz * sizeof(uint32_t));
+        if (!rc && !H.identity)
+            rc = copy_h2d(ctx, p->perm, H.perm.data(), (size_t)nnz * sizeof(uint32_t));
+        if (!rc)
+            rc = copy_h2d(ctx, p->splits, H.splits.data(), H.splits.size() * sizeof(SplitRow));
+        if (rc) {
+            plan_free_device(p);
+            delete p;
+            return rc;
+        }
+        p->magic = kMagicPlan;
     }
-    p->magic = kMagicPlan;
     if (vv) {
         rc = spc3d_plan_set_values(p, vv);
         if (rc) {
@@ -745,6 +844,46 @@ int spc3d_plan_create_ex(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t nco
     }
     *out = p;
     return SPC3D_OK;
+}
+
+int spc3d_plan_download(spc3d_plan *plan, uint32_t *col, uint32_t *perm, uint32_t *segs,
+                        uint32_t seg_cap, uint32_t *splits, uint32_t split_cap)
+{
+    if (!live(plan))
+        return fail(SPC3D_ERR_INVALID_ARG, "plan is NULL or destroyed");
+    const spc3d_plan_info &I = plan->info;
+    if ((segs && seg_cap < I.nsegments_padded) || (splits && split_cap < I.nsplit_rows))
+        return fail(SPC3D_ERR_SIZE_MISMATCH, "output capacity is smaller than the plan");
+    int rc = use_device(plan->ctx);
+    if (rc)
+        return rc;
+    const size_t nnz = (size_t)I.nnz;
+    if (col && nnz)
+        rc = copy_d2h(plan->ctx, col, plan->col, nnz * sizeof(uint32_t));
+    if (!rc && perm && nnz) {
+        if (plan->perm)
+            rc = copy_d2h(plan->ctx, perm, plan->perm, nnz * sizeof(uint32_t));
+        else
+            for (size_t e = 0; e < nnz; ++e)
+                perm[e] = (uint32_t)e;
+    }
+    if (!rc && segs && I.nsegments_padded)
+        rc = copy_d2h(plan->ctx, segs, plan->segs, (size_t)I.nsegments_padded * sizeof(Seg));
+    if (!rc && splits && I.nsplit_rows) {
+        std::vector<SplitRow> tmp;
+        try {
+            tmp.resize(I.nsplit_rows);
+        } catch (const std::bad_alloc &) {
+            return fail(SPC3D_ERR_ALLOC, "host allocation failed");
+        }
+        rc = copy_d2h(plan->ctx, tmp.data(), plan->splits, tmp.size() * sizeof(SplitRow));
+        for (size_t i = 0; !rc && i < tmp.size(); ++i) {
+            splits[3 * i + 0] = tmp[i].row;
+            splits[3 * i + 1] = tmp[i].first_slot;
+            splits[3 * i + 2] = tmp[i].nslots;
+        }
+    }
+    return rc;
 }
 
 int spc3d_plan_create(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t ncols, uint64_t nnz,
@@ -761,6 +900,8 @@ int spc3d_plan_create(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t ncols,
                {"SPC3D_L2_HOT_BYTES", &o.l2_hot_bytes},
                {"SPC3D_HUB_MIN", &o.hub_min},
                {"SPC3D_XCD_SLICES", &o.xcd_slices}};
+    if (const char *b = std::getenv("SPC3D_PLAN_BUILDER"))
+        o.builder = std::strcmp(b, "host") == 0 ? 1u : 2u;
     for (auto &e : env)
         if (const char *s = std::getenv(e.name)) {
             const long long v = std::atoll(s);

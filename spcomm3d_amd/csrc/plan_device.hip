@@ -1,0 +1,768 @@
+// Device-side plan construction (see plan_device.h).  Every step restates one
+// step of build_host_plan (plan_host.cpp) with a parallel primitive that gives
+// the same result: histograms by atomics, prefix sums by device scans, the
+// stable counting sorts by stable radix sorts.
+#include "plan_device.h"
+
+#include <hip/hip_runtime.h>
+#include <hipcub/hipcub.hpp>
+
+#include <algorithm>
+#include <cstdio>
+
+#include "../../include/spcomm3d_hip.h"
+
+namespace spc3d {
+namespace {
+
+constexpr int kTB = 256;
+
+struct Counters { // one device-resident block, zeroed (first_bad: all ones) before use
+    uint32_t first_bad;
+    uint32_t rows_touched, max_row, cols_touched, max_cdeg;
+    uint32_t not_identity;
+    uint32_t qcount[kSlices], qlong[kSlices];
+    uint32_t nlong;
+    uint32_t pad;
+    unsigned long long covered;
+    unsigned long long load[kSlices];
+    unsigned long long any_load;
+};
+
+// Owning device buffer; freed on scope exit unless released.
+template <typename T> struct DBuf {
+    T *p = nullptr;
+    DBuf() = default;
+    DBuf(const DBuf &) = delete;
+    DBuf &operator=(const DBuf &) = delete;
+    ~DBuf() { reset(); }
+    void reset()
+    {
+        if (p)
+            (void)hipFree(p);
+        p = nullptr;
+    }
+    hipError_t alloc(size_t count)
+    {
+        reset();
+        if (count == 0)
+            return hipSuccess;
+        return hipMalloc((void **)&p, count * sizeof(T));
+    }
+    T *release()
+    {
+        T *r = p;
+        p = nullptr;
+        return r;
+    }
+};
+
+inline uint32_t grid_for(uint64_t n)
+{
+    const uint64_t want = (n + kTB - 1) / kTB;
+    const uint64_t cap = 256 * 32;
+    return (uint32_t)(want < 1 ? 1 : (want > cap ? cap : want));
+}
+
+inline int bits_for(uint64_t max_value) // bits needed to hold max_value (at least 1)
+{
+    int b = 1;
+    while (b < 64 && (max_value >> b) != 0)
+        ++b;
+    return b;
+}
+
+#define GRID_STRIDE(i, n)                                                                         \
+    for (uint64_t i = (uint64_t)blockIdx.x * kTB + threadIdx.x; i < (n);                         \
+         i += (uint64_t)gridDim.x * kTB)
+
+template <typename T> __device__ __forceinline__ T wave_sum(T v)
+{
+    for (int s = 32; s >= 1; s >>= 1)
+        v += __shfl_xor(v, s, 64);
+    return v;
+}
+
+template <typename T> __global__ void fill_k(T *p, uint64_t n, T v)
+{
+    GRID_STRIDE(i, n) p[i] = v;
+}
+
+__global__ void iota_k(uint32_t *p, uint64_t n)
+{
+    GRID_STRIDE(i, n) p[i] = (uint32_t)i;
+}
+
+// Row and column histograms; the first out-of-range entry, if any.
+__global__ void hist_k(const uint32_t *__restrict__ ii, const uint32_t *__restrict__ jj,
+                       uint64_t nnz, uint32_t nrows, uint32_t ncols, uint32_t *rowcnt,
+                       uint32_t *coldeg, Counters *C)
+{
+    GRID_STRIDE(e, nnz)
+    {
+        const uint32_t r = ii[e], c = jj[e];
+        if (r >= nrows || c >= ncols) {
+            atomicMin(&C->first_bad, (uint32_t)e);
+        } else {
+            atomicAdd(rowcnt + r, 1u);
+            atomicAdd(coldeg + c, 1u);
+        }
+    }
+}
+
+// Number of non-zero counts and the largest count.
+__global__ void stats_k(const uint32_t *__restrict__ cnt, uint64_t n, uint32_t *touched,
+                        uint32_t *maxv)
+{
+    uint32_t t = 0, m = 0;
+    GRID_STRIDE(i, n)
+    {
+        const uint32_t v = cnt[i];
+        t += v != 0;
+        m = m > v ? m : v;
+    }
+    for (int s = 32; s >= 1; s >>= 1) {
+        t += __shfl_xor(t, s, 64);
+        const uint32_t o = __shfl_xor(m, s, 64);
+        m = m > o ? m : o;
+    }
+    if ((threadIdx.x & 63) == 0) {
+        if (t)
+            atomicAdd(touched, t);
+        if (m)
+            atomicMax(maxv, m);
+    }
+}
+
+__global__ void sum_first_k(const uint32_t *__restrict__ v, uint64_t n, unsigned long long *out)
+{
+    unsigned long long s = 0;
+    GRID_STRIDE(i, n) s += v[i];
+    for (int k = 32; k >= 1; k >>= 1)
+        s += __shfl_xor(s, k, 64);
+    if ((threadIdx.x & 63) == 0 && s)
+        atomicAdd(out, s);
+}
+
+// Classes of the htot hottest columns (order[] = columns by degree, highest first).
+__global__ void classify_k(const uint32_t *__restrict__ order, uint64_t htot, uint32_t hrep,
+                           uint8_t *cls)
+{
+    GRID_STRIDE(i, htot)
+    cls[order[i]] = i < hrep ? kClsRep : slice_of_rank(i - hrep);
+}
+
+__global__ void hubflag_k(const uint32_t *__restrict__ rowcnt, uint32_t nrows, uint32_t hub_min,
+                          uint32_t *flag)
+{
+    GRID_STRIDE(r, (uint64_t)nrows + 1) flag[r] = (r < nrows && rowcnt[r] >= hub_min) ? 1u : 0u;
+}
+
+// Per hub row, the number of entries in each of the 9 groups.
+__global__ void hubcount_k(const uint32_t *__restrict__ ii, const uint32_t *__restrict__ jj,
+                           uint64_t nnz, const uint32_t *__restrict__ hubflag,
+                           const uint32_t *__restrict__ hubpos, const uint8_t *__restrict__ cls,
+                           uint32_t *hubcnt)
+{
+    GRID_STRIDE(e, nnz)
+    {
+        const uint32_t r = ii[e];
+        if (hubflag[r])
+            atomicAdd(hubcnt + (size_t)hubpos[r] * 9 + hub_group(r, cls[jj[e]]), 1u);
+    }
+}
+
+// Sort key of entry e: its row, then (hub rows of the sliced layout) its group.
+template <typename KeyT>
+__global__ void keys_k(const uint32_t *__restrict__ ii, const uint32_t *__restrict__ jj,
+                       uint64_t nnz, bool slices, const uint32_t *__restrict__ hubflag,
+                       const uint8_t *__restrict__ cls, KeyT *key)
+{
+    GRID_STRIDE(e, nnz)
+    {
+        const uint32_t r = ii[e];
+        if (!slices) {
+            key[e] = (KeyT)r;
+        } else {
+            const uint32_t g = hubflag[r] ? hub_group(r, cls[jj[e]]) : 0u;
+            key[e] = (KeyT)(((KeyT)r << 4) | (KeyT)g);
+        }
+    }
+}
+
+// col[p] = jj[perm[p]]; flags an order that is not the identity.
+__global__ void gather_cols_k(const uint32_t *__restrict__ jj, const uint32_t *__restrict__ perm,
+                              uint64_t nnz, uint32_t *col, Counters *C)
+{
+    bool moved = false;
+    GRID_STRIDE(p, nnz)
+    {
+        const uint32_t e = perm[p];
+        col[p] = jj[e];
+        moved |= e != (uint32_t)p;
+    }
+    if (__any(moved) && (threadIdx.x & 63) == 0)
+        atomicOr(&C->not_identity, 1u);
+}
+
+__device__ __forceinline__ uint32_t parts_of(uint32_t len, uint32_t seg_max)
+{
+    return len == 0 ? 0u : (len + seg_max - 1) / seg_max;
+}
+
+// Pieces per row; rows cut into several pieces also count as a split row and
+// take one partial-sum slot per piece.
+__global__ void count_pieces_k(const uint32_t *__restrict__ rowcnt, uint32_t nrows,
+                               uint32_t seg_max, bool slices,
+                               const uint32_t *__restrict__ hubflag,
+                               const uint32_t *__restrict__ hubpos,
+                               const uint32_t *__restrict__ hubcnt, uint32_t *npieces,
+                               uint32_t *issplit, uint32_t *nslot)
+{
+    GRID_STRIDE(r, (uint64_t)nrows + 1)
+    {
+        uint32_t np = 0;
+        if (r < nrows) {
+            if (slices && hubflag[r]) {
+                for (uint32_t k = 0; k < 9; ++k)
+                    np += parts_of(hubcnt[(size_t)hubpos[r] * 9 + k], seg_max);
+            } else {
+                np = parts_of(rowcnt[r], seg_max);
+            }
+        }
+        npieces[r] = np;
+        issplit[r] = np > 1;
+        nslot[r] = np > 1 ? np : 0u;
+    }
+}
+
+// Writes the pieces of every row, in row order: balanced parts of at most
+// seg_max entries per range (a non-hub row is one range, a hub row one per group).
+__global__ void emit_pieces_k(const uint32_t *__restrict__ rowptr, uint32_t nrows,
+                              uint32_t seg_max, bool slices,
+                              const uint32_t *__restrict__ hubflag,
+                              const uint32_t *__restrict__ hubpos,
+                              const uint32_t *__restrict__ hubcnt,
+                              const uint32_t *__restrict__ piece_off,
+                              const uint32_t *__restrict__ split_off,
+                              const uint32_t *__restrict__ slot_off, Seg *pseg, uint8_t *pqueue,
+                              SplitRow *splits)
+{
+    GRID_STRIDE(r, nrows)
+    {
+        const uint32_t np = piece_off[r + 1] - piece_off[r];
+        if (np == 0)
+            continue;
+        const uint32_t s = rowptr[r], len = rowptr[r + 1] - s;
+        const bool hub = slices && hubflag[r];
+        uint32_t at = piece_off[r];
+        uint32_t slot = np > 1 ? slot_off[r] : kWholeRow;
+        if (np > 1)
+            splits[split_off[r]] = SplitRow{(uint32_t)r, slot_off[r], np, 0u};
+        uint32_t start = s;
+        const uint32_t ngroups = hub ? 9u : 1u;
+        for (uint32_t k = 0; k < ngroups; ++k) {
+            const uint32_t n = hub ? hubcnt[(size_t)hubpos[r] * 9 + k] : len;
+            if (n == 0)
+                continue;
+            const uint8_t queue = (hub && k < 8) ? (uint8_t)k : kAnyQueue;
+            const uint32_t parts = (n + seg_max - 1) / seg_max;
+            const uint32_t base = n / parts, rem = n % parts;
+            for (uint32_t q = 0; q < parts; ++q) {
+                const uint32_t l = base + (q < rem ? 1u : 0u);
+                pseg[at] = Seg{(uint32_t)r, start, l, slot};
+                pqueue[at] = queue;
+                ++at;
+                start += l;
+                if (np > 1)
+                    ++slot;
+            }
+        }
+    }
+}
+
+// Unsliced layout: key for "longest first", and the number of long pieces.
+__global__ void len_keys_k(const Seg *__restrict__ pseg, uint64_t n, uint32_t seg_max,
+                           uint32_t *key, Counters *C)
+{
+    uint32_t nl = 0;
+    GRID_STRIDE(i, n)
+    {
+        const uint32_t l = pseg[i].len;
+        key[i] = seg_max - l;
+        nl += l >= kLongSegment;
+    }
+    for (int s = 32; s >= 1; s >>= 1)
+        nl += __shfl_xor(nl, s, 64);
+    if ((threadIdx.x & 63) == 0 && nl)
+        atomicAdd(&C->nlong, nl);
+}
+
+__global__ void gather_segs_k(const Seg *__restrict__ pseg, const uint32_t *__restrict__ idx,
+                              uint64_t n, Seg *out)
+{
+    GRID_STRIDE(i, n) out[i] = pseg[idx[i]];
+}
+
+// Sliced layout, step 1: which pieces are free (any queue), the work already
+// bound to each queue, and the work that is free.
+__global__ void any_flags_k(const Seg *__restrict__ pseg, const uint8_t *__restrict__ pqueue,
+                            uint64_t n, uint32_t *anyflag, Counters *C)
+{
+    unsigned long long w[kSlices + 1] = {0}; // [8] = free work
+    GRID_STRIDE(i, (uint64_t)n + 1)
+    {
+        if (i == n) {
+            anyflag[i] = 0;
+            continue;
+        }
+        const uint8_t q = pqueue[i];
+        const unsigned long long wi = (unsigned long long)pseg[i].len + kSegCost;
+        anyflag[i] = q == kAnyQueue;
+#pragma unroll
+        for (uint32_t k = 0; k <= kSlices; ++k)
+            w[k] += (k == kSlices ? q == kAnyQueue : q == k) ? wi : 0ull;
+    }
+#pragma unroll
+    for (uint32_t k = 0; k <= kSlices; ++k) {
+        const unsigned long long t = wave_sum(w[k]);
+        if ((threadIdx.x & 63) == 0 && t)
+            atomicAdd(k == kSlices ? &C->any_load : &C->load[k], t);
+    }
+}
+
+// Step 2: the free pieces, compacted in piece order, with their length keys.
+__global__ void compact_any_k(const Seg *__restrict__ pseg, const uint32_t *__restrict__ anyflag,
+                              const uint32_t *__restrict__ anypos, uint64_t n, uint32_t seg_max,
+                              uint32_t *any_idx, uint32_t *any_key)
+{
+    GRID_STRIDE(i, n)
+    if (anyflag[i]) {
+        any_idx[anypos[i]] = (uint32_t)i;
+        any_key[anypos[i]] = seg_max - pseg[i].len;
+    }
+}
+
+struct Upto {
+    uint32_t v[kDealQueues];
+};
+
+// Step 3: every piece gets its queue.  The combined list is [bound pieces in piece
+// order | free pieces longest first]; its key is (queue, seg_max - len).
+__global__ void combine_k(const Seg *__restrict__ pseg, const uint8_t *__restrict__ pqueue,
+                          const uint32_t *__restrict__ anyflag,
+                          const uint32_t *__restrict__ anypos,
+                          const uint32_t *__restrict__ any_sorted, uint64_t npieces,
+                          uint64_t nany, uint32_t seg_max, Upto upto, uint32_t *comb_idx,
+                          uint32_t *comb_key, Counters *C)
+{
+    const uint64_t nbound = npieces - nany;
+    uint32_t cnt[kSlices] = {0}, lng[kSlices] = {0};
+    GRID_STRIDE(t, npieces + nany)
+    {
+        uint32_t piece, q;
+        uint64_t at;
+        if (t < npieces) { // a bound piece, at its rank among the bound ones
+            if (anyflag[t])
+                continue;
+            piece = (uint32_t)t;
+            q = pqueue[t];
+            at = t - anypos[t];
+        } else { // the free piece of rank j
+            const uint64_t j = t - npieces;
+            piece = any_sorted[j];
+            q = deal_queue((uint32_t)j, upto.v);
+            at = nbound + j;
+        }
+        const uint32_t l = pseg[piece].len;
+        comb_idx[at] = piece;
+        comb_key[at] = q * (seg_max + 1) + (seg_max - l);
+#pragma unroll
+        for (uint32_t k = 0; k < kSlices; ++k) {
+            cnt[k] += q == k;
+            lng[k] += q == k && l >= kLongSegment;
+        }
+    }
+#pragma unroll
+    for (uint32_t k = 0; k < kSlices; ++k) {
+        const uint32_t c = wave_sum(cnt[k]), g = wave_sum(lng[k]);
+        if ((threadIdx.x & 63) == 0) {
+            if (c)
+                atomicAdd(&C->qcount[k], c);
+            if (g)
+                atomicAdd(&C->qlong[k], g);
+        }
+    }
+}
+
+struct QStart {
+    uint32_t v[kSlices];
+};
+
+// Step 4: piece of rank i in queue q goes to chunk i / 64 of that queue, which is
+// global chunk (i / 64) * 8 + q.
+__global__ void scatter_segs_k(const Seg *__restrict__ pseg, const uint32_t *__restrict__ idx,
+                               const uint32_t *__restrict__ key, uint64_t n, uint32_t seg_max,
+                               QStart qstart, Seg *out)
+{
+    GRID_STRIDE(s, n)
+    {
+        const uint32_t q = key[s] / (seg_max + 1);
+        const uint64_t i = s - qstart.v[q];
+        out[((i / kChunk) * kSlices + q) * kChunk + i % kChunk] = pseg[idx[s]];
+    }
+}
+
+#define HIP_OK(expr)                                                                              \
+    do {                                                                                          \
+        const hipError_t e_ = (expr);                                                             \
+        if (e_ != hipSuccess) {                                                                   \
+            err = std::string("device plan: ") + #expr + ": " + hipGetErrorString(e_);            \
+            return e_ == hipErrorOutOfMemory ? SPC3D_ERR_ALLOC : SPC3D_ERR_HIP;                   \
+        }                                                                                         \
+    } while (0)
+
+// Scratch for the device-wide primitives, grown on demand.
+struct Temp {
+    DBuf<unsigned char> buf;
+    size_t cap = 0;
+    hipError_t need(size_t bytes)
+    {
+        bytes = bytes < 256 ? 256 : bytes; // never null: a null pointer asks for the size again
+        if (bytes <= cap)
+            return hipSuccess;
+        const hipError_t e = buf.alloc(bytes);
+        cap = e == hipSuccess ? bytes : 0;
+        return e;
+    }
+};
+
+template <typename T>
+int exclusive_sum(Temp &tmp, const T *in, T *out, size_t n, hipStream_t st, std::string &err)
+{
+    size_t bytes = 0;
+    HIP_OK(hipcub::DeviceScan::ExclusiveSum(nullptr, bytes, in, out, n, st));
+    HIP_OK(tmp.need(bytes));
+    HIP_OK(hipcub::DeviceScan::ExclusiveSum(tmp.buf.p, bytes, in, out, n, st));
+    return SPC3D_OK;
+}
+
+// Stable ascending sort of (key, value) pairs on key bits [0, bits).
+template <typename KeyT>
+int sort_pairs(Temp &tmp, const KeyT *kin, KeyT *kout, const uint32_t *vin, uint32_t *vout,
+               uint32_t n, int bits, bool descending, hipStream_t st, std::string &err)
+{
+    size_t bytes = 0;
+    if (descending) {
+        HIP_OK(hipcub::DeviceRadixSort::SortPairsDescending(nullptr, bytes, kin, kout, vin, vout,
+                                                            n, 0, bits, st));
+        HIP_OK(tmp.need(bytes));
+        HIP_OK(hipcub::DeviceRadixSort::SortPairsDescending(tmp.buf.p, bytes, kin, kout, vin,
+                                                            vout, n, 0, bits, st));
+    } else {
+        HIP_OK(hipcub::DeviceRadixSort::SortPairs(nullptr, bytes, kin, kout, vin, vout, n, 0,
+                                                  bits, st));
+        HIP_OK(tmp.need(bytes));
+        HIP_OK(hipcub::DeviceRadixSort::SortPairs(tmp.buf.p, bytes, kin, kout, vin, vout, n, 0,
+                                                  bits, st));
+    }
+    return SPC3D_OK;
+}
+
+#define LAUNCH(kernel, n, ...)                                                                    \
+    hipLaunchKernelGGL(kernel, dim3(grid_for(n)), dim3(kTB), 0, st, __VA_ARGS__)
+
+#define TRY(expr)                                                                                 \
+    do {                                                                                          \
+        const int rc_ = (expr);                                                                   \
+        if (rc_ != SPC3D_OK)                                                                      \
+            return rc_;                                                                           \
+    } while (0)
+
+int fetch(hipStream_t st, void *host, const void *dev, size_t bytes, std::string &err)
+{
+    HIP_OK(hipGetLastError());
+    HIP_OK(hipMemcpyAsync(host, dev, bytes, hipMemcpyDeviceToHost, st));
+    HIP_OK(hipStreamSynchronize(st));
+    return SPC3D_OK;
+}
+
+// Sorts the entries into kernel order: perm (kernel position -> caller's
+// position) and col.  KeyT is wide enough for (row << 4 | group).
+template <typename KeyT>
+int order_entries(Temp &tmp, hipStream_t st, uint64_t nnz, int key_bits, bool slices,
+                  const uint32_t *d_ii, const uint32_t *d_jj, const uint32_t *hubflag,
+                  const uint8_t *cls, uint32_t *perm, uint32_t *col, Counters *C, std::string &err)
+{
+    DBuf<KeyT> key, key_out;
+    DBuf<uint32_t> ident;
+    HIP_OK(key.alloc(nnz));
+    HIP_OK(key_out.alloc(nnz));
+    HIP_OK(ident.alloc(nnz));
+    LAUNCH((keys_k<KeyT>), nnz, d_ii, d_jj, nnz, slices, hubflag, cls, key.p);
+    LAUNCH(iota_k, nnz, ident.p, nnz);
+    TRY(sort_pairs<KeyT>(tmp, key.p, key_out.p, ident.p, perm, (uint32_t)nnz, key_bits, false, st,
+                         err));
+    LAUNCH(gather_cols_k, nnz, d_jj, perm, nnz, col, C);
+    HIP_OK(hipGetLastError());
+    HIP_OK(hipStreamSynchronize(st)); // key buffers are freed on return
+    return SPC3D_OK;
+}
+
+} // namespace
+
+int build_device_plan(hipStream_t st, uint32_t nrows, uint32_t ncols, uint64_t nnz,
+                      const uint32_t *d_ii, const uint32_t *d_jj, const PlanOpts &opts,
+                      HostPlan &meta, DevPlanArrays &out, std::string &err)
+{
+    if (nnz >= (1ull << 32)) {
+        err = "nnz >= 2^32 is not supported";
+        return SPC3D_ERR_TOO_LARGE;
+    }
+    if (nnz > 0 && (d_ii == nullptr || d_jj == nullptr)) {
+        err = "ii/jj is NULL with nnz > 0";
+        return SPC3D_ERR_INVALID_ARG;
+    }
+    const uint32_t seg_max =
+        std::min<uint32_t>(opts.seg_max ? opts.seg_max : default_seg_max(nnz), 1u << 30);
+    const uint32_t hub_min = opts.hub_min ? opts.hub_min : kDefaultHubMin;
+    const bool want_slices = opts.xcd_slices == 0 || opts.xcd_slices == kSlices;
+
+    HostPlan P;
+    P.nrows = nrows;
+    P.ncols = ncols;
+    P.nnz = nnz;
+    P.seg_max = seg_max;
+    out = DevPlanArrays{};
+    if (nnz == 0) {
+        meta = std::move(P);
+        return SPC3D_OK;
+    }
+
+    Temp tmp;
+    DBuf<Counters> dC;
+    Counters hC;
+    HIP_OK(dC.alloc(1));
+    HIP_OK(hipMemsetAsync(dC.p, 0, sizeof(Counters), st));
+    HIP_OK(hipMemsetAsync(&dC.p->first_bad, 0xFF, sizeof(uint32_t), st));
+
+    // ---- histograms, validation ------------------------------------------------
+    DBuf<uint32_t> rowcnt, rowptr, coldeg;
+    HIP_OK(rowcnt.alloc((size_t)nrows + 1));
+    HIP_OK(rowptr.alloc((size_t)nrows + 1));
+    HIP_OK(coldeg.alloc(ncols));
+    HIP_OK(hipMemsetAsync(rowcnt.p, 0, ((size_t)nrows + 1) * sizeof(uint32_t), st));
+    HIP_OK(hipMemsetAsync(coldeg.p, 0, (size_t)ncols * sizeof(uint32_t), st));
+    LAUNCH(hist_k, nnz, d_ii, d_jj, nnz, nrows, ncols, rowcnt.p, coldeg.p, dC.p);
+    LAUNCH(stats_k, nrows, rowcnt.p, (uint64_t)nrows, &dC.p->rows_touched, &dC.p->max_row);
+    LAUNCH(stats_k, ncols, coldeg.p, (uint64_t)ncols, &dC.p->cols_touched, &dC.p->max_cdeg);
+    TRY(exclusive_sum(tmp, rowcnt.p, rowptr.p, (size_t)nrows + 1, st, err));
+    TRY(fetch(st, &hC, dC.p, sizeof hC, err));
+    if (hC.first_bad != 0xFFFFFFFFu) {
+        uint32_t r = 0, c = 0;
+        TRY(fetch(st, &r, d_ii + hC.first_bad, sizeof r, err));
+        TRY(fetch(st, &c, d_jj + hC.first_bad, sizeof c, err));
+        char buf[160];
+        std::snprintf(buf, sizeof buf, "entry %llu = (%u, %u) is outside the %u x %u pattern",
+                      (unsigned long long)hC.first_bad, r, c, nrows, ncols);
+        err = buf;
+        return SPC3D_ERR_BAD_INDEX;
+    }
+    P.rows_touched = hC.rows_touched;
+    P.cols_touched = hC.cols_touched;
+    P.max_row_nnz = hC.max_row;
+    const uint32_t ctouched = hC.cols_touched, maxcdeg = hC.max_cdeg;
+
+    // ---- column classes (XCD slicing only) ---------------------------------------
+    DBuf<uint8_t> cls;
+    bool slices = false;
+    if (want_slices && opts.hot_cols > 0 && ctouched > opts.hot_cols) {
+        const uint32_t h1 = opts.hot_cols;
+        const uint32_t hrep = std::max<uint32_t>(h1 / 6, 1);
+        const uint64_t htot =
+            std::min<uint64_t>((uint64_t)hrep + (uint64_t)(h1 - hrep) * kSlices, ctouched);
+        // Columns by degree, highest first, ties in column order (a stable sort);
+        // the untouched columns end up last.
+        DBuf<uint32_t> colid, order, deg_sorted;
+        HIP_OK(colid.alloc(ncols));
+        HIP_OK(order.alloc(ncols));
+        HIP_OK(deg_sorted.alloc(ncols));
+        LAUNCH(iota_k, ncols, colid.p, (uint64_t)ncols);
+        TRY(sort_pairs<uint32_t>(tmp, coldeg.p, deg_sorted.p, colid.p, order.p, ncols,
+                                 bits_for(maxcdeg), true, st, err));
+        LAUNCH(sum_first_k, htot, deg_sorted.p, htot, &dC.p->covered);
+        TRY(fetch(st, &hC, dC.p, sizeof hC, err));
+        const uint64_t covered = hC.covered;
+        const double coverage = (double)covered / (double)nnz;
+        const double share = (double)htot / (double)ctouched;
+        if (coverage >= 0.2 && coverage >= 2.0 * share) {
+            slices = true;
+            HIP_OK(cls.alloc(ncols));
+            LAUNCH(fill_k<uint8_t>, ncols, cls.p, (uint64_t)ncols, kClsCold);
+            LAUNCH(classify_k, htot, order.p, htot, hrep, cls.p);
+            P.hot_cols = (uint32_t)htot;
+            P.hot_entries = covered;
+        }
+        HIP_OK(hipGetLastError());
+        HIP_OK(hipStreamSynchronize(st)); // the sort buffers are freed here
+    }
+
+    // ---- hub rows: group counts ---------------------------------------------------
+    DBuf<uint32_t> hubflag, hubpos, hubcnt;
+    uint32_t nh = 0;
+    if (slices) {
+        HIP_OK(hubflag.alloc((size_t)nrows + 1));
+        HIP_OK(hubpos.alloc((size_t)nrows + 1));
+        LAUNCH(hubflag_k, (uint64_t)nrows + 1, rowcnt.p, nrows, hub_min, hubflag.p);
+        TRY(exclusive_sum(tmp, hubflag.p, hubpos.p, (size_t)nrows + 1, st, err));
+        TRY(fetch(st, &nh, hubpos.p + nrows, sizeof nh, err));
+        P.hub_rows = nh;
+        HIP_OK(hubcnt.alloc((size_t)nh * 9 + 1));
+        HIP_OK(hipMemsetAsync(hubcnt.p, 0, ((size_t)nh * 9 + 1) * sizeof(uint32_t), st));
+        LAUNCH(hubcount_k, nnz, d_ii, d_jj, nnz, hubflag.p, hubpos.p, cls.p, hubcnt.p);
+    }
+
+    // ---- stable sort into kernel order ------------------------------------------------
+    DBuf<uint32_t> perm, col;
+    HIP_OK(perm.alloc(nnz));
+    HIP_OK(col.alloc(nnz));
+    {
+        const int row_bits = bits_for(nrows ? nrows - 1 : 0);
+        const int key_bits = row_bits + (slices ? 4 : 0);
+        if (key_bits <= 32)
+            TRY(order_entries<uint32_t>(tmp, st, nnz, key_bits, slices, d_ii, d_jj, hubflag.p,
+                                        cls.p, perm.p, col.p, dC.p, err));
+        else
+            TRY(order_entries<unsigned long long>(tmp, st, nnz, key_bits, slices, d_ii, d_jj,
+                                                  hubflag.p, cls.p, perm.p, col.p, dC.p, err));
+    }
+
+    // ---- segments --------------------------------------------------------------------
+    DBuf<uint32_t> npieces, issplit, nslot, piece_off, split_off, slot_off;
+    const size_t nr1 = (size_t)nrows + 1;
+    HIP_OK(npieces.alloc(nr1));
+    HIP_OK(issplit.alloc(nr1));
+    HIP_OK(nslot.alloc(nr1));
+    HIP_OK(piece_off.alloc(nr1));
+    HIP_OK(split_off.alloc(nr1));
+    HIP_OK(slot_off.alloc(nr1));
+    LAUNCH(count_pieces_k, nr1, rowcnt.p, nrows, seg_max, slices, hubflag.p, hubpos.p, hubcnt.p,
+           npieces.p, issplit.p, nslot.p);
+    TRY(exclusive_sum(tmp, npieces.p, piece_off.p, (size_t)nrows + 1, st, err));
+    TRY(exclusive_sum(tmp, issplit.p, split_off.p, (size_t)nrows + 1, st, err));
+    TRY(exclusive_sum(tmp, nslot.p, slot_off.p, (size_t)nrows + 1, st, err));
+    uint32_t totals[3] = {0, 0, 0};
+    TRY(fetch(st, &totals[0], piece_off.p + nrows, sizeof(uint32_t), err));
+    TRY(fetch(st, &totals[1], split_off.p + nrows, sizeof(uint32_t), err));
+    TRY(fetch(st, &totals[2], slot_off.p + nrows, sizeof(uint32_t), err));
+    const uint32_t np_total = totals[0], nsplit = totals[1];
+    P.nslots = totals[2];
+    P.nseg_real = np_total;
+
+    DBuf<Seg> pseg;
+    DBuf<uint8_t> pqueue;
+    DBuf<SplitRow> splits;
+    HIP_OK(pseg.alloc(np_total));
+    HIP_OK(pqueue.alloc(np_total));
+    HIP_OK(splits.alloc(nsplit));
+    LAUNCH(emit_pieces_k, nrows, rowptr.p, nrows, seg_max, slices, hubflag.p, hubpos.p, hubcnt.p,
+           piece_off.p, split_off.p, slot_off.p, pseg.p, pqueue.p, splits.p);
+
+    // ---- order and deal --------------------------------------------------------------
+    DBuf<Seg> segs;
+    uint32_t nseg_padded = 0;
+    const int len_bits = bits_for(seg_max);
+    if (!slices) {
+        DBuf<uint32_t> key, key_out, idx, idx_out;
+        HIP_OK(key.alloc(np_total));
+        HIP_OK(key_out.alloc(np_total));
+        HIP_OK(idx.alloc(np_total));
+        HIP_OK(idx_out.alloc(np_total));
+        HIP_OK(segs.alloc(np_total));
+        LAUNCH(len_keys_k, np_total, pseg.p, (uint64_t)np_total, seg_max, key.p, dC.p);
+        LAUNCH(iota_k, np_total, idx.p, (uint64_t)np_total);
+        TRY(sort_pairs<uint32_t>(tmp, key.p, key_out.p, idx.p, idx_out.p, np_total, len_bits,
+                                 false, st, err));
+        LAUNCH(gather_segs_k, np_total, pseg.p, idx_out.p, (uint64_t)np_total, segs.p);
+        TRY(fetch(st, &hC, dC.p, sizeof hC, err));
+        P.nqueues = 1;
+        nseg_padded = np_total;
+        P.nseg_long = hC.nlong / kChunk * kChunk;
+    } else {
+        DBuf<uint32_t> anyflag, anypos;
+        HIP_OK(anyflag.alloc((size_t)np_total + 1));
+        HIP_OK(anypos.alloc((size_t)np_total + 1));
+        LAUNCH(any_flags_k, (uint64_t)np_total + 1, pseg.p, pqueue.p, (uint64_t)np_total,
+               anyflag.p, dC.p);
+        TRY(exclusive_sum(tmp, anyflag.p, anypos.p, (size_t)np_total + 1, st, err));
+        uint32_t nany = 0;
+        TRY(fetch(st, &nany, anypos.p + np_total, sizeof nany, err));
+        TRY(fetch(st, &hC, dC.p, sizeof hC, err));
+
+        DBuf<uint32_t> any_idx, any_key, any_key_out, any_sorted;
+        HIP_OK(any_idx.alloc(nany));
+        HIP_OK(any_key.alloc(nany));
+        HIP_OK(any_key_out.alloc(nany));
+        HIP_OK(any_sorted.alloc(nany));
+        if (nany) {
+            LAUNCH(compact_any_k, np_total, pseg.p, anyflag.p, anypos.p, (uint64_t)np_total,
+                   seg_max, any_idx.p, any_key.p);
+            TRY(sort_pairs<uint32_t>(tmp, any_key.p, any_key_out.p, any_idx.p, any_sorted.p, nany,
+                                     len_bits, false, st, err));
+        }
+        uint64_t load[kDealQueues];
+        for (uint32_t q = 0; q < kDealQueues; ++q)
+            load[q] = hC.load[q];
+        Upto upto;
+        deal_thresholds(load, hC.any_load, upto.v);
+
+        DBuf<uint32_t> comb_idx, comb_key, comb_idx_out, comb_key_out;
+        HIP_OK(comb_idx.alloc(np_total));
+        HIP_OK(comb_key.alloc(np_total));
+        HIP_OK(comb_idx_out.alloc(np_total));
+        HIP_OK(comb_key_out.alloc(np_total));
+        LAUNCH(combine_k, (uint64_t)np_total + nany, pseg.p, pqueue.p, anyflag.p, anypos.p,
+               any_sorted.p, (uint64_t)np_total, (uint64_t)nany, seg_max, upto, comb_idx.p,
+               comb_key.p, dC.p);
+        const int comb_bits = bits_for((uint64_t)kSlices * ((uint64_t)seg_max + 1) - 1);
+        TRY(sort_pairs<uint32_t>(tmp, comb_key.p, comb_key_out.p, comb_idx.p, comb_idx_out.p,
+                                 np_total, comb_bits, false, st, err));
+        TRY(fetch(st, &hC, dC.p, sizeof hC, err));
+        QStart qs;
+        uint32_t at = 0, nchunks = 0, rounds = 0xFFFFFFFFu;
+        for (uint32_t q = 0; q < kSlices; ++q) {
+            qs.v[q] = at;
+            at += hC.qcount[q];
+            nchunks = std::max(nchunks, (hC.qcount[q] + kChunk - 1) / kChunk);
+            rounds = std::min(rounds, hC.qlong[q] / kChunk);
+        }
+        const uint64_t padded = (uint64_t)nchunks * kSlices * kChunk;
+        if (padded >= (1ull << 32)) {
+            err = "the padded segment list does not fit 32 bits";
+            return SPC3D_ERR_TOO_LARGE;
+        }
+        nseg_padded = (uint32_t)padded;
+        HIP_OK(segs.alloc(nseg_padded));
+        LAUNCH(fill_k<Seg>, nseg_padded, segs.p, (uint64_t)nseg_padded, (Seg{0, 0, 0, kWholeRow}));
+        LAUNCH(scatter_segs_k, np_total, pseg.p, comb_idx_out.p, comb_key_out.p,
+               (uint64_t)np_total, seg_max, qs, segs.p);
+        HIP_OK(hipGetLastError());
+        HIP_OK(hipStreamSynchronize(st));
+        P.nqueues = kSlices;
+        P.nseg_long = rounds * kSlices * kChunk;
+    }
+    HIP_OK(hipGetLastError());
+    HIP_OK(hipStreamSynchronize(st));
+    P.identity = hC.not_identity == 0;
+
+    out.segs = segs.release();
+    out.nseg_padded = nseg_padded;
+    out.col = col.release();
+    out.perm = P.identity ? nullptr : perm.release();
+    out.splits = splits.release();
+    out.nsplit = nsplit;
+    meta = std::move(P);
+    return SPC3D_OK;
+}
+
+} // namespace spc3d

@@ -42,31 +42,12 @@ int validate_coo(uint32_t nrows, uint32_t ncols, uint64_t nnz, const uint32_t *i
 
 namespace {
 
-// Column classes (XCD slicing).  A "replicated" column is hot enough that every
-// L2 keeps its dense row; a "slice s" column is meant to be kept by the L2 of
-// XCD s, so the entries of hub rows in it are queued to XCD s; "cold" columns
-// are not expected to stay in any L2.
-constexpr uint8_t kRep = 8, kCold = 9;
-constexpr uint8_t kAnyQueue = 0xFF;
-constexpr uint32_t kSlices = 8;
+constexpr uint8_t kRep = kClsRep, kCold = kClsCold;
 
 struct Piece {
     Seg seg;
     uint8_t queue;
 };
-
-// Columns are dealt to slices in degree order, back and forth (0..7, 7..0, ...),
-// so that no slice collects the larger column of every round.
-inline uint8_t slice_of_rank(uint64_t i)
-{
-    const uint32_t pos = (uint32_t)(i % kSlices);
-    return (uint8_t)(((i / kSlices) & 1) ? kSlices - 1 - pos : pos);
-}
-
-// Replicated-hot entries of a hub row ride with one of its slices; a hash of
-// the row id picks it (low row-id bits correlate with degree in R-MAT-like
-// graphs, so they would not spread the rows evenly).
-inline uint32_t rep_slice(uint32_t row) { return (row * 2654435761u) >> 29; }
 
 inline uint32_t seg_len(const Seg &s) { return s.len; }
 
@@ -178,10 +159,7 @@ int build_host_plan(uint32_t nrows, uint32_t ncols, uint64_t nnz, const uint32_t
         // keep the caller's order.
         std::vector<int32_t> hubidx;
         std::vector<uint32_t> hubcnt; // 9 group counts per hub row
-        auto group_of = [&](uint32_t r, uint32_t c) -> uint32_t {
-            const uint8_t k = cls[c];
-            return k == kRep ? rep_slice(r) : (k == kCold ? 8u : k);
-        };
+        auto group_of = [&](uint32_t r, uint32_t c) -> uint32_t { return hub_group(r, cls[c]); };
         if (slices) {
             hubidx.assign((size_t)nrows, -1);
             uint32_t nh = 0;

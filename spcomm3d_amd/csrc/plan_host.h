@@ -5,6 +5,12 @@
 #include <string>
 #include <vector>
 
+#if defined(__HIPCC__)
+#define SPC3D_HD __host__ __device__
+#else
+#define SPC3D_HD
+#endif
+
 namespace spc3d {
 
 // One unit of work for a lane group: `len` consecutive entries of one row in
@@ -61,6 +67,34 @@ struct HostPlan {
 
 constexpr uint32_t kDefaultHubMin = 128;
 
+// ---- column classes of the XCD-sliced layout ---------------------------------
+// A "replicated" column is hot enough that every L2 keeps its dense row; a
+// "slice s" column (class s < 8) is meant to be kept by the L2 of XCD s, so the
+// entries of hub rows in it are queued to XCD s; "cold" columns are not expected
+// to stay in any L2.
+constexpr uint8_t kClsRep = 8, kClsCold = 9;
+constexpr uint8_t kAnyQueue = 0xFF;
+constexpr uint32_t kSlices = 8;
+
+// Columns are dealt to slices in degree order, back and forth (0..7, 7..0, ...),
+// so that no slice collects the larger column of every round.
+SPC3D_HD inline uint8_t slice_of_rank(uint64_t i)
+{
+    const uint32_t pos = (uint32_t)(i % kSlices);
+    return (uint8_t)(((i / kSlices) & 1) ? kSlices - 1 - pos : pos);
+}
+
+// Replicated-hot entries of a hub row ride with one of its slices; a hash of
+// the row id picks it (low row-id bits correlate with degree in R-MAT-like
+// graphs, so they would not spread the rows evenly).
+SPC3D_HD inline uint32_t rep_slice(uint32_t row) { return (row * 2654435761u) >> 29; }
+
+// Group (0..7: slice, 8: cold) of an entry of hub row `row` in a column of class `cls`.
+SPC3D_HD inline uint32_t hub_group(uint32_t row, uint8_t cls)
+{
+    return cls == kClsRep ? rep_slice(row) : (cls == kClsCold ? 8u : cls);
+}
+
 // ---- dealing of free segments to the 8 XCD queues -------------------------
 // A segment weighs its length plus kSegCost (descriptor, dense row, write-back).
 constexpr uint32_t kSegCost = 4;
@@ -109,7 +143,7 @@ inline void deal_thresholds(const uint64_t (&load)[kDealQueues], uint64_t free_l
 
 // Queue of the i-th free segment (longest first): the share that holds the i-th
 // point of the golden-ratio sequence i * 0x9E3779B9 mod 2^32.
-inline uint32_t deal_queue(uint32_t i, const uint32_t (&upto)[kDealQueues])
+SPC3D_HD inline uint32_t deal_queue(uint32_t i, const uint32_t (&upto)[kDealQueues])
 {
     const uint32_t x = i * 0x9E3779B9u;
     uint32_t q = 0;

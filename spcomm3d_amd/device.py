@@ -28,10 +28,15 @@ def _vp(a: np.ndarray | None):
     return None if a is None else a.ctypes.data_as(ctypes.c_void_p)
 
 
+_BUILDERS = {None: 0, "device": 2, "host": 1}
+
+
 def make_opts(seg_max=None, k_hint=None, l2_hot_bytes=None, hub_min=None,
-              xcd_slices=None) -> PlanOpts:
-    """``spc3d_plan_opts``; ``None`` keeps the library default."""
+              xcd_slices=None, builder=None) -> PlanOpts:
+    """``spc3d_plan_opts``; ``None`` keeps the library default.  ``builder``:
+    ``"device"`` or ``"host"`` (where ``spc3d_plan_create_ex`` builds the plan)."""
     o = PlanOpts()
+    o.builder = _BUILDERS[builder]
     o.seg_max = int(seg_max or 0)
     o.k_hint = int(k_hint or 0)
     o.l2_hot_bytes = int(l2_hot_bytes or 0)
@@ -228,6 +233,12 @@ class Vals:
     def fill(self, value: float):
         check(self.ctx._lib.spc3d_vals_fill(self._h, float(value)), "spc3d_vals_fill")
 
+    def device_ptr(self) -> int:
+        p = ctypes.c_void_p()
+        check(self.ctx._lib.spc3d_vals_device_ptr(self._h, ctypes.byref(p)),
+              "spc3d_vals_device_ptr")
+        return p.value or 0
+
     def close(self):
         if getattr(self, "_h", None) and getattr(self.ctx, "_h", None):
             self.ctx._lib.spc3d_vals_destroy(self._h)
@@ -274,6 +285,36 @@ class Plan:
         check(rc, "spc3d_plan_create")
         self._h = h
         self.nnz = int(ii.size)
+
+    @classmethod
+    def from_device(cls, ctx: Context, nrows, ncols, ii: "Vals", jj: "Vals", nnz: int, dtype,
+                    **opts) -> "Plan":
+        """Plan of a pattern whose ``ii`` / ``jj`` already live on the device, as the
+        first ``nnz`` 32-bit words of two value vectors (``spc3d_plan_create_from_device``)."""
+        self = cls.__new__(cls)
+        self.ctx = ctx
+        self.code = dtype_code(dtype)
+        self.dtype = _NP[self.code]
+        h = ctypes.c_void_p()
+        check(ctx._lib.spc3d_plan_create_from_device(
+            ctx._h, self.code, int(nrows), int(ncols), int(nnz), ii.device_ptr(), jj.device_ptr(),
+            ctypes.byref(make_opts(**opts)), ctypes.byref(h)), "spc3d_plan_create_from_device")
+        self._h = h
+        self.nnz = int(nnz)
+        return self
+
+    def download(self) -> dict:
+        """The plan's arrays as they are on the device, in the layout of
+        :func:`plan_build_host` (``spc3d_plan_download``)."""
+        info = self.info
+        col = np.empty(self.nnz, dtype=np.uint32)
+        perm = np.empty(self.nnz, dtype=np.uint32)
+        segs = np.empty((info.nsegments_padded, 4), dtype=np.uint32)
+        splits = np.empty((info.nsplit_rows, 3), dtype=np.uint32)
+        check(self.ctx._lib.spc3d_plan_download(self._h, _vp(col), _vp(perm), _vp(segs),
+                                                info.nsegments_padded, _vp(splits),
+                                                info.nsplit_rows), "spc3d_plan_download")
+        return {"info": info, "col": col, "perm": perm, "segs": segs, "splits": splits}
 
     def set_values(self, vv: np.ndarray):
         vv = np.ascontiguousarray(vv)
