@@ -38,10 +38,10 @@ METRIC = "SDDMM & SpMM GFLOP/s + % HBM roofline on 1 MI355X, RMAT-20 K=64"
 # on (default plan options) and left null for any other: long-segment launch +
 # short-segment launch (+ fix-up for spmm).
 MEASURED_TRAFFIC = {
-    ("rmat20_ef16", 64, "sorted", "f64"): {"sddmm": 4675.3e6 + 1289.8e6,
-                                           "spmm": 4143.0e6 + 1328.7e6 + 123.1e6},
-    ("rmat20_ef16", 64, "sorted", "f32"): {"sddmm": 2358.9e6 + 796.0e6,
-                                           "spmm": 1885.2e6 + 724.9e6 + 61.8e6},
+    ("rmat20_ef16", 64, "sorted", "f64"): {"sddmm": 4603.5e6 + 1168.5e6,
+                                           "spmm": 4089.7e6 + 1326.8e6 + 123.1e6},
+    ("rmat20_ef16", 64, "sorted", "f32"): {"sddmm": 2277.0e6 + 675.6e6,
+                                           "spmm": 1840.7e6 + 723.9e6 + 61.8e6},
 }
 
 
@@ -229,7 +229,9 @@ def main():
                    "rows_touched": main_r["rows_touched"], "cols_touched": main_r["cols_touched"]},
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": kd["strict_gbs"],
                      "peak": roofline.HBM_PEAK_GBS, "unit": "GB/s", "frac": kd["strict_frac"],
-                     "traffic": traffic, "bytes_per_launch": kd["strict_bytes"],
+                     "traffic": traffic,
+                     "traffic_gbs": None if traffic is None else traffic / kd["ms_avg"] / 1e6,
+                     "bytes_per_launch": kd["strict_bytes"],
                      "ms_per_launch": kd["ms_avg"], "model": "strict (each operand once)"},
         "cpu_baseline": cpu,
         "kernels": main_r["kernels"],
