@@ -98,6 +98,12 @@ template <typename T> class Vals {
     Vals &operator=(const Vals &) = delete;
     spc3d_vals *get() const { return h_; }
     uint64_t size() const { return n_; }
+    void *device_ptr() const
+    {
+        void *p = nullptr;
+        check(spc3d_vals_device_ptr(h_, &p), "spc3d_vals_device_ptr");
+        return p;
+    }
     void upload(const T *host) { check(spc3d_vals_upload(h_, host), "spc3d_vals_upload"); }
     void download(T *host) { check(spc3d_vals_download(h_, host), "spc3d_vals_download"); }
     void fill(double v) { check(spc3d_vals_fill(h_, v), "spc3d_vals_fill"); }
@@ -118,6 +124,16 @@ template <typename T> class Plan {
                    : spc3d_plan_create(ctx.get(), dtype_of<T>(), nrows, ncols, nnz, ii, jj, vv,
                                        &h_),
               "spc3d_plan_create");
+    }
+    // A pattern that already lives on the device: dev_ii, dev_jj are device pointers
+    // to nnz uint32 each.  The plan has no values until set_values.
+    struct FromDevice {};
+    Plan(FromDevice, Context &ctx, uint32_t nrows, uint32_t ncols, uint64_t nnz,
+         const void *dev_ii, const void *dev_jj, const spc3d_plan_opts *opts = nullptr)
+    {
+        check(spc3d_plan_create_from_device(ctx.get(), dtype_of<T>(), nrows, ncols, nnz, dev_ii,
+                                            dev_jj, opts, &h_),
+              "spc3d_plan_create_from_device");
     }
     ~Plan()
     {
@@ -142,6 +158,51 @@ template <typename T> class Plan {
   private:
     spc3d_plan *h_ = nullptr;
 };
+
+// Buffer slot i <-> dense row rows[i] of a panel with panel_rows rows: the device
+// form of SparseComm::sendptr / recvptr (src/comm.hpp:41,49).
+class RowMap {
+  public:
+    RowMap(Context &ctx, uint32_t panel_rows, uint64_t n, const uint32_t *rows) : n_(n)
+    {
+        check(spc3d_rowmap_create(ctx.get(), panel_rows, n, rows, &h_), "spc3d_rowmap_create");
+    }
+    ~RowMap()
+    {
+        if (h_)
+            spc3d_rowmap_destroy(h_);
+    }
+    RowMap(const RowMap &) = delete;
+    RowMap &operator=(const RowMap &) = delete;
+    spc3d_rowmap *get() const { return h_; }
+    uint64_t size() const { return n_; }
+
+  private:
+    spc3d_rowmap *h_ = nullptr;
+    uint64_t n_;
+};
+
+// buf[i,:] = P[rows[i],:]  (SparseComm::copy_to_sendbuff, src/comm.hpp:90-103)
+template <typename T>
+void rows_pack(Context &ctx, const Panel<T> &P, const RowMap &map, Vals<T> &buf)
+{
+    check(spc3d_rows_pack(ctx.get(), P.get(), map.get(), buf.get()), "spc3d_rows_pack");
+}
+
+// P[rows[i],:] = buf[i,:]  (SparseComm::copy_from_recvbuff, src/comm.hpp:166-177)
+template <typename T>
+void rows_unpack(Context &ctx, Panel<T> &P, const RowMap &map, const Vals<T> &buf)
+{
+    check(spc3d_rows_unpack(ctx.get(), P.get(), map.get(), buf.get()), "spc3d_rows_unpack");
+}
+
+// P[rows[i],:] += buf[i,:] in slot order  (SparseComm::SUM_from_recvbuff, src/comm.hpp:178-189)
+template <typename T>
+void rows_unpack_sum(Context &ctx, Panel<T> &P, const RowMap &map, const Vals<T> &buf)
+{
+    check(spc3d_rows_unpack_sum(ctx.get(), P.get(), map.get(), buf.get()),
+          "spc3d_rows_unpack_sum");
+}
 
 // C = S .* (A B^T) on resident operands; asynchronous on the context's stream.
 template <typename T>

@@ -18,6 +18,7 @@
 #include <string>
 
 #include "spc3d/core_ops.hpp"
+#include "spc3d/device.hpp"
 #include "spc3d/distributed_comp.hpp"
 
 extern "C" {
@@ -359,6 +360,72 @@ static void test_dist_wrappers_single_rank()
     std::fclose(f);
 }
 
+// The resident-operand handles: SDDMM whose result feeds SpMM without leaving the
+// device, a plan made from a pattern that is already there, and the pack /
+// sum-unpack pair either side of a sparse exchange (src/comm.hpp:90-103,178-189),
+// here sending every partial Y row back onto itself twice.
+static void test_resident_handles_and_row_exchange()
+{
+    const idx_t m = 300, n = 257, k = 24;
+    cooMat S = random_coo(m, n, 5000, 41);
+    denseMatrix A = random_panel(m, k, 42), B = random_panel(n, k, 43), Y0 = random_panel(m, k, 44);
+    spc3d::Context ctx(0);
+    spc3d::Panel<real_t> dA(ctx, m, k), dB(ctx, n, k), dY(ctx, m, k);
+    dA.upload(A.data.data());
+    dB.upload(B.data.data());
+    dY.upload(Y0.data.data());
+    // the pattern goes up as 32-bit words and is planned where it lies
+    static_assert(sizeof(float) == sizeof(idx_t), "index words travel as 32-bit values");
+    spc3d::Vals<float> dii(ctx, S.nnz), djj(ctx, S.nnz);
+    dii.upload(reinterpret_cast<const float *>(S.ii.data()));
+    djj.upload(reinterpret_cast<const float *>(S.jj.data()));
+    spc3d::Plan<real_t> P(spc3d::Plan<real_t>::FromDevice{}, ctx, m, n, S.nnz, dii.device_ptr(),
+                          djj.device_ptr());
+    P.set_values(S.vv.data());
+    spc3d::Vals<real_t> dC(ctx, S.nnz);
+    spc3d::sddmm(ctx, P, dA, dB, dC);
+    std::vector<real_t> c(S.nnz), cref;
+    dC.download(c.data());
+    oracle_sddmm(A, B, S, cref);
+    CHECK(max_rel(c, cref, k * 1.0) < kTol);
+    // C becomes the sparse operand of SpMM on the device
+    P.set_values(dC);
+    spc3d::spmm(ctx, P, dB, dY);
+    cooMat S2 = S;
+    S2.vv = cref;
+    std::vector<real_t> yref = Y0.data;
+    oracle_spmm(B, S2, yref, m);
+    std::vector<real_t> y((size_t)m * k);
+    dY.download(y.data());
+    CHECK(max_rel(y, yref, 100.0) < 10 * kTol);
+
+    // pack rows (with repeats), then sum them back: Y[r] += (times r is listed) * Y[r]
+    std::vector<idx_t> rows;
+    for (idx_t r = 0; r < m; r += 3) {
+        rows.push_back(r);
+        if (r % 2 == 0)
+            rows.push_back(r);
+    }
+    spc3d::RowMap map(ctx, m, rows.size(), rows.data());
+    spc3d::Vals<real_t> buf(ctx, rows.size() * (uint64_t)k);
+    spc3d::rows_pack(ctx, dY, map, buf);
+    spc3d::rows_unpack_sum(ctx, dY, map, buf);
+    std::vector<real_t> y2((size_t)m * k), want = y;
+    dY.download(y2.data());
+    for (idx_t r : rows)
+        for (idx_t j = 0; j < k; ++j)
+            want[(size_t)r * k + j] += y[(size_t)r * k + j]; // sequential, slot order
+    CHECK(y2 == want); // copies and ordered adds: bit for bit
+    bool threw = false;
+    try {
+        idx_t bad = m;
+        spc3d::RowMap nope(ctx, m, 1, &bad);
+    } catch (const std::out_of_range &) {
+        threw = true;
+    }
+    CHECK(threw);
+}
+
 int main(int argc, char **argv)
 {
     const bool host_only = argc > 1 && std::strcmp(argv[1], "--host") == 0;
@@ -370,6 +437,7 @@ int main(int argc, char **argv)
             test_bench_fill_and_five_calls();
             test_random_against_oracle_and_remap();
             test_dist_wrappers_single_rank();
+            test_resident_handles_and_row_exchange();
             hip::shutdown();
         } catch (const std::exception &e) {
             std::printf("FAIL: exception: %s\n", e.what());
