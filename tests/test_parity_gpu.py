@@ -135,6 +135,42 @@ def test_cut_rows_with_ragged_k(ctx, dtype, k):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("k", [64, 20])
+def test_rows_the_pattern_never_names_are_never_read(ctx, dtype, k):
+    # the reference touches A[ii[e]], B[jj[e]] and Y[ii[e]] only (core_ops.cpp:16,32): NaN
+    # in every other dense row must not reach any result, whatever the batching loads
+    m, n, nnz = 90, 120, 1500
+    ii, jj, vv, A, B, Y0 = rand_case(77 + k, m, n, k, nnz, dtype, hub=400)
+    ii = (ii // 2 * 2).astype(np.uint32)       # odd rows are never named
+    jj = (jj // 3 * 3).astype(np.uint32)       # two columns in three are never named
+    A[1::2] = np.nan
+    B[np.arange(n) % 3 != 0] = np.nan
+    C = gpu_sddmm(ctx, m, n, ii, jj, vv, A, B)
+    assert np.all(np.isfinite(C))
+    Aclean, Bclean = np.nan_to_num(A), np.nan_to_num(B)
+    check_sddmm(Aclean, Bclean, ii, jj, vv, C)
+    Y0[1::2] = np.nan
+    Y = gpu_spmm(ctx, m, n, ii, jj, vv, B, Y0)
+    assert np.all(np.isnan(Y[1::2])) and np.all(np.isfinite(Y[0::2]))
+    check_spmm(Bclean, ii, jj, vv, np.nan_to_num(Y0), np.nan_to_num(Y))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_non_finite_inputs_propagate_as_in_the_reference(ctx, dtype):
+    # an infinite X row named with weight a gives a * inf in Y, not NaN from 0 * inf
+    m, n, k = 8, 8, 64
+    ii = np.array([0, 0, 0, 0, 0, 3], dtype=np.uint32)
+    jj = np.array([1, 2, 3, 4, 5, 5], dtype=np.uint32)
+    vv = np.array([1, 1, 1, 1, 2, 1], dtype=dtype)
+    X = np.ones((n, k), dtype=dtype)
+    X[5] = np.inf
+    Y = gpu_spmm(ctx, m, n, ii, jj, vv, X, np.zeros((m, k), dtype=dtype))
+    assert np.all(np.isposinf(Y[0])) and np.all(np.isposinf(Y[3])) and np.all(Y[1] == 0)
+    C = gpu_sddmm(ctx, m, n, ii, jj, vv, np.ones((m, k), dtype=dtype), X)
+    assert np.array_equal(C[:4], np.full(4, k, dtype=dtype)) and np.all(np.isposinf(C[4:]))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("nnz", [0, 1, 2, 15, 16, 17, 63, 65])
 def test_tiny_and_ragged(ctx, dtype, nnz):
     ii, jj, vv, A, B, Y0 = rand_case(nnz, 5, 9, 64, nnz, dtype)
