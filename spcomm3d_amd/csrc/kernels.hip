@@ -5,18 +5,18 @@
 //
 // Both are gather-bound (about 0.25 flop per byte): no MFMA.  The unit of work
 // is a row segment (plan_host.h): at most seg_max consecutive entries of one
-// row.  A dense row of K reals is covered by LPR lanes holding VPL 16-byte
-// vectors each (K * sizeof(T) = LPR * VPL * 16, so K is a compile-time
-// constant of each instantiation), one wavefront works on 64 / LPR segments at
-// once and every global load instruction moves 64 x 16 B.  Segments arrive
-// sorted longest first, so the lane groups of a wavefront run the same trip
-// count.
+// row.  A dense row of K reals is nvec 16-byte vectors, covered by LPR lanes
+// holding VPL vectors each (nvec = LPR * VPL with the row stride a compile-time
+// constant, or nvec < LPR * VPL given at run time in the "ragged" variants, whose
+// spare lanes idle); one wavefront works on 64 / LPR segments at once and every
+// global load instruction moves 64 x 16 B.  Segments arrive sorted longest
+// first, so the lane groups of a wavefront run the same trip count.
 //
-// A segment is walked in batches of UB entries, then one batch each of
-// UB/2, ..., 2, 1 entries as the remaining length requires: every batch size
-// is its own straight-line code with no per-entry predicates.  Within a batch
-// all gathers are issued before any arithmetic (a scheduling barrier keeps the
-// compiler from serialising them).
+// A segment is walked in batches of UB entries; what remains is one masked
+// batch (the missing entries repeat the last one's loads and store nothing), or,
+// in SpMM's short-segment launch, exact batches of UB/2, ..., 2, 1.  Every batch
+// is straight-line code: within it all gathers are issued before any arithmetic
+// (a scheduling barrier keeps the compiler from serialising them).
 //
 //   sddmm: the group keeps its A row slice in registers, gathers the B row
 //          slices of a batch, and reduces the per-lane partial dot products
