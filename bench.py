@@ -11,8 +11,9 @@ the same run and reported under "also".
 Prints one JSON line.  `value` is (flops of both kernels) / (wall time per
 step).  `roofline` is the slower of the two kernels: strict-model bytes per
 launch over its mean launch time, measured with HIP events on the library's
-stream inside the timed region, against 8 TB/s.  `cpu_baseline` is the CPU
-oracle (a serial restatement of the reference's loops) timed on one host core
+stream inside the timed region, against 8 TB/s.  `cpu_baseline` is the
+reference's own kernels (where their build is present, fp64) or else the CPU
+oracle (a serial restatement of the reference's loops), timed on one host core
 on the same workload.
 """
 from __future__ import annotations
@@ -134,6 +135,41 @@ def run_gpu(w, dtype, steps, warmup, seg_max=None, max_timed=1300, copies=0):
     return out
 
 
+def run_reference_baseline(w):
+    """The reference's own core_ops.cpp (compiled into oracle/_ref where the
+    reference tree was available; fp64 only, its real_t is a fixed macro) over
+    the same workload: one SDDMM + SpMM pass on one core, timed inside the shim
+    as the reference times its kernels.  None if that build is not there."""
+    import ctypes
+
+    from tests import _oracle as oracle
+
+    if not oracle.have_ref():
+        return None
+    try:
+        lib = ctypes.CDLL(oracle.REF_LIB)
+        fn = lib.ref_time_f64
+    except (OSError, AttributeError):
+        return None
+    fn.restype = ctypes.c_int
+    fn.argtypes = ([ctypes.c_uint32] * 3 + [ctypes.c_void_p] * 3 + [ctypes.c_uint64] +
+                   [ctypes.c_void_p] * 3 + [ctypes.POINTER(ctypes.c_double)] * 3)
+    A, B, Y0, vv = w.panel_A("f64"), w.panel_B("f64"), w.panel_Y0("f64"), w.values("f64")
+    vp = lambda a: a.ctypes.data_as(ctypes.c_void_p)  # noqa: E731
+    ts, tp, cs = ctypes.c_double(), ctypes.c_double(), ctypes.c_double()
+    if fn(w.nrows, w.ncols, w.k, vp(A), vp(B), vp(Y0), w.nnz, vp(w.ii), vp(w.jj), vp(vv),
+          ctypes.byref(ts), ctypes.byref(tp), ctypes.byref(cs)) != 0:
+        return None
+    fl = 2 * w.nnz * w.k
+    return {"value": 2 * fl / (ts.value + tp.value) / 1e9, "unit": "GFLOP/s", "cores": 1,
+            "kind": "reference",
+            "sample": f"one full SDDMM+SpMM pass of the reference's core_ops.cpp over {w.name} "
+                      f"K={w.k} f64 ({w.order} COO, nnz={w.nnz})",
+            "sddmm_s": ts.value, "spmm_s": tp.value,
+            "sddmm_gflops": fl / ts.value / 1e9, "spmm_gflops": fl / tp.value / 1e9,
+            "host_cores": os.cpu_count(), "flags": "g++ -O3 -ffp-contract=off"}
+
+
 def run_cpu_baseline(w, dtype):
     """The CPU oracle (serial, one core, as the reference's per-rank path is:
     no threads anywhere in it) on the same workload, one SDDMM + SpMM pass."""
@@ -209,7 +245,11 @@ def main():
         other = "f32" if args.dtype == "f64" else "f64"
         also[other] = run_gpu(w, other, args.steps, args.warmup, args.seg_max)
         log(json.dumps(also[other]))
-    cpu = None if args.no_cpu else run_cpu_baseline(w, args.dtype)
+    cpu = None
+    if not args.no_cpu:
+        port = run_cpu_baseline(w, args.dtype)
+        ref = run_reference_baseline(w) if args.dtype == "f64" else None
+        cpu = dict(ref, port=port) if ref else port
 
     dom = max(main_r["kernels"], key=lambda k: main_r["kernels"][k]["ms_avg"])
     kd = main_r["kernels"][dom]

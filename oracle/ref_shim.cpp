@@ -7,6 +7,7 @@
 //
 // This file contains no reference code; it includes the reference headers by
 // path (-I<reference>/src) and links the reference's core_ops.cpp.
+#include <chrono>
 #include <cstdint>
 #include <cstring>
 #include <exception>
@@ -73,6 +74,44 @@ ref_spmm_f64(uint32_t ncols, uint32_t nrows, uint32_t k, const double *X,
         fill_coo(A, nrows, ncols, nnz, ii, jj, avv);
         spmm(x, A, y);
         std::memcpy(Y, y.data.data(), (size_t)nrows * k * sizeof(double));
+        return 0;
+    } catch (const std::exception &) {
+        return -1;
+    }
+}
+
+// One SDDMM then one SpMM of the reference over the same operands, timed as the
+// reference times its kernel (a chrono pair around the call,
+// src/distributed_comp.cpp:176-179); building the reference's objects from the
+// caller's arrays is outside the timed regions.  The results are discarded but
+// for one checksum each, so that the calls cannot be optimised away.
+__attribute__((visibility("default"))) int
+ref_time_f64(uint32_t m, uint32_t n, uint32_t k, const double *A, const double *B,
+             const double *Y0, uint64_t nnz, const uint32_t *ii, const uint32_t *jj,
+             const double *vv, double *sddmm_seconds, double *spmm_seconds, double *checksum)
+{
+    try {
+        denseMatrix a, b, y;
+        cooMat S, C;
+        fill_panel(a, m, k, A);
+        fill_panel(b, n, k, B);
+        fill_panel(y, m, k, Y0);
+        fill_coo(S, m, n, nnz, ii, jj, vv);
+        C = S;
+        using clock = std::chrono::steady_clock;
+        const auto t0 = clock::now();
+        sddmm(a, b, S, C);
+        const auto t1 = clock::now();
+        spmm(b, S, y);
+        const auto t2 = clock::now();
+        *sddmm_seconds = std::chrono::duration<double>(t1 - t0).count();
+        *spmm_seconds = std::chrono::duration<double>(t2 - t1).count();
+        double sum = 0;
+        for (uint64_t e = 0; e < nnz; ++e)
+            sum += C.vv[e];
+        for (double v : y.data)
+            sum += v;
+        *checksum = sum;
         return 0;
     } catch (const std::exception &) {
         return -1;
