@@ -67,6 +67,25 @@ def test_f64_bit_exact_vs_live_reference_build(seed):
 
 
 @pytest.mark.skipif(not oracle.have_ref(), reason="oracle/_ref is only built where the reference is mounted")
+def test_timed_reference_pass_computes_what_the_oracle_computes():
+    # the entry bench.py times as the CPU baseline: SDDMM, then SpMM with the same values
+    import ctypes
+
+    ref = oracle.load_ref()
+    ii, jj, vv, A, B, Y0 = _rand_case(9, 120, 120, 16, 3000)
+    p = lambda a: a.ctypes.data_as(oracle._vp)  # noqa: E731
+    ts, tp, cs = ctypes.c_double(), ctypes.c_double(), ctypes.c_double()
+    ref.ref_time_f64.restype = ctypes.c_int
+    ref.ref_time_f64.argtypes = ([ctypes.c_uint32] * 3 + [oracle._vp] * 3 + [ctypes.c_uint64] +
+                                 [oracle._vp] * 3 + [ctypes.POINTER(ctypes.c_double)] * 3)
+    assert ref.ref_time_f64(120, 120, 16, p(A), p(B), p(Y0), ii.size, p(ii), p(jj), p(vv),
+                            ctypes.byref(ts), ctypes.byref(tp), ctypes.byref(cs)) == 0
+    want = float(np.sum(oracle.sddmm(A, B, ii, jj, vv))) + float(np.sum(oracle.spmm(B, ii, jj, vv, Y0)))
+    assert abs(cs.value - want) <= 1e-9 * max(1.0, abs(want))
+    assert ts.value > 0 and tp.value > 0
+
+
+@pytest.mark.skipif(not oracle.have_ref(), reason="oracle/_ref is only built where the reference is mounted")
 def test_reference_rejects_bad_index_like_oracle():
     ref = oracle.load_ref()
     ii, jj, vv, A, B, _ = _rand_case(5, 10, 10, 4, 20)
