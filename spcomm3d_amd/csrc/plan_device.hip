@@ -93,20 +93,45 @@ __global__ void iota_k(uint32_t *p, uint64_t n)
     GRID_STRIDE(i, n) p[i] = (uint32_t)i;
 }
 
+// Adds 1 to cnt[key] for every lane with a valid key, with one atomic per run of
+// equal keys in consecutive lanes (sorted COO puts a whole wavefront on one row,
+// and same-address atomics of a wavefront are served one after the other).
+__device__ __forceinline__ void count_runs(uint32_t *cnt, uint32_t key, bool valid)
+{
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t prev = __shfl_up(key, 1, 64);
+    const bool prev_valid = __shfl_up((int)valid, 1, 64) != 0;
+    const bool head = valid && (lane == 0 || !prev_valid || prev != key);
+    // a run ends where the next head starts or where the keys stop being valid
+    const unsigned long long stops = __ballot(head || !valid);
+    if (head) {
+        const unsigned long long above = lane == 63 ? 0ull : stops >> (lane + 1);
+        const uint32_t len = above ? (uint32_t)__ffsll((long long)above) : 64u - lane;
+        atomicAdd(cnt + key, len);
+    }
+}
+
 // Row and column histograms; the first out-of-range entry, if any.
 __global__ void hist_k(const uint32_t *__restrict__ ii, const uint32_t *__restrict__ jj,
                        uint64_t nnz, uint32_t nrows, uint32_t ncols, uint32_t *rowcnt,
                        uint32_t *coldeg, Counters *C)
 {
-    GRID_STRIDE(e, nnz)
-    {
-        const uint32_t r = ii[e], c = jj[e];
-        if (r >= nrows || c >= ncols) {
-            atomicMin(&C->first_bad, (uint32_t)e);
-        } else {
-            atomicAdd(rowcnt + r, 1u);
-            atomicAdd(coldeg + c, 1u);
+    // whole wavefronts walk the entries together, so that lanes can pool their counts
+    const uint64_t stride = (uint64_t)gridDim.x * kTB;
+    for (uint64_t base = (uint64_t)blockIdx.x * kTB + (threadIdx.x & ~63u); base < nnz;
+         base += stride) {
+        const uint64_t e = base + (threadIdx.x & 63u);
+        uint32_t r = 0, c = 0;
+        bool ok = false;
+        if (e < nnz) {
+            r = ii[e];
+            c = jj[e];
+            ok = r < nrows && c < ncols;
+            if (!ok)
+                atomicMin(&C->first_bad, (uint32_t)e);
         }
+        count_runs(rowcnt, r, ok);
+        count_runs(coldeg, c, ok);
     }
 }
 
