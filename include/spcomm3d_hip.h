@@ -199,6 +199,20 @@ SPC3D_API int spc3d_plan_create_from_device(spc3d_ctx *ctx, int dtype, uint32_t 
                                   uint32_t ncols, uint64_t nnz, const void *dev_ii,
                                   const void *dev_jj, const spc3d_plan_opts *opts,
                                   spc3d_plan **out);
+/* The index transforms the reference runs before its kernels, for index arrays
+ * that live on the GPU (device pointers to n uint32 of the context's device).
+ * spc3d_localize_device = COOMatrix::localizeIndices (src/SparseMatrix.hpp:69-99)
+ * for one of the two arrays: every distinct value gets the next local id the
+ * first time it appears in the array, dev_idx[e] is replaced by its local id,
+ * dev_ltg[local] (capacity n) receives the value and *nlocal the number of ids
+ * (the reference's nrows / ncols and ltgR / ltgC; call it once for ii, once for
+ * jj).  spc3d_remap_device = COOMatrix::ReMapIndices (src/SparseMatrix.hpp:100-106):
+ * dev_idx[e] = dev_map[dev_idx[e]]; an index >= map_len gives SPC3D_ERR_BAD_INDEX
+ * (the reference's .at()) and changes nothing.  Both synchronous. */
+SPC3D_API int spc3d_localize_device(spc3d_ctx *ctx, uint64_t n, void *dev_idx, void *dev_ltg,
+                          uint32_t *nlocal);
+SPC3D_API int spc3d_remap_device(spc3d_ctx *ctx, uint64_t n, void *dev_idx, const void *dev_map,
+                       uint32_t map_len);
 /* Copies a plan's arrays back from the device, in the layout of
  * spc3d_plan_build_host (each output may be NULL; perm is the identity when the
  * plan stores none).  For inspection and tests.  Synchronous. */

@@ -74,6 +74,8 @@ SIGNATURES = {
                                       P(PlanInfo), c_vp, c_vp, c_vp, c_u32, c_vp, c_u32]),
     "spc3d_plan_create_from_device": (c_int, [c_vp, c_int, c_u32, c_u32, c_u64, c_vp, c_vp,
                                               P(PlanOpts), P(c_vp)]),
+    "spc3d_localize_device": (c_int, [c_vp, c_u64, c_vp, c_vp, P(c_u32)]),
+    "spc3d_remap_device": (c_int, [c_vp, c_u64, c_vp, c_vp, c_u32]),
     "spc3d_plan_download": (c_int, [c_vp, c_vp, c_vp, c_vp, c_u32, c_vp, c_u32]),
     "spc3d_plan_destroy": (c_int, [c_vp]),
     "spc3d_plan_set_values": (c_int, [c_vp, c_vp]),

@@ -846,6 +846,38 @@ int spc3d_plan_create_ex(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t nco
     return SPC3D_OK;
 }
 
+int spc3d_localize_device(spc3d_ctx *ctx, uint64_t n, void *dev_idx, void *dev_ltg,
+                          uint32_t *nlocal)
+{
+    if (!live(ctx) || !nlocal)
+        return fail(SPC3D_ERR_INVALID_ARG, "context or nlocal is NULL");
+    *nlocal = 0;
+    if (n && (!dev_idx || !dev_ltg))
+        return fail(SPC3D_ERR_INVALID_ARG, "index or map pointer is NULL");
+    int rc = use_device(ctx);
+    if (rc)
+        return rc;
+    std::string err;
+    rc = localize_device(ctx->stream, n, (uint32_t *)dev_idx, (uint32_t *)dev_ltg, nlocal, err);
+    return rc == SPC3D_OK ? rc : fail(rc, err);
+}
+
+int spc3d_remap_device(spc3d_ctx *ctx, uint64_t n, void *dev_idx, const void *dev_map,
+                       uint32_t map_len)
+{
+    if (!live(ctx))
+        return fail(SPC3D_ERR_INVALID_ARG, "context is NULL or destroyed");
+    if (n && (!dev_idx || (!dev_map && map_len)))
+        return fail(SPC3D_ERR_INVALID_ARG, "index or map pointer is NULL");
+    int rc = use_device(ctx);
+    if (rc)
+        return rc;
+    std::string err;
+    rc = remap_device(ctx->stream, n, (uint32_t *)dev_idx, (const uint32_t *)dev_map, map_len,
+                      err);
+    return rc == SPC3D_OK ? rc : fail(rc, err);
+}
+
 int spc3d_plan_download(spc3d_plan *plan, uint32_t *col, uint32_t *perm, uint32_t *segs,
                         uint32_t seg_cap, uint32_t *splits, uint32_t split_cap)
 {

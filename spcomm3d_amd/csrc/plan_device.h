@@ -30,4 +30,15 @@ int build_device_plan(hipStream_t stream, uint32_t nrows, uint32_t ncols, uint64
                       const uint32_t *d_ii, const uint32_t *d_jj, const PlanOpts &opts,
                       HostPlan &meta, DevPlanArrays &out, std::string &err);
 
+// COOMatrix::localizeIndices (src/SparseMatrix.hpp:69-99) on one device array of n
+// indices: every distinct value gets the next local id the first time it
+// appears, d_idx[e] becomes its local id, d_ltg[local] (capacity n) the value.
+int localize_device(hipStream_t stream, uint64_t n, uint32_t *d_idx, uint32_t *d_ltg,
+                    uint32_t *nlocal, std::string &err);
+
+// COOMatrix::ReMapIndices (src/SparseMatrix.hpp:100-106): d_idx[e] = d_map[d_idx[e]];
+// an index >= map_len is SPC3D_ERR_BAD_INDEX and nothing is changed.
+int remap_device(hipStream_t stream, uint64_t n, uint32_t *d_idx, const uint32_t *d_map,
+                 uint32_t map_len, std::string &err);
+
 } // namespace spc3d

@@ -438,6 +438,60 @@ __global__ void scatter_segs_k(const Seg *__restrict__ pseg, const uint32_t *__r
     }
 }
 
+// ---- localizeIndices / ReMapIndices on the device -----------------------------
+// head[i] = 1 where a run of equal sorted keys starts (i == n: 0, the scan's total slot)
+__global__ void heads_k(const uint32_t *__restrict__ key, uint64_t n, uint32_t *head)
+{
+    GRID_STRIDE(i, n + 1) head[i] = (i < n && (i == 0 || key[i] != key[i - 1])) ? 1u : 0u;
+}
+
+// For every run: the position at which its value first appears in the caller's
+// array (the sort is stable, so the head of the run holds it) and the value.
+__global__ void run_firsts_k(const uint32_t *__restrict__ key, const uint32_t *__restrict__ pos,
+                             const uint32_t *__restrict__ head,
+                             const uint32_t *__restrict__ run_of, uint64_t n, uint32_t *first_pos,
+                             uint32_t *run_key)
+{
+    GRID_STRIDE(i, n)
+    if (head[i]) {
+        first_pos[run_of[i]] = pos[i];
+        run_key[run_of[i]] = key[i];
+    }
+}
+
+// Runs in order of first appearance: the r-th gets local id r.
+__global__ void run_ranks_k(const uint32_t *__restrict__ run_order,
+                            const uint32_t *__restrict__ run_key, uint64_t nruns,
+                            uint32_t *rank_of, uint32_t *ltg)
+{
+    GRID_STRIDE(r, nruns)
+    {
+        rank_of[run_order[r]] = (uint32_t)r;
+        ltg[r] = run_key[run_order[r]];
+    }
+}
+
+__global__ void write_local_k(const uint32_t *__restrict__ pos, const uint32_t *__restrict__ head,
+                              const uint32_t *__restrict__ run_of,
+                              const uint32_t *__restrict__ rank_of, uint64_t n, uint32_t *idx)
+{
+    // run_of[] is the exclusive scan of head[]: inside a run it already counts the head
+    GRID_STRIDE(i, n) idx[pos[i]] = rank_of[run_of[i] + head[i] - 1];
+}
+
+__global__ void remap_check_k(const uint32_t *__restrict__ idx, uint64_t n, uint32_t map_len,
+                              Counters *C)
+{
+    GRID_STRIDE(e, n)
+    if (idx[e] >= map_len)
+        atomicMin(&C->first_bad, (uint32_t)e);
+}
+
+__global__ void remap_apply_k(uint32_t *idx, uint64_t n, const uint32_t *__restrict__ map)
+{
+    GRID_STRIDE(e, n) idx[e] = map[idx[e]];
+}
+
 #define HIP_OK(expr)                                                                              \
     do {                                                                                          \
         const hipError_t e_ = (expr);                                                             \
@@ -787,6 +841,79 @@ int build_device_plan(hipStream_t st, uint32_t nrows, uint32_t ncols, uint64_t n
     out.splits = splits.release();
     out.nsplit = nsplit;
     meta = std::move(P);
+    return SPC3D_OK;
+}
+
+int localize_device(hipStream_t st, uint64_t n, uint32_t *d_idx, uint32_t *d_ltg,
+                    uint32_t *nlocal, std::string &err)
+{
+    *nlocal = 0;
+    if (n == 0)
+        return SPC3D_OK;
+    if (n >= (1ull << 32)) {
+        err = "more than 2^32 - 1 indices are not supported";
+        return SPC3D_ERR_TOO_LARGE;
+    }
+    Temp tmp;
+    DBuf<uint32_t> ident, key, pos, head, run_of;
+    HIP_OK(ident.alloc(n));
+    HIP_OK(key.alloc(n));
+    HIP_OK(pos.alloc(n));
+    HIP_OK(head.alloc(n + 1));
+    HIP_OK(run_of.alloc(n + 1));
+    LAUNCH(iota_k, n, ident.p, n);
+    TRY(sort_pairs<uint32_t>(tmp, d_idx, key.p, ident.p, pos.p, (uint32_t)n, 32, false, st, err));
+    LAUNCH(heads_k, n + 1, key.p, n, head.p);
+    TRY(exclusive_sum(tmp, head.p, run_of.p, (size_t)n + 1, st, err));
+    uint32_t nruns = 0;
+    TRY(fetch(st, &nruns, run_of.p + n, sizeof nruns, err));
+
+    DBuf<uint32_t> first_pos, run_key, first_sorted, run_order, rank_of;
+    HIP_OK(first_pos.alloc(nruns));
+    HIP_OK(run_key.alloc(nruns));
+    HIP_OK(first_sorted.alloc(nruns));
+    HIP_OK(run_order.alloc(nruns));
+    HIP_OK(rank_of.alloc(nruns));
+    // run_of[i] of a head is its run's index; of the other members it is one more
+    LAUNCH(run_firsts_k, n, key.p, pos.p, head.p, run_of.p, n, first_pos.p, run_key.p);
+    LAUNCH(iota_k, nruns, ident.p, (uint64_t)nruns);
+    TRY(sort_pairs<uint32_t>(tmp, first_pos.p, first_sorted.p, ident.p, run_order.p, nruns,
+                             bits_for(n - 1), false, st, err));
+    LAUNCH(run_ranks_k, nruns, run_order.p, run_key.p, (uint64_t)nruns, rank_of.p, d_ltg);
+    LAUNCH(write_local_k, n, pos.p, head.p, run_of.p, rank_of.p, n, d_idx);
+    HIP_OK(hipGetLastError());
+    HIP_OK(hipStreamSynchronize(st));
+    *nlocal = nruns;
+    return SPC3D_OK;
+}
+
+int remap_device(hipStream_t st, uint64_t n, uint32_t *d_idx, const uint32_t *d_map,
+                 uint32_t map_len, std::string &err)
+{
+    if (n == 0)
+        return SPC3D_OK;
+    if (n >= (1ull << 32)) {
+        err = "more than 2^32 - 1 indices are not supported";
+        return SPC3D_ERR_TOO_LARGE;
+    }
+    DBuf<Counters> dC;
+    Counters hC;
+    HIP_OK(dC.alloc(1));
+    HIP_OK(hipMemsetAsync(dC.p, 0xFF, sizeof(Counters), st));
+    LAUNCH(remap_check_k, n, d_idx, n, map_len, dC.p);
+    TRY(fetch(st, &hC, dC.p, sizeof hC, err));
+    if (hC.first_bad != 0xFFFFFFFFu) {
+        uint32_t v = 0;
+        TRY(fetch(st, &v, d_idx + hC.first_bad, sizeof v, err));
+        char buf[128];
+        std::snprintf(buf, sizeof buf, "index %llu = %u is outside the map of %u entries",
+                      (unsigned long long)hC.first_bad, v, map_len);
+        err = buf;
+        return SPC3D_ERR_BAD_INDEX;
+    }
+    LAUNCH(remap_apply_k, n, d_idx, n, d_map);
+    HIP_OK(hipGetLastError());
+    HIP_OK(hipStreamSynchronize(st));
     return SPC3D_OK;
 }
 

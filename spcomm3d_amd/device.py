@@ -383,6 +383,25 @@ class RowMap:
             pass
 
 
+def localize_device(ctx: Context, idx: Vals, n: int) -> tuple[int, Vals]:
+    """``COOMatrix::localizeIndices`` (``src/SparseMatrix.hpp:69-99``) for one index
+    array held as the first ``n`` 32-bit words of ``idx``: rewrites it to local ids
+    in order of first appearance; returns their number and the local -> global map
+    (a value vector of ``n`` words, the first ``nlocal`` of which are used)."""
+    ltg = Vals(ctx, max(int(n), 1), np.float32)
+    nlocal = ctypes.c_uint32()
+    check(ctx._lib.spc3d_localize_device(ctx._h, int(n), idx.device_ptr(), ltg.device_ptr(),
+                                         ctypes.byref(nlocal)), "spc3d_localize_device")
+    return int(nlocal.value), ltg
+
+
+def remap_device(ctx: Context, idx: Vals, n: int, mapping: Vals, map_len: int) -> None:
+    """``COOMatrix::ReMapIndices`` (``src/SparseMatrix.hpp:100-106``):
+    ``idx[e] = mapping[idx[e]]`` on the device."""
+    check(ctx._lib.spc3d_remap_device(ctx._h, int(n), idx.device_ptr(), mapping.device_ptr(),
+                                      int(map_len)), "spc3d_remap_device")
+
+
 def coo_validate(nrows: int, ncols: int, ii, jj) -> None:
     """Host-only bounds check of a pattern; raises :class:`BadIndexError`."""
     ii = _as_idx(ii, "ii")

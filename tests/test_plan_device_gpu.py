@@ -3,6 +3,7 @@ plan built by the host builder: the same arrays bit for bit (index work, so no
 tolerance), for every layout the host builder produces.  The host builder
 itself is checked without a GPU in test_capi_host.py."""
 import ctypes
+import os
 
 import numpy as np
 import pytest
@@ -12,6 +13,8 @@ from spcomm3d_amd import device
 from spcomm3d_amd import workloads as W
 
 pytestmark = pytest.mark.gpu
+GOLDEN_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden",
+                           "core_ops_golden.npz")
 
 INFO_FIELDS = [name for name, _ in capi.PlanInfo._fields_ if name != "reserved"]
 
@@ -137,6 +140,55 @@ def test_pattern_already_on_the_device(ctx):
     assert np.array_equal(c1.download(), c2.download())
     for h in (S, H, dA, dB, c1, c2, dii, djj):
         h.close()
+
+
+def _words(ctx, a):
+    v = ctx.vals(max(a.size, 1), np.float32)
+    if a.size:
+        v.upload(np.ascontiguousarray(a, dtype=np.uint32).view(np.float32))
+    return v
+
+
+def _first_appearance(a):
+    ids, ltg, out = {}, [], np.empty(a.size, dtype=np.uint32)
+    for e, g in enumerate(a.tolist()):  # src/SparseMatrix.hpp:69-99, one array
+        if g not in ids:
+            ids[g] = len(ltg)
+            ltg.append(g)
+        out[e] = ids[g]
+    return out, np.array(ltg, dtype=np.uint32)
+
+
+def test_localize_on_device_matches_the_reference_vectors(ctx):
+    # tests/golden: the reference's own localizeIndices on an 80-entry pattern
+    g = np.load(GOLDEN_PATH)
+    for glob, loc, ltg in (("localize.gi", "localize.li", "localize.ltgR"),
+                           ("localize.gj", "localize.lj", "localize.ltgC")):
+        d = _words(ctx, g[glob])
+        nlocal, dl = device.localize_device(ctx, d, g[glob].size)
+        assert nlocal == g[ltg].size
+        assert np.array_equal(d.download().view(np.uint32)[:g[glob].size], g[loc])
+        assert np.array_equal(dl.download().view(np.uint32)[:nlocal], g[ltg])
+
+
+@pytest.mark.parametrize("n,span", [(1, 5), (1000, 50), (100000, 2 ** 32 - 1), (300000, 70000)])
+def test_localize_and_remap_on_device_random(ctx, n, span):
+    rng = np.random.default_rng(n)
+    a = rng.integers(0, span, n, dtype=np.uint64).astype(np.uint32)
+    want, ltg = _first_appearance(a)
+    d = _words(ctx, a)
+    nlocal, dl = device.localize_device(ctx, d, n)
+    assert nlocal == ltg.size
+    assert np.array_equal(d.download().view(np.uint32)[:n], want)
+    assert np.array_equal(dl.download().view(np.uint32)[:nlocal], ltg)
+    # ReMapIndices with the inverse map gives the global ids back
+    device.remap_device(ctx, d, n, dl, nlocal)
+    assert np.array_equal(d.download().view(np.uint32)[:n], a)
+    # an index outside the map is refused and nothing changes
+    if nlocal > 1:
+        with pytest.raises(capi.BadIndexError):
+            device.remap_device(ctx, d, n, dl, int(a.max()))
+        assert np.array_equal(d.download().view(np.uint32)[:n], a)
 
 
 def test_download_refuses_short_buffers(ctx):
