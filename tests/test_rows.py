@@ -3,6 +3,7 @@
 src/comm.hpp:90-103,166-189): oracle pinned on the CPU, HIP kernels checked
 against it bit for bit on the GPU (they only move and add in a fixed order)."""
 import ctypes
+import os
 
 import numpy as np
 import pytest
@@ -63,6 +64,57 @@ def test_oracle_rows_against_numpy(dtype):
     assert p[0, 0] == dtype(0)  # (0 + 1 + big) - big == 0 because 1 is absorbed
     with pytest.raises(IndexError):
         oracle_rows(0, P, np.array([40], np.uint32), buf[:1])
+
+
+GOLDEN = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden",
+                              "rows_golden.npz"))
+REF_ROWS = os.path.join(oracle.ORACLE_DIR, "_ref", "libref_rows.so")
+
+
+@pytest.mark.parametrize("name", ["k1", "k6", "k64"])
+def test_oracle_rows_against_the_reference_vectors(name):
+    # tests/golden/rows_golden.npz: the reference's own SparseComm copies (src/comm.hpp:90-103,
+    # 166-189) on seeded inputs with repeated rows; bit for bit
+    g = {k: GOLDEN[f"{name}.{k}"] for k in ("P", "rows", "buf", "packed", "unpacked", "summed")}
+    assert np.array_equal(oracle_rows(0, g["P"], g["rows"], g["buf"])[1], g["packed"])
+    assert np.array_equal(oracle_rows(1, g["P"], g["rows"], g["buf"])[0], g["unpacked"])
+    assert np.array_equal(oracle_rows(2, g["P"], g["rows"], g["buf"])[0], g["summed"])
+
+
+@pytest.mark.skipif(not os.path.exists(REF_ROWS),
+                    reason="oracle/_ref is only built where the reference is mounted")
+@pytest.mark.parametrize("seed", [1, 2])
+def test_oracle_rows_bit_exact_vs_live_reference_build(seed):
+    lib = ctypes.CDLL(REF_ROWS)
+    lib.ref_rows_f64.restype = ctypes.c_int
+    lib.ref_rows_f64.argtypes = [ctypes.c_int, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_void_p,
+                                 ctypes.c_uint64, ctypes.c_void_p, ctypes.c_void_p]
+    P, rows, buf = case(seed, 200, 17, 900, np.float64)
+    vp = lambda a: a.ctypes.data_as(ctypes.c_void_p)  # noqa: E731
+    for op in (0, 1, 2):
+        p, b = P.copy(), buf.copy()
+        assert lib.ref_rows_f64(op, 200, 17, vp(p), rows.size, vp(rows), vp(b)) == 0
+        op_, ob = oracle_rows(op, P, rows, buf)
+        assert np.array_equal(op_, p) and np.array_equal(ob, b)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["k1", "k6", "k64"])
+def test_rows_kernels_match_the_reference_vectors(ctx, name):
+    from spcomm3d_amd import device
+
+    g = {k: GOLDEN[f"{name}.{k}"] for k in ("P", "rows", "buf", "packed", "unpacked", "summed")}
+    k = g["P"].shape[1]
+    rm = device.RowMap(ctx, g["P"].shape[0], g["rows"])
+    dP, dB = ctx.panel_from(g["P"]), ctx.vals(g["rows"].size * k, np.float64)
+    rm.pack(dP, dB)
+    assert np.array_equal(dB.download().reshape(-1, k), g["packed"])
+    dB.upload(g["buf"].ravel())
+    rm.unpack(dP, dB)
+    assert np.array_equal(dP.download(), g["unpacked"])
+    dP.upload(g["P"])
+    rm.unpack_sum(dP, dB)
+    assert np.array_equal(dP.download(), g["summed"])
 
 
 def test_rowmap_validation_needs_no_gpu():
