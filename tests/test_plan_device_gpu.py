@@ -110,6 +110,30 @@ def test_uniform_and_banded_patterns_stay_unsliced(ctx):
     both(ctx, w.nrows, w.ncols, w.ii, w.jj)
 
 
+def test_random_patterns_and_options_differential(ctx):
+    # many small skewed patterns under random tuning: every layout decision of the two
+    # builders (slicing on/off, hub rows, cut rows, dealing, padding) must coincide
+    rng = np.random.default_rng(2024)
+    sliced = 0
+    for _ in range(60):
+        m, n = int(rng.integers(1, 400)), int(rng.integers(40, 400))
+        nnz = int(rng.integers(1, 6000))
+        # Zipf-like rows and columns so that hubs and hot columns exist
+        ii = np.minimum((rng.pareto(0.7, nnz)).astype(np.int64), m - 1).astype(np.uint32)
+        jj = np.minimum((rng.pareto(0.5, nnz) * 3).astype(np.int64), n - 1).astype(np.uint32)
+        if rng.random() < 0.5:
+            o = np.lexsort((jj, ii))
+            ii, jj = ii[o], jj[o]
+        opts = dict(seg_max=int(rng.choice([1, 3, 16, 64, 500])),
+                    hub_min=int(rng.choice([1, 2, 8, 32, 128])),
+                    l2_hot_bytes=int(rng.choice([64, 256, 1024, 4096])),
+                    k_hint=int(rng.choice([1, 16, 64])),
+                    xcd_slices=int(rng.choice([0, 8, 8, 1])))
+        P = both(ctx, m, n, ii, jj, **opts)
+        sliced += P["info"].nqueues == 8
+    assert sliced >= 10  # the sliced layout was exercised, not only the plain one
+
+
 def test_bad_index_is_reported_as_by_the_host_check(ctx):
     ii = np.array([0, 1, 1, 9, 1], dtype=np.uint32)
     jj = np.array([0, 1, 5, 0, 7], dtype=np.uint32)
