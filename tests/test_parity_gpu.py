@@ -135,6 +135,42 @@ def test_cut_rows_with_ragged_k(ctx, dtype, k):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_random_shapes_widths_and_plan_options(ctx, dtype):
+    # every knob at once: skewed patterns, sorted or not, exact / ragged / generic row widths,
+    # cut rows, the sliced layout on small inputs, both plan builders
+    rng = np.random.default_rng(99)
+    for case in range(40):
+        m, n = int(rng.integers(1, 300)), int(rng.integers(40, 300))
+        nnz = int(rng.integers(1, 5000))
+        k = int(rng.choice([1, 2, 4, 5, 8, 12, 16, 24, 32, 40, 64, 68, 96, 128, 160, 256, 516]))
+        ii = np.minimum(rng.pareto(0.7, nnz).astype(np.int64), m - 1).astype(np.uint32)
+        jj = np.minimum((rng.pareto(0.5, nnz) * 3).astype(np.int64), n - 1).astype(np.uint32)
+        if rng.random() < 0.5:
+            o = np.lexsort((jj, ii))
+            ii, jj = np.ascontiguousarray(ii[o]), np.ascontiguousarray(jj[o])
+        vv = rng.uniform(-1, 1, nnz).astype(dtype)
+        A = rng.uniform(-1, 1, (m, k)).astype(dtype)
+        B = rng.uniform(-1, 1, (n, k)).astype(dtype)
+        Y0 = rng.uniform(-1, 1, (m, k)).astype(dtype)
+        opts = dict(seg_max=int(rng.choice([1, 5, 16, 64, 500])),
+                    hub_min=int(rng.choice([1, 8, 32, 128])),
+                    l2_hot_bytes=int(rng.choice([64, 256, 4096])), k_hint=k,
+                    xcd_slices=int(rng.choice([0, 8, 1])),
+                    builder=str(rng.choice(["device", "host"])))
+        S = ctx.plan(m, n, ii, jj, vv, **opts)
+        dA, dB, dY, dC = ctx.panel_from(A), ctx.panel_from(B), ctx.panel_from(Y0), ctx.vals(nnz, dtype)
+        ctx.sddmm(S, dA, dB, dC)
+        ctx.spmm(S, dB, dY)
+        try:
+            check_sddmm(A, B, ii, jj, vv, dC.download())
+            check_spmm(B, ii, jj, vv, Y0, dY.download())
+        except AssertionError as e:
+            raise AssertionError(f"case {case}: m={m} n={n} nnz={nnz} k={k} {opts}: {e}") from None
+        for h in (S, dA, dB, dY, dC):
+            h.close()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("k", [64, 20])
 def test_rows_the_pattern_never_names_are_never_read(ctx, dtype, k):
     # the reference touches A[ii[e]], B[jj[e]] and Y[ii[e]] only (core_ops.cpp:16,32): NaN
