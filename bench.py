@@ -14,7 +14,9 @@ launch over its mean launch time, measured with HIP events on the library's
 stream inside the timed region, against 8 TB/s.  `cpu_baseline` is the
 reference's own kernels (where their build is present, fp64) or else the CPU
 oracle (a serial restatement of the reference's loops), timed on one host core
-on the same workload.
+on the same workload.  `fused_step` is the same step through the one-pass entry
+point spc3d_sddmm_spmm (an extension without counterpart in the reference); it is
+reported beside `value`, which always comes from the two separate calls.
 """
 from __future__ import annotations
 
@@ -108,6 +110,16 @@ def run_gpu(w, dtype, steps, warmup, seg_max=None, max_timed=1300, copies=0):
         wall = time.perf_counter() - t0
         sd = np.array([ctx.elapsed_ms(3 * i, 3 * i + 1) for i in range(ntimed)])
         sp = np.array([ctx.elapsed_ms(3 * i + 1, 3 * i + 2) for i in range(ntimed)])
+        # The same step through the fused entry point (both results from one pass over
+        # the gathered rows); reported beside the headline, never as it.
+        for _ in range(warmup):
+            ctx.sddmm_spmm(S, dA, dB, dC, dY)
+        ctx.sync()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            ctx.sddmm_spmm(S, dA, dB, dC, dY)
+        ctx.sync()
+        fused_wall = time.perf_counter() - t0
         for h in (S, dA, dB, dY, dC):
             h.close()
 
@@ -118,6 +130,10 @@ def run_gpu(w, dtype, steps, warmup, seg_max=None, max_timed=1300, copies=0):
            "upload_s": upload_s, "nsegments": info.nsegments, "nsplit_rows": info.nsplit_rows,
            "seg_max": info.seg_max, "rows_touched": m_t, "cols_touched": n_t,
            "gflops": 2 * fl / (wall / steps) / 1e9, "kernels": {}}
+    fb = roofline.fused_bytes(w.nrows, w.nnz, w.k, wbytes, m_t, n_t, with_perm)
+    out["fused_step"] = {"entry": "spc3d_sddmm_spmm", "ms_per_step": fused_wall / steps * 1e3,
+                         "gflops": 2 * fl / (fused_wall / steps) / 1e9, "strict_bytes": int(fb),
+                         "strict_frac": fb / (fused_wall / steps) / 1e9 / roofline.HBM_PEAK_GBS}
     for name, ms, strict, gather in (
             ("sddmm", sd,
              roofline.sddmm_bytes(w.nrows, w.nnz, w.k, wbytes, m_t, n_t, with_perm),
@@ -275,6 +291,7 @@ def main():
                      "ms_per_launch": kd["ms_avg"], "model": "strict (each operand once)"},
         "cpu_baseline": cpu,
         "kernels": main_r["kernels"],
+        "fused_step": main_r["fused_step"],
         "plan": {k: main_r[k] for k in ("plan_build_s", "upload_s", "nsegments", "nsplit_rows",
                                         "seg_max")},
         "also": also,

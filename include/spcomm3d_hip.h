@@ -235,6 +235,22 @@ SPC3D_API int spc3d_plan_get_info(const spc3d_plan *plan, spc3d_plan_info *info)
 SPC3D_API int spc3d_sddmm(spc3d_ctx *ctx, spc3d_plan *S, const spc3d_panel *A,
                 const spc3d_panel *B, spc3d_vals *C);
 SPC3D_API int spc3d_spmm(spc3d_ctx *ctx, spc3d_plan *A, const spc3d_panel *X, spc3d_panel *Y);
+/* Both kernels over one pattern and one dense operand B in a single pass, so that
+ * each gathered row of B is used twice: C as spc3d_sddmm(ctx, S, A, B, C), and
+ *   chained == 0:  Y += S B, as spc3d_spmm(ctx, S, B, Y) with S's own values;
+ *   chained != 0:  Y += C B, the SpMM whose sparse values are the SDDMM result
+ *                  just computed (what calling spc3d_plan_set_values_device(S, C)
+ *                  and spc3d_spmm(ctx, S, B, Y) afterwards would give, without
+ *                  changing the plan's values).
+ * Same results as the separate calls within the summation-order tolerance;
+ * requires A.n == B.n == Y.n, Y.m >= nrows, Y aliasing neither A nor B.  The
+ * chained form needs K * sizeof(real) to be a multiple of 16 bytes up to 4096
+ * (SPC3D_ERR_INVALID_ARG otherwise); the other falls back to the two calls.
+ * Has no counterpart in the reference, which runs its two kernels in separate
+ * passes (miniapp/bench_both.cpp:202-203; miniapp/bench_spmm.cpp:185-186).
+ * Asynchronous on the context's stream. */
+SPC3D_API int spc3d_sddmm_spmm(spc3d_ctx *ctx, spc3d_plan *S, const spc3d_panel *A,
+                     const spc3d_panel *B, spc3d_vals *C, spc3d_panel *Y, int chained);
 
 /* ---- the copies either side of a sparse exchange ---------------------------
  * A row map ties buffer slot i to dense row rows[i] of a panel: the device form

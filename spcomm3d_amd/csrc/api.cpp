@@ -1013,6 +1013,23 @@ int spc3d_plan_get_info(const spc3d_plan *plan, spc3d_plan_info *info)
     return SPC3D_OK;
 }
 
+// Partial-sum rows of cut rows; sized on first use for this K.
+static int ensure_partial(spc3d_plan *p, uint32_t K)
+{
+    if (!p->info.npartial_slots || p->partial_k >= K)
+        return SPC3D_OK;
+    HIP_TRY(hipStreamSynchronize(p->ctx->stream));
+    if (p->partial)
+        (void)hipFree(p->partial);
+    p->partial = nullptr;
+    p->partial_k = 0;
+    int rc = dev_alloc_bytes(&p->partial, (size_t)p->info.npartial_slots * K * elem_size(p->dtype));
+    if (rc)
+        return rc;
+    p->partial_k = K;
+    return SPC3D_OK;
+}
+
 /* ---- hot path ------------------------------------------------------------ */
 int spc3d_sddmm(spc3d_ctx *ctx, spc3d_plan *S, const spc3d_panel *A, const spc3d_panel *B,
                 spc3d_vals *C)
@@ -1070,20 +1087,60 @@ int spc3d_spmm(spc3d_ctx *ctx, spc3d_plan *Ap, const spc3d_panel *X, spc3d_panel
     int rc = use_device(ctx);
     if (rc)
         return rc;
-    if (Ap->info.npartial_slots && Ap->partial_k < K) {
-        // Partial-sum rows of cut rows; sized on first use for this K.
-        HIP_TRY(hipStreamSynchronize(ctx->stream));
-        if (Ap->partial)
-            (void)hipFree(Ap->partial);
-        Ap->partial = nullptr;
-        Ap->partial_k = 0;
-        rc = dev_alloc_bytes(&Ap->partial,
-                             (size_t)Ap->info.npartial_slots * K * elem_size(Ap->dtype));
-        if (rc)
-            return rc;
-        Ap->partial_k = K;
-    }
+    rc = ensure_partial(Ap, K);
+    if (rc)
+        return rc;
     HIP_TRY(launch_spmm(Ap->dtype, view_of(Ap), X->dev, Y->dev, K, streams_of(ctx)));
+    return SPC3D_OK;
+}
+
+int spc3d_sddmm_spmm(spc3d_ctx *ctx, spc3d_plan *S, const spc3d_panel *A, const spc3d_panel *B,
+                     spc3d_vals *C, spc3d_panel *Y, int chained)
+{
+    if (!live(ctx) || !live(S) || !live(A) || !live(B) || !live(C) || !live(Y))
+        return fail(SPC3D_ERR_INVALID_ARG, "a handle is NULL or destroyed");
+    if (S->ctx != ctx || A->ctx != ctx || B->ctx != ctx || C->ctx != ctx || Y->ctx != ctx)
+        return fail(SPC3D_ERR_INVALID_ARG, "operands belong to different contexts");
+    if (A->dtype != S->dtype || B->dtype != S->dtype || C->dtype != S->dtype ||
+        Y->dtype != S->dtype)
+        return fail(SPC3D_ERR_SIZE_MISMATCH, "operand dtypes differ from the plan's");
+    const uint32_t K = A->n;
+    if (B->n != K || Y->n != K)
+        return fail(SPC3D_ERR_SIZE_MISMATCH, "A.n, B.n and Y.n differ");
+    if (S->info.nnz == 0)
+        return SPC3D_OK;
+    if (A->m < S->info.nrows || B->m < S->info.ncols || Y->m < S->info.nrows)
+        return fail(SPC3D_ERR_SIZE_MISMATCH, "panel has fewer rows than the pattern addresses");
+    if (C->n < S->info.nnz)
+        return fail(SPC3D_ERR_SIZE_MISMATCH, "C.vv is shorter than nnz");
+    if (Y->dev == A->dev || Y->dev == B->dev)
+        return fail(SPC3D_ERR_INVALID_ARG, "Y must not alias A or B");
+    if (!S->has_values)
+        return fail(SPC3D_ERR_INVALID_ARG, "plan has no values (spc3d_plan_set_values)");
+    int rc = use_device(ctx);
+    if (rc)
+        return rc;
+    if (K == 0) { // empty dot products, nothing to add
+        HIP_TRY(launch_fill(C->dtype, C->dev, S->info.nnz, 0.0, ctx->stream));
+        return SPC3D_OK;
+    }
+    rc = ensure_partial(S, K);
+    if (rc)
+        return rc;
+    hipError_t e = launch_sddmm_spmm(S->dtype, chained != 0, view_of(S), A->dev, B->dev, C->dev,
+                                     Y->dev, K, streams_of(ctx));
+    if (e == hipErrorNotSupported) {
+        (void)hipGetLastError();
+        if (chained)
+            return fail(SPC3D_ERR_INVALID_ARG,
+                        "the chained form needs K * sizeof(real) to be a multiple of 16 bytes, "
+                        "at most 4096");
+        // No vector kernel for this K: the two calls one after the other.
+        HIP_TRY(launch_sddmm(S->dtype, view_of(S), A->dev, B->dev, C->dev, K, streams_of(ctx)));
+        HIP_TRY(launch_spmm(S->dtype, view_of(S), B->dev, Y->dev, K, streams_of(ctx)));
+        return SPC3D_OK;
+    }
+    HIP_TRY(e);
     return SPC3D_OK;
 }
 

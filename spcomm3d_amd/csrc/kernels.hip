@@ -154,6 +154,16 @@ template <int LPR, int NB> __device__ __forceinline__ bool is_writer(uint32_t su
     return (sub & mask) == 0;
 }
 
+// Lane (within the group) that stores entry u after group_reduce<LPR, NB>.
+template <int LPR, int NB> __device__ __forceinline__ constexpr int writer_lane(int u)
+{
+    int lane = 0;
+    for (int t = 0; t < ilog2(NB); ++t)
+        if ((u >> (ilog2(NB) - 1 - t)) & 1)
+            lane |= Strides<LPR>::s[t];
+    return lane;
+}
+
 // Segment this lane group works on.  Segments are stored in chunks of kChunk;
 // with nq == 8, chunk v belongs to queue v % 8.  The hardware deals the
 // workgroups of a dispatch to the 8 XCDs round-robin by workgroup id, starting
@@ -208,12 +218,17 @@ __device__ __forceinline__ bool lane_on(uint32_t sub, int v, uint32_t nvec)
 // exist; the others repeat entry n - 1 (loads without branches, from addresses
 // that are being read anyway) and store nothing, so that a tail of any length
 // costs one round of gathers.
-template <typename T, int LPR, int VPL, int NB, bool RG, bool MK>
+//
+// FZ ("fused"): the gathered B rows also feed the SpMM of the same pattern,
+// acc += w_u * B[c_u,:] in kernel order, with w_u = S.vv (FZ == 1) or the SDDMM
+// result just computed (FZ == 2); the weight of entry u is broadcast from the lane
+// that stores it.
+template <typename T, int LPR, int VPL, int NB, bool RG, bool MK, int FZ>
 __device__ __forceinline__ void
-sddmm_batch(const typename Vec<T>::type (&a)[VPL], const uint32_t *__restrict__ col,
-            const uint32_t *__restrict__ perm, const T *__restrict__ sval,
-            const T *__restrict__ B, T *__restrict__ C, uint32_t p0, uint32_t n, uint32_t sub,
-            uint32_t nvec)
+sddmm_batch(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type (&acc)[VPL],
+            const uint32_t *__restrict__ col, const uint32_t *__restrict__ perm,
+            const T *__restrict__ sval, const T *__restrict__ B, T *__restrict__ C, uint32_t p0,
+            uint32_t n, uint32_t sub, uint32_t nvec)
 {
     using V = typename Vec<T>::type;
     static_assert(NB <= LPR, "batch must fit the lane group");
@@ -248,72 +263,85 @@ sddmm_batch(const typename Vec<T>::type (&a)[VPL], const uint32_t *__restrict__ 
     T part[NB];
 #pragma unroll
     for (int u = 0; u < NB; ++u) {
-        T acc = (T)0;
+        T dot = (T)0;
 #pragma unroll
         for (int v = 0; v < VPL; ++v)
 #pragma unroll
             for (int i = 0; i < Vec<T>::N; ++i)
-                acc += a[v][i] * b[u][v][i];
-        part[u] = acc;
+                dot += a[v][i] * b[u][v][i];
+        part[u] = dot;
     }
     group_reduce<T, LPR, NB>(part, sub);
+    const T result = part[0] * sv;
     // Results in the caller's order: when that is the kernel order the stores of a
     // batch fill whole lines and stream out; when it is not they are scattered, and
     // plain stores let the L2 merge neighbours into lines before writing back.
     if (writer) {
         if (perm)
-            C[dst] = part[0] * sv;
+            C[dst] = result;
         else
-            nt_store(part[0] * sv, C + dst);
+            nt_store(result, C + dst);
+    }
+    if constexpr (FZ != 0) {
+        const T mine = FZ == 2 ? result : sv; // valid on the writer lanes
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+            const bool on = !MK || (uint32_t)u < n;
+            const T w = on ? __shfl(mine, writer_lane<LPR, NB>(u), LPR) : (T)0;
+#pragma unroll
+            for (int v = 0; v < VPL; ++v)
+                acc[v] += (on ? b[u][v] : V{}) * w;
+        }
     }
 }
 
 // n consecutive entries from p.  WIDE: full batches of UB, then one masked batch
 // of the smallest size in {4, 8, 16} that holds the rest.  !WIDE (segments known
 // to be short, run at twice the occupancy): masked batches of UB throughout.
-template <typename T, int LPR, int VPL, int UB, bool RG, bool WIDE>
+template <typename T, int LPR, int VPL, int UB, bool RG, bool WIDE, int FZ>
 __device__ __forceinline__ void
-sddmm_walk(const typename Vec<T>::type (&a)[VPL], const uint32_t *__restrict__ col,
-           const uint32_t *__restrict__ perm, const T *__restrict__ sval,
-           const T *__restrict__ B, T *__restrict__ C, uint32_t p, uint32_t n, uint32_t sub,
-           uint32_t nvec)
+sddmm_walk(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type (&acc)[VPL],
+           const uint32_t *__restrict__ col, const uint32_t *__restrict__ perm,
+           const T *__restrict__ sval, const T *__restrict__ B, T *__restrict__ C, uint32_t p,
+           uint32_t n, uint32_t sub, uint32_t nvec)
 {
     if constexpr (WIDE) {
         for (; n >= UB; n -= UB, p += UB)
-            sddmm_batch<T, LPR, VPL, UB, RG, false>(a, col, perm, sval, B, C, p, UB, sub, nvec);
+            sddmm_batch<T, LPR, VPL, UB, RG, false, FZ>(a, acc, col, perm, sval, B, C, p, UB, sub, nvec);
         if (n == 0)
             return;
         if constexpr (UB > 8) {
             if (n > 8) {
-                sddmm_batch<T, LPR, VPL, UB, RG, true>(a, col, perm, sval, B, C, p, n, sub, nvec);
+                sddmm_batch<T, LPR, VPL, UB, RG, true, FZ>(a, acc, col, perm, sval, B, C, p, n, sub, nvec);
                 return;
             }
         }
         if constexpr (UB > 4) {
             if (n > 4) {
-                sddmm_batch<T, LPR, VPL, 8, RG, true>(a, col, perm, sval, B, C, p, n, sub, nvec);
+                sddmm_batch<T, LPR, VPL, 8, RG, true, FZ>(a, acc, col, perm, sval, B, C, p, n, sub, nvec);
                 return;
             }
         }
-        sddmm_batch<T, LPR, VPL, (UB < 4 ? UB : 4), RG, true>(a, col, perm, sval, B, C, p, n, sub,
-                                                              nvec);
+        sddmm_batch<T, LPR, VPL, (UB < 4 ? UB : 4), RG, true, FZ>(a, acc, col, perm, sval, B, C, p, n, sub, nvec);
     } else {
 #pragma nounroll
         while (n > 0) {
             const uint32_t m = n < (uint32_t)UB ? n : (uint32_t)UB;
-            sddmm_batch<T, LPR, VPL, UB, RG, true>(a, col, perm, sval, B, C, p, m, sub, nvec);
+            sddmm_batch<T, LPR, VPL, UB, RG, true, FZ>(a, acc, col, perm, sval, B, C, p, m, sub, nvec);
             n -= m;
             p += m;
         }
     }
 }
 
-template <typename T, int LPR, int VPL, int UB, bool RG, bool WIDE>
+// FZ != 0: also Y[row,:] += sum of the segment's w_u * B[c_u,:] (partial-sum slot for
+// a cut row, as in spmm_seg_kernel); Y and partial are unused otherwise.
+template <typename T, int LPR, int VPL, int UB, bool RG, bool WIDE, int FZ>
 __global__ void __launch_bounds__(kBlock)
 sddmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint32_t rot,
                  const uint32_t *__restrict__ col, const uint32_t *__restrict__ perm,
                  const T *__restrict__ sval, const T *__restrict__ A, const T *__restrict__ B,
-                 T *__restrict__ C, uint32_t nvec)
+                 T *__restrict__ C, T *__restrict__ Y, T *__restrict__ partial, uint32_t nvec)
 {
     static_assert(UB <= LPR && UB <= 16 && LPR <= 64, "batch must fit the lane group");
     using V = typename Vec<T>::type;
@@ -325,14 +353,31 @@ sddmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint3
     if (sg[2] == 0)
         return;
 
-    V a[VPL];
+    V a[VPL], acc[VPL];
     {
         const V *arow = row_ptr<T, LPR, VPL, RG>(A, sg[0], sub, nvec);
 #pragma unroll
-        for (int v = 0; v < VPL; ++v)
+        for (int v = 0; v < VPL; ++v) {
             a[v] = lane_on<LPR, RG>(sub, v, nvec) ? nt_load(arow + v * LPR) : V{};
+            acc[v] = V{};
+        }
     }
-    sddmm_walk<T, LPR, VPL, UB, RG, WIDE>(a, col, perm, sval, B, C, sg[1], sg[2], sub, nvec);
+    sddmm_walk<T, LPR, VPL, UB, RG, WIDE, FZ>(a, acc, col, perm, sval, B, C, sg[1], sg[2], sub,
+                                              nvec);
+    if constexpr (FZ != 0) {
+        const bool whole = sg[3] == kWholeRow;
+        V *dst = const_cast<V *>(whole ? row_ptr<T, LPR, VPL, RG>(Y, sg[0], sub, nvec)
+                                       : row_ptr<T, LPR, VPL, RG>(partial, sg[3], sub, nvec));
+#pragma unroll
+        for (int v = 0; v < VPL; ++v) {
+            if (!lane_on<LPR, RG>(sub, v, nvec))
+                continue;
+            if (whole)
+                nt_store(nt_load(dst + v * LPR) + acc[v], dst + v * LPR);
+            else
+                dst[v * LPR] = acc[v]; // read back by spmm_fixup right after
+        }
+    }
 }
 
 // Any K: one wavefront per segment, lanes stride over K, scalar loads.
@@ -732,23 +777,23 @@ inline hipError_t join_aux(const Streams &S)
     return hipStreamSynchronize(S.aux);
 }
 
-template <typename T, int LPR, int VPL, int UB, int US, bool RG>
-hipError_t run_sddmm(const DevPlanView &P, const T *A, const T *B, T *C, const Streams &S,
+template <typename T, int LPR, int VPL, int UB, int US, bool RG, int FZ>
+hipError_t run_sddmm(const DevPlanView &P, const T *A, const T *B, T *C, T *Y, const Streams &S,
                      uint32_t nvec)
 {
     const uint32_t nl = P.nseg_long, ns = P.nseg - P.nseg_long;
     const bool both = nl && ns && fork_aux(S);
     if (nl)
-        hipLaunchKernelGGL((sddmm_seg_kernel<T, LPR, VPL, UB, RG, true>),
+        hipLaunchKernelGGL((sddmm_seg_kernel<T, LPR, VPL, UB, RG, true, FZ>),
                            dim3(blocks_for_groups(nl, P.nqueues, 64 / LPR)), dim3(kBlock), 0,
                            S.main, P.segs, nl, P.nqueues, 0u, P.col, P.perm, (const T *)P.sval,
-                           A, B, C, nvec);
+                           A, B, C, Y, (T *)P.partial, nvec);
     if (ns)
-        hipLaunchKernelGGL((sddmm_seg_kernel<T, LPR, VPL, US, RG, false>),
+        hipLaunchKernelGGL((sddmm_seg_kernel<T, LPR, VPL, US, RG, false, FZ>),
                            dim3(blocks_for_groups(ns, P.nqueues, 64 / LPR)), dim3(kBlock), 0,
                            both ? S.aux : S.main, P.segs + nl, ns, P.nqueues,
-                           both ? S.aux_rot : 0u, P.col, P.perm, (const T *)P.sval, A, B, C,
-                           nvec);
+                           both ? S.aux_rot : 0u, P.col, P.perm, (const T *)P.sval, A, B, C, Y,
+                           (T *)P.partial, nvec);
     const hipError_t launched = hipGetLastError();
     const hipError_t joined = both ? join_aux(S) : hipSuccess;
     return launched != hipSuccess ? launched : joined;
@@ -787,9 +832,28 @@ hipError_t run_spmm(const DevPlanView &P, const T *X, T *Y, const Streams &S, ui
     X(4, 1, 4, 4, 4) X(8, 1, 8, 8, 4) X(16, 1, 16, 8, 4) X(32, 1, 16, 8, 4) X(64, 1, 16, 8, 4)    \
     X(64, 2, 8, 4, 2) X(64, 4, 4, 2, 1)
 
+// Adds the partial sums of cut rows into Y (after the segment kernels of an SpMM or
+// a fused call).
 template <typename T>
-hipError_t sddmm_typed(const DevPlanView &P, const void *A, const void *B, void *C, uint32_t K,
-                       const Streams &SS)
+hipError_t launch_fixup(const DevPlanView &P, T *Y, uint32_t K, hipStream_t st)
+{
+    if (!P.nsplit)
+        return hipSuccess;
+    uint32_t lanes = 4;
+    while (lanes < (uint32_t)kBlock && lanes < K)
+        lanes *= 2;
+    const uint32_t rows_per_block = kBlock / lanes;
+    hipLaunchKernelGGL((spmm_fixup_kernel<T>),
+                       dim3((P.nsplit + rows_per_block - 1) / rows_per_block), dim3(kBlock), 0, st,
+                       P.splits, P.nsplit, (const T *)P.partial, Y, K, lanes);
+    return hipGetLastError();
+}
+
+// FZ == 0: SDDMM.  FZ == 1, 2: SDDMM fused with the SpMM of the same pattern over
+// the same B (vector kernels only: hipErrorNotSupported for other K).
+template <typename T, int FZ>
+hipError_t sddmm_typed(const DevPlanView &P, const void *A, const void *B, void *C, void *Y,
+                       uint32_t K, const Streams &SS)
 {
     const hipStream_t st = SS.main;
     if (P.nseg == 0)
@@ -799,26 +863,32 @@ hipError_t sddmm_typed(const DevPlanView &P, const void *A, const void *B, void 
     hipError_t e = hipSuccess;
 #define X(L, V, U, S, S2)                                                                         \
     if (!done && !sh.ragged && sh.lpr == L && sh.vpl == V) {                                      \
-        e = run_sddmm<T, L, V, U, S, false>(P, (const T *)A, (const T *)B, (T *)C, SS, sh.nvec);  \
+        e = run_sddmm<T, L, V, U, S, false, FZ>(P, (const T *)A, (const T *)B, (T *)C, (T *)Y,    \
+                                                SS, sh.nvec);                                     \
         done = true;                                                                              \
     }
     SPC3D_FOR_SHAPES(X)
 #undef X
 #define X(L, V, U, S, S2)                                                                         \
     if (!done && sh.ragged && sh.lpr == L && sh.vpl == V) {                                       \
-        e = run_sddmm<T, L, V, U, S, true>(P, (const T *)A, (const T *)B, (T *)C, SS, sh.nvec);   \
+        e = run_sddmm<T, L, V, U, S, true, FZ>(P, (const T *)A, (const T *)B, (T *)C, (T *)Y, SS, \
+                                               sh.nvec);                                          \
         done = true;                                                                              \
     }
     SPC3D_FOR_RAGGED_SHAPES(X)
 #undef X
     if (!done) {
+        if (FZ != 0)
+            return hipErrorNotSupported;
         const uint32_t grid = blocks_for_groups(P.nseg, P.nqueues, 1);
         hipLaunchKernelGGL((sddmm_generic_kernel<T>), dim3(grid), dim3(kBlock), 0, st, P.segs,
-                           P.nseg, P.nqueues, 0u, P.col, P.perm, (const T *)P.sval, (const T *)A, (const T *)B,
-                           (T *)C, K);
+                           P.nseg, P.nqueues, 0u, P.col, P.perm, (const T *)P.sval, (const T *)A,
+                           (const T *)B, (T *)C, K);
     }
     const hipError_t last = hipGetLastError();
-    return e != hipSuccess ? e : last;
+    if (e != hipSuccess || last != hipSuccess)
+        return e != hipSuccess ? e : last;
+    return FZ != 0 ? launch_fixup<T>(P, (T *)Y, K, st) : hipSuccess;
 }
 
 template <typename T>
@@ -855,17 +925,7 @@ hipError_t spmm_typed(const DevPlanView &P, const void *X_, void *Y, uint32_t K,
         e = hipGetLastError();
     if (e != hipSuccess)
         return e;
-    if (P.nsplit) {
-        uint32_t lanes = 4;
-        while (lanes < (uint32_t)kBlock && lanes < K)
-            lanes *= 2;
-        const uint32_t rows_per_block = kBlock / lanes;
-        hipLaunchKernelGGL((spmm_fixup_kernel<T>),
-                           dim3((P.nsplit + rows_per_block - 1) / rows_per_block), dim3(kBlock), 0,
-                           st, P.splits, P.nsplit, (const T *)P.partial, (T *)Y, K, lanes);
-        e = hipGetLastError();
-    }
-    return e;
+    return launch_fixup<T>(P, (T *)Y, K, st);
 }
 
 inline uint32_t stream_grid(uint64_t n)
@@ -880,8 +940,18 @@ inline uint32_t stream_grid(uint64_t n)
 hipError_t launch_sddmm(int dtype, const DevPlanView &P, const void *A, const void *B, void *C,
                         uint32_t K, const Streams &stream)
 {
-    return dtype == 1 ? sddmm_typed<double>(P, A, B, C, K, stream)
-                      : sddmm_typed<float>(P, A, B, C, K, stream);
+    return dtype == 1 ? sddmm_typed<double, 0>(P, A, B, C, nullptr, K, stream)
+                      : sddmm_typed<float, 0>(P, A, B, C, nullptr, K, stream);
+}
+
+hipError_t launch_sddmm_spmm(int dtype, int chained, const DevPlanView &P, const void *A,
+                             const void *B, void *C, void *Y, uint32_t K, const Streams &stream)
+{
+    if (dtype == 1)
+        return chained ? sddmm_typed<double, 2>(P, A, B, C, Y, K, stream)
+                       : sddmm_typed<double, 1>(P, A, B, C, Y, K, stream);
+    return chained ? sddmm_typed<float, 2>(P, A, B, C, Y, K, stream)
+                   : sddmm_typed<float, 1>(P, A, B, C, Y, K, stream);
 }
 
 hipError_t launch_spmm(int dtype, const DevPlanView &P, const void *X, void *Y, uint32_t K,

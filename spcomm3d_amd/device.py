@@ -109,6 +109,14 @@ class Context:
             opts["seg_max"] = seg_max
         return Plan(self, nrows, ncols, ii, jj, vv, dtype, opts or None)
 
+    def sddmm_spmm(self, S: "Plan", A: "Panel", B: "Panel", C: "Vals", Y: "Panel",
+                   chained: bool = False):
+        """SDDMM and the SpMM of the same pattern over ``B`` in one pass
+        (``spc3d_sddmm_spmm``): ``C`` as :meth:`sddmm`; ``Y += S B``, or ``Y += C B`` when
+        ``chained``."""
+        check(self._lib.spc3d_sddmm_spmm(self._h, S._h, A._h, B._h, C._h, Y._h, int(chained)),
+              "spc3d_sddmm_spmm")
+
     def probe_xcd(self, nblocks: int) -> np.ndarray:
         """XCD id each workgroup of an ``nblocks``-wide grid ran on (``spc3d_ctx_probe_xcd``)."""
         out = np.zeros(nblocks, dtype=np.uint32)

@@ -217,4 +217,14 @@ template <typename T> void spmm(Context &ctx, Plan<T> &A, const Panel<T> &X, Pan
     check(spc3d_spmm(ctx.get(), A.get(), X.get(), Y.get()), "spc3d_spmm");
 }
 
+// Both of the above over one pattern and one B in a single pass (spc3d_sddmm_spmm):
+// C as sddmm; Y += S B, or Y += C B when chained.
+template <typename T>
+void sddmm_spmm(Context &ctx, Plan<T> &S, const Panel<T> &A, const Panel<T> &B, Vals<T> &C,
+                Panel<T> &Y, bool chained = false)
+{
+    check(spc3d_sddmm_spmm(ctx.get(), S.get(), A.get(), B.get(), C.get(), Y.get(), chained ? 1 : 0),
+          "spc3d_sddmm_spmm");
+}
+
 } // namespace spc3d

@@ -34,3 +34,11 @@ def sddmm_bytes(nrows, nnz, k, w, m_t, n_t, with_perm=False, gather=False) -> in
 def spmm_bytes(nrows, nnz, k, w, m_t, n_t, gather=False) -> int:
     x_side = nnz if gather else n_t
     return index_bytes(nrows, nnz, False) + w * nnz + w * k * x_side + 2 * w * k * m_t
+
+
+def fused_bytes(nrows, nnz, k, w, m_t, n_t, with_perm=False, gather=False) -> int:
+    """SDDMM and the SpMM of the same pattern over the same B in one pass: every
+    operand of either kernel once (A, B, the Y read-modify-write, S.vv, C.vv)."""
+    b_side = nnz if gather else n_t
+    return (index_bytes(nrows, nnz, with_perm) + 2 * w * nnz + w * k * m_t + w * k * b_side +
+            2 * w * k * m_t)

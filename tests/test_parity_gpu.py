@@ -134,6 +134,51 @@ def test_cut_rows_with_ragged_k(ctx, dtype, k):
     check_spmm(B, ii, jj, vv, Y0, gpu_spmm(ctx, 40, 300, ii, jj, vv, B, Y0, seg_max=64))
 
 
+# ---- both kernels in one pass over the gathered rows ---------------------------------
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("chained", [False, True])
+@pytest.mark.parametrize("k", [4, 20, 64, 100, 256])
+def test_fused_sddmm_spmm_equals_the_two_calls(ctx, dtype, chained, k):
+    m, n, nnz = 120, 90, 4000
+    ii, jj, vv, A, B, Y0 = rand_case(500 + k, m, n, k, nnz, dtype, hub=900)
+    S = ctx.plan(m, n, ii, jj, vv, seg_max=64)  # cut rows: partial sums and the fix-up
+    dA, dB, dY, dC = ctx.panel_from(A), ctx.panel_from(B), ctx.panel_from(Y0), ctx.vals(nnz, dtype)
+    ctx.sddmm_spmm(S, dA, dB, dC, dY, chained=chained)
+    C, Y = dC.download(), dY.download()
+    check_sddmm(A, B, ii, jj, vv, C)
+    # the SpMM half against the oracle, with the weights it is defined to use
+    w = oracle.sddmm(A, B, ii, jj, vv) if chained else vv
+    check_spmm(B, ii, jj, w.astype(dtype), Y0, Y)
+    # and the plan's own values are untouched: a plain SpMM afterwards still uses S.vv
+    dY.upload(Y0)
+    ctx.spmm(S, dB, dY)
+    check_spmm(B, ii, jj, vv, Y0, dY.download())
+    for h in (S, dA, dB, dY, dC):
+        h.close()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_fused_call_on_the_sliced_layout_and_odd_widths(ctx, dtype):
+    w = W.rmat(14, 16, 64).shuffled()
+    A, B, Y0, vv = w.panel_A(dtype), w.panel_B(dtype), w.panel_Y0(dtype), w.values(dtype)
+    S = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, vv, xcd_slices=8, l2_hot_bytes=64 * 1024,
+                 hub_min=32, seg_max=256)
+    assert S.info.nqueues == 8
+    dA, dB, dY, dC = ctx.panel_from(A), ctx.panel_from(B), ctx.panel_from(Y0), ctx.vals(w.nnz, dtype)
+    ctx.sddmm_spmm(S, dA, dB, dC, dY)
+    check_sddmm(A, B, w.ii, w.jj, vv, dC.download())
+    check_spmm(B, w.ii, w.jj, vv, Y0, dY.download())
+    # K without a vector kernel: the plain form falls back to the two calls, the chained one refuses
+    ii, jj, vv, A, B, Y0 = rand_case(3, 30, 30, 5, 200, dtype)
+    S2 = ctx.plan(30, 30, ii, jj, vv)
+    dA, dB, dY, dC = ctx.panel_from(A), ctx.panel_from(B), ctx.panel_from(Y0), ctx.vals(200, dtype)
+    ctx.sddmm_spmm(S2, dA, dB, dC, dY)
+    check_sddmm(A, B, ii, jj, vv, dC.download())
+    check_spmm(B, ii, jj, vv, Y0, dY.download())
+    with pytest.raises(capi.Spc3dError):
+        ctx.sddmm_spmm(S2, dA, dB, dC, dY, chained=True)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_random_shapes_widths_and_plan_options(ctx, dtype):
     # every knob at once: skewed patterns, sorted or not, exact / ragged / generic row widths,
