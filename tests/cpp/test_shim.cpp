@@ -399,6 +399,20 @@ static void test_resident_handles_and_row_exchange()
     dY.download(y.data());
     CHECK(max_rel(y, yref, 100.0) < 10 * kTol);
 
+    // the same two results from the one-pass call, chained: Y0 += C B
+    {
+        spc3d::Panel<real_t> dY2(ctx, m, k);
+        spc3d::Vals<real_t> dC2(ctx, S.nnz);
+        dY2.upload(Y0.data.data());
+        P.set_values(S.vv.data());
+        spc3d::sddmm_spmm(ctx, P, dA, dB, dC2, dY2, true);
+        std::vector<real_t> c2(S.nnz), y2((size_t)m * k);
+        dC2.download(c2.data());
+        dY2.download(y2.data());
+        CHECK(max_rel(c2, cref, k * 1.0) < kTol);
+        CHECK(max_rel(y2, yref, 100.0) < 10 * kTol);
+    }
+
     // pack rows (with repeats), then sum them back: Y[r] += (times r is listed) * Y[r]
     std::vector<idx_t> rows;
     for (idx_t r = 0; r < m; r += 3) {
