@@ -1,0 +1,61 @@
+"""The contract of bench.py and __graft_entry__ that can be checked without a GPU."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_bench_refuses_more_than_one_gpu():
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"],
+                       capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0
+    assert "one GPU" in r.stderr and r.stdout.strip() == ""
+
+
+def test_entry_points_exist():
+    sys.path.insert(0, ROOT)
+    import __graft_entry__ as g
+
+    assert callable(g.build) and callable(g.smoke)
+
+
+def test_byte_models_of_the_roofline():
+    from spcomm3d_amd import roofline
+
+    # R-MAT 20, K = 64, fp64, with the output permutation read: the figures the bench line
+    # and the profiles quote
+    nnz, m, mt, nt = 16086740, 1048576, 547169, 547037
+    sd = roofline.sddmm_bytes(m, nnz, 64, 8, mt, nt, True)
+    sp = roofline.spmm_bytes(m, nnz, 64, 8, mt, nt)
+    fz = roofline.fused_bytes(m, nnz, 64, 8, mt, nt, True)
+    index = 4 * (m + 1) + 4 * nnz
+    assert sd == index + 4 * nnz + 2 * 8 * nnz + 8 * 64 * (mt + nt) == 950509540
+    assert sp == index + 8 * nnz + 8 * 64 * nt + 2 * 8 * 64 * mt == 1037619188
+    assert fz == sd + 2 * 8 * 64 * mt
+    assert roofline.flops(nnz, 64) == 2 * nnz * 64
+
+
+@pytest.mark.gpu
+def test_bench_line_has_the_contract_fields():
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--config", "er16k",
+                        "--steps", "5", "--warmup", "1"], capture_output=True, text=True,
+                       timeout=600)
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = [ln for ln in r.stdout.splitlines() if ln.strip()]
+    assert len(lines) == 1
+    d = json.loads(lines[0])
+    for k in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step",
+              "higher_is_better", "scaling", "vs_baseline", "dtype", "data", "config", "roofline",
+              "cpu_baseline"):
+        assert k in d, k
+    assert d["n_gpus"] == 1 and d["steps"] == 5 and d["vs_baseline"] is None
+    assert d["dtype"] == "f64" and "workload" in d["config"]
+    assert set(("bound", "achieved", "peak", "unit", "frac", "traffic")) <= set(d["roofline"])
+    assert d["roofline"]["bound"] == "hbm" and d["roofline"]["peak"] == 8000.0
+    assert abs(d["roofline"]["frac"] - d["roofline"]["achieved"] / 8000.0) < 1e-12
+    assert set(("value", "unit", "cores", "kind", "sample")) <= set(d["cpu_baseline"])
+    assert d["cpu_baseline"]["kind"] in ("reference", "port")
