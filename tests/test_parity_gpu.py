@@ -146,9 +146,9 @@ def test_fused_sddmm_spmm_equals_the_two_calls(ctx, dtype, chained, k):
     ctx.sddmm_spmm(S, dA, dB, dC, dY, chained=chained)
     C, Y = dC.download(), dY.download()
     check_sddmm(A, B, ii, jj, vv, C)
-    # the SpMM half against the oracle, with the weights it is defined to use
-    w = oracle.sddmm(A, B, ii, jj, vv) if chained else vv
-    check_spmm(B, ii, jj, w.astype(dtype), Y0, Y)
+    # the SpMM half against the oracle, with the weights it is defined to use: S.vv, or
+    # the C this very call produced (C itself was held to the SDDMM oracle above)
+    check_spmm(B, ii, jj, C if chained else vv, Y0, Y)
     # and the plan's own values are untouched: a plain SpMM afterwards still uses S.vv
     dY.upload(Y0)
     ctx.spmm(S, dB, dY)
@@ -168,6 +168,10 @@ def test_fused_call_on_the_sliced_layout_and_odd_widths(ctx, dtype):
     ctx.sddmm_spmm(S, dA, dB, dC, dY)
     check_sddmm(A, B, w.ii, w.jj, vv, dC.download())
     check_spmm(B, w.ii, w.jj, vv, Y0, dY.download())
+    dY.upload(Y0)
+    ctx.sddmm_spmm(S, dA, dB, dC, dY, chained=True)
+    check_sddmm(A, B, w.ii, w.jj, vv, dC.download())
+    check_spmm(B, w.ii, w.jj, dC.download(), Y0, dY.download())
     # K without a vector kernel: the plain form falls back to the two calls, the chained one refuses
     ii, jj, vv, A, B, Y0 = rand_case(3, 30, 30, 5, 200, dtype)
     S2 = ctx.plan(30, 30, ii, jj, vv)
