@@ -225,7 +225,7 @@ __device__ __forceinline__ bool lane_on(uint32_t sub, int v, uint32_t nvec)
 // that stores it.
 template <typename T, int LPR, int VPL, int NB, bool RG, bool MK, int FZ>
 __device__ __forceinline__ void
-sddmm_batch(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type (&acc)[VPL],
+sddmm_batch_one(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type (&acc)[VPL],
             const uint32_t *__restrict__ col, const uint32_t *__restrict__ perm,
             const T *__restrict__ sval, const T *__restrict__ B, T *__restrict__ C, uint32_t p0,
             uint32_t n, uint32_t sub, uint32_t nvec)
@@ -295,6 +295,111 @@ sddmm_batch(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type (&acc)[
     }
 }
 
+template <typename T, int LPR, int VPL, int NB, bool RG, bool MK, int FZ>
+__device__ __forceinline__ void
+sddmm_batch_rounds(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type (&acc)[VPL],
+            const uint32_t *__restrict__ col, const uint32_t *__restrict__ perm,
+            const T *__restrict__ sval, const T *__restrict__ B, T *__restrict__ C, uint32_t p0,
+            uint32_t n, uint32_t sub, uint32_t nvec)
+{
+    using V = typename Vec<T>::type;
+    // A group of LPR lanes reduces at most LPR entries at a time: the NB entries of
+    // the batch are R rounds of G, all gathered before the first round is reduced, so
+    // that narrow rows (LPR = 4, 8) keep as many gathers in flight as wide ones.
+    constexpr int G = NB < LPR ? NB : LPR;
+    constexpr int R = NB / G;
+    static_assert(R * G == NB, "a batch is a whole number of rounds");
+
+    // Lane u of the group fetches the column of entry u of each round; the writer
+    // lanes fetch what they need for the store.  These head the dependency chain.
+    const uint32_t uo = entry_of<LPR, G>(sub);
+    const bool wlane = is_writer<LPR, G>(sub);
+    uint32_t cme[R], dst[R];
+    T sv[R];
+    bool writer[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        uint32_t e = (uint32_t)r * G + (sub & (G - 1));
+        if (MK)
+            e = e < n ? e : n - 1;
+        cme[r] = nt_load(col + p0 + e);
+        const uint32_t mine = (uint32_t)r * G + uo;
+        writer[r] = wlane && (!MK || mine < n);
+        sv[r] = (T)0;
+        dst[r] = p0 + mine;
+        if (writer[r]) {
+            sv[r] = nt_load(sval + p0 + mine);
+            if (perm)
+                dst[r] = nt_load(perm + p0 + mine);
+        }
+    }
+
+    V b[NB][VPL];
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+        const uint32_t c = __shfl(cme[j / G], j % G, LPR);
+        const V *brow = row_ptr<T, LPR, VPL, RG>(B, c, sub, nvec);
+#pragma unroll
+        for (int v = 0; v < VPL; ++v)
+            b[j][v] = lane_on<LPR, RG>(sub, v, nvec) ? brow[v * LPR] : V{};
+    }
+    __builtin_amdgcn_sched_barrier(0); // all gathers in flight before the first use
+
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        T part[G];
+#pragma unroll
+        for (int u = 0; u < G; ++u) {
+            T dot = (T)0;
+#pragma unroll
+            for (int v = 0; v < VPL; ++v)
+#pragma unroll
+                for (int i = 0; i < Vec<T>::N; ++i)
+                    dot += a[v][i] * b[r * G + u][v][i];
+            part[u] = dot;
+        }
+        group_reduce<T, LPR, G>(part, sub);
+        const T result = part[0] * sv[r];
+        // Results in the caller's order: when that is the kernel order the stores of a
+        // batch fill whole lines and stream out; when it is not they are scattered, and
+        // plain stores let the L2 merge neighbours into lines before writing back.
+        if (writer[r]) {
+            if (perm)
+                C[dst[r]] = result;
+            else
+                nt_store(result, C + dst[r]);
+        }
+        if constexpr (FZ != 0) {
+            const T mine = FZ == 2 ? result : sv[r]; // valid on the writer lanes
+#pragma unroll
+            for (int u = 0; u < G; ++u) {
+                const bool on = !MK || (uint32_t)(r * G + u) < n;
+                const T w = on ? __shfl(mine, writer_lane<LPR, G>(u), LPR) : (T)0;
+#pragma unroll
+                for (int v = 0; v < VPL; ++v)
+                    acc[v] += (on ? b[r * G + u][v] : V{}) * w;
+            }
+        }
+    }
+}
+
+// A batch of NB entries: one round when the lane group can reduce them at once,
+// several otherwise.
+template <typename T, int LPR, int VPL, int NB, bool RG, bool MK, int FZ>
+__device__ __forceinline__ void
+sddmm_batch(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type (&acc)[VPL],
+            const uint32_t *__restrict__ col, const uint32_t *__restrict__ perm,
+            const T *__restrict__ sval, const T *__restrict__ B, T *__restrict__ C, uint32_t p0,
+            uint32_t n, uint32_t sub, uint32_t nvec)
+{
+    if constexpr (NB <= LPR)
+        sddmm_batch_one<T, LPR, VPL, NB, RG, MK, FZ>(a, acc, col, perm, sval, B, C, p0, n, sub,
+                                                     nvec);
+    else
+        sddmm_batch_rounds<T, LPR, VPL, NB, RG, MK, FZ>(a, acc, col, perm, sval, B, C, p0, n, sub,
+                                                        nvec);
+}
+
 // n consecutive entries from p.  WIDE: full batches of UB, then one masked batch
 // of the smallest size in {4, 8, 16} that holds the rest.  !WIDE (segments known
 // to be short, run at twice the occupancy): masked batches of UB throughout.
@@ -343,7 +448,7 @@ sddmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint3
                  const T *__restrict__ sval, const T *__restrict__ A, const T *__restrict__ B,
                  T *__restrict__ C, T *__restrict__ Y, T *__restrict__ partial, uint32_t nvec)
 {
-    static_assert(UB <= LPR && UB <= 16 && LPR <= 64, "batch must fit the lane group");
+    static_assert(UB <= 16 && LPR <= 64, "at most 16 entries in flight per lane");
     using V = typename Vec<T>::type;
     const uint32_t sub = threadIdx.x & (LPR - 1);
     const uint64_t sid = seg_index<64 / LPR>(nq, rot);
@@ -414,7 +519,7 @@ sddmm_generic_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, u
 // entry n - 1 and add zero times zero.
 template <typename T, int LPR, int VPL, int NB, bool RG, bool MK>
 __device__ __forceinline__ void
-spmm_batch(typename Vec<T>::type (&acc)[VPL], const uint32_t *__restrict__ col,
+spmm_batch_one(typename Vec<T>::type (&acc)[VPL], const uint32_t *__restrict__ col,
            const T *__restrict__ sval, const T *__restrict__ X, uint32_t p0, uint32_t n,
            uint32_t sub, uint32_t nvec)
 {
@@ -447,6 +552,64 @@ spmm_batch(typename Vec<T>::type (&acc)[VPL], const uint32_t *__restrict__ col,
         for (int v = 0; v < VPL; ++v)
             acc[v] += (on ? x[u][v] : V{}) * a;
     }
+}
+
+template <typename T, int LPR, int VPL, int NB, bool RG, bool MK>
+__device__ __forceinline__ void
+spmm_batch_rounds(typename Vec<T>::type (&acc)[VPL], const uint32_t *__restrict__ col,
+           const T *__restrict__ sval, const T *__restrict__ X, uint32_t p0, uint32_t n,
+           uint32_t sub, uint32_t nvec)
+{
+    using V = typename Vec<T>::type;
+    // Lane u of the group fetches column and value of entry u of each of the R rounds
+    // of G <= LPR entries (see sddmm_batch).
+    constexpr int G = NB < LPR ? NB : LPR;
+    constexpr int R = NB / G;
+    static_assert(R * G == NB, "a batch is a whole number of rounds");
+    uint32_t cme[R];
+    T vme[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        uint32_t e = (uint32_t)r * G + (sub & (G - 1));
+        if (MK)
+            e = e < n ? e : n - 1;
+        cme[r] = nt_load(col + p0 + e);
+        vme[r] = nt_load(sval + p0 + e);
+    }
+
+    V x[NB][VPL];
+    T av[NB];
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+        const uint32_t c = __shfl(cme[j / G], j % G, LPR);
+        av[j] = __shfl(vme[j / G], j % G, LPR);
+        const V *xrow = row_ptr<T, LPR, VPL, RG>(X, c, sub, nvec);
+#pragma unroll
+        for (int v = 0; v < VPL; ++v)
+            x[j][v] = lane_on<LPR, RG>(sub, v, nvec) ? xrow[v * LPR] : V{};
+    }
+    __builtin_amdgcn_sched_barrier(0); // all gathers in flight before the first use
+    // Entries are added in kernel order.
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+        const bool on = !MK || (uint32_t)j < n;
+        const T w = on ? av[j] : (T)0;
+#pragma unroll
+        for (int v = 0; v < VPL; ++v)
+            acc[v] += (on ? x[j][v] : V{}) * w;
+    }
+}
+
+template <typename T, int LPR, int VPL, int NB, bool RG, bool MK>
+__device__ __forceinline__ void
+spmm_batch(typename Vec<T>::type (&acc)[VPL], const uint32_t *__restrict__ col,
+           const T *__restrict__ sval, const T *__restrict__ X, uint32_t p0, uint32_t n,
+           uint32_t sub, uint32_t nvec)
+{
+    if constexpr (NB <= LPR)
+        spmm_batch_one<T, LPR, VPL, NB, RG, MK>(acc, col, sval, X, p0, n, sub, nvec);
+    else
+        spmm_batch_rounds<T, LPR, VPL, NB, RG, MK>(acc, col, sval, X, p0, n, sub, nvec);
 }
 
 template <typename T, int LPR, int VPL, int UB, bool RG, bool WIDE>
@@ -508,7 +671,7 @@ spmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint32
                 const T *__restrict__ X, T *__restrict__ Y, T *__restrict__ partial,
                 uint32_t nvec)
 {
-    static_assert(UB <= LPR && UB <= 16 && LPR <= 64, "batch must fit the lane group");
+    static_assert(UB <= 16 && LPR <= 64, "at most 16 entries in flight per lane");
     using V = typename Vec<T>::type;
     const uint32_t sub = threadIdx.x & (LPR - 1);
     const uint64_t sid = seg_index<64 / LPR>(nq, rot);
@@ -823,17 +986,15 @@ hipError_t run_spmm(const DevPlanView &P, const T *X, T *Y, const Streams &S, ui
 // (LPR, VPL, UB, US_SDDMM, US_SPMM): UB * VPL 16-byte gathers are in flight per
 // lane in the long-segment launch, US * VPL in the short-segment one.
 #define SPC3D_FOR_SHAPES(X)                                                                       \
-    X(4, 1, 4, 4, 4) X(8, 1, 8, 8, 4) X(16, 1, 16, 8, 4) X(32, 1, 16, 8, 4) X(64, 1, 16, 8, 4)    \
-    X(4, 2, 4, 4, 2) X(8, 2, 8, 4, 2) X(16, 2, 8, 4, 2) X(32, 2, 8, 4, 2) X(64, 2, 8, 4, 2)       \
+    X(4, 1, 16, 8, 4) X(8, 1, 16, 8, 4) X(16, 1, 16, 8, 4) X(32, 1, 16, 8, 4) X(64, 1, 16, 8, 4)  \
+    X(4, 2, 8, 4, 2) X(8, 2, 8, 4, 2) X(16, 2, 8, 4, 2) X(32, 2, 8, 4, 2) X(64, 2, 8, 4, 2)       \
     X(4, 4, 4, 2, 1) X(8, 4, 4, 2, 1) X(16, 4, 4, 2, 1) X(32, 4, 4, 2, 1) X(64, 4, 4, 2, 1)
 // Rows that do not fill a shape: the smallest power-of-two LPR covering the row,
 // then 64 lanes with 2 or 4 vectors each.
 #define SPC3D_FOR_RAGGED_SHAPES(X)                                                                \
-    X(4, 1, 4, 4, 4) X(8, 1, 8, 8, 4) X(16, 1, 16, 8, 4) X(32, 1, 16, 8, 4) X(64, 1, 16, 8, 4)    \
+    X(4, 1, 16, 8, 4) X(8, 1, 16, 8, 4) X(16, 1, 16, 8, 4) X(32, 1, 16, 8, 4) X(64, 1, 16, 8, 4)  \
     X(64, 2, 8, 4, 2) X(64, 4, 4, 2, 1)
 
-// Adds the partial sums of cut rows into Y (after the segment kernels of an SpMM or
-// a fused call).
 template <typename T>
 hipError_t launch_fixup(const DevPlanView &P, T *Y, uint32_t K, hipStream_t st)
 {
