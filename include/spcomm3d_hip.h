@@ -29,8 +29,11 @@
  *    (src/basic.hpp:36), so its behaviour is defined only for m*n < 2^32.
  *    This library uses 64-bit offsets; nnz must be < 2^32.
  *  - A context is used by one host thread at a time and owns one HIP stream
- *    (default priority).  Kernel-launching calls are asynchronous on that
- *    stream; *_download and *_host calls return with host memory valid.
+ *    (default priority), plus an internal one of the same priority on which
+ *    part of an SDDMM / SpMM call runs, forked from and joined back to the
+ *    first by events inside the call.  Kernel-launching calls are asynchronous
+ *    on the context's stream; *_download and *_host calls return with host
+ *    memory valid.
  *  - Nothing here falls back to the CPU: without a usable GPU every device
  *    call fails with SPC3D_ERR_NO_DEVICE.
  */
