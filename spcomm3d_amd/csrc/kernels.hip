@@ -384,7 +384,10 @@ sddmm_batch_rounds(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type 
 }
 
 // A batch of NB entries: one round when the lane group can reduce them at once,
-// several otherwise.
+// several otherwise.  The two forms are kept apart on purpose: written as the
+// R = 1 case of the rounds form, the single round compiles to 24 more VGPRs
+// (100 -> 124 in the wide launch, 62 -> 74 and two wavefronts per SIMD fewer in
+// the short one), which cost the 5-entry rows of a stencil 20 %.
 template <typename T, int LPR, int VPL, int NB, bool RG, bool MK, int FZ>
 __device__ __forceinline__ void
 sddmm_batch(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type (&acc)[VPL],
