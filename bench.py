@@ -17,6 +17,9 @@ oracle (a serial restatement of the reference's loops), timed on one host core
 on the same workload.  `fused_step` is the same step through the one-pass entry
 point spc3d_sddmm_spmm (an extension without counterpart in the reference); it is
 reported beside `value`, which always comes from the two separate calls.
+`row_copies` times the pack and sum-unpack copies of a sparse exchange over the
+touched rows of Y (algorithmic bytes: rows read + buffer written; buffer read +
+rows read and written).
 """
 from __future__ import annotations
 
@@ -120,6 +123,34 @@ def run_gpu(w, dtype, steps, warmup, seg_max=None, max_timed=1300, copies=0):
             ctx.sddmm_spmm(S, dA, dB, dC, dY)
         ctx.sync()
         fused_wall = time.perf_counter() - t0
+        # The copies either side of a sparse exchange on the same panel: every touched
+        # row of Y packed into a buffer, and the buffer summed back (src/comm.hpp:90-103,
+        # 178-189), `steps` times each.
+        touched = np.flatnonzero(np.bincount(w.ii, minlength=w.nrows)).astype(np.uint32)
+        rmap = device.RowMap(ctx, w.nrows, touched)
+        dbuf = ctx.vals(touched.size * w.k, dtype)
+        for _ in range(warmup):
+            rmap.pack(dY, dbuf)
+            rmap.unpack_sum(dY, dbuf)
+        ctx.sync()
+        ctx.mark(4000)
+        for _ in range(steps):
+            rmap.pack(dY, dbuf)
+        ctx.mark(4001)
+        for _ in range(steps):
+            rmap.unpack_sum(dY, dbuf)
+        ctx.mark(4002)
+        pack_ms = ctx.elapsed_ms(4000, 4001) / steps
+        sum_ms = ctx.elapsed_ms(4001, 4002) / steps
+        nrow_bytes = touched.size * w.k * wbytes
+        rows = {"rows": int(touched.size),
+                "pack": {"ms": pack_ms, "bytes": int(2 * nrow_bytes + 4 * touched.size)},
+                "unpack_sum": {"ms": sum_ms, "bytes": int(3 * nrow_bytes + 4 * touched.size)}}
+        for v in (rows["pack"], rows["unpack_sum"]):
+            v["gbs"] = v["bytes"] / v["ms"] / 1e6
+            v["frac"] = v["gbs"] / roofline.HBM_PEAK_GBS
+        rmap.close()
+        dbuf.close()
         for h in (S, dA, dB, dY, dC):
             h.close()
 
@@ -134,6 +165,7 @@ def run_gpu(w, dtype, steps, warmup, seg_max=None, max_timed=1300, copies=0):
     out["fused_step"] = {"entry": "spc3d_sddmm_spmm", "ms_per_step": fused_wall / steps * 1e3,
                          "gflops": 2 * fl / (fused_wall / steps) / 1e9, "strict_bytes": int(fb),
                          "strict_frac": fb / (fused_wall / steps) / 1e9 / roofline.HBM_PEAK_GBS}
+    out["row_copies"] = rows
     for name, ms, strict, gather in (
             ("sddmm", sd,
              roofline.sddmm_bytes(w.nrows, w.nnz, w.k, wbytes, m_t, n_t, with_perm),
@@ -292,6 +324,7 @@ def main():
         "cpu_baseline": cpu,
         "kernels": main_r["kernels"],
         "fused_step": main_r["fused_step"],
+        "row_copies": main_r["row_copies"],
         "plan": {k: main_r[k] for k in ("plan_build_s", "upload_s", "nsegments", "nsplit_rows",
                                         "seg_max")},
         "also": also,
