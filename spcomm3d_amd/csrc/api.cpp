@@ -918,10 +918,9 @@ int spc3d_plan_download(spc3d_plan *plan, uint32_t *col, uint32_t *perm, uint32_
     return rc;
 }
 
-int spc3d_plan_create(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t ncols, uint64_t nnz,
-                      const uint32_t *ii, const uint32_t *jj, const void *vv, spc3d_plan **out)
+// Library defaults, each overridable from the environment for tuning runs.
+static spc3d_plan_opts opts_from_env()
 {
-    // Defaults, each overridable from the environment for tuning runs.
     spc3d_plan_opts o;
     std::memset(&o, 0, sizeof o);
     struct {
@@ -932,14 +931,21 @@ int spc3d_plan_create(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t ncols,
                {"SPC3D_L2_HOT_BYTES", &o.l2_hot_bytes},
                {"SPC3D_HUB_MIN", &o.hub_min},
                {"SPC3D_XCD_SLICES", &o.xcd_slices}};
-    if (const char *b = std::getenv("SPC3D_PLAN_BUILDER"))
-        o.builder = std::strcmp(b, "host") == 0 ? 1u : 2u;
     for (auto &e : env)
         if (const char *s = std::getenv(e.name)) {
             const long long v = std::atoll(s);
             if (v > 0 && v <= 0xFFFFFFFFll)
                 *e.field = (uint32_t)v;
         }
+    if (const char *b = std::getenv("SPC3D_PLAN_BUILDER"))
+        o.builder = std::strcmp(b, "host") == 0 ? 1u : 2u;
+    return o;
+}
+
+int spc3d_plan_create(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t ncols, uint64_t nnz,
+                      const uint32_t *ii, const uint32_t *jj, const void *vv, spc3d_plan **out)
+{
+    const spc3d_plan_opts o = opts_from_env();
     return spc3d_plan_create_ex(ctx, dtype, nrows, ncols, nnz, ii, jj, vv, &o, out);
 }
 
@@ -1286,7 +1292,10 @@ int spc3d_sddmm_host(spc3d_ctx *ctx, int dtype, uint32_t m, uint32_t n, uint32_t
     spc3d_plan *S = nullptr;
     spc3d_panel *a = nullptr, *b = nullptr;
     spc3d_vals *c = nullptr;
-    int rc = spc3d_plan_create(ctx, dtype, m, n, nnz, ii, jj, svv, &S);
+    spc3d_plan_opts o = opts_from_env();
+    if (!o.k_hint)
+        o.k_hint = k; // the one width this plan will ever run with
+    int rc = spc3d_plan_create_ex(ctx, dtype, m, n, nnz, ii, jj, svv, &o, &S);
     if (!rc) rc = spc3d_panel_create(ctx, dtype, m, k, &a);
     if (!rc) rc = spc3d_panel_create(ctx, dtype, n, k, &b);
     if (!rc) rc = spc3d_vals_create(ctx, dtype, nnz, &c);
@@ -1310,7 +1319,10 @@ int spc3d_spmm_host(spc3d_ctx *ctx, int dtype, uint32_t ncols, uint32_t nrows, u
         return fail(SPC3D_ERR_INVALID_ARG, "avv is NULL");
     spc3d_plan *S = nullptr;
     spc3d_panel *x = nullptr, *y = nullptr;
-    int rc = spc3d_plan_create(ctx, dtype, nrows, ncols, nnz, ii, jj, avv, &S);
+    spc3d_plan_opts o = opts_from_env();
+    if (!o.k_hint)
+        o.k_hint = k;
+    int rc = spc3d_plan_create_ex(ctx, dtype, nrows, ncols, nnz, ii, jj, avv, &o, &S);
     if (!rc) rc = spc3d_panel_create(ctx, dtype, ncols, k, &x);
     if (!rc) rc = spc3d_panel_create(ctx, dtype, nrows, k, &y);
     if (!rc) rc = spc3d_panel_upload(x, X);

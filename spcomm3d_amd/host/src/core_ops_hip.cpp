@@ -43,7 +43,7 @@ uint64_t fingerprint(const void *data, size_t bytes, uint64_t seed)
 struct CachedPlan {
     uint64_t pattern_fp = 0, values_fp = 0;
     uint64_t nnz = 0;
-    uint32_t nrows = 0, ncols = 0;
+    uint32_t nrows = 0, ncols = 0, k = 0;
     uint64_t last_use = 0;
     std::unique_ptr<Plan<real_t>> plan;
 };
@@ -83,7 +83,9 @@ struct Shim {
         return *c;
     }
 
-    Plan<real_t> &plan_for(const cooMat &S, uint32_t nrows, uint32_t ncols)
+    // k: the row width the plan will run with (it sizes the set of dense rows planned
+    // for L2); a pattern used with another width is planned again.
+    Plan<real_t> &plan_for(const cooMat &S, uint32_t nrows, uint32_t ncols, uint32_t k)
     {
         const uint64_t nnz = S.nnz;
         if (S.ii.size() < nnz || S.jj.size() < nnz || S.vv.size() < nnz)
@@ -93,7 +95,8 @@ struct Shim {
         const uint64_t vfp = fingerprint(S.vv.data(), nnz * sizeof(real_t), 2);
         ++clock;
         for (CachedPlan &e : plans) {
-            if (e.pattern_fp == pfp && e.nnz == nnz && e.nrows == nrows && e.ncols == ncols) {
+            if (e.pattern_fp == pfp && e.nnz == nnz && e.nrows == nrows && e.ncols == ncols &&
+                e.k == k) {
                 if (e.values_fp != vfp) {
                     e.plan->set_values(S.vv.data());
                     e.values_fp = vfp;
@@ -116,11 +119,14 @@ struct Shim {
         e.nnz = nnz;
         e.nrows = nrows;
         e.ncols = ncols;
+        e.k = k;
         e.last_use = clock;
         // Validates every index against the panel heights: a bad one throws
         // std::out_of_range here, as the reference's .at() would at that entry.
+        spc3d_plan_opts opts = {};
+        opts.k_hint = k;
         e.plan.reset(new Plan<real_t>(context(), nrows, ncols, nnz, S.ii.data(), S.jj.data(),
-                                      S.vv.data()));
+                                      S.vv.data(), &opts));
         plans.push_back(std::move(e));
         return *plans.back().plan;
     }
@@ -154,7 +160,7 @@ void sddmm(denseMatrix &A, denseMatrix &B, cooMat &S, cooMat &C)
     if (B.n != A.n)
         throw std::runtime_error("sddmm: B.n != A.n is not supported");
     Shim &s = shim();
-    Plan<real_t> &plan = s.plan_for(S, A.m, B.m);
+    Plan<real_t> &plan = s.plan_for(S, A.m, B.m, A.n);
     Panel<real_t> &a = s.panel(s.a, A.m, A.n);
     Panel<real_t> &b = s.panel(s.b, B.m, B.n);
     Vals<real_t> &c = s.vals(S.nnz);
@@ -183,7 +189,7 @@ void spmm(denseMatrix &X, cooMat &A, denseMatrix &Y)
     if (Y.n != X.n)
         throw std::runtime_error("spmm: Y.n != X.n is not supported");
     Shim &s = shim();
-    Plan<real_t> &plan = s.plan_for(A, Y.m, X.m);
+    Plan<real_t> &plan = s.plan_for(A, Y.m, X.m, X.n);
     Panel<real_t> &x = s.panel(s.b, X.m, X.n);
     Panel<real_t> &y = s.panel(s.y, Y.m, Y.n);
     x.upload(X.data.data());
