@@ -72,7 +72,9 @@ def run_gpu(w, dtype, steps, warmup, seg_max=None, max_timed=1300, copies=0):
     A, B, Y0, vv = w.panel_A(dtype), w.panel_B(dtype), w.panel_Y0(dtype), w.values(dtype)
     with device.Context(0) as ctx:
         t0 = time.perf_counter()
-        S = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, vv, seg_max=seg_max)
+        # the plan sizes its L2-resident set for K = 64 unless told the width it will run with
+        hint = {} if w.k == 64 else {"k_hint": w.k}
+        S = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, vv, seg_max=seg_max, **hint)
         ctx.sync()
         plan_s = time.perf_counter() - t0
         info = S.info
