@@ -924,6 +924,14 @@ inline uint32_t blocks_for_groups(uint32_t nseg, uint32_t nq, int groups_per_wav
 // rows of a stencil 1.6x faster with US = 4 than with 16, R-MAT hub segments
 // 1.5x slower.  With an auxiliary stream the two run side by side.
 
+// A pattern this small does not keep the chip busy for long enough to repay a
+// second launch with its fork and join (about 20 us when the kernels are short):
+// when it has segments of both kinds, all of them go to the wide launch (either
+// kernel handles segments of any length; the long ones hold most of the entries).
+// Measured on R-MAT 14 .. 19: one launch wins up to about 180 k segments (11 against
+// 32 us at 12 k), two from 400 k on.
+constexpr uint32_t kOneLaunchSegments = 196608;
+
 // Makes the auxiliary stream wait for everything queued on the main stream so
 // far.  On failure nothing was queued on aux and the caller stays on main.
 inline bool fork_aux(const Streams &S)
@@ -947,7 +955,9 @@ template <typename T, int LPR, int VPL, int UB, int US, bool RG, int FZ>
 hipError_t run_sddmm(const DevPlanView &P, const T *A, const T *B, T *C, T *Y, const Streams &S,
                      uint32_t nvec)
 {
-    const uint32_t nl = P.nseg_long, ns = P.nseg - P.nseg_long;
+    uint32_t nl = P.nseg_long, ns = P.nseg - P.nseg_long;
+    if (nl && ns && P.nseg <= kOneLaunchSegments)
+        nl = P.nseg, ns = 0;
     const bool both = nl && ns && fork_aux(S);
     if (nl)
         hipLaunchKernelGGL((sddmm_seg_kernel<T, LPR, VPL, UB, RG, true, FZ>),
@@ -968,7 +978,9 @@ hipError_t run_sddmm(const DevPlanView &P, const T *A, const T *B, T *C, T *Y, c
 template <typename T, int LPR, int VPL, int UB, int US, bool RG>
 hipError_t run_spmm(const DevPlanView &P, const T *X, T *Y, const Streams &S, uint32_t nvec)
 {
-    const uint32_t nl = P.nseg_long, ns = P.nseg - P.nseg_long;
+    uint32_t nl = P.nseg_long, ns = P.nseg - P.nseg_long;
+    if (nl && ns && P.nseg <= kOneLaunchSegments)
+        nl = P.nseg, ns = 0;
     const bool both = nl && ns && fork_aux(S);
     if (nl)
         hipLaunchKernelGGL((spmm_seg_kernel<T, LPR, VPL, UB, RG, true>),
