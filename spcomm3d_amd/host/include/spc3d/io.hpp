@@ -136,6 +136,12 @@ inline void read_binary(const std::string &inFN, cooMat &C, bool single_rank = t
     f.read(reinterpret_cast<char *>(&n), 8);
     if (!f)
         throw std::runtime_error("read_binary: " + inFN + " has no header");
+    // a header that promises more triplets than the file holds must not size the arrays
+    f.seekg(0, std::ios::end);
+    const std::uint64_t file_bytes = (std::uint64_t)f.tellg();
+    f.seekg(16, std::ios::beg);
+    if (n > (file_bytes - 16) / 16)
+        throw std::runtime_error("read_binary: " + inFN + " ends before its last entry");
     C.gnrows = r;
     C.gncols = c;
     C.gnnz = n;

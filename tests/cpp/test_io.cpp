@@ -5,6 +5,7 @@
 //
 //   test_io <dir with the golden files>
 #include <cstdio>
+#include <cstring>
 #include <fstream>
 #include <iterator>
 #include <string>
@@ -99,6 +100,20 @@ int main(int argc, char **argv)
         std::vector<char> ref = slurp(dir + "/general.bin");
         std::ofstream(cut, std::ios::binary).write(ref.data(), 100);
         read_binary(cut, R);
+    } catch (const std::runtime_error &) {
+        threw = true;
+    }
+    CHECK(threw);
+    // a header that promises 2^40 triplets is refused before anything is sized by it
+    threw = false;
+    try {
+        cooMat R;
+        const std::string lie = "/tmp/spc3d_test_io_lie.bin";
+        std::vector<char> ref = slurp(dir + "/general.bin");
+        const std::uint64_t huge = 1ull << 40;
+        std::memcpy(&ref[8], &huge, 8);
+        std::ofstream(lie, std::ios::binary).write(ref.data(), (std::streamsize)ref.size());
+        read_binary(lie, R);
     } catch (const std::runtime_error &) {
         threw = true;
     }
