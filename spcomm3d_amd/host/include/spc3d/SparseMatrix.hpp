@@ -9,10 +9,17 @@
 //     time it appears in the entry stream; only touched rows / columns get
 //     ids; ltgR / ltgC invert the maps.
 //   ReMapIndices (:100-106): ii[i] = mapR[ii[i]], jj[i] = mapC[jj[i]].
+//   self_generate_random (:49-67): distinct random positions, value 1.
 #pragma once
 
+#include <chrono>
+#include <cstdint>
+#include <iostream>
+#include <random>
+#include <stdexcept>
 #include <string>
 #include <unordered_map>
+#include <unordered_set>
 #include <vector>
 
 #include "basic.hpp"
@@ -53,6 +60,29 @@ template <typename T, typename IdxT> class COOMatrix : public SparseMatrix<T, Id
         const idx_large_t n = count == 0 ? this->nnz : static_cast<idx_large_t>(count);
         for (idx_large_t i = 0; i < n; ++i)
             std::cout << ii[i] << " " << jj[i] << " " << vv[i] << std::endl;
+    }
+
+    // Appends count entries of value 1 at distinct random positions of the
+    // gnrows x gncols pattern (SparseMatrix.hpp:49-67 seeds from the clock; a seed can
+    // be given here so that a run can be repeated).  nnz stays the caller's to set.
+    void self_generate_random(IdxT count, std::uint64_t seed = 0)
+    {
+        const std::uint64_t cells = (std::uint64_t)this->gnrows * this->gncols;
+        if (count > cells)
+            throw std::out_of_range("self_generate_random: more entries than cells");
+        std::mt19937_64 rng(seed ? seed
+                                 : (std::uint64_t)std::chrono::steady_clock::now()
+                                       .time_since_epoch()
+                                       .count());
+        std::unordered_set<std::uint64_t> used;
+        used.reserve(count * 2);
+        for (IdxT made = 0; made < count;) {
+            const std::uint64_t cell = rng() % cells;
+            if (!used.insert(cell).second)
+                continue; // a position is used once
+            addEntry((IdxT)(cell / this->gncols), (IdxT)(cell % this->gncols), (T)1);
+            ++made;
+        }
     }
 
     void localizeIndices() override

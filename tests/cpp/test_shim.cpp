@@ -145,6 +145,41 @@ static void test_types_and_index_transforms()
     CHECK(Cc.vv == S.vv && Cc.nnz == S.nnz);
 }
 
+static void test_random_pattern_generator()
+{
+    cooMat S;
+    S.gnrows = 37;
+    S.gncols = 11;
+    S.self_generate_random(300, 5);
+    CHECK(S.ii.size() == 300 && S.jj.size() == 300 && S.vv.size() == 300);
+    std::vector<char> seen(37 * 11, 0);
+    bool ok = true;
+    for (size_t i = 0; i < 300; ++i) {
+        ok = ok && S.ii[i] < 37 && S.jj[i] < 11 && S.vv[i] == (real_t)1;
+        ok = ok && !seen[S.ii[i] * 11 + S.jj[i]];
+        seen[S.ii[i] * 11 + S.jj[i]] = 1;
+    }
+    CHECK(ok); // in range, value 1, no position twice
+    cooMat T;
+    T.gnrows = 37;
+    T.gncols = 11;
+    T.self_generate_random(300, 5);
+    CHECK(T.ii == S.ii && T.jj == S.jj); // same seed, same pattern
+    // every cell may be asked for; one more than that may not
+    cooMat U;
+    U.gnrows = 2;
+    U.gncols = 2;
+    U.self_generate_random(4, 1);
+    CHECK(U.ii.size() == 4);
+    bool threw = false;
+    try {
+        U.self_generate_random(5, 1);
+    } catch (const std::out_of_range &) {
+        threw = true;
+    }
+    CHECK(threw);
+}
+
 static void test_errors_without_touching_the_gpu()
 {
     // C.vv too short: the reference's C.vv.at(i) throws (core_ops.cpp:18)
@@ -444,6 +479,7 @@ int main(int argc, char **argv)
 {
     const bool host_only = argc > 1 && std::strcmp(argv[1], "--host") == 0;
     test_types_and_index_transforms();
+    test_random_pattern_generator();
     test_errors_without_touching_the_gpu();
     if (!host_only) {
         try {
