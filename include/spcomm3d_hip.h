@@ -127,6 +127,25 @@ SPC3D_API int spc3d_ctx_stream(spc3d_ctx *ctx, void **hip_stream); /* the hipStr
  * caller check that on its machine.  Synchronous. */
 SPC3D_API int spc3d_ctx_probe_xcd(spc3d_ctx *ctx, uint32_t nblocks, uint32_t *xcd);
 
+/* A sequence of kernel-launching calls recorded once and replayed with one launch
+ * (a HIP graph): for steps so short that launch latency dominates them (the
+ * reference's 16384 x 16384 case runs one kernel in under 10 us).  Between
+ * spc3d_capture_begin and spc3d_capture_end the calls that only queue kernels -
+ * spc3d_sddmm, spc3d_spmm, spc3d_sddmm_spmm, spc3d_rows_*, spc3d_panel_fill,
+ * spc3d_panel_copy, spc3d_vals_fill, spc3d_plan_set_values_device - are recorded
+ * instead of run; every other call on the context (anything that allocates,
+ * copies to or from the host, waits or times) returns SPC3D_ERR_INVALID_ARG and
+ * leaves the recording intact.  An SpMM over a plan with cut rows must have run
+ * once with the same K before it is recorded (its partial-sum rows are
+ * allocated on first use).  spc3d_graph_launch replays the sequence on the
+ * context's stream, asynchronously, over the same operands; their contents at
+ * launch time are what the kernels read.  Has no counterpart in the reference. */
+typedef struct spc3d_graph spc3d_graph;
+SPC3D_API int spc3d_capture_begin(spc3d_ctx *ctx);
+SPC3D_API int spc3d_capture_end(spc3d_ctx *ctx, spc3d_graph **out);
+SPC3D_API int spc3d_graph_launch(spc3d_graph *graph);
+SPC3D_API int spc3d_graph_destroy(spc3d_graph *graph);
+
 /* Timing on the context's stream (the reference times the call with chrono in
  * integer ms, src/distributed_comp.cpp:176-179; a kernel here lasts well under
  * one).  spc3d_timer_mark records event `slot` (0..4095) on the stream;

@@ -52,6 +52,10 @@ SIGNATURES = {
     "spc3d_ctx_probe_xcd": (c_int, [c_vp, c_u32, c_vp]),
     "spc3d_timer_mark": (c_int, [c_vp, c_int]),
     "spc3d_timer_elapsed_ms": (c_int, [c_vp, c_int, c_int, P(c_float)]),
+    "spc3d_capture_begin": (c_int, [c_vp]),
+    "spc3d_capture_end": (c_int, [c_vp, P(c_vp)]),
+    "spc3d_graph_launch": (c_int, [c_vp]),
+    "spc3d_graph_destroy": (c_int, [c_vp]),
     "spc3d_panel_create": (c_int, [c_vp, c_int, c_u32, c_u32, P(c_vp)]),
     "spc3d_panel_destroy": (c_int, [c_vp]),
     "spc3d_panel_upload": (c_int, [c_vp, c_vp]),

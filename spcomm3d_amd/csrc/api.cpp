@@ -51,6 +51,7 @@ constexpr uint32_t kMagicPanel = 0x53433350; // stale or foreign pointer is refu
 constexpr uint32_t kMagicVals = 0x53433356;  // instead of dereferenced further
 constexpr uint32_t kMagicPlan = 0x5343334c;
 constexpr uint32_t kMagicRowMap = 0x5343334d;
+constexpr uint32_t kMagicGraph = 0x53433347;
 constexpr int kTimerSlots = 4096;
 
 inline size_t elem_size(int dtype) { return dtype == SPC3D_F64 ? 8 : 4; }
@@ -65,6 +66,7 @@ struct spc3d_ctx {
     hipStream_t aux_stream; // short-segment launches run here, beside the long-segment ones
     hipEvent_t fork_event, join_event;
     uint32_t aux_rot; // (XCD of workgroup 0 on aux - XCD of workgroup 0 on main) mod 8
+    bool capturing;   // between spc3d_capture_begin and spc3d_capture_end
     hipEvent_t timers[kTimerSlots];
     bool timer_set[kTimerSlots];
 };
@@ -93,6 +95,13 @@ struct spc3d_rowmap {
     uint32_t *rows, *urows, *ptr, *slots; // device
 };
 
+struct spc3d_graph {
+    uint32_t magic;
+    spc3d_ctx *ctx;
+    hipGraph_t graph;
+    hipGraphExec_t exec;
+};
+
 struct spc3d_plan {
     uint32_t magic;
     spc3d_ctx *ctx;
@@ -117,8 +126,17 @@ bool live(const spc3d_vals *v) { return v && v->magic == kMagicVals && live(v->c
 bool live(const spc3d_plan *p) { return p && p->magic == kMagicPlan && live(p->ctx); }
 bool live(const spc3d_rowmap *p) { return p && p->magic == kMagicRowMap && live(p->ctx); }
 
-int use_device(const spc3d_ctx *ctx)
+bool live(const spc3d_graph *g) { return g && g->magic == kMagicGraph && live(g->ctx); }
+
+// Makes the context's device current.  While the context records a graph only the
+// calls that merely queue kernels may run (capturable); everything that allocates,
+// copies to or from the host or waits is refused.
+int use_device(const spc3d_ctx *ctx, bool capturable = false)
 {
+    if (ctx->capturing && !capturable)
+        return fail(SPC3D_ERR_INVALID_ARG,
+                    "this call allocates, copies or waits: not allowed between "
+                    "spc3d_capture_begin and spc3d_capture_end");
     HIP_TRY(hipSetDevice(ctx->device));
     return SPC3D_OK;
 }
@@ -290,6 +308,7 @@ int spc3d_ctx_create(int device, spc3d_ctx **out)
     // Each hardware queue starts its round-robin over the XCDs at its own XCD:
     // measure where workgroup 0 lands on either stream.
     c->aux_rot = 0;
+    c->capturing = false;
     if (c->aux_stream) {
         uint32_t *probe = nullptr, host[2] = {0, 0};
         e = hipMalloc((void **)&probe, 2 * sizeof(uint32_t));
@@ -323,6 +342,14 @@ int spc3d_ctx_destroy(spc3d_ctx *ctx)
 {
     if (!live(ctx))
         return fail(SPC3D_ERR_INVALID_ARG, "context is NULL or destroyed");
+    if (ctx->capturing) { // drop the unfinished recording
+        hipGraph_t g = nullptr;
+        (void)hipStreamEndCapture(ctx->stream, &g);
+        if (g)
+            (void)hipGraphDestroy(g);
+        (void)hipGetLastError();
+        ctx->capturing = false;
+    }
     (void)hipSetDevice(ctx->device);
     (void)hipStreamSynchronize(ctx->stream);
     for (int i = 0; i < kTimerSlots; ++i)
@@ -340,11 +367,102 @@ int spc3d_ctx_destroy(spc3d_ctx *ctx)
     return SPC3D_OK;
 }
 
+static int refuse_while_capturing(const spc3d_ctx *ctx)
+{
+    if (ctx->capturing)
+        return fail(SPC3D_ERR_INVALID_ARG,
+                    "not allowed between spc3d_capture_begin and spc3d_capture_end");
+    return SPC3D_OK;
+}
+
 int spc3d_ctx_sync(spc3d_ctx *ctx)
 {
     if (!live(ctx))
         return fail(SPC3D_ERR_INVALID_ARG, "context is NULL or destroyed");
+    if (int rc = refuse_while_capturing(ctx))
+        return rc;
     HIP_TRY(hipStreamSynchronize(ctx->stream));
+    return SPC3D_OK;
+}
+
+/* ---- recorded sequences of calls ------------------------------------------- */
+int spc3d_capture_begin(spc3d_ctx *ctx)
+{
+    if (!live(ctx))
+        return fail(SPC3D_ERR_INVALID_ARG, "context is NULL or destroyed");
+    if (ctx->capturing)
+        return fail(SPC3D_ERR_INVALID_ARG, "the context is recording already");
+    int rc = use_device(ctx);
+    if (rc)
+        return rc;
+    HIP_TRY(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+    ctx->capturing = true;
+    return SPC3D_OK;
+}
+
+int spc3d_capture_end(spc3d_ctx *ctx, spc3d_graph **out)
+{
+    if (!out)
+        return fail(SPC3D_ERR_INVALID_ARG, "out is NULL");
+    *out = nullptr;
+    if (!live(ctx))
+        return fail(SPC3D_ERR_INVALID_ARG, "context is NULL or destroyed");
+    if (!ctx->capturing)
+        return fail(SPC3D_ERR_INVALID_ARG, "the context is not recording");
+    ctx->capturing = false;
+    hipGraph_t graph = nullptr;
+    hipError_t e = hipStreamEndCapture(ctx->stream, &graph);
+    if (e != hipSuccess || !graph) {
+        (void)hipGetLastError();
+        if (graph)
+            (void)hipGraphDestroy(graph);
+        return fail_hip(e != hipSuccess ? e : hipErrorUnknown, "hipStreamEndCapture");
+    }
+    hipGraphExec_t exec = nullptr;
+    e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        (void)hipGraphDestroy(graph);
+        return fail_hip(e, "hipGraphInstantiate");
+    }
+    spc3d_graph *g = new (std::nothrow) spc3d_graph();
+    if (!g) {
+        (void)hipGraphExecDestroy(exec);
+        (void)hipGraphDestroy(graph);
+        return fail(SPC3D_ERR_ALLOC, "host allocation failed");
+    }
+    g->ctx = ctx;
+    g->graph = graph;
+    g->exec = exec;
+    g->magic = kMagicGraph;
+    *out = g;
+    return SPC3D_OK;
+}
+
+int spc3d_graph_launch(spc3d_graph *g)
+{
+    if (!live(g))
+        return fail(SPC3D_ERR_INVALID_ARG, "graph is NULL or destroyed");
+    if (g->ctx->capturing)
+        return fail(SPC3D_ERR_INVALID_ARG, "the context is recording");
+    int rc = use_device(g->ctx);
+    if (rc)
+        return rc;
+    HIP_TRY(hipGraphLaunch(g->exec, g->ctx->stream));
+    return SPC3D_OK;
+}
+
+int spc3d_graph_destroy(spc3d_graph *g)
+{
+    if (!live(g))
+        return fail(SPC3D_ERR_INVALID_ARG, "graph is NULL or destroyed");
+    if (int rc = refuse_while_capturing(g->ctx))
+        return rc;
+    (void)hipSetDevice(g->ctx->device);
+    (void)hipStreamSynchronize(g->ctx->stream);
+    (void)hipGraphExecDestroy(g->exec);
+    (void)hipGraphDestroy(g->graph);
+    g->magic = 0;
+    delete g;
     return SPC3D_OK;
 }
 
@@ -385,6 +503,8 @@ int spc3d_timer_mark(spc3d_ctx *ctx, int slot)
         return fail(SPC3D_ERR_INVALID_ARG, "context is NULL or destroyed");
     if (slot < 0 || slot >= kTimerSlots)
         return fail(SPC3D_ERR_INVALID_ARG, "timer slot out of range");
+    if (int rc = refuse_while_capturing(ctx))
+        return rc;
     if (!ctx->timers[slot])
         HIP_TRY(hipEventCreate(&ctx->timers[slot]));
     HIP_TRY(hipEventRecord(ctx->timers[slot], ctx->stream));
@@ -438,6 +558,8 @@ int spc3d_panel_destroy(spc3d_panel *p)
 {
     if (!live(p))
         return fail(SPC3D_ERR_INVALID_ARG, "panel is NULL or destroyed");
+    if (int rc = refuse_while_capturing(p->ctx))
+        return rc;
     (void)hipSetDevice(p->ctx->device);
     (void)hipStreamSynchronize(p->ctx->stream);
     if (p->dev)
@@ -473,7 +595,7 @@ int spc3d_panel_fill(spc3d_panel *p, double value)
 {
     if (!live(p))
         return fail(SPC3D_ERR_INVALID_ARG, "panel is NULL or destroyed");
-    int rc = use_device(p->ctx);
+    int rc = use_device(p->ctx, true);
     if (rc)
         return rc;
     HIP_TRY(launch_fill(p->dtype, p->dev, (uint64_t)p->m * p->n, value, p->ctx->stream));
@@ -490,7 +612,7 @@ int spc3d_panel_copy(spc3d_panel *dst, const spc3d_panel *src)
         return fail(SPC3D_ERR_SIZE_MISMATCH, "panels differ in shape or dtype");
     if (dst->dev == src->dev)
         return SPC3D_OK;
-    int rc = use_device(dst->ctx);
+    int rc = use_device(dst->ctx, true);
     if (rc)
         return rc;
     HIP_TRY(launch_copy(dst->dev, src->dev, (uint64_t)dst->m * dst->n * elem_size(dst->dtype),
@@ -551,6 +673,8 @@ int spc3d_vals_destroy(spc3d_vals *v)
 {
     if (!live(v))
         return fail(SPC3D_ERR_INVALID_ARG, "value vector is NULL or destroyed");
+    if (int rc = refuse_while_capturing(v->ctx))
+        return rc;
     (void)hipSetDevice(v->ctx->device);
     (void)hipStreamSynchronize(v->ctx->stream);
     if (v->dev)
@@ -584,7 +708,7 @@ int spc3d_vals_fill(spc3d_vals *v, double value)
 {
     if (!live(v))
         return fail(SPC3D_ERR_INVALID_ARG, "value vector is NULL or destroyed");
-    int rc = use_device(v->ctx);
+    int rc = use_device(v->ctx, true);
     if (rc)
         return rc;
     HIP_TRY(launch_fill(v->dtype, v->dev, v->n, value, v->ctx->stream));
@@ -953,6 +1077,8 @@ int spc3d_plan_destroy(spc3d_plan *plan)
 {
     if (!live(plan))
         return fail(SPC3D_ERR_INVALID_ARG, "plan is NULL or destroyed");
+    if (int rc = refuse_while_capturing(plan->ctx))
+        return rc;
     (void)hipSetDevice(plan->ctx->device);
     (void)hipStreamSynchronize(plan->ctx->stream);
     plan_free_device(plan);
@@ -1002,7 +1128,7 @@ int spc3d_plan_set_values_device(spc3d_plan *plan, const spc3d_vals *vv)
     if (vv->dtype != plan->dtype || vv->n < plan->info.nnz || vv->ctx != plan->ctx)
         return fail(SPC3D_ERR_SIZE_MISMATCH,
                     "value vector dtype / length / context does not fit the plan");
-    int rc = use_device(plan->ctx);
+    int rc = use_device(plan->ctx, true);
     if (rc)
         return rc;
     HIP_TRY(launch_gather_vals(plan->dtype, vv->dev, plan->perm, plan->sval, plan->info.nnz,
@@ -1024,6 +1150,10 @@ static int ensure_partial(spc3d_plan *p, uint32_t K)
 {
     if (!p->info.npartial_slots || p->partial_k >= K)
         return SPC3D_OK;
+    if (p->ctx->capturing)
+        return fail(SPC3D_ERR_INVALID_ARG,
+                    "the plan's partial-sum rows are not allocated for this K yet: run the call "
+                    "once before recording it");
     HIP_TRY(hipStreamSynchronize(p->ctx->stream));
     if (p->partial)
         (void)hipFree(p->partial);
@@ -1058,13 +1188,13 @@ int spc3d_sddmm(spc3d_ctx *ctx, spc3d_plan *S, const spc3d_panel *A, const spc3d
     if (!S->has_values)
         return fail(SPC3D_ERR_INVALID_ARG, "plan has no values (spc3d_plan_set_values)");
     if (K == 0) { // empty dot product: every result is 0 * S.vv = 0
-        int rc = use_device(ctx);
+        int rc = use_device(ctx, true);
         if (rc)
             return rc;
         HIP_TRY(launch_fill(C->dtype, C->dev, S->info.nnz, 0.0, ctx->stream));
         return SPC3D_OK;
     }
-    int rc = use_device(ctx);
+    int rc = use_device(ctx, true);
     if (rc)
         return rc;
     HIP_TRY(launch_sddmm(S->dtype, view_of(S), A->dev, B->dev, C->dev, K, streams_of(ctx)));
@@ -1090,7 +1220,7 @@ int spc3d_spmm(spc3d_ctx *ctx, spc3d_plan *Ap, const spc3d_panel *X, spc3d_panel
         return fail(SPC3D_ERR_INVALID_ARG, "X and Y must not alias");
     if (!Ap->has_values)
         return fail(SPC3D_ERR_INVALID_ARG, "plan has no values (spc3d_plan_set_values)");
-    int rc = use_device(ctx);
+    int rc = use_device(ctx, true);
     if (rc)
         return rc;
     rc = ensure_partial(Ap, K);
@@ -1123,7 +1253,7 @@ int spc3d_sddmm_spmm(spc3d_ctx *ctx, spc3d_plan *S, const spc3d_panel *A, const 
         return fail(SPC3D_ERR_INVALID_ARG, "Y must not alias A or B");
     if (!S->has_values)
         return fail(SPC3D_ERR_INVALID_ARG, "plan has no values (spc3d_plan_set_values)");
-    int rc = use_device(ctx);
+    int rc = use_device(ctx, true);
     if (rc)
         return rc;
     if (K == 0) { // empty dot products, nothing to add
@@ -1228,6 +1358,8 @@ int spc3d_rowmap_destroy(spc3d_rowmap *m)
 {
     if (!live(m))
         return fail(SPC3D_ERR_INVALID_ARG, "row map is NULL or destroyed");
+    if (int rc = refuse_while_capturing(m->ctx))
+        return rc;
     (void)hipSetDevice(m->ctx->device);
     (void)hipStreamSynchronize(m->ctx->stream);
     if (m->rows) (void)hipFree(m->rows);
@@ -1252,7 +1384,7 @@ static int rows_op(int op, spc3d_ctx *ctx, const spc3d_panel *P, const spc3d_row
         return fail(SPC3D_ERR_SIZE_MISMATCH, "panel has fewer rows than the row map was made for");
     if (buf->n < (uint64_t)map->nslots * P->n)
         return fail(SPC3D_ERR_SIZE_MISMATCH, "buffer holds fewer than n * K reals");
-    int rc = use_device(ctx);
+    int rc = use_device(ctx, true);
     if (rc)
         return rc;
     RowMapView v;

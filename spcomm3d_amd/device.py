@@ -117,6 +117,15 @@ class Context:
         check(self._lib.spc3d_sddmm_spmm(self._h, S._h, A._h, B._h, C._h, Y._h, int(chained)),
               "spc3d_sddmm_spmm")
 
+    def capture_begin(self):
+        """Start recording kernel-launching calls instead of running them (``spc3d_capture_begin``)."""
+        check(self._lib.spc3d_capture_begin(self._h), "spc3d_capture_begin")
+
+    def capture_end(self) -> "Graph":
+        h = ctypes.c_void_p()
+        check(self._lib.spc3d_capture_end(self._h, ctypes.byref(h)), "spc3d_capture_end")
+        return Graph(self, h)
+
     def probe_xcd(self, nblocks: int) -> np.ndarray:
         """XCD id each workgroup of an ``nblocks``-wide grid ran on (``spc3d_ctx_probe_xcd``)."""
         out = np.zeros(nblocks, dtype=np.uint32)
@@ -343,6 +352,27 @@ class Plan:
     def close(self):
         if getattr(self, "_h", None) and getattr(self.ctx, "_h", None):
             self.ctx._lib.spc3d_plan_destroy(self._h)
+        self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class Graph:
+    """A recorded sequence of calls, replayed with one launch (``spc3d_graph``)."""
+
+    def __init__(self, ctx: Context, h):
+        self.ctx, self._h = ctx, h
+
+    def launch(self):
+        check(self.ctx._lib.spc3d_graph_launch(self._h), "spc3d_graph_launch")
+
+    def close(self):
+        if getattr(self, "_h", None) and getattr(self.ctx, "_h", None):
+            self.ctx._lib.spc3d_graph_destroy(self._h)
         self._h = None
 
     def __del__(self):

@@ -1,0 +1,115 @@
+"""Recorded call sequences (HIP graphs) through the C ABI: every replay must give
+what the same calls give when run eagerly, bit for bit (the kernels are
+reproducible run to run), with other work and synchronisations between replays."""
+import time
+
+import numpy as np
+import pytest
+
+from spcomm3d_amd import _capi as capi
+from spcomm3d_amd import workloads as W
+
+pytestmark = pytest.mark.gpu
+
+
+def operands(ctx, w, dtype):
+    vv = w.values(dtype)
+    S = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, vv, k_hint=w.k)
+    dA, dB = ctx.panel_from(w.panel_A(dtype)), ctx.panel_from(w.panel_B(dtype))
+    return S, dA, dB
+
+
+@pytest.mark.parametrize("maker,dtype", [
+    (lambda: W.erdos_renyi(16384, 16, 32), np.float64),          # one launch per call
+    (lambda: W.rmat(15, 16, 64).shuffled(), np.float32),         # cut rows, fix-up, one launch
+    (lambda: W.rmat(19, 16, 16), np.float32),                    # two launches on two streams
+])
+def test_replays_equal_eager_runs(ctx, maker, dtype):
+    w = maker()
+    S, dA, dB = operands(ctx, w, dtype)
+    Y0 = w.panel_Y0(dtype)
+    eY, gY = ctx.panel_from(Y0), ctx.panel_from(Y0)
+    eC, gC = ctx.vals(w.nnz, dtype), ctx.vals(w.nnz, dtype)
+    other = ctx.vals(w.nnz, dtype)
+
+    def step(C, Y):
+        ctx.sddmm(S, dA, dB, C)
+        ctx.spmm(S, dB, Y)
+
+    step(other, ctx.panel_from(Y0))  # first use allocates the plan's partial-sum rows
+    ctx.sync()
+    ctx.capture_begin()
+    step(gC, gY)
+    g = ctx.capture_end()
+    gC.fill(-3.0)  # nothing ran while recording
+    assert np.all(gC.download() == -3.0) and np.array_equal(gY.download(), Y0)
+    for replay in range(4):
+        step(eC, eY)          # eager twin of this replay
+        g.launch()
+        ctx.sddmm(S, dB if w.nrows == w.ncols else dA, dB, other)  # unrelated work in between
+        ctx.sync()
+        assert np.array_equal(gC.download(), eC.download()), replay
+        assert np.array_equal(gY.download(), eY.download()), replay  # Y accumulates per replay
+        gC.fill(0.0)          # the next replay must write it again
+    g.close()
+
+
+def test_calls_that_cannot_be_recorded_are_refused_and_leave_the_recording_intact(ctx):
+    w = W.rmat(13, 16, 64)
+    S, dA, dB = operands(ctx, w, np.float64)
+    dY, dC = ctx.panel_from(w.panel_Y0("f64")), ctx.vals(w.nnz, np.float64)
+    cut = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, w.values("f64"), seg_max=16)  # never run: no partial rows yet
+    ctx.capture_begin()
+    with pytest.raises(capi.Spc3dError):
+        ctx.capture_begin()                      # already recording
+    with pytest.raises(capi.Spc3dError):
+        dC.download()                            # copies to the host
+    with pytest.raises(capi.Spc3dError):
+        ctx.sync()                               # waits
+    with pytest.raises(capi.Spc3dError):
+        ctx.vals(10, np.float64)                 # allocates
+    with pytest.raises(capi.Spc3dError) as e:
+        ctx.spmm(cut, dB, dY)                    # would allocate its partial-sum rows
+    assert "once before" in str(e.value)
+    ctx.sddmm(S, dA, dB, dC)                     # the recording is still good
+    g = ctx.capture_end()
+    with pytest.raises(capi.Spc3dError):
+        ctx.capture_end()                        # not recording any more
+    g.launch()
+    ctx.sync()
+    eC = ctx.vals(w.nnz, np.float64)
+    ctx.sddmm(S, dA, dB, eC)
+    assert np.array_equal(dC.download(), eC.download())
+    g.close()
+
+
+def test_replay_of_a_short_step_costs_less_than_its_eager_calls(ctx):
+    w = W.erdos_renyi(16384, 16, 32)
+    S, dA, dB = operands(ctx, w, np.float64)
+    dY, dC = ctx.panel_from(w.panel_Y0("f64")), ctx.vals(w.nnz, np.float64)
+
+    def step():
+        ctx.sddmm(S, dA, dB, dC)
+        ctx.spmm(S, dB, dY)
+
+    step()
+    ctx.sync()
+    ctx.capture_begin()
+    for _ in range(10):
+        step()
+    g = ctx.capture_end()
+
+    def timed(fn, n):
+        fn()
+        ctx.sync()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        ctx.sync()
+        return (time.perf_counter() - t0) / n
+
+    eager = timed(lambda: [step() for _ in range(10)], 50)
+    replay = timed(g.launch, 50)
+    print(f"ER 16384 K=32 fp64, 10 steps: eager {eager * 1e6:.1f} us, one replay {replay * 1e6:.1f} us")
+    assert replay < eager * 1.5  # never a regression worth the name; usually well below
+    g.close()
