@@ -8,7 +8,8 @@
 // row.  A dense row of K reals is nvec 16-byte vectors, covered by LPR lanes
 // holding VPL vectors each (nvec = LPR * VPL with the row stride a compile-time
 // constant, or nvec < LPR * VPL given at run time in the "ragged" variants, whose
-// spare lanes idle); one wavefront works on 64 / LPR segments at once and every
+// spare lanes idle, or a row that ends inside its last vector in the "odd"
+// variants); one wavefront works on 64 / LPR segments at once and every
 // global load instruction moves 64 x 16 B.  Segments arrive sorted longest
 // first, so the lane groups of a wavefront run the same trip count.
 //
@@ -45,10 +46,12 @@ namespace {
 template <typename T> struct Vec;
 template <> struct Vec<float> {
     typedef float type __attribute__((ext_vector_type(4)));
+    typedef type loose __attribute__((aligned(4))); // same vector at element alignment
     static constexpr int N = 4;
 };
 template <> struct Vec<double> {
     typedef double type __attribute__((ext_vector_type(2)));
+    typedef type loose __attribute__((aligned(8)));
     static constexpr int N = 2;
 };
 
@@ -194,10 +197,10 @@ template <int G> __device__ __forceinline__ uint64_t seg_index(uint32_t nq, uint
            (threadIdx.x & 63u) / (64 / G);
 }
 
-// RG ("ragged"): a dense row is nvec 16-byte vectors with nvec < LPR * VPL, given at
-// run time; lanes whose vector index is >= nvec idle.  !RG: nvec == LPR * VPL
-// exactly and the row stride is a compile-time constant.
-template <typename T, int LPR, int VPL, bool RG>
+// RG == 1 ("ragged"): a dense row is nvec 16-byte vectors with nvec < LPR * VPL,
+// given at run time; lanes whose vector index is >= nvec idle.  RG == 0: nvec ==
+// LPR * VPL exactly and the row stride is a compile-time constant.  RG == 2: below.
+template <typename T, int LPR, int VPL, int RG>
 __device__ __forceinline__ const typename Vec<T>::type *row_ptr(const T *base, uint32_t row,
                                                                 uint32_t sub, uint32_t nvec)
 {
@@ -207,10 +210,142 @@ __device__ __forceinline__ const typename Vec<T>::type *row_ptr(const T *base, u
            sub;
 }
 
-template <int LPR, bool RG>
+template <int LPR, int RG>
 __device__ __forceinline__ bool lane_on(uint32_t sub, int v, uint32_t nvec)
 {
     return !RG || sub + (uint32_t)v * LPR < nvec;
+}
+
+// RG == 2 ("odd"): a dense row of K reals is no whole number of 16-byte vectors
+// (the kernels' `nvec` argument carries K).  Rows start at element alignment only,
+// and the last vector of a row would reach past its end, so: the lane that holds the
+// row's end loads the 16 bytes that END there (the leading elements of that vector
+// belong to the lane before and are not counted), and lanes past the end load the
+// same vector and count nothing.  Every load stays inside the row, without a
+// branch.  Vector loads and stores at 4- or 8-byte alignment are what global memory
+// accesses on this GPU allow.
+// 16-byte accesses at element alignment.  (Not through nt_load / nt_store: template
+// argument deduction would drop the typedef's alignment.)
+template <typename T> __device__ __forceinline__ typename Vec<T>::type loose_load(const char *p)
+{
+    return *reinterpret_cast<const typename Vec<T>::loose *>(p);
+}
+template <typename T> __device__ __forceinline__ typename Vec<T>::type loose_load_nt(const char *p)
+{
+    return __builtin_nontemporal_load(reinterpret_cast<const typename Vec<T>::loose *>(p));
+}
+template <typename T>
+__device__ __forceinline__ void loose_store(typename Vec<T>::type v, char *p)
+{
+    *reinterpret_cast<typename Vec<T>::loose *>(p) = v;
+}
+template <typename T>
+__device__ __forceinline__ void loose_store_nt(typename Vec<T>::type v, char *p)
+{
+    __builtin_nontemporal_store(v, reinterpret_cast<typename Vec<T>::loose *>(p));
+}
+
+template <typename T, int VPL, int RG> struct Odd {};
+template <typename T, int VPL> struct Odd<T, VPL, 2> {
+    uint32_t off[VPL];             // byte offset within a row of this lane's vector v
+    bool keep[VPL][Vec<T>::N];     // the elements of it that are this lane's
+    bool all[VPL];                 // every element is
+};
+
+template <typename T, int LPR, int VPL, int RG>
+__device__ __forceinline__ Odd<T, VPL, RG> odd_lanes(uint32_t sub, uint32_t K)
+{
+    Odd<T, VPL, RG> o;
+    if constexpr (RG == 2) {
+        const uint32_t bytes = K * (uint32_t)sizeof(T); // >= 16: see pick_shape
+#pragma unroll
+        for (int v = 0; v < VPL; ++v) {
+            const uint32_t first = (sub + (uint32_t)v * LPR) * 16;
+            const uint32_t start = first < bytes - 16 ? first : bytes - 16;
+            o.off[v] = start;
+            o.all[v] = start == first;
+#pragma unroll
+            for (int i = 0; i < Vec<T>::N; ++i)
+                o.keep[v][i] = start + (uint32_t)i * sizeof(T) >= first;
+        }
+    }
+    return o;
+}
+
+template <typename T, int RG>
+__device__ __forceinline__ const char *odd_row(const T *base, uint32_t row, uint32_t K)
+{
+    static_assert(RG == 2, "rows of K reals at element alignment");
+    return reinterpret_cast<const char *>(base) + (uint64_t)row * ((uint64_t)K * sizeof(T));
+}
+
+// out[v] = this lane's vectors of dense row `row`.  RG == 2 loads every element of
+// them; what is not the lane's to count is left out by the caller (SDDMM: in the
+// dot product; SpMM: at the store).
+template <typename T, int LPR, int VPL, int RG>
+__device__ __forceinline__ void gather_row(typename Vec<T>::type (&out)[VPL], const T *base,
+                                           uint32_t row, uint32_t sub, uint32_t nvec,
+                                           const Odd<T, VPL, RG> &odd)
+{
+    using V = typename Vec<T>::type;
+    if constexpr (RG == 2) {
+        const char *r = odd_row<T, RG>(base, row, nvec);
+#pragma unroll
+        for (int v = 0; v < VPL; ++v)
+            out[v] = loose_load<T>(r + odd.off[v]);
+    } else {
+        const V *r = row_ptr<T, LPR, VPL, RG>(base, row, sub, nvec);
+#pragma unroll
+        for (int v = 0; v < VPL; ++v)
+            out[v] = lane_on<LPR, RG>(sub, v, nvec) ? r[v * LPR] : V{};
+    }
+}
+
+// a . b over the elements that are this lane's.
+template <typename T, int VPL, int RG>
+__device__ __forceinline__ T lane_dot(const typename Vec<T>::type (&a)[VPL],
+                                      const typename Vec<T>::type (&b)[VPL],
+                                      const Odd<T, VPL, RG> &odd)
+{
+    T dot = (T)0;
+#pragma unroll
+    for (int v = 0; v < VPL; ++v)
+#pragma unroll
+        for (int i = 0; i < Vec<T>::N; ++i) {
+            if constexpr (RG == 2)
+                dot += a[v][i] * (odd.keep[v][i] ? b[v][i] : (T)0);
+            else
+                dot += a[v][i] * b[v][i];
+        }
+    return dot;
+}
+
+// Writes y0 + acc (whole rows of Y) or acc (partial-sum slots, read back by
+// spmm_fixup right after) to this lane's part of the row at drow: one vector store
+// where the whole vector is the lane's, element stores for the lane at the row's end.
+template <typename T, int VPL>
+__device__ __forceinline__ void odd_store(char *drow, bool whole,
+                                          const typename Vec<T>::type (&y0)[VPL],
+                                          const typename Vec<T>::type (&acc)[VPL],
+                                          const Odd<T, VPL, 2> &odd)
+{
+    using V = typename Vec<T>::type;
+#pragma unroll
+    for (int v = 0; v < VPL; ++v) {
+        const V r = y0[v] + acc[v]; // y0 is zero for a slot
+        if (odd.all[v]) {
+            if (whole)
+                loose_store_nt<T>(r, drow + odd.off[v]);
+            else
+                loose_store<T>(r, drow + odd.off[v]);
+        } else {
+            T *d = reinterpret_cast<T *>(drow + odd.off[v]);
+#pragma unroll
+            for (int i = 0; i < Vec<T>::N; ++i)
+                if (odd.keep[v][i])
+                    d[i] = r[i];
+        }
+    }
 }
 
 // ---------------------------------------------------------------- SDDMM ----
@@ -223,12 +358,13 @@ __device__ __forceinline__ bool lane_on(uint32_t sub, int v, uint32_t nvec)
 // acc += w_u * B[c_u,:] in kernel order, with w_u = S.vv (FZ == 1) or the SDDMM
 // result just computed (FZ == 2); the weight of entry u is broadcast from the lane
 // that stores it.
-template <typename T, int LPR, int VPL, int NB, bool RG, bool MK, int FZ>
+template <typename T, int LPR, int VPL, int NB, int RG, bool MK, int FZ>
 __device__ __forceinline__ void
 sddmm_batch_one(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type (&acc)[VPL],
             const uint32_t *__restrict__ col, const uint32_t *__restrict__ perm,
             const T *__restrict__ sval, const T *__restrict__ B, T *__restrict__ C, uint32_t p0,
-            uint32_t n, uint32_t sub, uint32_t nvec)
+            uint32_t n, uint32_t sub, uint32_t nvec,
+            const Odd<T, VPL, RG> &odd)
 {
     using V = typename Vec<T>::type;
     static_assert(NB <= LPR, "batch must fit the lane group");
@@ -253,23 +389,14 @@ sddmm_batch_one(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type (&a
 #pragma unroll
     for (int u = 0; u < NB; ++u) {
         const uint32_t c = __shfl(cme, u, LPR);
-        const V *brow = row_ptr<T, LPR, VPL, RG>(B, c, sub, nvec);
-#pragma unroll
-        for (int v = 0; v < VPL; ++v)
-            b[u][v] = lane_on<LPR, RG>(sub, v, nvec) ? brow[v * LPR] : V{};
+        gather_row<T, LPR, VPL, RG>(b[u], B, c, sub, nvec, odd);
     }
     __builtin_amdgcn_sched_barrier(0); // all gathers in flight before the first use
 
     T part[NB];
 #pragma unroll
     for (int u = 0; u < NB; ++u) {
-        T dot = (T)0;
-#pragma unroll
-        for (int v = 0; v < VPL; ++v)
-#pragma unroll
-            for (int i = 0; i < Vec<T>::N; ++i)
-                dot += a[v][i] * b[u][v][i];
-        part[u] = dot;
+        part[u] = lane_dot<T, VPL, RG>(a, b[u], odd);
     }
     group_reduce<T, LPR, NB>(part, sub);
     const T result = part[0] * sv;
@@ -295,12 +422,13 @@ sddmm_batch_one(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type (&a
     }
 }
 
-template <typename T, int LPR, int VPL, int NB, bool RG, bool MK, int FZ>
+template <typename T, int LPR, int VPL, int NB, int RG, bool MK, int FZ>
 __device__ __forceinline__ void
 sddmm_batch_rounds(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type (&acc)[VPL],
             const uint32_t *__restrict__ col, const uint32_t *__restrict__ perm,
             const T *__restrict__ sval, const T *__restrict__ B, T *__restrict__ C, uint32_t p0,
-            uint32_t n, uint32_t sub, uint32_t nvec)
+            uint32_t n, uint32_t sub, uint32_t nvec,
+            const Odd<T, VPL, RG> &odd)
 {
     using V = typename Vec<T>::type;
     // A group of LPR lanes reduces at most LPR entries at a time: the NB entries of
@@ -338,10 +466,7 @@ sddmm_batch_rounds(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type 
 #pragma unroll
     for (int j = 0; j < NB; ++j) {
         const uint32_t c = __shfl(cme[j / G], j % G, LPR);
-        const V *brow = row_ptr<T, LPR, VPL, RG>(B, c, sub, nvec);
-#pragma unroll
-        for (int v = 0; v < VPL; ++v)
-            b[j][v] = lane_on<LPR, RG>(sub, v, nvec) ? brow[v * LPR] : V{};
+        gather_row<T, LPR, VPL, RG>(b[j], B, c, sub, nvec, odd);
     }
     __builtin_amdgcn_sched_barrier(0); // all gathers in flight before the first use
 
@@ -350,13 +475,7 @@ sddmm_batch_rounds(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type 
         T part[G];
 #pragma unroll
         for (int u = 0; u < G; ++u) {
-            T dot = (T)0;
-#pragma unroll
-            for (int v = 0; v < VPL; ++v)
-#pragma unroll
-                for (int i = 0; i < Vec<T>::N; ++i)
-                    dot += a[v][i] * b[r * G + u][v][i];
-            part[u] = dot;
+            part[u] = lane_dot<T, VPL, RG>(a, b[r * G + u], odd);
         }
         group_reduce<T, LPR, G>(part, sub);
         const T result = part[0] * sv[r];
@@ -388,54 +507,56 @@ sddmm_batch_rounds(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type 
 // R = 1 case of the rounds form, the single round compiles to 24 more VGPRs
 // (100 -> 124 in the wide launch, 62 -> 74 and two wavefronts per SIMD fewer in
 // the short one), which cost the 5-entry rows of a stencil 20 %.
-template <typename T, int LPR, int VPL, int NB, bool RG, bool MK, int FZ>
+template <typename T, int LPR, int VPL, int NB, int RG, bool MK, int FZ>
 __device__ __forceinline__ void
 sddmm_batch(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type (&acc)[VPL],
             const uint32_t *__restrict__ col, const uint32_t *__restrict__ perm,
             const T *__restrict__ sval, const T *__restrict__ B, T *__restrict__ C, uint32_t p0,
-            uint32_t n, uint32_t sub, uint32_t nvec)
+            uint32_t n, uint32_t sub, uint32_t nvec,
+            const Odd<T, VPL, RG> &odd)
 {
     if constexpr (NB <= LPR)
         sddmm_batch_one<T, LPR, VPL, NB, RG, MK, FZ>(a, acc, col, perm, sval, B, C, p0, n, sub,
-                                                     nvec);
+                                                     nvec, odd);
     else
         sddmm_batch_rounds<T, LPR, VPL, NB, RG, MK, FZ>(a, acc, col, perm, sval, B, C, p0, n, sub,
-                                                        nvec);
+                                                        nvec, odd);
 }
 
 // n consecutive entries from p.  WIDE: full batches of UB, then one masked batch
 // of the smallest size in {4, 8, 16} that holds the rest.  !WIDE (segments known
 // to be short, run at twice the occupancy): masked batches of UB throughout.
-template <typename T, int LPR, int VPL, int UB, bool RG, bool WIDE, int FZ>
+template <typename T, int LPR, int VPL, int UB, int RG, bool WIDE, int FZ>
 __device__ __forceinline__ void
 sddmm_walk(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type (&acc)[VPL],
            const uint32_t *__restrict__ col, const uint32_t *__restrict__ perm,
            const T *__restrict__ sval, const T *__restrict__ B, T *__restrict__ C, uint32_t p,
-           uint32_t n, uint32_t sub, uint32_t nvec)
+           uint32_t n, uint32_t sub, uint32_t nvec,
+            const Odd<T, VPL, RG> &odd)
 {
     if constexpr (WIDE) {
         for (; n >= UB; n -= UB, p += UB)
-            sddmm_batch<T, LPR, VPL, UB, RG, false, FZ>(a, acc, col, perm, sval, B, C, p, UB, sub, nvec);
+            sddmm_batch<T, LPR, VPL, UB, RG, false, FZ>(a, acc, col, perm, sval, B, C, p, UB, sub, nvec, odd);
         if (n == 0)
             return;
         if constexpr (UB > 8) {
             if (n > 8) {
-                sddmm_batch<T, LPR, VPL, UB, RG, true, FZ>(a, acc, col, perm, sval, B, C, p, n, sub, nvec);
+                sddmm_batch<T, LPR, VPL, UB, RG, true, FZ>(a, acc, col, perm, sval, B, C, p, n, sub, nvec, odd);
                 return;
             }
         }
         if constexpr (UB > 4) {
             if (n > 4) {
-                sddmm_batch<T, LPR, VPL, 8, RG, true, FZ>(a, acc, col, perm, sval, B, C, p, n, sub, nvec);
+                sddmm_batch<T, LPR, VPL, 8, RG, true, FZ>(a, acc, col, perm, sval, B, C, p, n, sub, nvec, odd);
                 return;
             }
         }
-        sddmm_batch<T, LPR, VPL, (UB < 4 ? UB : 4), RG, true, FZ>(a, acc, col, perm, sval, B, C, p, n, sub, nvec);
+        sddmm_batch<T, LPR, VPL, (UB < 4 ? UB : 4), RG, true, FZ>(a, acc, col, perm, sval, B, C, p, n, sub, nvec, odd);
     } else {
 #pragma nounroll
         while (n > 0) {
             const uint32_t m = n < (uint32_t)UB ? n : (uint32_t)UB;
-            sddmm_batch<T, LPR, VPL, UB, RG, true, FZ>(a, acc, col, perm, sval, B, C, p, m, sub, nvec);
+            sddmm_batch<T, LPR, VPL, UB, RG, true, FZ>(a, acc, col, perm, sval, B, C, p, m, sub, nvec, odd);
             n -= m;
             p += m;
         }
@@ -444,7 +565,7 @@ sddmm_walk(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type (&acc)[V
 
 // FZ != 0: also Y[row,:] += sum of the segment's w_u * B[c_u,:] (partial-sum slot for
 // a cut row, as in spmm_seg_kernel); Y and partial are unused otherwise.
-template <typename T, int LPR, int VPL, int UB, bool RG, bool WIDE, int FZ>
+template <typename T, int LPR, int VPL, int UB, int RG, bool WIDE, int FZ>
 __global__ void __launch_bounds__(kBlock)
 sddmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint32_t rot,
                  const uint32_t *__restrict__ col, const uint32_t *__restrict__ perm,
@@ -461,8 +582,19 @@ sddmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint3
     if (sg[2] == 0)
         return;
 
+    const Odd<T, VPL, RG> odd = odd_lanes<T, LPR, VPL, RG>(sub, nvec);
     V a[VPL], acc[VPL];
-    {
+    if constexpr (RG == 2) {
+        const char *arow = odd_row<T, RG>(A, sg[0], nvec);
+#pragma unroll
+        for (int v = 0; v < VPL; ++v) {
+            a[v] = loose_load_nt<T>(arow + odd.off[v]);
+#pragma unroll
+            for (int i = 0; i < Vec<T>::N; ++i)
+                a[v][i] = odd.keep[v][i] ? a[v][i] : (T)0;
+            acc[v] = V{};
+        }
+    } else {
         const V *arow = row_ptr<T, LPR, VPL, RG>(A, sg[0], sub, nvec);
 #pragma unroll
         for (int v = 0; v < VPL; ++v) {
@@ -471,8 +603,17 @@ sddmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint3
         }
     }
     sddmm_walk<T, LPR, VPL, UB, RG, WIDE, FZ>(a, acc, col, perm, sval, B, C, sg[1], sg[2], sub,
-                                              nvec);
-    if constexpr (FZ != 0) {
+                                              nvec, odd);
+    if constexpr (FZ != 0 && RG == 2) {
+        const bool whole = sg[3] == kWholeRow;
+        char *drow = const_cast<char *>(whole ? odd_row<T, RG>(Y, sg[0], nvec)
+                                              : odd_row<T, RG>(partial, sg[3], nvec));
+        V y0[VPL];
+#pragma unroll
+        for (int v = 0; v < VPL; ++v)
+            y0[v] = whole ? loose_load_nt<T>(drow + odd.off[v]) : V{};
+        odd_store<T, VPL>(drow, whole, y0, acc, odd);
+    } else if constexpr (FZ != 0) {
         const bool whole = sg[3] == kWholeRow;
         V *dst = const_cast<V *>(whole ? row_ptr<T, LPR, VPL, RG>(Y, sg[0], sub, nvec)
                                        : row_ptr<T, LPR, VPL, RG>(partial, sg[3], sub, nvec));
@@ -520,11 +661,12 @@ sddmm_generic_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, u
 // ----------------------------------------------------------------- SpMM ----
 // MK: only the first n of the NB entries exist; the others repeat the loads of
 // entry n - 1 and add zero times zero.
-template <typename T, int LPR, int VPL, int NB, bool RG, bool MK>
+template <typename T, int LPR, int VPL, int NB, int RG, bool MK>
 __device__ __forceinline__ void
 spmm_batch_one(typename Vec<T>::type (&acc)[VPL], const uint32_t *__restrict__ col,
            const T *__restrict__ sval, const T *__restrict__ X, uint32_t p0, uint32_t n,
-           uint32_t sub, uint32_t nvec)
+           uint32_t sub, uint32_t nvec,
+            const Odd<T, VPL, RG> &odd)
 {
     using V = typename Vec<T>::type;
     static_assert(NB <= LPR, "batch must fit the lane group");
@@ -540,10 +682,7 @@ spmm_batch_one(typename Vec<T>::type (&acc)[VPL], const uint32_t *__restrict__ c
     for (int u = 0; u < NB; ++u) {
         const uint32_t c = __shfl(cme, u, LPR);
         av[u] = __shfl(vme, u, LPR);
-        const V *xrow = row_ptr<T, LPR, VPL, RG>(X, c, sub, nvec);
-#pragma unroll
-        for (int v = 0; v < VPL; ++v)
-            x[u][v] = lane_on<LPR, RG>(sub, v, nvec) ? xrow[v * LPR] : V{};
+        gather_row<T, LPR, VPL, RG>(x[u], X, c, sub, nvec, odd);
     }
     __builtin_amdgcn_sched_barrier(0); // all gathers in flight before the first use
     // Entries are added in kernel order.
@@ -557,11 +696,12 @@ spmm_batch_one(typename Vec<T>::type (&acc)[VPL], const uint32_t *__restrict__ c
     }
 }
 
-template <typename T, int LPR, int VPL, int NB, bool RG, bool MK>
+template <typename T, int LPR, int VPL, int NB, int RG, bool MK>
 __device__ __forceinline__ void
 spmm_batch_rounds(typename Vec<T>::type (&acc)[VPL], const uint32_t *__restrict__ col,
            const T *__restrict__ sval, const T *__restrict__ X, uint32_t p0, uint32_t n,
-           uint32_t sub, uint32_t nvec)
+           uint32_t sub, uint32_t nvec,
+            const Odd<T, VPL, RG> &odd)
 {
     using V = typename Vec<T>::type;
     // Lane u of the group fetches column and value of entry u of each of the R rounds
@@ -586,10 +726,7 @@ spmm_batch_rounds(typename Vec<T>::type (&acc)[VPL], const uint32_t *__restrict_
     for (int j = 0; j < NB; ++j) {
         const uint32_t c = __shfl(cme[j / G], j % G, LPR);
         av[j] = __shfl(vme[j / G], j % G, LPR);
-        const V *xrow = row_ptr<T, LPR, VPL, RG>(X, c, sub, nvec);
-#pragma unroll
-        for (int v = 0; v < VPL; ++v)
-            x[j][v] = lane_on<LPR, RG>(sub, v, nvec) ? xrow[v * LPR] : V{};
+        gather_row<T, LPR, VPL, RG>(x[j], X, c, sub, nvec, odd);
     }
     __builtin_amdgcn_sched_barrier(0); // all gathers in flight before the first use
     // Entries are added in kernel order.
@@ -603,23 +740,25 @@ spmm_batch_rounds(typename Vec<T>::type (&acc)[VPL], const uint32_t *__restrict_
     }
 }
 
-template <typename T, int LPR, int VPL, int NB, bool RG, bool MK>
+template <typename T, int LPR, int VPL, int NB, int RG, bool MK>
 __device__ __forceinline__ void
 spmm_batch(typename Vec<T>::type (&acc)[VPL], const uint32_t *__restrict__ col,
            const T *__restrict__ sval, const T *__restrict__ X, uint32_t p0, uint32_t n,
-           uint32_t sub, uint32_t nvec)
+           uint32_t sub, uint32_t nvec,
+            const Odd<T, VPL, RG> &odd)
 {
     if constexpr (NB <= LPR)
-        spmm_batch_one<T, LPR, VPL, NB, RG, MK>(acc, col, sval, X, p0, n, sub, nvec);
+        spmm_batch_one<T, LPR, VPL, NB, RG, MK>(acc, col, sval, X, p0, n, sub, nvec, odd);
     else
-        spmm_batch_rounds<T, LPR, VPL, NB, RG, MK>(acc, col, sval, X, p0, n, sub, nvec);
+        spmm_batch_rounds<T, LPR, VPL, NB, RG, MK>(acc, col, sval, X, p0, n, sub, nvec, odd);
 }
 
-template <typename T, int LPR, int VPL, int UB, bool RG, bool WIDE>
+template <typename T, int LPR, int VPL, int UB, int RG, bool WIDE>
 __device__ __forceinline__ void
 spmm_walk(typename Vec<T>::type (&acc)[VPL], const uint32_t *__restrict__ col,
           const T *__restrict__ sval, const T *__restrict__ X, uint32_t p, uint32_t n,
-          uint32_t sub, uint32_t nvec)
+          uint32_t sub, uint32_t nvec,
+            const Odd<T, VPL, RG> &odd)
 {
     // Short segments: exact batches of UB, then UB/2 ... 1 as n requires.  Measured
     // against masked batches here (which cost registers, hence occupancy): 3 % faster
@@ -627,47 +766,47 @@ spmm_walk(typename Vec<T>::type (&acc)[VPL], const uint32_t *__restrict__ col,
     // read-modify-write stream, not by rounds of gathers.
     if constexpr (!WIDE) {
         for (; n >= UB; n -= UB, p += UB)
-            spmm_batch<T, LPR, VPL, UB, RG, false>(acc, col, sval, X, p, UB, sub, nvec);
+            spmm_batch<T, LPR, VPL, UB, RG, false>(acc, col, sval, X, p, UB, sub, nvec, odd);
         if constexpr (UB > 8)
             if (n & 8) {
-                spmm_batch<T, LPR, VPL, 8, RG, false>(acc, col, sval, X, p, 8, sub, nvec);
+                spmm_batch<T, LPR, VPL, 8, RG, false>(acc, col, sval, X, p, 8, sub, nvec, odd);
                 p += 8;
             }
         if constexpr (UB > 4)
             if (n & 4) {
-                spmm_batch<T, LPR, VPL, 4, RG, false>(acc, col, sval, X, p, 4, sub, nvec);
+                spmm_batch<T, LPR, VPL, 4, RG, false>(acc, col, sval, X, p, 4, sub, nvec, odd);
                 p += 4;
             }
         if constexpr (UB > 2)
             if (n & 2) {
-                spmm_batch<T, LPR, VPL, 2, RG, false>(acc, col, sval, X, p, 2, sub, nvec);
+                spmm_batch<T, LPR, VPL, 2, RG, false>(acc, col, sval, X, p, 2, sub, nvec, odd);
                 p += 2;
             }
         if constexpr (UB > 1)
             if (n & 1)
-                spmm_batch<T, LPR, VPL, 1, RG, false>(acc, col, sval, X, p, 1, sub, nvec);
+                spmm_batch<T, LPR, VPL, 1, RG, false>(acc, col, sval, X, p, 1, sub, nvec, odd);
     } else {
         for (; n >= UB; n -= UB, p += UB)
-            spmm_batch<T, LPR, VPL, UB, RG, false>(acc, col, sval, X, p, UB, sub, nvec);
+            spmm_batch<T, LPR, VPL, UB, RG, false>(acc, col, sval, X, p, UB, sub, nvec, odd);
         if (n == 0)
             return;
         if constexpr (UB > 8) {
             if (n > 8) {
-                spmm_batch<T, LPR, VPL, UB, RG, true>(acc, col, sval, X, p, n, sub, nvec);
+                spmm_batch<T, LPR, VPL, UB, RG, true>(acc, col, sval, X, p, n, sub, nvec, odd);
                 return;
             }
         }
         if constexpr (UB > 4) {
             if (n > 4) {
-                spmm_batch<T, LPR, VPL, 8, RG, true>(acc, col, sval, X, p, n, sub, nvec);
+                spmm_batch<T, LPR, VPL, 8, RG, true>(acc, col, sval, X, p, n, sub, nvec, odd);
                 return;
             }
         }
-        spmm_batch<T, LPR, VPL, (UB < 4 ? UB : 4), RG, true>(acc, col, sval, X, p, n, sub, nvec);
+        spmm_batch<T, LPR, VPL, (UB < 4 ? UB : 4), RG, true>(acc, col, sval, X, p, n, sub, nvec, odd);
     }
 }
 
-template <typename T, int LPR, int VPL, int UB, bool RG, bool WIDE>
+template <typename T, int LPR, int VPL, int UB, int RG, bool WIDE>
 __global__ void __launch_bounds__(kBlock)
 spmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint32_t rot,
                 const uint32_t *__restrict__ col, const T *__restrict__ sval,
@@ -684,8 +823,7 @@ spmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint32
     if (sg[2] == 0)
         return;
     const bool whole = sg[3] == kWholeRow;
-    V *dst = const_cast<V *>(whole ? row_ptr<T, LPR, VPL, RG>(Y, sg[0], sub, nvec)
-                                   : row_ptr<T, LPR, VPL, RG>(partial, sg[3], sub, nvec));
+    const Odd<T, VPL, RG> odd = odd_lanes<T, LPR, VPL, RG>(sub, nvec);
 
     V acc[VPL], y0[VPL];
 #pragma unroll
@@ -693,21 +831,35 @@ spmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint32
         acc[v] = V{};
         y0[v] = V{};
     }
-    if (whole) {
+    if constexpr (RG == 2) {
+        char *drow = const_cast<char *>(whole ? odd_row<T, RG>(Y, sg[0], nvec)
+                                              : odd_row<T, RG>(partial, sg[3], nvec));
+        if (whole) {
 #pragma unroll
-        for (int v = 0; v < VPL; ++v)
-            if (lane_on<LPR, RG>(sub, v, nvec))
-                y0[v] = nt_load(dst + v * LPR);
-    }
-    spmm_walk<T, LPR, VPL, UB, RG, WIDE>(acc, col, sval, X, sg[1], sg[2], sub, nvec);
+            for (int v = 0; v < VPL; ++v)
+                y0[v] = loose_load_nt<T>(drow + odd.off[v]);
+        }
+        spmm_walk<T, LPR, VPL, UB, RG, WIDE>(acc, col, sval, X, sg[1], sg[2], sub, nvec, odd);
+        odd_store<T, VPL>(drow, whole, y0, acc, odd);
+    } else {
+        V *dst = const_cast<V *>(whole ? row_ptr<T, LPR, VPL, RG>(Y, sg[0], sub, nvec)
+                                       : row_ptr<T, LPR, VPL, RG>(partial, sg[3], sub, nvec));
+        if (whole) {
 #pragma unroll
-    for (int v = 0; v < VPL; ++v) {
-        if (!lane_on<LPR, RG>(sub, v, nvec))
-            continue;
-        if (whole)
-            nt_store(y0[v] + acc[v], dst + v * LPR);
-        else
-            dst[v * LPR] = acc[v]; // read back by spmm_fixup right after
+            for (int v = 0; v < VPL; ++v)
+                if (lane_on<LPR, RG>(sub, v, nvec))
+                    y0[v] = nt_load(dst + v * LPR);
+        }
+        spmm_walk<T, LPR, VPL, UB, RG, WIDE>(acc, col, sval, X, sg[1], sg[2], sub, nvec, odd);
+#pragma unroll
+        for (int v = 0; v < VPL; ++v) {
+            if (!lane_on<LPR, RG>(sub, v, nvec))
+                continue;
+            if (whole)
+                nt_store(y0[v] + acc[v], dst + v * LPR);
+            else
+                dst[v * LPR] = acc[v]; // read back by spmm_fixup right after
+        }
     }
 }
 
@@ -872,37 +1024,41 @@ copy_kernel(u32x4 *__restrict__ dst, const u32x4 *__restrict__ src, uint64_t nve
 // ------------------------------------------------------------- dispatch ----
 struct Shape {
     int lpr, vpl;  // lpr == 0: generic kernel
-    bool ragged;   // fewer vectors per row than lpr * vpl
-    uint32_t nvec; // 16-byte vectors per dense row
+    int mode;      // the kernels' RG: 0 exact, 1 ragged, 2 odd
+    uint32_t nvec; // 16-byte vectors per dense row; mode 2: K, the reals per row
 };
 
-// A dense row of K reals must be a whole number nvec <= 256 of 16-byte vectors;
-// anything else takes the generic kernels.  nvec == LPR * VPL with LPR a power of
-// two in [4, 64] and VPL in {1, 2, 4} runs a kernel with the row stride compiled
-// in; other nvec run the "ragged" variant of the smallest shape that covers a row,
-// in which the lanes past the row's end idle.
+// A dense row of K reals of at least 16 and at most 4096 bytes runs the vector
+// kernels; anything else takes the generic ones.  A whole number nvec of 16-byte
+// vectors with nvec == LPR * VPL, LPR a power of two in [4, 64] and VPL in {1, 2, 4},
+// runs a kernel with the row stride compiled in; other nvec run the "ragged" variant
+// of the smallest shape that covers a row, in which the lanes past the row's end
+// idle; rows that are no whole number of vectors run the "odd" variant of that shape.
 Shape pick_shape(size_t elem, uint32_t K)
 {
     const size_t bytes = (size_t)K * elem;
-    if (K == 0 || bytes % 16 || bytes / 16 > 256)
-        return {0, 0, false, 0};
-    const uint32_t nvec = (uint32_t)(bytes / 16);
-    for (int lpr = 64; lpr >= 4; lpr >>= 1) {
+    if (bytes < 16 || bytes > 4096)
+        return {0, 0, 0, 0};
+    const uint32_t nvec = (uint32_t)((bytes + 15) / 16);
+    const bool odd = bytes % 16 != 0;
+    for (int lpr = 64; lpr >= 4 && !odd; lpr >>= 1) {
         if (nvec % lpr)
             continue;
         const uint32_t vpl = nvec / lpr;
         if (vpl == 1 || vpl == 2 || vpl == 4)
-            return {lpr, (int)vpl, false, nvec};
+            return {lpr, (int)vpl, 0, nvec};
         break;
     }
+    const int mode = odd ? 2 : 1;
+    const uint32_t arg = odd ? K : nvec;
     if (nvec > 128)
-        return {64, 4, true, nvec};
+        return {64, 4, mode, arg};
     if (nvec > 64)
-        return {64, 2, true, nvec};
+        return {64, 2, mode, arg};
     int lpr = 4;
     while ((uint32_t)lpr < nvec)
         lpr *= 2;
-    return {lpr, 1, true, nvec};
+    return {lpr, 1, mode, arg};
 }
 
 // Workgroups needed to cover nseg segments (a whole number of chunks, and of
@@ -951,7 +1107,7 @@ inline hipError_t join_aux(const Streams &S)
     return hipStreamSynchronize(S.aux);
 }
 
-template <typename T, int LPR, int VPL, int UB, int US, bool RG, int FZ>
+template <typename T, int LPR, int VPL, int UB, int US, int RG, int FZ>
 hipError_t run_sddmm(const DevPlanView &P, const T *A, const T *B, T *C, T *Y, const Streams &S,
                      uint32_t nvec)
 {
@@ -975,7 +1131,7 @@ hipError_t run_sddmm(const DevPlanView &P, const T *A, const T *B, T *C, T *Y, c
     return launched != hipSuccess ? launched : joined;
 }
 
-template <typename T, int LPR, int VPL, int UB, int US, bool RG>
+template <typename T, int LPR, int VPL, int UB, int US, int RG>
 hipError_t run_spmm(const DevPlanView &P, const T *X, T *Y, const Streams &S, uint32_t nvec)
 {
     uint32_t nl = P.nseg_long, ns = P.nseg - P.nseg_long;
@@ -1038,17 +1194,19 @@ hipError_t sddmm_typed(const DevPlanView &P, const void *A, const void *B, void 
     bool done = false;
     hipError_t e = hipSuccess;
 #define X(L, V, U, S, S2)                                                                         \
-    if (!done && !sh.ragged && sh.lpr == L && sh.vpl == V) {                                      \
-        e = run_sddmm<T, L, V, U, S, false, FZ>(P, (const T *)A, (const T *)B, (T *)C, (T *)Y,    \
-                                                SS, sh.nvec);                                     \
+    if (!done && sh.mode == 0 && sh.lpr == L && sh.vpl == V) {                                    \
+        e = run_sddmm<T, L, V, U, S, 0, FZ>(P, (const T *)A, (const T *)B, (T *)C, (T *)Y, SS,    \
+                                            sh.nvec);                                             \
         done = true;                                                                              \
     }
     SPC3D_FOR_SHAPES(X)
 #undef X
 #define X(L, V, U, S, S2)                                                                         \
-    if (!done && sh.ragged && sh.lpr == L && sh.vpl == V) {                                       \
-        e = run_sddmm<T, L, V, U, S, true, FZ>(P, (const T *)A, (const T *)B, (T *)C, (T *)Y, SS, \
-                                               sh.nvec);                                          \
+    if (!done && sh.mode != 0 && sh.lpr == L && sh.vpl == V) {                                    \
+        e = sh.mode == 1 ? run_sddmm<T, L, V, U, S, 1, FZ>(P, (const T *)A, (const T *)B,         \
+                                                           (T *)C, (T *)Y, SS, sh.nvec)           \
+                         : run_sddmm<T, L, V, U, S, 2, FZ>(P, (const T *)A, (const T *)B,         \
+                                                           (T *)C, (T *)Y, SS, sh.nvec);          \
         done = true;                                                                              \
     }
     SPC3D_FOR_RAGGED_SHAPES(X)
@@ -1078,15 +1236,16 @@ hipError_t spmm_typed(const DevPlanView &P, const void *X_, void *Y, uint32_t K,
     bool done = false;
     hipError_t e = hipSuccess;
 #define X(L, V, U, S, S2)                                                                         \
-    if (!done && !sh.ragged && sh.lpr == L && sh.vpl == V) {                                      \
-        e = run_spmm<T, L, V, U, S2, false>(P, (const T *)X_, (T *)Y, SS, sh.nvec);               \
+    if (!done && sh.mode == 0 && sh.lpr == L && sh.vpl == V) {                                    \
+        e = run_spmm<T, L, V, U, S2, 0>(P, (const T *)X_, (T *)Y, SS, sh.nvec);                   \
         done = true;                                                                              \
     }
     SPC3D_FOR_SHAPES(X)
 #undef X
 #define X(L, V, U, S, S2)                                                                         \
-    if (!done && sh.ragged && sh.lpr == L && sh.vpl == V) {                                       \
-        e = run_spmm<T, L, V, U, S2, true>(P, (const T *)X_, (T *)Y, SS, sh.nvec);                \
+    if (!done && sh.mode != 0 && sh.lpr == L && sh.vpl == V) {                                    \
+        e = sh.mode == 1 ? run_spmm<T, L, V, U, S2, 1>(P, (const T *)X_, (T *)Y, SS, sh.nvec)     \
+                         : run_spmm<T, L, V, U, S2, 2>(P, (const T *)X_, (T *)Y, SS, sh.nvec);    \
         done = true;                                                                              \
     }
     SPC3D_FOR_RAGGED_SHAPES(X)
@@ -1229,7 +1388,7 @@ const char *kernel_variant(int dtype, uint32_t K)
         snprintf(buf, sizeof buf, "generic<%s>", dtype == 1 ? "f64" : "f32");
     else
         snprintf(buf, sizeof buf, "seg<%s,LPR=%d,VPL=%d%s>", dtype == 1 ? "f64" : "f32", sh.lpr,
-                 sh.vpl, sh.ragged ? ",ragged" : "");
+                 sh.vpl, sh.mode == 1 ? ",ragged" : (sh.mode == 2 ? ",odd" : ""));
     return buf;
 }
 

@@ -107,10 +107,12 @@ def test_golden_numcheck_closed_form(ctx):
 
 # ---- K sweep: rows that fill a kernel shape exactly (a power of two of 16-byte
 # vectors), rows that do not (the "ragged" variants: 12, 20, 48, 100, 300 ...), rows
-# that are no whole number of vectors or longer than 4 KiB (the generic kernels)
+# that are no whole number of vectors (the "odd" variants: 5, 7, 50, 63, 65, 1023 ...),
+# rows shorter than 16 bytes or longer than 4 KiB (the generic kernels)
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("k", [1, 2, 3, 4, 6, 8, 10, 12, 16, 20, 24, 32, 36, 48, 64, 72, 96, 100,
-                               128, 130, 200, 256, 300, 384, 512, 1024, 1028])
+@pytest.mark.parametrize("k", [1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 15, 16, 17, 20, 24, 31, 32,
+                               33, 36, 48, 50, 63, 64, 65, 72, 96, 100, 127, 128, 129, 130, 200,
+                               255, 256, 257, 300, 384, 511, 512, 513, 1023, 1024, 1025, 1028])
 def test_k_sweep_random_unsorted(ctx, dtype, k):
     ii, jj, vv, A, B, Y0 = rand_case(100 + k, 300, 257, k, 6000, dtype, hub=700)
     check_sddmm(A, B, ii, jj, vv, gpu_sddmm(ctx, 300, 257, ii, jj, vv, A, B, prefill=-5.0))
@@ -126,9 +128,10 @@ def test_segment_lengths_and_cut_rows(ctx, dtype, seg_max):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("k", [12, 48, 100, 136, 264])
+@pytest.mark.parametrize("k", [5, 7, 12, 48, 50, 63, 65, 100, 129, 136, 257, 264, 511])
 def test_cut_rows_with_ragged_k(ctx, dtype, k):
     # partial rows of cut segments and the fix-up pass at row widths that leave lanes idle
+    # or end inside a 16-byte vector
     ii, jj, vv, A, B, Y0 = rand_case(11 + k, 40, 300, k, 4000, dtype, hub=1500)
     check_sddmm(A, B, ii, jj, vv, gpu_sddmm(ctx, 40, 300, ii, jj, vv, A, B, seg_max=64))
     check_spmm(B, ii, jj, vv, Y0, gpu_spmm(ctx, 40, 300, ii, jj, vv, B, Y0, seg_max=64))
@@ -137,7 +140,7 @@ def test_cut_rows_with_ragged_k(ctx, dtype, k):
 # ---- both kernels in one pass over the gathered rows ---------------------------------
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("chained", [False, True])
-@pytest.mark.parametrize("k", [4, 20, 64, 100, 256])
+@pytest.mark.parametrize("k", [4, 5, 20, 50, 63, 64, 100, 256, 257, 511])
 def test_fused_sddmm_spmm_equals_the_two_calls(ctx, dtype, chained, k):
     m, n, nnz = 120, 90, 4000
     ii, jj, vv, A, B, Y0 = rand_case(500 + k, m, n, k, nnz, dtype, hub=900)
@@ -173,7 +176,7 @@ def test_fused_call_on_the_sliced_layout_and_odd_widths(ctx, dtype):
     check_sddmm(A, B, w.ii, w.jj, vv, dC.download())
     check_spmm(B, w.ii, w.jj, dC.download(), Y0, dY.download())
     # K without a vector kernel: the plain form falls back to the two calls, the chained one refuses
-    ii, jj, vv, A, B, Y0 = rand_case(3, 30, 30, 5, 200, dtype)
+    ii, jj, vv, A, B, Y0 = rand_case(3, 30, 30, 1, 200, dtype)
     S2 = ctx.plan(30, 30, ii, jj, vv)
     dA, dB, dY, dC = ctx.panel_from(A), ctx.panel_from(B), ctx.panel_from(Y0), ctx.vals(200, dtype)
     ctx.sddmm_spmm(S2, dA, dB, dC, dY)
@@ -191,7 +194,8 @@ def test_random_shapes_widths_and_plan_options(ctx, dtype):
     for case in range(40):
         m, n = int(rng.integers(1, 300)), int(rng.integers(40, 300))
         nnz = int(rng.integers(1, 5000))
-        k = int(rng.choice([1, 2, 4, 5, 8, 12, 16, 24, 32, 40, 64, 68, 96, 128, 160, 256, 516]))
+        k = int(rng.choice([1, 2, 4, 5, 7, 8, 12, 16, 19, 24, 32, 40, 50, 64, 65, 68, 96, 127, 128, 160,
+                            250, 256, 516, 1030]))
         ii = np.minimum(rng.pareto(0.7, nnz).astype(np.int64), m - 1).astype(np.uint32)
         jj = np.minimum((rng.pareto(0.5, nnz) * 3).astype(np.int64), n - 1).astype(np.uint32)
         if rng.random() < 0.5:
@@ -220,7 +224,7 @@ def test_random_shapes_widths_and_plan_options(ctx, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("k", [64, 20])
+@pytest.mark.parametrize("k", [64, 20, 50, 7, 129])
 def test_rows_the_pattern_never_names_are_never_read(ctx, dtype, k):
     # the reference touches A[ii[e]], B[jj[e]] and Y[ii[e]] only (core_ops.cpp:16,32): NaN
     # in every other dense row must not reach any result, whatever the batching loads
@@ -241,9 +245,12 @@ def test_rows_the_pattern_never_names_are_never_read(ctx, dtype, k):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_non_finite_inputs_propagate_as_in_the_reference(ctx, dtype):
+@pytest.mark.parametrize("k", [64, 50, 7, 129])
+def test_non_finite_inputs_propagate_as_in_the_reference(ctx, dtype, k):
     # an infinite X row named with weight a gives a * inf in Y, not NaN from 0 * inf
-    m, n, k = 8, 8, 64
+    # (nor, at widths that end inside a vector, from the elements a lane loads but does
+    # not count)
+    m, n = 8, 8
     ii = np.array([0, 0, 0, 0, 0, 3], dtype=np.uint32)
     jj = np.array([1, 2, 3, 4, 5, 5], dtype=np.uint32)
     vv = np.array([1, 1, 1, 1, 2, 1], dtype=dtype)
@@ -253,6 +260,20 @@ def test_non_finite_inputs_propagate_as_in_the_reference(ctx, dtype):
     assert np.all(np.isposinf(Y[0])) and np.all(np.isposinf(Y[3])) and np.all(Y[1] == 0)
     C = gpu_sddmm(ctx, m, n, ii, jj, vv, np.ones((m, k), dtype=dtype), X)
     assert np.array_equal(C[:4], np.full(4, k, dtype=dtype)) and np.all(np.isposinf(C[4:]))
+    # one infinite element at a time, in each of the last positions of a row (those a lane
+    # may hold twice at such widths): inf in C and in that one element of Y, never NaN
+    for back in range(1, min(k, 5)):
+        X = np.ones((n, k), dtype=dtype)
+        X[6, k - back] = np.inf
+        A = np.ones((m, k), dtype=dtype)
+        A[2, k - back] = np.inf
+        ii2, jj2 = np.array([1, 2], dtype=np.uint32), np.array([6, 0], dtype=np.uint32)
+        C = gpu_sddmm(ctx, m, n, ii2, jj2, np.ones(2, dtype=dtype), A, X)
+        assert np.all(np.isposinf(C)), (back, C)
+        Y = gpu_spmm(ctx, m, n, ii2, jj2, np.ones(2, dtype=dtype), X, np.zeros((m, k), dtype=dtype))
+        want = np.zeros((m, k), dtype=dtype)
+        want[1], want[2] = X[6], X[0]
+        assert np.array_equal(Y, want), back
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
