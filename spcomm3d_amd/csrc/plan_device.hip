@@ -23,7 +23,7 @@ struct Counters { // one device-resident block, zeroed (first_bad: all ones) bef
     uint32_t not_identity;
     uint32_t qcount[kSlices], qlong[kSlices];
     uint32_t nlong;
-    uint32_t pad;
+    uint32_t rows_unsorted;
     unsigned long long covered;
     unsigned long long load[kSlices];
     unsigned long long any_load;
@@ -57,11 +57,79 @@ template <typename T> struct DBuf {
     }
 };
 
+// Scratch device memory of one call: a few large blocks, handed out front to back
+// and freed together when the call returns.  (hipFree waits for the device: forty
+// hipMalloc / hipFree pairs per build cost more than all of its kernels.)
+class Arena {
+  public:
+    Arena() = default;
+    Arena(const Arena &) = delete;
+    Arena &operator=(const Arena &) = delete;
+    ~Arena()
+    {
+        for (int i = 0; i < nblocks_; ++i)
+            (void)hipFree(blocks_[i]);
+    }
+    // Makes sure that the next `bytes` come out of one block.
+    hipError_t reserve(size_t bytes)
+    {
+        if (bytes <= left_)
+            return hipSuccess;
+        if (nblocks_ == kMaxBlocks)
+            return hipErrorOutOfMemory;
+        void *b = nullptr;
+        const hipError_t e = hipMalloc(&b, bytes);
+        if (e != hipSuccess)
+            return e;
+        blocks_[nblocks_++] = b;
+        cur_ = static_cast<char *>(b);
+        left_ = bytes;
+        return hipSuccess;
+    }
+    hipError_t take(void **p, size_t bytes)
+    {
+        *p = nullptr;
+        if (bytes == 0)
+            return hipSuccess;
+        bytes = (bytes + 255) / 256 * 256;
+        const hipError_t e = reserve(bytes > left_ && bytes < kMinBlock ? kMinBlock : bytes);
+        if (e != hipSuccess)
+            return e;
+        *p = cur_;
+        cur_ += bytes;
+        left_ -= bytes;
+        return hipSuccess;
+    }
+
+  private:
+    static constexpr int kMaxBlocks = 64;
+    static constexpr size_t kMinBlock = (size_t)4 << 20;
+    void *blocks_[kMaxBlocks] = {};
+    int nblocks_ = 0;
+    char *cur_ = nullptr;
+    size_t left_ = 0;
+};
+
+// An array in the arena; nothing to free.
+template <typename T> struct SBuf {
+    T *p = nullptr;
+    hipError_t alloc(Arena &a, size_t count)
+    {
+        return a.take(reinterpret_cast<void **>(&p), count * sizeof(T));
+    }
+};
+
 inline uint32_t grid_for(uint64_t n)
 {
     const uint64_t want = (n + kTB - 1) / kTB;
     const uint64_t cap = 256 * 32;
     return (uint32_t)(want < 1 ? 1 : (want > cap ? cap : want));
+}
+
+inline uint32_t small_grid_for(uint64_t n) // kernels that end in one atomic per workgroup
+{
+    const uint32_t g = grid_for(n);
+    return g > 1024 ? 1024 : g;
 }
 
 inline int bits_for(uint64_t max_value) // bits needed to hold max_value (at least 1)
@@ -81,6 +149,43 @@ template <typename T> __device__ __forceinline__ T wave_sum(T v)
     for (int s = 32; s >= 1; s >>= 1)
         v += __shfl_xor(v, s, 64);
     return v;
+}
+
+// Sum (maximum) of v over the workgroup, valid in thread 0; every thread of the
+// workgroup calls.  The kernels that count into the Counters block add one value
+// per workgroup and run on a small grid: device-wide atomics on a handful of
+// addresses are served one after the other, and one per wavefront of a full-size
+// grid cost more than the rest of the kernel.
+template <typename T> __device__ __forceinline__ T block_sum(T v)
+{
+    __shared__ T part[kTB / 64];
+    v = wave_sum(v);
+    __syncthreads(); // an earlier call's part[] has been read
+    if ((threadIdx.x & 63) == 0)
+        part[threadIdx.x >> 6] = v;
+    __syncthreads();
+    T t = 0;
+    if (threadIdx.x == 0)
+        for (int w = 0; w < kTB / 64; ++w)
+            t += part[w];
+    return t;
+}
+__device__ __forceinline__ uint32_t block_max(uint32_t v)
+{
+    __shared__ uint32_t part[kTB / 64];
+    for (int s = 32; s >= 1; s >>= 1) {
+        const uint32_t o = __shfl_xor(v, s, 64);
+        v = v > o ? v : o;
+    }
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0)
+        part[threadIdx.x >> 6] = v;
+    __syncthreads();
+    uint32_t t = 0;
+    if (threadIdx.x == 0)
+        for (int w = 0; w < kTB / 64; ++w)
+            t = t > part[w] ? t : part[w];
+    return t;
 }
 
 template <typename T> __global__ void fill_k(T *p, uint64_t n, T v)
@@ -111,27 +216,66 @@ __device__ __forceinline__ void count_runs(uint32_t *cnt, uint32_t key, bool val
     }
 }
 
-// Row and column histograms; the first out-of-range entry, if any.
-__global__ void hist_k(const uint32_t *__restrict__ ii, const uint32_t *__restrict__ jj,
-                       uint64_t nnz, uint32_t nrows, uint32_t ncols, uint32_t *rowcnt,
-                       uint32_t *coldeg, Counters *C)
+// The first out-of-range entry, if any; whether the rows ever step down.
+__global__ void check_k(const uint32_t *__restrict__ ii, const uint32_t *__restrict__ jj,
+                        uint64_t nnz, uint32_t nrows, uint32_t ncols, Counters *C)
 {
-    // whole wavefronts walk the entries together, so that lanes can pool their counts
+    uint32_t bad = 0xFFFFFFFFu;
+    int down = 0;
+    GRID_STRIDE(e, nnz)
+    {
+        const uint32_t r = ii[e];
+        if ((r >= nrows || jj[e] >= ncols) && (uint32_t)e < bad)
+            bad = (uint32_t)e;
+        down |= e > 0 && ii[e - 1] > r;
+    }
+    if (bad != 0xFFFFFFFFu)
+        atomicMin(&C->first_bad, bad); // rare: the build fails
+    down = __syncthreads_or(down);
+    if (threadIdx.x == 0 && down)
+        atomicOr(&C->rows_unsorted, 1u);
+}
+
+// Row histogram of entries sorted by row: whole wavefronts walk the entries
+// together and pool their counts, one atomic per run of equal rows.
+__global__ void hist_sorted_k(const uint32_t *__restrict__ ii, uint64_t nnz, uint32_t *rowcnt)
+{
     const uint64_t stride = (uint64_t)gridDim.x * kTB;
     for (uint64_t base = (uint64_t)blockIdx.x * kTB + (threadIdx.x & ~63u); base < nnz;
          base += stride) {
         const uint64_t e = base + (threadIdx.x & 63u);
-        uint32_t r = 0, c = 0;
-        bool ok = false;
-        if (e < nnz) {
-            r = ii[e];
-            c = jj[e];
-            ok = r < nrows && c < ncols;
-            if (!ok)
-                atomicMin(&C->first_bad, (uint32_t)e);
-        }
-        count_runs(rowcnt, r, ok);
-        count_runs(coldeg, c, ok);
+        const bool ok = e < nnz;
+        count_runs(rowcnt, ok ? ii[e] : 0u, ok);
+    }
+}
+
+// Histogram from sorted ids: the columns', and the rows' of a pattern that is not
+// sorted by row (a device-wide atomic per entry is served at the memory side, 1.5 ms
+// for 16 M entries; the radix sort and these two passes take a third of that).
+// Where a run of equal ids starts, its position goes to start[id]; where it ends,
+// the position after it goes to deg[id] (zeroed before); deg[id] -= start[id] then
+// leaves the run's length.  The ids were checked against nbins before.
+__global__ void run_bounds_k(const uint32_t *__restrict__ sorted, uint64_t n, uint32_t nbins,
+                             uint32_t *start, uint32_t *deg)
+{
+    GRID_STRIDE(i, n)
+    {
+        const uint32_t k = sorted[i];
+        if (k >= nbins)
+            continue;
+        if (i == 0 || sorted[i - 1] != k)
+            start[k] = (uint32_t)i;
+        if (i + 1 == n || sorted[i + 1] != k)
+            deg[k] = (uint32_t)(i + 1);
+    }
+}
+__global__ void run_lengths_k(const uint32_t *__restrict__ start, uint64_t nbins, uint32_t *deg)
+{
+    GRID_STRIDE(c, nbins)
+    {
+        const uint32_t end = deg[c];
+        if (end)
+            deg[c] = end - start[c];
     }
 }
 
@@ -146,12 +290,9 @@ __global__ void stats_k(const uint32_t *__restrict__ cnt, uint64_t n, uint32_t *
         t += v != 0;
         m = m > v ? m : v;
     }
-    for (int s = 32; s >= 1; s >>= 1) {
-        t += __shfl_xor(t, s, 64);
-        const uint32_t o = __shfl_xor(m, s, 64);
-        m = m > o ? m : o;
-    }
-    if ((threadIdx.x & 63) == 0) {
+    t = block_sum(t);
+    m = block_max(m);
+    if (threadIdx.x == 0) {
         if (t)
             atomicAdd(touched, t);
         if (m)
@@ -163,9 +304,8 @@ __global__ void sum_first_k(const uint32_t *__restrict__ v, uint64_t n, unsigned
 {
     unsigned long long s = 0;
     GRID_STRIDE(i, n) s += v[i];
-    for (int k = 32; k >= 1; k >>= 1)
-        s += __shfl_xor(s, k, 64);
-    if ((threadIdx.x & 63) == 0 && s)
+    s = block_sum(s);
+    if (threadIdx.x == 0 && s)
         atomicAdd(out, s);
 }
 
@@ -183,17 +323,43 @@ __global__ void hubflag_k(const uint32_t *__restrict__ rowcnt, uint32_t nrows, u
     GRID_STRIDE(r, (uint64_t)nrows + 1) flag[r] = (r < nrows && rowcnt[r] >= hub_min) ? 1u : 0u;
 }
 
-// Per hub row, the number of entries in each of the 9 groups.
+// Per hub row, the number of entries in each of the 9 groups.  Whole wavefronts
+// walk the entries together: per group, the lanes that share the row of the first
+// such lane add their count with one atomic (sorted COO puts a wavefront on one or
+// two rows), the others one each.
 __global__ void hubcount_k(const uint32_t *__restrict__ ii, const uint32_t *__restrict__ jj,
                            uint64_t nnz, const uint32_t *__restrict__ hubflag,
                            const uint32_t *__restrict__ hubpos, const uint8_t *__restrict__ cls,
                            uint32_t *hubcnt)
 {
-    GRID_STRIDE(e, nnz)
-    {
-        const uint32_t r = ii[e];
-        if (hubflag[r])
-            atomicAdd(hubcnt + (size_t)hubpos[r] * 9 + hub_group(r, cls[jj[e]]), 1u);
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint64_t stride = (uint64_t)gridDim.x * kTB;
+    for (uint64_t base = (uint64_t)blockIdx.x * kTB + (threadIdx.x & ~63u); base < nnz;
+         base += stride) {
+        const uint64_t e = base + lane;
+        uint32_t r = 0, grp = 0;
+        bool hub = false;
+        if (e < nnz) {
+            r = ii[e];
+            hub = hubflag[r] != 0;
+            if (hub)
+                grp = hub_group(r, cls[jj[e]]);
+        }
+        if (!__any(hub))
+            continue;
+        for (uint32_t g = 0; g < 9; ++g) {
+            const bool mine = hub && grp == g;
+            const unsigned long long m = __ballot(mine);
+            if (m == 0)
+                continue;
+            const int lead = __ffsll((long long)m) - 1;
+            const uint32_t r0 = __shfl(r, lead, 64);
+            const unsigned long long same = __ballot(mine && r == r0);
+            if ((int)lane == lead)
+                atomicAdd(hubcnt + (size_t)hubpos[r] * 9 + g, (uint32_t)__popcll(same));
+            else if (mine && r != r0)
+                atomicAdd(hubcnt + (size_t)hubpos[r] * 9 + g, 1u);
+        }
     }
 }
 
@@ -317,9 +483,8 @@ __global__ void len_keys_k(const Seg *__restrict__ pseg, uint64_t n, uint32_t se
         key[i] = seg_max - l;
         nl += l >= kLongSegment;
     }
-    for (int s = 32; s >= 1; s >>= 1)
-        nl += __shfl_xor(nl, s, 64);
-    if ((threadIdx.x & 63) == 0 && nl)
+    nl = block_sum(nl);
+    if (threadIdx.x == 0 && nl)
         atomicAdd(&C->nlong, nl);
 }
 
@@ -350,8 +515,8 @@ __global__ void any_flags_k(const Seg *__restrict__ pseg, const uint8_t *__restr
     }
 #pragma unroll
     for (uint32_t k = 0; k <= kSlices; ++k) {
-        const unsigned long long t = wave_sum(w[k]);
-        if ((threadIdx.x & 63) == 0 && t)
+        const unsigned long long t = block_sum(w[k]);
+        if (threadIdx.x == 0 && t)
             atomicAdd(k == kSlices ? &C->any_load : &C->load[k], t);
     }
 }
@@ -410,8 +575,8 @@ __global__ void combine_k(const Seg *__restrict__ pseg, const uint8_t *__restric
     }
 #pragma unroll
     for (uint32_t k = 0; k < kSlices; ++k) {
-        const uint32_t c = wave_sum(cnt[k]), g = wave_sum(lng[k]);
-        if ((threadIdx.x & 63) == 0) {
+        const uint32_t c = block_sum(cnt[k]), g = block_sum(lng[k]);
+        if (threadIdx.x == 0) {
             if (c)
                 atomicAdd(&C->qcount[k], c);
             if (g)
@@ -503,14 +668,16 @@ __global__ void remap_apply_k(uint32_t *idx, uint64_t n, const uint32_t *__restr
 
 // Scratch for the device-wide primitives, grown on demand.
 struct Temp {
-    DBuf<unsigned char> buf;
+    Arena &arena;
+    unsigned char *p = nullptr;
     size_t cap = 0;
+    explicit Temp(Arena &a) : arena(a) {}
     hipError_t need(size_t bytes)
     {
         bytes = bytes < 256 ? 256 : bytes; // never null: a null pointer asks for the size again
         if (bytes <= cap)
             return hipSuccess;
-        const hipError_t e = buf.alloc(bytes);
+        const hipError_t e = arena.take(reinterpret_cast<void **>(&p), bytes);
         cap = e == hipSuccess ? bytes : 0;
         return e;
     }
@@ -522,7 +689,7 @@ int exclusive_sum(Temp &tmp, const T *in, T *out, size_t n, hipStream_t st, std:
     size_t bytes = 0;
     HIP_OK(hipcub::DeviceScan::ExclusiveSum(nullptr, bytes, in, out, n, st));
     HIP_OK(tmp.need(bytes));
-    HIP_OK(hipcub::DeviceScan::ExclusiveSum(tmp.buf.p, bytes, in, out, n, st));
+    HIP_OK(hipcub::DeviceScan::ExclusiveSum(tmp.p, bytes, in, out, n, st));
     return SPC3D_OK;
 }
 
@@ -536,20 +703,33 @@ int sort_pairs(Temp &tmp, const KeyT *kin, KeyT *kout, const uint32_t *vin, uint
         HIP_OK(hipcub::DeviceRadixSort::SortPairsDescending(nullptr, bytes, kin, kout, vin, vout,
                                                             n, 0, bits, st));
         HIP_OK(tmp.need(bytes));
-        HIP_OK(hipcub::DeviceRadixSort::SortPairsDescending(tmp.buf.p, bytes, kin, kout, vin,
+        HIP_OK(hipcub::DeviceRadixSort::SortPairsDescending(tmp.p, bytes, kin, kout, vin,
                                                             vout, n, 0, bits, st));
     } else {
         HIP_OK(hipcub::DeviceRadixSort::SortPairs(nullptr, bytes, kin, kout, vin, vout, n, 0,
                                                   bits, st));
         HIP_OK(tmp.need(bytes));
-        HIP_OK(hipcub::DeviceRadixSort::SortPairs(tmp.buf.p, bytes, kin, kout, vin, vout, n, 0,
+        HIP_OK(hipcub::DeviceRadixSort::SortPairs(tmp.p, bytes, kin, kout, vin, vout, n, 0,
                                                   bits, st));
     }
     return SPC3D_OK;
 }
 
+// Ascending sort of keys on key bits [0, bits).
+int sort_keys(Temp &tmp, const uint32_t *kin, uint32_t *kout, uint32_t n, int bits,
+              hipStream_t st, std::string &err)
+{
+    size_t bytes = 0;
+    HIP_OK(hipcub::DeviceRadixSort::SortKeys(nullptr, bytes, kin, kout, n, 0, bits, st));
+    HIP_OK(tmp.need(bytes));
+    HIP_OK(hipcub::DeviceRadixSort::SortKeys(tmp.p, bytes, kin, kout, n, 0, bits, st));
+    return SPC3D_OK;
+}
+
 #define LAUNCH(kernel, n, ...)                                                                    \
     hipLaunchKernelGGL(kernel, dim3(grid_for(n)), dim3(kTB), 0, st, __VA_ARGS__)
+#define LAUNCH_SMALL(kernel, n, ...)                                                              \
+    hipLaunchKernelGGL(kernel, dim3(small_grid_for(n)), dim3(kTB), 0, st, __VA_ARGS__)
 
 #define TRY(expr)                                                                                 \
     do {                                                                                          \
@@ -569,22 +749,21 @@ int fetch(hipStream_t st, void *host, const void *dev, size_t bytes, std::string
 // Sorts the entries into kernel order: perm (kernel position -> caller's
 // position) and col.  KeyT is wide enough for (row << 4 | group).
 template <typename KeyT>
-int order_entries(Temp &tmp, hipStream_t st, uint64_t nnz, int key_bits, bool slices,
+int order_entries(Arena &arena, Temp &tmp, hipStream_t st, uint64_t nnz, int key_bits, bool slices,
                   const uint32_t *d_ii, const uint32_t *d_jj, const uint32_t *hubflag,
                   const uint8_t *cls, uint32_t *perm, uint32_t *col, Counters *C, std::string &err)
 {
-    DBuf<KeyT> key, key_out;
-    DBuf<uint32_t> ident;
-    HIP_OK(key.alloc(nnz));
-    HIP_OK(key_out.alloc(nnz));
-    HIP_OK(ident.alloc(nnz));
+    SBuf<KeyT> key, key_out;
+    SBuf<uint32_t> ident;
+    HIP_OK(key.alloc(arena, nnz));
+    HIP_OK(key_out.alloc(arena, nnz));
+    HIP_OK(ident.alloc(arena, nnz));
     LAUNCH((keys_k<KeyT>), nnz, d_ii, d_jj, nnz, slices, hubflag, cls, key.p);
     LAUNCH(iota_k, nnz, ident.p, nnz);
     TRY(sort_pairs<KeyT>(tmp, key.p, key_out.p, ident.p, perm, (uint32_t)nnz, key_bits, false, st,
                          err));
     LAUNCH(gather_cols_k, nnz, d_jj, perm, nnz, col, C);
     HIP_OK(hipGetLastError());
-    HIP_OK(hipStreamSynchronize(st)); // key buffers are freed on return
     return SPC3D_OK;
 }
 
@@ -618,24 +797,28 @@ int build_device_plan(hipStream_t st, uint32_t nrows, uint32_t ncols, uint64_t n
         return SPC3D_OK;
     }
 
-    Temp tmp;
-    DBuf<Counters> dC;
+    // One block for everything whose size is known now: ten arrays per row, five and
+    // a class byte per column, the sorted column ids, two keys and an index per entry,
+    // the primitives' scratch.
+    Arena arena;
+    const size_t key_bytes = bits_for(nrows ? nrows - 1 : 0) + 4 > 32 ? 8 : 4;
+    HIP_OK(arena.reserve(((size_t)nrows + 1) * 40 + (size_t)ncols * 17 + (size_t)std::max(nrows, ncols) * 4 +
+                         (size_t)nnz * (2 * key_bytes + 8) + (size_t)nnz / 2 + ((size_t)8 << 20)));
+    Temp tmp(arena);
+    SBuf<Counters> dC;
     Counters hC;
-    HIP_OK(dC.alloc(1));
+    HIP_OK(dC.alloc(arena, 1));
     HIP_OK(hipMemsetAsync(dC.p, 0, sizeof(Counters), st));
     HIP_OK(hipMemsetAsync(&dC.p->first_bad, 0xFF, sizeof(uint32_t), st));
 
     // ---- histograms, validation ------------------------------------------------
-    DBuf<uint32_t> rowcnt, rowptr, coldeg;
-    HIP_OK(rowcnt.alloc((size_t)nrows + 1));
-    HIP_OK(rowptr.alloc((size_t)nrows + 1));
-    HIP_OK(coldeg.alloc(ncols));
+    SBuf<uint32_t> rowcnt, rowptr, coldeg;
+    HIP_OK(rowcnt.alloc(arena, (size_t)nrows + 1));
+    HIP_OK(rowptr.alloc(arena, (size_t)nrows + 1));
+    HIP_OK(coldeg.alloc(arena, ncols));
     HIP_OK(hipMemsetAsync(rowcnt.p, 0, ((size_t)nrows + 1) * sizeof(uint32_t), st));
     HIP_OK(hipMemsetAsync(coldeg.p, 0, (size_t)ncols * sizeof(uint32_t), st));
-    LAUNCH(hist_k, nnz, d_ii, d_jj, nnz, nrows, ncols, rowcnt.p, coldeg.p, dC.p);
-    LAUNCH(stats_k, nrows, rowcnt.p, (uint64_t)nrows, &dC.p->rows_touched, &dC.p->max_row);
-    LAUNCH(stats_k, ncols, coldeg.p, (uint64_t)ncols, &dC.p->cols_touched, &dC.p->max_cdeg);
-    TRY(exclusive_sum(tmp, rowcnt.p, rowptr.p, (size_t)nrows + 1, st, err));
+    LAUNCH_SMALL(check_k, nnz, d_ii, d_jj, nnz, nrows, ncols, dC.p);
     TRY(fetch(st, &hC, dC.p, sizeof hC, err));
     if (hC.first_bad != 0xFFFFFFFFu) {
         uint32_t r = 0, c = 0;
@@ -647,13 +830,34 @@ int build_device_plan(hipStream_t st, uint32_t nrows, uint32_t ncols, uint64_t n
         err = buf;
         return SPC3D_ERR_BAD_INDEX;
     }
+    {
+        SBuf<uint32_t> sorted, start;
+        HIP_OK(sorted.alloc(arena, nnz));
+        HIP_OK(start.alloc(arena, std::max<size_t>(ncols, nrows)));
+        if (hC.rows_unsorted) {
+            TRY(sort_keys(tmp, d_ii, sorted.p, (uint32_t)nnz, bits_for(nrows ? nrows - 1 : 0), st,
+                          err));
+            LAUNCH(run_bounds_k, nnz, sorted.p, nnz, nrows, start.p, rowcnt.p);
+            LAUNCH(run_lengths_k, nrows, start.p, (uint64_t)nrows, rowcnt.p);
+        } else {
+            LAUNCH(hist_sorted_k, nnz, d_ii, nnz, rowcnt.p);
+        }
+        TRY(sort_keys(tmp, d_jj, sorted.p, (uint32_t)nnz, bits_for(ncols ? ncols - 1 : 0), st,
+                      err));
+        LAUNCH(run_bounds_k, nnz, sorted.p, nnz, ncols, start.p, coldeg.p);
+        LAUNCH(run_lengths_k, ncols, start.p, (uint64_t)ncols, coldeg.p);
+    }
+    LAUNCH_SMALL(stats_k, nrows, rowcnt.p, (uint64_t)nrows, &dC.p->rows_touched, &dC.p->max_row);
+    LAUNCH_SMALL(stats_k, ncols, coldeg.p, (uint64_t)ncols, &dC.p->cols_touched, &dC.p->max_cdeg);
+    TRY(exclusive_sum(tmp, rowcnt.p, rowptr.p, (size_t)nrows + 1, st, err));
+    TRY(fetch(st, &hC, dC.p, sizeof hC, err));
     P.rows_touched = hC.rows_touched;
     P.cols_touched = hC.cols_touched;
     P.max_row_nnz = hC.max_row;
     const uint32_t ctouched = hC.cols_touched, maxcdeg = hC.max_cdeg;
 
     // ---- column classes (XCD slicing only) ---------------------------------------
-    DBuf<uint8_t> cls;
+    SBuf<uint8_t> cls;
     bool slices = false;
     if (want_slices && opts.hot_cols > 0 && ctouched > opts.hot_cols) {
         const uint32_t h1 = opts.hot_cols;
@@ -662,41 +866,40 @@ int build_device_plan(hipStream_t st, uint32_t nrows, uint32_t ncols, uint64_t n
             std::min<uint64_t>((uint64_t)hrep + (uint64_t)(h1 - hrep) * kSlices, ctouched);
         // Columns by degree, highest first, ties in column order (a stable sort);
         // the untouched columns end up last.
-        DBuf<uint32_t> colid, order, deg_sorted;
-        HIP_OK(colid.alloc(ncols));
-        HIP_OK(order.alloc(ncols));
-        HIP_OK(deg_sorted.alloc(ncols));
+        SBuf<uint32_t> colid, order, deg_sorted;
+        HIP_OK(colid.alloc(arena, ncols));
+        HIP_OK(order.alloc(arena, ncols));
+        HIP_OK(deg_sorted.alloc(arena, ncols));
         LAUNCH(iota_k, ncols, colid.p, (uint64_t)ncols);
         TRY(sort_pairs<uint32_t>(tmp, coldeg.p, deg_sorted.p, colid.p, order.p, ncols,
                                  bits_for(maxcdeg), true, st, err));
-        LAUNCH(sum_first_k, htot, deg_sorted.p, htot, &dC.p->covered);
+        LAUNCH_SMALL(sum_first_k, htot, deg_sorted.p, htot, &dC.p->covered);
         TRY(fetch(st, &hC, dC.p, sizeof hC, err));
         const uint64_t covered = hC.covered;
         const double coverage = (double)covered / (double)nnz;
         const double share = (double)htot / (double)ctouched;
         if (coverage >= 0.2 && coverage >= 2.0 * share) {
             slices = true;
-            HIP_OK(cls.alloc(ncols));
+            HIP_OK(cls.alloc(arena, ncols));
             LAUNCH(fill_k<uint8_t>, ncols, cls.p, (uint64_t)ncols, kClsCold);
             LAUNCH(classify_k, htot, order.p, htot, hrep, cls.p);
             P.hot_cols = (uint32_t)htot;
             P.hot_entries = covered;
         }
         HIP_OK(hipGetLastError());
-        HIP_OK(hipStreamSynchronize(st)); // the sort buffers are freed here
     }
 
     // ---- hub rows: group counts ---------------------------------------------------
-    DBuf<uint32_t> hubflag, hubpos, hubcnt;
+    SBuf<uint32_t> hubflag, hubpos, hubcnt;
     uint32_t nh = 0;
     if (slices) {
-        HIP_OK(hubflag.alloc((size_t)nrows + 1));
-        HIP_OK(hubpos.alloc((size_t)nrows + 1));
+        HIP_OK(hubflag.alloc(arena, (size_t)nrows + 1));
+        HIP_OK(hubpos.alloc(arena, (size_t)nrows + 1));
         LAUNCH(hubflag_k, (uint64_t)nrows + 1, rowcnt.p, nrows, hub_min, hubflag.p);
         TRY(exclusive_sum(tmp, hubflag.p, hubpos.p, (size_t)nrows + 1, st, err));
         TRY(fetch(st, &nh, hubpos.p + nrows, sizeof nh, err));
         P.hub_rows = nh;
-        HIP_OK(hubcnt.alloc((size_t)nh * 9 + 1));
+        HIP_OK(hubcnt.alloc(arena, (size_t)nh * 9 + 1));
         HIP_OK(hipMemsetAsync(hubcnt.p, 0, ((size_t)nh * 9 + 1) * sizeof(uint32_t), st));
         LAUNCH(hubcount_k, nnz, d_ii, d_jj, nnz, hubflag.p, hubpos.p, cls.p, hubcnt.p);
     }
@@ -709,22 +912,22 @@ int build_device_plan(hipStream_t st, uint32_t nrows, uint32_t ncols, uint64_t n
         const int row_bits = bits_for(nrows ? nrows - 1 : 0);
         const int key_bits = row_bits + (slices ? 4 : 0);
         if (key_bits <= 32)
-            TRY(order_entries<uint32_t>(tmp, st, nnz, key_bits, slices, d_ii, d_jj, hubflag.p,
+            TRY(order_entries<uint32_t>(arena, tmp, st, nnz, key_bits, slices, d_ii, d_jj, hubflag.p,
                                         cls.p, perm.p, col.p, dC.p, err));
         else
-            TRY(order_entries<unsigned long long>(tmp, st, nnz, key_bits, slices, d_ii, d_jj,
+            TRY(order_entries<unsigned long long>(arena, tmp, st, nnz, key_bits, slices, d_ii, d_jj,
                                                   hubflag.p, cls.p, perm.p, col.p, dC.p, err));
     }
 
     // ---- segments --------------------------------------------------------------------
-    DBuf<uint32_t> npieces, issplit, nslot, piece_off, split_off, slot_off;
+    SBuf<uint32_t> npieces, issplit, nslot, piece_off, split_off, slot_off;
     const size_t nr1 = (size_t)nrows + 1;
-    HIP_OK(npieces.alloc(nr1));
-    HIP_OK(issplit.alloc(nr1));
-    HIP_OK(nslot.alloc(nr1));
-    HIP_OK(piece_off.alloc(nr1));
-    HIP_OK(split_off.alloc(nr1));
-    HIP_OK(slot_off.alloc(nr1));
+    HIP_OK(npieces.alloc(arena, nr1));
+    HIP_OK(issplit.alloc(arena, nr1));
+    HIP_OK(nslot.alloc(arena, nr1));
+    HIP_OK(piece_off.alloc(arena, nr1));
+    HIP_OK(split_off.alloc(arena, nr1));
+    HIP_OK(slot_off.alloc(arena, nr1));
     LAUNCH(count_pieces_k, nr1, rowcnt.p, nrows, seg_max, slices, hubflag.p, hubpos.p, hubcnt.p,
            npieces.p, issplit.p, nslot.p);
     TRY(exclusive_sum(tmp, npieces.p, piece_off.p, (size_t)nrows + 1, st, err));
@@ -738,11 +941,13 @@ int build_device_plan(hipStream_t st, uint32_t nrows, uint32_t ncols, uint64_t n
     P.nslots = totals[2];
     P.nseg_real = np_total;
 
-    DBuf<Seg> pseg;
-    DBuf<uint8_t> pqueue;
+    // and one for everything sized by the number of pieces
+    HIP_OK(arena.reserve((size_t)np_total * 64 + ((size_t)4 << 20)));
+    SBuf<Seg> pseg;
+    SBuf<uint8_t> pqueue;
     DBuf<SplitRow> splits;
-    HIP_OK(pseg.alloc(np_total));
-    HIP_OK(pqueue.alloc(np_total));
+    HIP_OK(pseg.alloc(arena, np_total));
+    HIP_OK(pqueue.alloc(arena, np_total));
     HIP_OK(splits.alloc(nsplit));
     LAUNCH(emit_pieces_k, nrows, rowptr.p, nrows, seg_max, slices, hubflag.p, hubpos.p, hubcnt.p,
            piece_off.p, split_off.p, slot_off.p, pseg.p, pqueue.p, splits.p);
@@ -752,13 +957,13 @@ int build_device_plan(hipStream_t st, uint32_t nrows, uint32_t ncols, uint64_t n
     uint32_t nseg_padded = 0;
     const int len_bits = bits_for(seg_max);
     if (!slices) {
-        DBuf<uint32_t> key, key_out, idx, idx_out;
-        HIP_OK(key.alloc(np_total));
-        HIP_OK(key_out.alloc(np_total));
-        HIP_OK(idx.alloc(np_total));
-        HIP_OK(idx_out.alloc(np_total));
+        SBuf<uint32_t> key, key_out, idx, idx_out;
+        HIP_OK(key.alloc(arena, np_total));
+        HIP_OK(key_out.alloc(arena, np_total));
+        HIP_OK(idx.alloc(arena, np_total));
+        HIP_OK(idx_out.alloc(arena, np_total));
         HIP_OK(segs.alloc(np_total));
-        LAUNCH(len_keys_k, np_total, pseg.p, (uint64_t)np_total, seg_max, key.p, dC.p);
+        LAUNCH_SMALL(len_keys_k, np_total, pseg.p, (uint64_t)np_total, seg_max, key.p, dC.p);
         LAUNCH(iota_k, np_total, idx.p, (uint64_t)np_total);
         TRY(sort_pairs<uint32_t>(tmp, key.p, key_out.p, idx.p, idx_out.p, np_total, len_bits,
                                  false, st, err));
@@ -768,21 +973,21 @@ int build_device_plan(hipStream_t st, uint32_t nrows, uint32_t ncols, uint64_t n
         nseg_padded = np_total;
         P.nseg_long = hC.nlong / kChunk * kChunk;
     } else {
-        DBuf<uint32_t> anyflag, anypos;
-        HIP_OK(anyflag.alloc((size_t)np_total + 1));
-        HIP_OK(anypos.alloc((size_t)np_total + 1));
-        LAUNCH(any_flags_k, (uint64_t)np_total + 1, pseg.p, pqueue.p, (uint64_t)np_total,
+        SBuf<uint32_t> anyflag, anypos;
+        HIP_OK(anyflag.alloc(arena, (size_t)np_total + 1));
+        HIP_OK(anypos.alloc(arena, (size_t)np_total + 1));
+        LAUNCH_SMALL(any_flags_k, (uint64_t)np_total + 1, pseg.p, pqueue.p, (uint64_t)np_total,
                anyflag.p, dC.p);
         TRY(exclusive_sum(tmp, anyflag.p, anypos.p, (size_t)np_total + 1, st, err));
         uint32_t nany = 0;
         TRY(fetch(st, &nany, anypos.p + np_total, sizeof nany, err));
         TRY(fetch(st, &hC, dC.p, sizeof hC, err));
 
-        DBuf<uint32_t> any_idx, any_key, any_key_out, any_sorted;
-        HIP_OK(any_idx.alloc(nany));
-        HIP_OK(any_key.alloc(nany));
-        HIP_OK(any_key_out.alloc(nany));
-        HIP_OK(any_sorted.alloc(nany));
+        SBuf<uint32_t> any_idx, any_key, any_key_out, any_sorted;
+        HIP_OK(any_idx.alloc(arena, nany));
+        HIP_OK(any_key.alloc(arena, nany));
+        HIP_OK(any_key_out.alloc(arena, nany));
+        HIP_OK(any_sorted.alloc(arena, nany));
         if (nany) {
             LAUNCH(compact_any_k, np_total, pseg.p, anyflag.p, anypos.p, (uint64_t)np_total,
                    seg_max, any_idx.p, any_key.p);
@@ -795,12 +1000,12 @@ int build_device_plan(hipStream_t st, uint32_t nrows, uint32_t ncols, uint64_t n
         Upto upto;
         deal_thresholds(load, hC.any_load, upto.v);
 
-        DBuf<uint32_t> comb_idx, comb_key, comb_idx_out, comb_key_out;
-        HIP_OK(comb_idx.alloc(np_total));
-        HIP_OK(comb_key.alloc(np_total));
-        HIP_OK(comb_idx_out.alloc(np_total));
-        HIP_OK(comb_key_out.alloc(np_total));
-        LAUNCH(combine_k, (uint64_t)np_total + nany, pseg.p, pqueue.p, anyflag.p, anypos.p,
+        SBuf<uint32_t> comb_idx, comb_key, comb_idx_out, comb_key_out;
+        HIP_OK(comb_idx.alloc(arena, np_total));
+        HIP_OK(comb_key.alloc(arena, np_total));
+        HIP_OK(comb_idx_out.alloc(arena, np_total));
+        HIP_OK(comb_key_out.alloc(arena, np_total));
+        LAUNCH_SMALL(combine_k, (uint64_t)np_total + nany, pseg.p, pqueue.p, anyflag.p, anypos.p,
                any_sorted.p, (uint64_t)np_total, (uint64_t)nany, seg_max, upto, comb_idx.p,
                comb_key.p, dC.p);
         const int comb_bits = bits_for((uint64_t)kSlices * ((uint64_t)seg_max + 1) - 1);
@@ -825,8 +1030,6 @@ int build_device_plan(hipStream_t st, uint32_t nrows, uint32_t ncols, uint64_t n
         LAUNCH(fill_k<Seg>, nseg_padded, segs.p, (uint64_t)nseg_padded, (Seg{0, 0, 0, kWholeRow}));
         LAUNCH(scatter_segs_k, np_total, pseg.p, comb_idx_out.p, comb_key_out.p,
                (uint64_t)np_total, seg_max, qs, segs.p);
-        HIP_OK(hipGetLastError());
-        HIP_OK(hipStreamSynchronize(st));
         P.nqueues = kSlices;
         P.nseg_long = rounds * kSlices * kChunk;
     }
@@ -854,13 +1057,15 @@ int localize_device(hipStream_t st, uint64_t n, uint32_t *d_idx, uint32_t *d_ltg
         err = "more than 2^32 - 1 indices are not supported";
         return SPC3D_ERR_TOO_LARGE;
     }
-    Temp tmp;
-    DBuf<uint32_t> ident, key, pos, head, run_of;
-    HIP_OK(ident.alloc(n));
-    HIP_OK(key.alloc(n));
-    HIP_OK(pos.alloc(n));
-    HIP_OK(head.alloc(n + 1));
-    HIP_OK(run_of.alloc(n + 1));
+    Arena arena;
+    HIP_OK(arena.reserve((size_t)n * 44 + ((size_t)8 << 20))); // ten arrays of at most n + 1, scratch
+    Temp tmp(arena);
+    SBuf<uint32_t> ident, key, pos, head, run_of;
+    HIP_OK(ident.alloc(arena, n));
+    HIP_OK(key.alloc(arena, n));
+    HIP_OK(pos.alloc(arena, n));
+    HIP_OK(head.alloc(arena, n + 1));
+    HIP_OK(run_of.alloc(arena, n + 1));
     LAUNCH(iota_k, n, ident.p, n);
     TRY(sort_pairs<uint32_t>(tmp, d_idx, key.p, ident.p, pos.p, (uint32_t)n, 32, false, st, err));
     LAUNCH(heads_k, n + 1, key.p, n, head.p);
@@ -868,12 +1073,12 @@ int localize_device(hipStream_t st, uint64_t n, uint32_t *d_idx, uint32_t *d_ltg
     uint32_t nruns = 0;
     TRY(fetch(st, &nruns, run_of.p + n, sizeof nruns, err));
 
-    DBuf<uint32_t> first_pos, run_key, first_sorted, run_order, rank_of;
-    HIP_OK(first_pos.alloc(nruns));
-    HIP_OK(run_key.alloc(nruns));
-    HIP_OK(first_sorted.alloc(nruns));
-    HIP_OK(run_order.alloc(nruns));
-    HIP_OK(rank_of.alloc(nruns));
+    SBuf<uint32_t> first_pos, run_key, first_sorted, run_order, rank_of;
+    HIP_OK(first_pos.alloc(arena, nruns));
+    HIP_OK(run_key.alloc(arena, nruns));
+    HIP_OK(first_sorted.alloc(arena, nruns));
+    HIP_OK(run_order.alloc(arena, nruns));
+    HIP_OK(rank_of.alloc(arena, nruns));
     // run_of[i] of a head is its run's index; of the other members it is one more
     LAUNCH(run_firsts_k, n, key.p, pos.p, head.p, run_of.p, n, first_pos.p, run_key.p);
     LAUNCH(iota_k, nruns, ident.p, (uint64_t)nruns);
