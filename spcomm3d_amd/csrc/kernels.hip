@@ -199,7 +199,7 @@ template <int G> __device__ __forceinline__ uint64_t seg_index(uint32_t nq, uint
 
 // RG == 1 ("ragged"): a dense row is nvec 16-byte vectors with nvec < LPR * VPL,
 // given at run time; lanes whose vector index is >= nvec idle.  RG == 0: nvec ==
-// LPR * VPL exactly and the row stride is a compile-time constant.  RG == 2: below.
+// LPR * VPL exactly and the row stride is a compile-time constant.  RG == 2, 3: below.
 template <typename T, int LPR, int VPL, int RG>
 __device__ __forceinline__ const typename Vec<T>::type *row_ptr(const T *base, uint32_t row,
                                                                 uint32_t sub, uint32_t nvec)
@@ -216,14 +216,6 @@ __device__ __forceinline__ bool lane_on(uint32_t sub, int v, uint32_t nvec)
     return !RG || sub + (uint32_t)v * LPR < nvec;
 }
 
-// RG == 2 ("odd"): a dense row of K reals is no whole number of 16-byte vectors
-// (the kernels' `nvec` argument carries K).  Rows start at element alignment only,
-// and the last vector of a row would reach past its end, so: the lane that holds the
-// row's end loads the 16 bytes that END there (the leading elements of that vector
-// belong to the lane before and are not counted), and lanes past the end load the
-// same vector and count nothing.  Every load stays inside the row, without a
-// branch.  Vector loads and stores at 4- or 8-byte alignment are what global memory
-// accesses on this GPU allow.
 // 16-byte accesses at element alignment.  (Not through nt_load / nt_store: template
 // argument deduction would drop the typedef's alignment.)
 template <typename T> __device__ __forceinline__ typename Vec<T>::type loose_load(const char *p)
@@ -245,12 +237,28 @@ __device__ __forceinline__ void loose_store_nt(typename Vec<T>::type v, char *p)
     __builtin_nontemporal_store(v, reinterpret_cast<typename Vec<T>::loose *>(p));
 }
 
-template <typename T, int VPL, int RG> struct Odd {};
-template <typename T, int VPL> struct Odd<T, VPL, 2> {
+// RG == 2 ("odd"): a dense row of K reals is no whole number of 16-byte vectors
+// (the kernels' `nvec` argument carries K).  Rows start at element alignment only,
+// and the last vector of a row would reach past its end, so: the lane that holds the
+// row's end loads the 16 bytes that END there (the leading elements of that vector
+// belong to the lane before and are not counted), and lanes past the end load the
+// same vector and count nothing.  Every load stays inside the row, without a
+// branch.  Vector loads and stores at 4- or 8-byte alignment are what global memory
+// accesses on this GPU allow.
+//
+// RG == 3 ("thin"): a dense row is shorter than 16 bytes (K < Vec<T>::N reals; `nvec`
+// carries K again).  The row is the first K elements of one vector, loaded element by
+// element (the elements past K repeat element K - 1: no branch, no access outside
+// the row) and counted by the first lane of the group only; the group's other lanes
+// load the same addresses and count nothing.  Runs the 4-lane shape.
+template <typename T, int VPL> struct OddLanes {
     uint32_t off[VPL];             // byte offset within a row of this lane's vector v
     bool keep[VPL][Vec<T>::N];     // the elements of it that are this lane's
     bool all[VPL];                 // every element is
 };
+template <typename T, int VPL, int RG> struct Odd {};
+template <typename T, int VPL> struct Odd<T, VPL, 2> : OddLanes<T, VPL> {};
+template <typename T, int VPL> struct Odd<T, VPL, 3> : OddLanes<T, VPL> {};
 
 template <typename T, int LPR, int VPL, int RG>
 __device__ __forceinline__ Odd<T, VPL, RG> odd_lanes(uint32_t sub, uint32_t K)
@@ -268,6 +276,15 @@ __device__ __forceinline__ Odd<T, VPL, RG> odd_lanes(uint32_t sub, uint32_t K)
             for (int i = 0; i < Vec<T>::N; ++i)
                 o.keep[v][i] = start + (uint32_t)i * sizeof(T) >= first;
         }
+    } else if constexpr (RG == 3) {
+#pragma unroll
+        for (int v = 0; v < VPL; ++v) {
+            o.off[v] = 0;
+            o.all[v] = false;
+#pragma unroll
+            for (int i = 0; i < Vec<T>::N; ++i)
+                o.keep[v][i] = v == 0 && sub == 0 && (uint32_t)i < K;
+        }
     }
     return o;
 }
@@ -275,11 +292,31 @@ __device__ __forceinline__ Odd<T, VPL, RG> odd_lanes(uint32_t sub, uint32_t K)
 template <typename T, int RG>
 __device__ __forceinline__ const char *odd_row(const T *base, uint32_t row, uint32_t K)
 {
-    static_assert(RG == 2, "rows of K reals at element alignment");
+    static_assert(RG >= 2, "rows of K reals at element alignment");
     return reinterpret_cast<const char *>(base) + (uint64_t)row * ((uint64_t)K * sizeof(T));
 }
 
-// out[v] = this lane's vectors of dense row `row`.  RG == 2 loads every element of
+// Vector v of the row at r as this lane loads it in the RG >= 2 variants (NT: a
+// row that is read once).
+template <typename T, int RG, int VPL, bool NT = false>
+__device__ __forceinline__ typename Vec<T>::type odd_load(const char *r, int v, uint32_t K,
+                                                          const Odd<T, VPL, RG> &odd)
+{
+    if constexpr (RG == 3) {
+        typename Vec<T>::type out{};
+        const T *e = reinterpret_cast<const T *>(r);
+#pragma unroll
+        for (int i = 0; i + 1 < Vec<T>::N; ++i) // K <= N - 1
+            out[i] = e[(uint32_t)i < K ? (uint32_t)i : K - 1];
+        return out;
+    } else if constexpr (NT) {
+        return loose_load_nt<T>(r + odd.off[v]);
+    } else {
+        return loose_load<T>(r + odd.off[v]);
+    }
+}
+
+// out[v] = this lane's vectors of dense row `row`.  RG >= 2 loads every element of
 // them; what is not the lane's to count is left out by the caller (SDDMM: in the
 // dot product; SpMM: at the store).
 template <typename T, int LPR, int VPL, int RG>
@@ -288,11 +325,11 @@ __device__ __forceinline__ void gather_row(typename Vec<T>::type (&out)[VPL], co
                                            const Odd<T, VPL, RG> &odd)
 {
     using V = typename Vec<T>::type;
-    if constexpr (RG == 2) {
+    if constexpr (RG >= 2) {
         const char *r = odd_row<T, RG>(base, row, nvec);
 #pragma unroll
         for (int v = 0; v < VPL; ++v)
-            out[v] = loose_load<T>(r + odd.off[v]);
+            out[v] = odd_load<T, RG, VPL>(r, v, nvec, odd);
     } else {
         const V *r = row_ptr<T, LPR, VPL, RG>(base, row, sub, nvec);
 #pragma unroll
@@ -312,7 +349,7 @@ __device__ __forceinline__ T lane_dot(const typename Vec<T>::type (&a)[VPL],
     for (int v = 0; v < VPL; ++v)
 #pragma unroll
         for (int i = 0; i < Vec<T>::N; ++i) {
-            if constexpr (RG == 2)
+            if constexpr (RG >= 2)
                 dot += a[v][i] * (odd.keep[v][i] ? b[v][i] : (T)0);
             else
                 dot += a[v][i] * b[v][i];
@@ -327,7 +364,7 @@ template <typename T, int VPL>
 __device__ __forceinline__ void odd_store(char *drow, bool whole,
                                           const typename Vec<T>::type (&y0)[VPL],
                                           const typename Vec<T>::type (&acc)[VPL],
-                                          const Odd<T, VPL, 2> &odd)
+                                          const OddLanes<T, VPL> &odd)
 {
     using V = typename Vec<T>::type;
 #pragma unroll
@@ -584,11 +621,11 @@ sddmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint3
 
     const Odd<T, VPL, RG> odd = odd_lanes<T, LPR, VPL, RG>(sub, nvec);
     V a[VPL], acc[VPL];
-    if constexpr (RG == 2) {
+    if constexpr (RG >= 2) {
         const char *arow = odd_row<T, RG>(A, sg[0], nvec);
 #pragma unroll
         for (int v = 0; v < VPL; ++v) {
-            a[v] = loose_load_nt<T>(arow + odd.off[v]);
+            a[v] = odd_load<T, RG, VPL, true>(arow, v, nvec, odd);
 #pragma unroll
             for (int i = 0; i < Vec<T>::N; ++i)
                 a[v][i] = odd.keep[v][i] ? a[v][i] : (T)0;
@@ -604,14 +641,14 @@ sddmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint3
     }
     sddmm_walk<T, LPR, VPL, UB, RG, WIDE, FZ>(a, acc, col, perm, sval, B, C, sg[1], sg[2], sub,
                                               nvec, odd);
-    if constexpr (FZ != 0 && RG == 2) {
+    if constexpr (FZ != 0 && RG >= 2) {
         const bool whole = sg[3] == kWholeRow;
         char *drow = const_cast<char *>(whole ? odd_row<T, RG>(Y, sg[0], nvec)
                                               : odd_row<T, RG>(partial, sg[3], nvec));
         V y0[VPL];
 #pragma unroll
         for (int v = 0; v < VPL; ++v)
-            y0[v] = whole ? loose_load_nt<T>(drow + odd.off[v]) : V{};
+            y0[v] = whole ? odd_load<T, RG, VPL, true>(drow, v, nvec, odd) : V{};
         odd_store<T, VPL>(drow, whole, y0, acc, odd);
     } else if constexpr (FZ != 0) {
         const bool whole = sg[3] == kWholeRow;
@@ -831,13 +868,13 @@ spmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint32
         acc[v] = V{};
         y0[v] = V{};
     }
-    if constexpr (RG == 2) {
+    if constexpr (RG >= 2) {
         char *drow = const_cast<char *>(whole ? odd_row<T, RG>(Y, sg[0], nvec)
                                               : odd_row<T, RG>(partial, sg[3], nvec));
         if (whole) {
 #pragma unroll
             for (int v = 0; v < VPL; ++v)
-                y0[v] = loose_load_nt<T>(drow + odd.off[v]);
+                y0[v] = odd_load<T, RG, VPL, true>(drow, v, nvec, odd);
         }
         spmm_walk<T, LPR, VPL, UB, RG, WIDE>(acc, col, sval, X, sg[1], sg[2], sub, nvec, odd);
         odd_store<T, VPL>(drow, whole, y0, acc, odd);
@@ -1024,21 +1061,24 @@ copy_kernel(u32x4 *__restrict__ dst, const u32x4 *__restrict__ src, uint64_t nve
 // ------------------------------------------------------------- dispatch ----
 struct Shape {
     int lpr, vpl;  // lpr == 0: generic kernel
-    int mode;      // the kernels' RG: 0 exact, 1 ragged, 2 odd
-    uint32_t nvec; // 16-byte vectors per dense row; mode 2: K, the reals per row
+    int mode;      // the kernels' RG: 0 exact, 1 ragged, 2 odd, 3 thin
+    uint32_t nvec; // 16-byte vectors per dense row; modes 2, 3: K, the reals per row
 };
 
-// A dense row of K reals of at least 16 and at most 4096 bytes runs the vector
-// kernels; anything else takes the generic ones.  A whole number nvec of 16-byte
+// A dense row of K reals of at most 4096 bytes runs the vector kernels; longer ones
+// take the generic kernels, rows under 16 bytes the "thin" variant of the 4-lane shape.  A whole number nvec of 16-byte
 // vectors with nvec == LPR * VPL, LPR a power of two in [4, 64] and VPL in {1, 2, 4},
 // runs a kernel with the row stride compiled in; other nvec run the "ragged" variant
 // of the smallest shape that covers a row, in which the lanes past the row's end
-// idle; rows that are no whole number of vectors run the "odd" variant of that shape.
+// idle; rows that are no whole number of vectors, or of at most 16, run the "odd"
+// variant of that shape.
 Shape pick_shape(size_t elem, uint32_t K)
 {
     const size_t bytes = (size_t)K * elem;
-    if (bytes < 16 || bytes > 4096)
+    if (K == 0 || bytes > 4096)
         return {0, 0, 0, 0};
+    if (bytes < 16)
+        return {4, 1, 3, K};
     const uint32_t nvec = (uint32_t)((bytes + 15) / 16);
     const bool odd = bytes % 16 != 0;
     for (int lpr = 64; lpr >= 4 && !odd; lpr >>= 1) {
@@ -1049,8 +1089,13 @@ Shape pick_shape(size_t elem, uint32_t K)
             return {lpr, (int)vpl, 0, nvec};
         break;
     }
-    const int mode = odd ? 2 : 1;
-    const uint32_t arg = odd ? K : nvec;
+    // Narrow rows that leave lanes idle also run the odd variant: its idle lanes load a
+    // vector of the row and count nothing, where the ragged variant's skip the load
+    // under a branch (measured on R-MAT 20, fp32 K = 4: SDDMM 644 -> 557 us, SpMM
+    // 467 -> 339 us; K = 20: 510 -> 446 and 404 -> 324; level at 9 to 16 vectors, and
+    // from 17 vectors on the selects in the dot product cost SDDMM 2 to 4 %).
+    const int mode = (odd || nvec <= 16) ? 2 : 1;
+    const uint32_t arg = mode == 2 ? K : nvec;
     if (nvec > 128)
         return {64, 4, mode, arg};
     if (nvec > 64)
@@ -1161,10 +1206,12 @@ hipError_t run_spmm(const DevPlanView &P, const T *X, T *Y, const Streams &S, ui
     X(4, 2, 8, 4, 2) X(8, 2, 8, 4, 2) X(16, 2, 8, 4, 2) X(32, 2, 8, 4, 2) X(64, 2, 8, 4, 2)       \
     X(4, 4, 4, 2, 1) X(8, 4, 4, 2, 1) X(16, 4, 4, 2, 1) X(32, 4, 4, 2, 1) X(64, 4, 4, 2, 1)
 // Rows that do not fill a shape: the smallest power-of-two LPR covering the row,
-// then 64 lanes with 2 or 4 vectors each.
-#define SPC3D_FOR_RAGGED_SHAPES(X)                                                                \
+// then 64 lanes with 2 or 4 vectors each.  The ragged variants are only used from
+// 17 vectors per row on.
+#define SPC3D_FOR_ODD_SHAPES(X)                                                                   \
     X(4, 1, 16, 8, 4) X(8, 1, 16, 8, 4) X(16, 1, 16, 8, 4) X(32, 1, 16, 8, 4) X(64, 1, 16, 8, 4)  \
     X(64, 2, 8, 4, 2) X(64, 4, 4, 2, 1)
+#define SPC3D_FOR_RAGGED_SHAPES(X) X(32, 1, 16, 8, 4) X(64, 1, 16, 8, 4) X(64, 2, 8, 4, 2) X(64, 4, 4, 2, 1)
 
 template <typename T>
 hipError_t launch_fixup(const DevPlanView &P, T *Y, uint32_t K, hipStream_t st)
@@ -1202,15 +1249,26 @@ hipError_t sddmm_typed(const DevPlanView &P, const void *A, const void *B, void 
     SPC3D_FOR_SHAPES(X)
 #undef X
 #define X(L, V, U, S, S2)                                                                         \
-    if (!done && sh.mode != 0 && sh.lpr == L && sh.vpl == V) {                                    \
-        e = sh.mode == 1 ? run_sddmm<T, L, V, U, S, 1, FZ>(P, (const T *)A, (const T *)B,         \
-                                                           (T *)C, (T *)Y, SS, sh.nvec)           \
-                         : run_sddmm<T, L, V, U, S, 2, FZ>(P, (const T *)A, (const T *)B,         \
-                                                           (T *)C, (T *)Y, SS, sh.nvec);          \
+    if (!done && sh.mode == 1 && sh.lpr == L && sh.vpl == V) {                                    \
+        e = run_sddmm<T, L, V, U, S, 1, FZ>(P, (const T *)A, (const T *)B, (T *)C, (T *)Y, SS,    \
+                                            sh.nvec);                                             \
         done = true;                                                                              \
     }
     SPC3D_FOR_RAGGED_SHAPES(X)
 #undef X
+#define X(L, V, U, S, S2)                                                                         \
+    if (!done && sh.mode == 2 && sh.lpr == L && sh.vpl == V) {                                    \
+        e = run_sddmm<T, L, V, U, S, 2, FZ>(P, (const T *)A, (const T *)B, (T *)C, (T *)Y, SS,    \
+                                            sh.nvec);                                             \
+        done = true;                                                                              \
+    }
+    SPC3D_FOR_ODD_SHAPES(X)
+#undef X
+    if (!done && sh.mode == 3) {
+        e = run_sddmm<T, 4, 1, 16, 8, 3, FZ>(P, (const T *)A, (const T *)B, (T *)C, (T *)Y, SS,
+                                             sh.nvec);
+        done = true;
+    }
     if (!done) {
         if (FZ != 0)
             return hipErrorNotSupported;
@@ -1243,13 +1301,23 @@ hipError_t spmm_typed(const DevPlanView &P, const void *X_, void *Y, uint32_t K,
     SPC3D_FOR_SHAPES(X)
 #undef X
 #define X(L, V, U, S, S2)                                                                         \
-    if (!done && sh.mode != 0 && sh.lpr == L && sh.vpl == V) {                                    \
-        e = sh.mode == 1 ? run_spmm<T, L, V, U, S2, 1>(P, (const T *)X_, (T *)Y, SS, sh.nvec)     \
-                         : run_spmm<T, L, V, U, S2, 2>(P, (const T *)X_, (T *)Y, SS, sh.nvec);    \
+    if (!done && sh.mode == 1 && sh.lpr == L && sh.vpl == V) {                                    \
+        e = run_spmm<T, L, V, U, S2, 1>(P, (const T *)X_, (T *)Y, SS, sh.nvec);                   \
         done = true;                                                                              \
     }
     SPC3D_FOR_RAGGED_SHAPES(X)
 #undef X
+#define X(L, V, U, S, S2)                                                                         \
+    if (!done && sh.mode == 2 && sh.lpr == L && sh.vpl == V) {                                    \
+        e = run_spmm<T, L, V, U, S2, 2>(P, (const T *)X_, (T *)Y, SS, sh.nvec);                   \
+        done = true;                                                                              \
+    }
+    SPC3D_FOR_ODD_SHAPES(X)
+#undef X
+    if (!done && sh.mode == 3) {
+        e = run_spmm<T, 4, 1, 16, 4, 3>(P, (const T *)X_, (T *)Y, SS, sh.nvec);
+        done = true;
+    }
     if (!done) {
         const uint32_t grid = blocks_for_groups(P.nseg, P.nqueues, 1);
         hipLaunchKernelGGL((spmm_generic_kernel<T>), dim3(grid), dim3(kBlock), 0, st, P.segs,
@@ -1388,7 +1456,7 @@ const char *kernel_variant(int dtype, uint32_t K)
         snprintf(buf, sizeof buf, "generic<%s>", dtype == 1 ? "f64" : "f32");
     else
         snprintf(buf, sizeof buf, "seg<%s,LPR=%d,VPL=%d%s>", dtype == 1 ? "f64" : "f32", sh.lpr,
-                 sh.vpl, sh.mode == 1 ? ",ragged" : (sh.mode == 2 ? ",odd" : ""));
+                 sh.vpl, sh.mode == 1 ? ",ragged" : (sh.mode == 2 ? ",odd" : (sh.mode == 3 ? ",thin" : "")));
     return buf;
 }
 

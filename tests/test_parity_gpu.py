@@ -108,7 +108,8 @@ def test_golden_numcheck_closed_form(ctx):
 # ---- K sweep: rows that fill a kernel shape exactly (a power of two of 16-byte
 # vectors), rows that do not (the "ragged" variants: 12, 20, 48, 100, 300 ...), rows
 # that are no whole number of vectors (the "odd" variants: 5, 7, 50, 63, 65, 1023 ...),
-# rows shorter than 16 bytes or longer than 4 KiB (the generic kernels)
+# rows shorter than 16 bytes (the "thin" variant: 1, 2, 3), rows longer than 4 KiB (the
+# generic kernels)
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("k", [1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 15, 16, 17, 20, 24, 31, 32,
                                33, 36, 48, 50, 63, 64, 65, 72, 96, 100, 127, 128, 129, 130, 200,
@@ -128,7 +129,7 @@ def test_segment_lengths_and_cut_rows(ctx, dtype, seg_max):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("k", [5, 7, 12, 48, 50, 63, 65, 100, 129, 136, 257, 264, 511])
+@pytest.mark.parametrize("k", [1, 2, 3, 5, 7, 12, 48, 50, 63, 65, 100, 129, 136, 257, 264, 511])
 def test_cut_rows_with_ragged_k(ctx, dtype, k):
     # partial rows of cut segments and the fix-up pass at row widths that leave lanes idle
     # or end inside a 16-byte vector
@@ -140,7 +141,7 @@ def test_cut_rows_with_ragged_k(ctx, dtype, k):
 # ---- both kernels in one pass over the gathered rows ---------------------------------
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("chained", [False, True])
-@pytest.mark.parametrize("k", [4, 5, 20, 50, 63, 64, 100, 256, 257, 511])
+@pytest.mark.parametrize("k", [1, 2, 3, 4, 5, 20, 50, 63, 64, 100, 256, 257, 511])
 def test_fused_sddmm_spmm_equals_the_two_calls(ctx, dtype, chained, k):
     m, n, nnz = 120, 90, 4000
     ii, jj, vv, A, B, Y0 = rand_case(500 + k, m, n, k, nnz, dtype, hub=900)
@@ -176,7 +177,7 @@ def test_fused_call_on_the_sliced_layout_and_odd_widths(ctx, dtype):
     check_sddmm(A, B, w.ii, w.jj, vv, dC.download())
     check_spmm(B, w.ii, w.jj, dC.download(), Y0, dY.download())
     # K without a vector kernel: the plain form falls back to the two calls, the chained one refuses
-    ii, jj, vv, A, B, Y0 = rand_case(3, 30, 30, 1, 200, dtype)
+    ii, jj, vv, A, B, Y0 = rand_case(3, 30, 30, 1030, 200, dtype)
     S2 = ctx.plan(30, 30, ii, jj, vv)
     dA, dB, dY, dC = ctx.panel_from(A), ctx.panel_from(B), ctx.panel_from(Y0), ctx.vals(200, dtype)
     ctx.sddmm_spmm(S2, dA, dB, dC, dY)
@@ -224,7 +225,7 @@ def test_random_shapes_widths_and_plan_options(ctx, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("k", [64, 20, 50, 7, 129])
+@pytest.mark.parametrize("k", [64, 20, 50, 7, 129, 1, 3])
 def test_rows_the_pattern_never_names_are_never_read(ctx, dtype, k):
     # the reference touches A[ii[e]], B[jj[e]] and Y[ii[e]] only (core_ops.cpp:16,32): NaN
     # in every other dense row must not reach any result, whatever the batching loads
@@ -245,7 +246,7 @@ def test_rows_the_pattern_never_names_are_never_read(ctx, dtype, k):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("k", [64, 50, 7, 129])
+@pytest.mark.parametrize("k", [64, 50, 7, 129, 3, 2, 1])
 def test_non_finite_inputs_propagate_as_in_the_reference(ctx, dtype, k):
     # an infinite X row named with weight a gives a * inf in Y, not NaN from 0 * inf
     # (nor, at widths that end inside a vector, from the elements a lane loads but does
