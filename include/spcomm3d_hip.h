@@ -95,8 +95,10 @@ typedef struct {
 /* Plan tuning; a zero field selects the default.  Only speed depends on these. */
 typedef struct {
     uint32_t seg_max;      /* longest segment in entries (default: nnz / 2048 rounded down to
-                              a power of two, within 64 .. 2048) */
-    uint32_t k_hint;       /* XCD slicing: K the plan will mostly run with (default 64) */
+                              a power of two, within 64 .. 2048; with k_hint given, at most
+                              1024 for dense rows of 128 bytes and 512 for 64 bytes and less) */
+    uint32_t k_hint;       /* K the plan will mostly run with: sizes the XCD slicing (default
+                              64) and the default seg_max */
     uint32_t l2_hot_bytes; /* XCD slicing: share of one XCD's 4 MiB L2 planned for dense rows
                               (default 2 MiB) */
     uint32_t hub_min;      /* XCD slicing: rows with at least this many entries are cut by

@@ -774,6 +774,7 @@ static int resolve_opts(int dtype, const spc3d_plan_opts *o, PlanOpts &out)
     const uint64_t k = z.k_hint ? z.k_hint : 64;
     const uint64_t bytes = z.l2_hot_bytes ? z.l2_hot_bytes : 2u << 20;
     out.hot_cols = (uint32_t)(bytes / (k * elem_size(dtype)));
+    out.row_bytes = (uint32_t)std::min<uint64_t>((uint64_t)z.k_hint * elem_size(dtype), 1u << 30);
     return SPC3D_OK;
 }
 

@@ -67,10 +67,17 @@ void sort_longest_first(std::vector<Piece> &v, uint32_t seg_max)
 
 } // namespace
 
-uint32_t default_seg_max(uint64_t nnz)
+// nnz / 2048 rounded down to a power of two, within 64 .. 2048; at most 1024 for dense
+// rows of 128 bytes and 512 for rows of 64 bytes and less.  One lane group walks a
+// segment batch after batch, two memory latencies per batch, and the narrower the rows
+// the more segments share a wavefront and the fewer wavefronts a launch has: the
+// longest segments then set its duration (R-MAT 20, fp32 K = 16: SDDMM 542 us at 2048,
+// 421 at 512; SpMM 322 and 244; at 256-byte rows and more 1024 and 2048 are level).
+uint32_t default_seg_max(uint64_t nnz, uint32_t row_bytes)
 {
+    const uint32_t cap = row_bytes == 0 || row_bytes > 128 ? 2048u : (row_bytes > 64 ? 1024u : 512u);
     uint32_t s = 64;
-    while (s < 2048 && (uint64_t)s * 2 * 2048 <= nnz)
+    while (s < cap && (uint64_t)s * 2 * 2048 <= nnz)
         s *= 2;
     return s;
 }
@@ -82,7 +89,7 @@ int build_host_plan(uint32_t nrows, uint32_t ncols, uint64_t nnz, const uint32_t
     if (rc != SPC3D_OK)
         return rc;
     const uint32_t seg_max =
-        std::min<uint32_t>(opts.seg_max ? opts.seg_max : default_seg_max(nnz), 1u << 30);
+        std::min<uint32_t>(opts.seg_max ? opts.seg_max : default_seg_max(nnz, opts.row_bytes), 1u << 30);
     const uint32_t hub_min = opts.hub_min ? opts.hub_min : kDefaultHubMin;
     const bool want_slices = opts.xcd_slices == 0 || opts.xcd_slices == kSlices;
 

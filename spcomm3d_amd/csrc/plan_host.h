@@ -38,7 +38,8 @@ struct SplitRow {
 
 // Zero in any field selects the default.
 struct PlanOpts {
-    uint32_t seg_max = 0;    // longest segment (default: by nnz, 64 .. 2048)
+    uint32_t seg_max = 0;    // longest segment (default: by nnz and row_bytes, 64 .. 2048)
+    uint32_t row_bytes = 0;  // bytes of the dense rows the plan will mostly run with (0: unknown)
     uint32_t xcd_slices = 0; // 8 (default): hot columns are dealt to the 8 XCD L2s; 1: off
     uint32_t hot_cols = 0;   // slicing: dense rows one L2 is expected to keep
     uint32_t hub_min = 0;    // slicing: rows with at least this many entries are cut by slice (default 128)
@@ -156,7 +157,7 @@ SPC3D_HD inline uint32_t deal_queue(uint32_t i, const uint32_t (&upto)[kDealQueu
 // partial-sum row in SpMM), short enough that the longest segments do not
 // outlast the rest of the grid: nnz / 2048 rounded down to a power of two,
 // within [64, 2048].
-uint32_t default_seg_max(uint64_t nnz);
+uint32_t default_seg_max(uint64_t nnz, uint32_t row_bytes);
 
 // Returns 0, or an spc3d_status value with `err` filled.
 int validate_coo(uint32_t nrows, uint32_t ncols, uint64_t nnz, const uint32_t *ii,

@@ -165,6 +165,16 @@ def test_plan_default_seg_max_follows_nnz():
     w = W.rmat(17, 16, 64)
     s = device.plan_build_host(w.nrows, w.ncols, w.ii, w.jj)["info"].seg_max
     assert s == 1 << int(np.log2(w.nnz / 2048)) and 64 <= s <= 2048
+    # narrow dense rows put more segments on a wavefront: the cap comes down with k_hint
+    n = 2048 * 2048
+    ii = (np.arange(n, dtype=np.uint32) // 4200).astype(np.uint32)
+    jj = (np.arange(n, dtype=np.uint32) % 777).astype(np.uint32)
+    def seg_max(**kw):
+        return device.plan_build_host(1000, 777, ii, jj, **kw)["info"].seg_max
+    assert seg_max() == 2048 and seg_max(dtype="f32", k_hint=64) == 2048
+    assert seg_max(dtype="f64", k_hint=16) == 1024 and seg_max(dtype="f32", k_hint=32) == 1024
+    assert seg_max(dtype="f32", k_hint=16) == 512 and seg_max(dtype="f32", k_hint=1) == 512
+    assert seg_max(dtype="f32", k_hint=16, seg_max=2048) == 2048  # an explicit value wins
 
 
 def test_plan_sorted_input_is_identity_and_empty_rows_are_skipped():
