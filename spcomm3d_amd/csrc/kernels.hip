@@ -23,7 +23,8 @@
 //          slices of a batch, and reduces the per-lane partial dot products
 //          across the group with a halving exchange (NB-1 exchanges for NB
 //          entries instead of NB*log2(LPR)); exchanges inside a 16-lane row
-//          are DPP moves.  The lane that ends up with entry u's dot product
+//          are DPP moves, those across rows the gfx950 row swaps
+//          (v_permlane16_swap, v_permlane32_swap).  The lane that ends up with entry u's dot product
 //          scales it by S.vv and stores it at the caller's position.
 //   spmm : lane = slice of K, no cross-lane reduction; the group accumulates
 //          a * X[c,:] in registers and does one read-modify-write of the Y
@@ -71,12 +72,14 @@ template <typename P> __device__ __forceinline__ void nt_store(P v, P *p)
 __device__ __forceinline__ constexpr int ilog2(int x) { return x <= 1 ? 0 : 1 + ilog2(x >> 1); }
 
 // ---- lane exchange ----------------------------------------------------------
-// xchg<S>(v): the value lane (id ^ S) holds.  S < 16 stays inside a 16-lane DPP
-// row: xor 1 and 2 are quad permutes, xor 8 is a rotation by 8, xor 4 is
+// xchg<S>(v): the value lane (id ^ S) holds.  S < 16 (the only strides the kernels
+// use it for; 16 and 32 go through swap_add below) stays inside a 16-lane DPP row: xor 1 and 2 are quad permutes, xor 8 is a rotation by 8, xor 4 is
 // half-row mirror (i -> 7 - i = i ^ 7) after quad reverse (i ^ 3).
 template <int CTRL> __device__ __forceinline__ int dpp_mov(int v)
 {
-    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, false);
+    // every lane is written (all rows and banks enabled, the patterns used here have
+    // no invalid source lane): no previous value to set up
+    return __builtin_amdgcn_mov_dpp(v, CTRL, 0xF, 0xF, false);
 }
 template <int S> __device__ __forceinline__ int xchg_i32(int v)
 {
@@ -102,15 +105,48 @@ template <int S> __device__ __forceinline__ double xchg(double v)
     return __hiloint2double(hi, lo);
 }
 
+// Halving step across stride 16 or 32: a and b are two partial sums of which the
+// lanes with bit S clear go on with a and those with bit S set with b.  One
+// v_permlane16_swap / v_permlane32_swap (gfx950) exchanges the odd 16-lane rows of a
+// with the even rows of b (the upper 32 lanes of a with the lower 32 of b): the two
+// results, added, are a summed over the stride in the lanes with bit S clear and b
+// in the others -- no selects and no second move, 2 instructions per 32-bit word
+// where the DPP form takes 4.  With b == a it is the all-reduce across the stride.
+template <int S> __device__ __forceinline__ void swap_rows(unsigned &a, unsigned &b)
+{
+    static_assert(S == 16 || S == 32, "row swaps exist for strides 16 and 32");
+    if constexpr (S == 16) {
+        const auto r = __builtin_amdgcn_permlane16_swap(a, b, false, false);
+        a = r[0], b = r[1];
+    } else {
+        const auto r = __builtin_amdgcn_permlane32_swap(a, b, false, false);
+        a = r[0], b = r[1];
+    }
+}
+template <int S> __device__ __forceinline__ float swap_add(float a, float b)
+{
+    unsigned x = __float_as_uint(a), y = __float_as_uint(b);
+    swap_rows<S>(x, y);
+    return __uint_as_float(x) + __uint_as_float(y);
+}
+template <int S> __device__ __forceinline__ double swap_add(double a, double b)
+{
+    unsigned xl = (unsigned)__double2loint(a), yl = (unsigned)__double2loint(b);
+    unsigned xh = (unsigned)__double2hiint(a), yh = (unsigned)__double2hiint(b);
+    swap_rows<S>(xl, yl);
+    swap_rows<S>(xh, yh);
+    return __hiloint2double((int)xh, (int)xl) + __hiloint2double((int)yh, (int)yl);
+}
+
 // Order in which the xor strides of an LPR-lane group are used: the steps that
-// move the most values come first and get the single-instruction exchanges;
-// strides 16 and 32 (LDS-crossbar permutes) come last.
+// move the most values come first and get the cheapest exchanges: the row swaps
+// of strides 32 and 16, then the single-instruction DPP moves.
 template <int LPR> struct Strides;
 template <> struct Strides<4> { static constexpr int s[2] = {2, 1}; };
 template <> struct Strides<8> { static constexpr int s[3] = {2, 1, 4}; };
 template <> struct Strides<16> { static constexpr int s[4] = {8, 2, 1, 4}; };
-template <> struct Strides<32> { static constexpr int s[5] = {8, 2, 1, 4, 16}; };
-template <> struct Strides<64> { static constexpr int s[6] = {8, 2, 1, 4, 16, 32}; };
+template <> struct Strides<32> { static constexpr int s[5] = {16, 8, 2, 1, 4}; };
+template <> struct Strides<64> { static constexpr int s[6] = {32, 16, 8, 2, 1, 4}; };
 
 // Halving exchange + finishing all-reduce over an LPR-lane group.
 // In: part[u] = this lane's partial sum for entry u, u < NB.  Out: part[0] =
@@ -125,13 +161,20 @@ __device__ __forceinline__ void group_reduce(T (&part)[NB], uint32_t sub)
             const bool upper = (sub & S) != 0;
 #pragma unroll
             for (int i = 0; i < N / 2; ++i) {
-                const T keep = upper ? part[i + N / 2] : part[i];
-                const T send = upper ? part[i] : part[i + N / 2];
-                part[i] = keep + xchg<S>(send);
+                if constexpr (S >= 16) {
+                    part[i] = swap_add<S>(part[i], part[i + N / 2]);
+                } else {
+                    const T keep = upper ? part[i + N / 2] : part[i];
+                    const T send = upper ? part[i] : part[i + N / 2];
+                    part[i] = keep + xchg<S>(send);
+                }
             }
             group_reduce<T, LPR, NB, STEP + 1, N / 2>(part, sub);
         } else {
-            part[0] += xchg<S>(part[0]);
+            if constexpr (S >= 16)
+                part[0] = swap_add<S>(part[0], part[0]);
+            else
+                part[0] += xchg<S>(part[0]);
             group_reduce<T, LPR, NB, STEP + 1, 1>(part, sub);
         }
     }
