@@ -268,8 +268,8 @@ SPC3D_API int spc3d_spmm(spc3d_ctx *ctx, spc3d_plan *A, const spc3d_panel *X, sp
  *                  changing the plan's values).
  * Same results as the separate calls within the summation-order tolerance;
  * requires A.n == B.n == Y.n, Y.m >= nrows, Y aliasing neither A nor B.  The
- * chained form needs K * sizeof(real) to be a multiple of 16 bytes up to 4096
- * (SPC3D_ERR_INVALID_ARG otherwise); the other falls back to the two calls.
+ * chained form needs dense rows of at most 4096 bytes (K <= 1024 in fp32, 512 in
+ * fp64; SPC3D_ERR_INVALID_ARG otherwise); the other falls back to the two calls.
  * Has no counterpart in the reference, which runs its two kernels in separate
  * passes (miniapp/bench_both.cpp:202-203; miniapp/bench_spmm.cpp:185-186).
  * Asynchronous on the context's stream. */

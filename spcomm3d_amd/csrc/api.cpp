@@ -1270,8 +1270,8 @@ int spc3d_sddmm_spmm(spc3d_ctx *ctx, spc3d_plan *S, const spc3d_panel *A, const 
         (void)hipGetLastError();
         if (chained)
             return fail(SPC3D_ERR_INVALID_ARG,
-                        "the chained form needs K * sizeof(real) to be a multiple of 16 bytes, "
-                        "at most 4096");
+                        "the chained form needs dense rows of at most 4096 bytes "
+                        "(K * sizeof(real))");
         // No vector kernel for this K: the two calls one after the other.
         HIP_TRY(launch_sddmm(S->dtype, view_of(S), A->dev, B->dev, C->dev, K, streams_of(ctx)));
         HIP_TRY(launch_spmm(S->dtype, view_of(S), B->dev, Y->dev, K, streams_of(ctx)));

@@ -42,7 +42,8 @@ hipError_t launch_spmm(int dtype, const DevPlanView &P, const void *X, void *Y, 
 // SDDMM and the SpMM of the same pattern over the same B in one pass over the
 // gathered rows: C as launch_sddmm, and Y += W B with W = the plan's values
 // (chained == 0) or the C just computed (chained != 0).  P.partial must hold the
-// plan's partial-sum rows for this K.  hipErrorNotSupported when K has no vector kernel.
+// plan's partial-sum rows for this K.  hipErrorNotSupported when K has no vector kernel
+// (dense rows over 4096 bytes).
 hipError_t launch_sddmm_spmm(int dtype, int chained, const DevPlanView &P, const void *A,
                              const void *B, void *C, void *Y, uint32_t K, const Streams &streams);
 // out[p] = in[perm[p]] (perm == null: copy)
