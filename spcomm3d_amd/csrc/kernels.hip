@@ -298,15 +298,24 @@ template <typename T, int VPL> struct OddLanes {
     uint32_t off[VPL];             // byte offset within a row of this lane's vector v
     bool keep[VPL][Vec<T>::N];     // the elements of it that are this lane's
     bool all[VPL];                 // every element is
+    uint32_t stride;               // reals from one dense row to the next (>= K: the kernel may
+                                   // be working on a slice of K columns of wider rows)
+    bool accum;                    // SDDMM adds to C instead of overwriting it (every slice of
+                                   // wide rows but the first)
 };
 template <typename T, int VPL, int RG> struct Odd {};
 template <typename T, int VPL> struct Odd<T, VPL, 2> : OddLanes<T, VPL> {};
 template <typename T, int VPL> struct Odd<T, VPL, 3> : OddLanes<T, VPL> {};
 
 template <typename T, int LPR, int VPL, int RG>
-__device__ __forceinline__ Odd<T, VPL, RG> odd_lanes(uint32_t sub, uint32_t K)
+__device__ __forceinline__ Odd<T, VPL, RG> odd_lanes(uint32_t sub, uint32_t K, uint32_t stride,
+                                                     uint32_t accum)
 {
     Odd<T, VPL, RG> o;
+    if constexpr (RG >= 2) {
+        o.stride = stride;
+        o.accum = accum != 0;
+    }
     if constexpr (RG == 2) {
         const uint32_t bytes = K * (uint32_t)sizeof(T); // >= 16: see pick_shape
 #pragma unroll
@@ -333,10 +342,10 @@ __device__ __forceinline__ Odd<T, VPL, RG> odd_lanes(uint32_t sub, uint32_t K)
 }
 
 template <typename T, int RG>
-__device__ __forceinline__ const char *odd_row(const T *base, uint32_t row, uint32_t K)
+__device__ __forceinline__ const char *odd_row(const T *base, uint32_t row, uint32_t stride)
 {
-    static_assert(RG >= 2, "rows of K reals at element alignment");
-    return reinterpret_cast<const char *>(base) + (uint64_t)row * ((uint64_t)K * sizeof(T));
+    static_assert(RG >= 2, "rows at element alignment, `stride` reals apart");
+    return reinterpret_cast<const char *>(base) + (uint64_t)row * ((uint64_t)stride * sizeof(T));
 }
 
 // Vector v of the row at r as this lane loads it in the RG >= 2 variants (NT: a
@@ -369,7 +378,7 @@ __device__ __forceinline__ void gather_row(typename Vec<T>::type (&out)[VPL], co
 {
     using V = typename Vec<T>::type;
     if constexpr (RG >= 2) {
-        const char *r = odd_row<T, RG>(base, row, nvec);
+        const char *r = odd_row<T, RG>(base, row, odd.stride);
 #pragma unroll
         for (int v = 0; v < VPL; ++v)
             out[v] = odd_load<T, RG, VPL>(r, v, nvec, odd);
@@ -479,11 +488,15 @@ sddmm_batch_one(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type (&a
         part[u] = lane_dot<T, VPL, RG>(a, b[u], odd);
     }
     group_reduce<T, LPR, NB>(part, sub);
-    const T result = part[0] * sv;
+    T result = part[0] * sv;
     // Results in the caller's order: when that is the kernel order the stores of a
     // batch fill whole lines and stream out; when it is not they are scattered, and
     // plain stores let the L2 merge neighbours into lines before writing back.
     if (writer) {
+        if constexpr (RG >= 2) {
+            if (odd.accum)
+                result += C[dst];
+        }
         if (perm)
             C[dst] = result;
         else
@@ -558,11 +571,15 @@ sddmm_batch_rounds(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type 
             part[u] = lane_dot<T, VPL, RG>(a, b[r * G + u], odd);
         }
         group_reduce<T, LPR, G>(part, sub);
-        const T result = part[0] * sv[r];
+        T result = part[0] * sv[r];
         // Results in the caller's order: when that is the kernel order the stores of a
         // batch fill whole lines and stream out; when it is not they are scattered, and
         // plain stores let the L2 merge neighbours into lines before writing back.
         if (writer[r]) {
+            if constexpr (RG >= 2) {
+                if (odd.accum)
+                    result += C[dst[r]];
+            }
             if (perm)
                 C[dst[r]] = result;
             else
@@ -650,7 +667,8 @@ __global__ void __launch_bounds__(kBlock)
 sddmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint32_t rot,
                  const uint32_t *__restrict__ col, const uint32_t *__restrict__ perm,
                  const T *__restrict__ sval, const T *__restrict__ A, const T *__restrict__ B,
-                 T *__restrict__ C, T *__restrict__ Y, T *__restrict__ partial, uint32_t nvec)
+                 T *__restrict__ C, T *__restrict__ Y, T *__restrict__ partial, uint32_t nvec,
+                 uint32_t stride, uint32_t accum)
 {
     static_assert(UB <= 16 && LPR <= 64, "at most 16 entries in flight per lane");
     using V = typename Vec<T>::type;
@@ -662,10 +680,10 @@ sddmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint3
     if (sg[2] == 0)
         return;
 
-    const Odd<T, VPL, RG> odd = odd_lanes<T, LPR, VPL, RG>(sub, nvec);
+    const Odd<T, VPL, RG> odd = odd_lanes<T, LPR, VPL, RG>(sub, nvec, stride, accum);
     V a[VPL], acc[VPL];
     if constexpr (RG >= 2) {
-        const char *arow = odd_row<T, RG>(A, sg[0], nvec);
+        const char *arow = odd_row<T, RG>(A, sg[0], stride);
 #pragma unroll
         for (int v = 0; v < VPL; ++v) {
             a[v] = odd_load<T, RG, VPL, true>(arow, v, nvec, odd);
@@ -686,8 +704,8 @@ sddmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint3
                                               nvec, odd);
     if constexpr (FZ != 0 && RG >= 2) {
         const bool whole = sg[3] == kWholeRow;
-        char *drow = const_cast<char *>(whole ? odd_row<T, RG>(Y, sg[0], nvec)
-                                              : odd_row<T, RG>(partial, sg[3], nvec));
+        char *drow = const_cast<char *>(whole ? odd_row<T, RG>(Y, sg[0], stride)
+                                              : odd_row<T, RG>(partial, sg[3], stride));
         V y0[VPL];
 #pragma unroll
         for (int v = 0; v < VPL; ++v)
@@ -706,35 +724,6 @@ sddmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint3
             else
                 dst[v * LPR] = acc[v]; // read back by spmm_fixup right after
         }
-    }
-}
-
-// Any K: one wavefront per segment, lanes stride over K, scalar loads.
-template <typename T>
-__global__ void __launch_bounds__(kBlock)
-sddmm_generic_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint32_t rot,
-                     const uint32_t *__restrict__ col, const uint32_t *__restrict__ perm,
-                     const T *__restrict__ sval, const T *__restrict__ A,
-                     const T *__restrict__ B, T *__restrict__ C, uint32_t K)
-{
-    const uint32_t lane = threadIdx.x & 63u;
-    const uint64_t sid = seg_index<1>(nq, rot);
-    if (sid >= nseg)
-        return;
-    const Seg sg = segs[sid];
-    const uint32_t len = sg.len;
-    const T *arow = A + (size_t)sg.row * K;
-    for (uint32_t i = 0; i < len; ++i) {
-        const uint32_t p = sg.start + i;
-        const T *brow = B + (size_t)col[p] * K;
-        T acc = (T)0;
-        for (uint32_t j = lane; j < K; j += 64)
-            acc += arow[j] * brow[j];
-#pragma unroll
-        for (int s = 32; s >= 1; s >>= 1)
-            acc += __shfl_xor(acc, s, 64);
-        if (lane == 0)
-            C[perm ? perm[p] : p] = acc * sval[p];
     }
 }
 
@@ -891,7 +880,7 @@ __global__ void __launch_bounds__(kBlock)
 spmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint32_t rot,
                 const uint32_t *__restrict__ col, const T *__restrict__ sval,
                 const T *__restrict__ X, T *__restrict__ Y, T *__restrict__ partial,
-                uint32_t nvec)
+                uint32_t nvec, uint32_t stride)
 {
     static_assert(UB <= 16 && LPR <= 64, "at most 16 entries in flight per lane");
     using V = typename Vec<T>::type;
@@ -903,7 +892,7 @@ spmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint32
     if (sg[2] == 0)
         return;
     const bool whole = sg[3] == kWholeRow;
-    const Odd<T, VPL, RG> odd = odd_lanes<T, LPR, VPL, RG>(sub, nvec);
+    const Odd<T, VPL, RG> odd = odd_lanes<T, LPR, VPL, RG>(sub, nvec, stride, 0u);
 
     V acc[VPL], y0[VPL];
 #pragma unroll
@@ -912,8 +901,8 @@ spmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint32
         y0[v] = V{};
     }
     if constexpr (RG >= 2) {
-        char *drow = const_cast<char *>(whole ? odd_row<T, RG>(Y, sg[0], nvec)
-                                              : odd_row<T, RG>(partial, sg[3], nvec));
+        char *drow = const_cast<char *>(whole ? odd_row<T, RG>(Y, sg[0], stride)
+                                              : odd_row<T, RG>(partial, sg[3], stride));
         if (whole) {
 #pragma unroll
             for (int v = 0; v < VPL; ++v)
@@ -940,33 +929,6 @@ spmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint32
             else
                 dst[v * LPR] = acc[v]; // read back by spmm_fixup right after
         }
-    }
-}
-
-template <typename T>
-__global__ void __launch_bounds__(kBlock)
-spmm_generic_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint32_t rot,
-                    const uint32_t *__restrict__ col, const T *__restrict__ sval,
-                    const T *__restrict__ X, T *__restrict__ Y, T *__restrict__ partial,
-                    uint32_t K)
-{
-    const uint32_t lane = threadIdx.x & 63u;
-    const uint64_t sid = seg_index<1>(nq, rot);
-    if (sid >= nseg)
-        return;
-    const Seg sg = segs[sid];
-    const uint32_t len = sg.len;
-    if (len == 0)
-        return;
-    const bool whole = sg.slot == kWholeRow;
-    T *dst = whole ? Y + (size_t)sg.row * K : partial + (size_t)sg.slot * K;
-    for (uint32_t j = lane; j < K; j += 64) {
-        T acc = (T)0;
-        for (uint32_t i = 0; i < len; ++i) {
-            const uint32_t p = sg.start + i;
-            acc += sval[p] * X[(size_t)col[p] * K + j];
-        }
-        dst[j] = whole ? dst[j] + acc : acc;
     }
 }
 
@@ -1103,13 +1065,13 @@ copy_kernel(u32x4 *__restrict__ dst, const u32x4 *__restrict__ src, uint64_t nve
 
 // ------------------------------------------------------------- dispatch ----
 struct Shape {
-    int lpr, vpl;  // lpr == 0: generic kernel
+    int lpr, vpl;  // lpr == 0: rows over 4 KiB, run slice by slice
     int mode;      // the kernels' RG: 0 exact, 1 ragged, 2 odd, 3 thin
     uint32_t nvec; // 16-byte vectors per dense row; modes 2, 3: K, the reals per row
 };
 
-// A dense row of K reals of at most 4096 bytes runs the vector kernels; longer ones
-// take the generic kernels, rows under 16 bytes the "thin" variant of the 4-lane shape.  A whole number nvec of 16-byte
+// A dense row of K reals of at most 4096 bytes runs in one launch (pair); longer ones
+// go slice by slice, rows under 16 bytes take the "thin" variant of the 4-lane shape.  A whole number nvec of 16-byte
 // vectors with nvec == LPR * VPL, LPR a power of two in [4, 64] and VPL in {1, 2, 4},
 // runs a kernel with the row stride compiled in; other nvec run the "ragged" variant
 // of the smallest shape that covers a row, in which the lanes past the row's end
@@ -1197,7 +1159,7 @@ inline hipError_t join_aux(const Streams &S)
 
 template <typename T, int LPR, int VPL, int UB, int US, int RG, int FZ>
 hipError_t run_sddmm(const DevPlanView &P, const T *A, const T *B, T *C, T *Y, const Streams &S,
-                     uint32_t nvec)
+                     uint32_t nvec, uint32_t stride = 0, uint32_t accum = 0)
 {
     uint32_t nl = P.nseg_long, ns = P.nseg - P.nseg_long;
     if (nl && ns && P.nseg <= kOneLaunchSegments)
@@ -1207,20 +1169,21 @@ hipError_t run_sddmm(const DevPlanView &P, const T *A, const T *B, T *C, T *Y, c
         hipLaunchKernelGGL((sddmm_seg_kernel<T, LPR, VPL, UB, RG, true, FZ>),
                            dim3(blocks_for_groups(nl, P.nqueues, 64 / LPR)), dim3(kBlock), 0,
                            S.main, P.segs, nl, P.nqueues, 0u, P.col, P.perm, (const T *)P.sval,
-                           A, B, C, Y, (T *)P.partial, nvec);
+                           A, B, C, Y, (T *)P.partial, nvec, stride ? stride : nvec, accum);
     if (ns)
         hipLaunchKernelGGL((sddmm_seg_kernel<T, LPR, VPL, US, RG, false, FZ>),
                            dim3(blocks_for_groups(ns, P.nqueues, 64 / LPR)), dim3(kBlock), 0,
                            both ? S.aux : S.main, P.segs + nl, ns, P.nqueues,
                            both ? S.aux_rot : 0u, P.col, P.perm, (const T *)P.sval, A, B, C, Y,
-                           (T *)P.partial, nvec);
+                           (T *)P.partial, nvec, stride ? stride : nvec, accum);
     const hipError_t launched = hipGetLastError();
     const hipError_t joined = both ? join_aux(S) : hipSuccess;
     return launched != hipSuccess ? launched : joined;
 }
 
 template <typename T, int LPR, int VPL, int UB, int US, int RG>
-hipError_t run_spmm(const DevPlanView &P, const T *X, T *Y, const Streams &S, uint32_t nvec)
+hipError_t run_spmm(const DevPlanView &P, const T *X, T *Y, const Streams &S, uint32_t nvec,
+                    uint32_t stride = 0, size_t slice_off = 0)
 {
     uint32_t nl = P.nseg_long, ns = P.nseg - P.nseg_long;
     if (nl && ns && P.nseg <= kOneLaunchSegments)
@@ -1230,13 +1193,13 @@ hipError_t run_spmm(const DevPlanView &P, const T *X, T *Y, const Streams &S, ui
         hipLaunchKernelGGL((spmm_seg_kernel<T, LPR, VPL, UB, RG, true>),
                            dim3(blocks_for_groups(nl, P.nqueues, 64 / LPR)), dim3(kBlock), 0,
                            S.main, P.segs, nl, P.nqueues, 0u, P.col, (const T *)P.sval, X, Y,
-                           (T *)P.partial, nvec);
+                           (T *)P.partial + slice_off, nvec, stride ? stride : nvec);
     if (ns)
         hipLaunchKernelGGL((spmm_seg_kernel<T, LPR, VPL, US, RG, false>),
                            dim3(blocks_for_groups(ns, P.nqueues, 64 / LPR)), dim3(kBlock), 0,
                            both ? S.aux : S.main, P.segs + nl, ns, P.nqueues,
-                           both ? S.aux_rot : 0u, P.col, (const T *)P.sval, X, Y, (T *)P.partial,
-                           nvec);
+                           both ? S.aux_rot : 0u, P.col, (const T *)P.sval, X, Y,
+                           (T *)P.partial + slice_off, nvec, stride ? stride : nvec);
     const hipError_t launched = hipGetLastError();
     const hipError_t joined = both ? join_aux(S) : hipSuccess;
     return launched != hipSuccess ? launched : joined;
@@ -1271,8 +1234,45 @@ hipError_t launch_fixup(const DevPlanView &P, T *Y, uint32_t K, hipStream_t st)
     return hipGetLastError();
 }
 
+// The shape of rows that end inside a vector (mode 2) or are shorter than one (mode
+// 3), for a slice of sh.nvec columns of rows `stride` reals apart.
+Shape odd_shape(size_t elem, uint32_t K)
+{
+    const size_t bytes = (size_t)K * elem;
+    if (bytes < 16)
+        return {4, 1, 3, K};
+    const uint32_t nvec = (uint32_t)((bytes + 15) / 16);
+    if (nvec > 128)
+        return {64, 4, 2, K};
+    if (nvec > 64)
+        return {64, 2, 2, K};
+    int lpr = 4;
+    while ((uint32_t)lpr < nvec)
+        lpr *= 2;
+    return {lpr, 1, 2, K};
+}
+
+template <typename T, int FZ>
+hipError_t run_sddmm_odd(const Shape &sh, const DevPlanView &P, const T *A, const T *B, T *C,
+                         T *Y, const Streams &SS, uint32_t stride, uint32_t accum)
+{
+#define X(L, V, U, S, S2)                                                                         \
+    if (sh.mode == 2 && sh.lpr == L && sh.vpl == V)                                               \
+        return run_sddmm<T, L, V, U, S, 2, FZ>(P, A, B, C, Y, SS, sh.nvec, stride, accum);
+    SPC3D_FOR_ODD_SHAPES(X)
+#undef X
+    if (sh.mode == 3)
+        return run_sddmm<T, 4, 1, 16, 8, 3, FZ>(P, A, B, C, Y, SS, sh.nvec, stride, accum);
+    return hipErrorInvalidValue;
+}
+
+// Rows over 4 KiB go slice by slice: whole 4 KiB slices of columns first (all 256
+// vector slots of the 64 x 4 shape busy), then what is left of the row, each slice a
+// launch over the whole pattern that adds its part of the dot products to C.
+constexpr uint32_t kSliceBytes = 4096;
+
 // FZ == 0: SDDMM.  FZ == 1, 2: SDDMM fused with the SpMM of the same pattern over
-// the same B (vector kernels only: hipErrorNotSupported for other K).
+// the same B (hipErrorNotSupported for rows over 4 KiB).
 template <typename T, int FZ>
 hipError_t sddmm_typed(const DevPlanView &P, const void *A, const void *B, void *C, void *Y,
                        uint32_t K, const Streams &SS)
@@ -1299,31 +1299,40 @@ hipError_t sddmm_typed(const DevPlanView &P, const void *A, const void *B, void 
     }
     SPC3D_FOR_RAGGED_SHAPES(X)
 #undef X
-#define X(L, V, U, S, S2)                                                                         \
-    if (!done && sh.mode == 2 && sh.lpr == L && sh.vpl == V) {                                    \
-        e = run_sddmm<T, L, V, U, S, 2, FZ>(P, (const T *)A, (const T *)B, (T *)C, (T *)Y, SS,    \
-                                            sh.nvec);                                             \
-        done = true;                                                                              \
-    }
-    SPC3D_FOR_ODD_SHAPES(X)
-#undef X
-    if (!done && sh.mode == 3) {
-        e = run_sddmm<T, 4, 1, 16, 8, 3, FZ>(P, (const T *)A, (const T *)B, (T *)C, (T *)Y, SS,
-                                             sh.nvec);
+    if (!done && sh.mode >= 2) {
+        e = run_sddmm_odd<T, FZ>(sh, P, (const T *)A, (const T *)B, (T *)C, (T *)Y, SS, K, 0u);
         done = true;
     }
     if (!done) {
-        if (FZ != 0)
+        if constexpr (FZ != 0) {
             return hipErrorNotSupported;
-        const uint32_t grid = blocks_for_groups(P.nseg, P.nqueues, 1);
-        hipLaunchKernelGGL((sddmm_generic_kernel<T>), dim3(grid), dim3(kBlock), 0, st, P.segs,
-                           P.nseg, P.nqueues, 0u, P.col, P.perm, (const T *)P.sval, (const T *)A,
-                           (const T *)B, (T *)C, K);
+        } else {
+            const uint32_t per = kSliceBytes / (uint32_t)sizeof(T);
+            for (uint32_t at = 0; at < K && e == hipSuccess; at += per) {
+                const uint32_t w = K - at < per ? K - at : per;
+                e = run_sddmm_odd<T, 0>(odd_shape(sizeof(T), w), P, (const T *)A + at,
+                                        (const T *)B + at, (T *)C, nullptr, SS, K, at != 0);
+            }
+        }
     }
     const hipError_t last = hipGetLastError();
     if (e != hipSuccess || last != hipSuccess)
         return e != hipSuccess ? e : last;
     return FZ != 0 ? launch_fixup<T>(P, (T *)Y, K, st) : hipSuccess;
+}
+
+template <typename T>
+hipError_t run_spmm_odd(const Shape &sh, const DevPlanView &P, const T *X, T *Y,
+                        const Streams &SS, uint32_t stride, size_t slice_off)
+{
+#define X(L, V, U, S, S2)                                                                         \
+    if (sh.mode == 2 && sh.lpr == L && sh.vpl == V)                                               \
+        return run_spmm<T, L, V, U, S2, 2>(P, X, Y, SS, sh.nvec, stride, slice_off);
+    SPC3D_FOR_ODD_SHAPES(X)
+#undef X
+    if (sh.mode == 3)
+        return run_spmm<T, 4, 1, 16, 4, 3>(P, X, Y, SS, sh.nvec, stride, slice_off);
+    return hipErrorInvalidValue;
 }
 
 template <typename T>
@@ -1350,22 +1359,19 @@ hipError_t spmm_typed(const DevPlanView &P, const void *X_, void *Y, uint32_t K,
     }
     SPC3D_FOR_RAGGED_SHAPES(X)
 #undef X
-#define X(L, V, U, S, S2)                                                                         \
-    if (!done && sh.mode == 2 && sh.lpr == L && sh.vpl == V) {                                    \
-        e = run_spmm<T, L, V, U, S2, 2>(P, (const T *)X_, (T *)Y, SS, sh.nvec);                   \
-        done = true;                                                                              \
-    }
-    SPC3D_FOR_ODD_SHAPES(X)
-#undef X
-    if (!done && sh.mode == 3) {
-        e = run_spmm<T, 4, 1, 16, 4, 3>(P, (const T *)X_, (T *)Y, SS, sh.nvec);
+    if (!done && sh.mode >= 2) {
+        e = run_spmm_odd<T>(sh, P, (const T *)X_, (T *)Y, SS, K, 0);
         done = true;
     }
     if (!done) {
-        const uint32_t grid = blocks_for_groups(P.nseg, P.nqueues, 1);
-        hipLaunchKernelGGL((spmm_generic_kernel<T>), dim3(grid), dim3(kBlock), 0, st, P.segs,
-                           P.nseg, P.nqueues, 0u, P.col, (const T *)P.sval, (const T *)X_, (T *)Y,
-                           (T *)P.partial, K);
+        // rows over 4 KiB, slice by slice (see sddmm_typed); the slices of Y and of the
+        // partial-sum rows are disjoint
+        const uint32_t per = kSliceBytes / (uint32_t)sizeof(T);
+        for (uint32_t at = 0; at < K && e == hipSuccess; at += per) {
+            const uint32_t w = K - at < per ? K - at : per;
+            e = run_spmm_odd<T>(odd_shape(sizeof(T), w), P, (const T *)X_ + at, (T *)Y + at, SS, K,
+                                at);
+        }
     }
     if (e == hipSuccess)
         e = hipGetLastError();
@@ -1496,7 +1502,8 @@ const char *kernel_variant(int dtype, uint32_t K)
     static thread_local char buf[64];
     const Shape sh = pick_shape(dtype == 1 ? 8 : 4, K);
     if (sh.lpr == 0)
-        snprintf(buf, sizeof buf, "generic<%s>", dtype == 1 ? "f64" : "f32");
+        snprintf(buf, sizeof buf, "seg<%s,LPR=64,VPL=4,odd> per 4 KiB slice",
+                 dtype == 1 ? "f64" : "f32");
     else
         snprintf(buf, sizeof buf, "seg<%s,LPR=%d,VPL=%d%s>", dtype == 1 ? "f64" : "f32", sh.lpr,
                  sh.vpl, sh.mode == 1 ? ",ragged" : (sh.mode == 2 ? ",odd" : (sh.mode == 3 ? ",thin" : "")));

@@ -108,12 +108,13 @@ def test_golden_numcheck_closed_form(ctx):
 # ---- K sweep: rows that fill a kernel shape exactly (a power of two of 16-byte
 # vectors), rows that do not (the "ragged" variants: 12, 20, 48, 100, 300 ...), rows
 # that are no whole number of vectors (the "odd" variants: 5, 7, 50, 63, 65, 1023 ...),
-# rows shorter than 16 bytes (the "thin" variant: 1, 2, 3), rows longer than 4 KiB (the
-# generic kernels)
+# rows shorter than 16 bytes (the "thin" variant: 1, 2, 3), rows longer than 4 KiB (run
+# as 4 KiB column slices plus a rest, which may be thin: 1025 in fp32, 513 in fp64)
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("k", [1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 15, 16, 17, 20, 24, 31, 32,
                                33, 36, 48, 50, 63, 64, 65, 72, 96, 100, 127, 128, 129, 130, 200,
-                               255, 256, 257, 300, 384, 511, 512, 513, 1023, 1024, 1025, 1028])
+                               255, 256, 257, 300, 384, 511, 512, 513, 1023, 1024, 1025, 1028, 1500,
+                               2048, 2500])
 def test_k_sweep_random_unsorted(ctx, dtype, k):
     ii, jj, vv, A, B, Y0 = rand_case(100 + k, 300, 257, k, 6000, dtype, hub=700)
     check_sddmm(A, B, ii, jj, vv, gpu_sddmm(ctx, 300, 257, ii, jj, vv, A, B, prefill=-5.0))
@@ -129,7 +130,8 @@ def test_segment_lengths_and_cut_rows(ctx, dtype, seg_max):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("k", [1, 2, 3, 5, 7, 12, 48, 50, 63, 65, 100, 129, 136, 257, 264, 511])
+@pytest.mark.parametrize("k", [1, 2, 3, 5, 7, 12, 48, 50, 63, 65, 100, 129, 136, 257, 264, 511, 1030,
+                               2051])
 def test_cut_rows_with_ragged_k(ctx, dtype, k):
     # partial rows of cut segments and the fix-up pass at row widths that leave lanes idle
     # or end inside a 16-byte vector
@@ -176,7 +178,7 @@ def test_fused_call_on_the_sliced_layout_and_odd_widths(ctx, dtype):
     ctx.sddmm_spmm(S, dA, dB, dC, dY, chained=True)
     check_sddmm(A, B, w.ii, w.jj, vv, dC.download())
     check_spmm(B, w.ii, w.jj, dC.download(), Y0, dY.download())
-    # K without a vector kernel: the plain form falls back to the two calls, the chained one refuses
+    # rows over 4 KiB: the plain form falls back to the two calls, the chained one refuses
     ii, jj, vv, A, B, Y0 = rand_case(3, 30, 30, 1030, 200, dtype)
     S2 = ctx.plan(30, 30, ii, jj, vv)
     dA, dB, dY, dC = ctx.panel_from(A), ctx.panel_from(B), ctx.panel_from(Y0), ctx.vals(200, dtype)
@@ -189,7 +191,7 @@ def test_fused_call_on_the_sliced_layout_and_odd_widths(ctx, dtype):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_random_shapes_widths_and_plan_options(ctx, dtype):
-    # every knob at once: skewed patterns, sorted or not, exact / ragged / generic row widths,
+    # every knob at once: skewed patterns, sorted or not, exact / ragged / odd / sliced row widths,
     # cut rows, the sliced layout on small inputs, both plan builders
     rng = np.random.default_rng(99)
     for case in range(40):
@@ -225,7 +227,7 @@ def test_random_shapes_widths_and_plan_options(ctx, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("k", [64, 20, 50, 7, 129, 1, 3])
+@pytest.mark.parametrize("k", [64, 20, 50, 7, 129, 1, 3, 1030])
 def test_rows_the_pattern_never_names_are_never_read(ctx, dtype, k):
     # the reference touches A[ii[e]], B[jj[e]] and Y[ii[e]] only (core_ops.cpp:16,32): NaN
     # in every other dense row must not reach any result, whatever the batching loads
@@ -246,7 +248,7 @@ def test_rows_the_pattern_never_names_are_never_read(ctx, dtype, k):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("k", [64, 50, 7, 129, 3, 2, 1])
+@pytest.mark.parametrize("k", [64, 50, 7, 129, 3, 2, 1, 1027])
 def test_non_finite_inputs_propagate_as_in_the_reference(ctx, dtype, k):
     # an infinite X row named with weight a gives a * inf in Y, not NaN from 0 * inf
     # (nor, at widths that end inside a vector, from the elements a lane loads but does
