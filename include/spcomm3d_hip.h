@@ -115,6 +115,14 @@ typedef struct {
 /* ---- library / errors ------------------------------------------------- */
 SPC3D_API const char *spc3d_version(void);
 SPC3D_API const char *spc3d_last_error(void);
+/* Which kernel variant spc3d_sddmm / spc3d_spmm run for dense rows of k reals of
+ * `dtype`, as text ("seg<f32,LPR=16,VPL=1>": 16 lanes per row, one 16-byte vector
+ * each; ",ragged" / ",odd" / ",thin": rows that leave lanes idle, end inside a
+ * vector, or are shorter than one; "... per 4 KiB slice": rows over 4 KiB).  A
+ * diagnostic with no counterpart in the reference; needs no GPU.  The string
+ * belongs to the calling thread and lasts until its next call.  NULL for an unknown
+ * dtype. */
+SPC3D_API const char *spc3d_kernel_variant(int dtype, uint32_t k);
 SPC3D_API const char *spc3d_status_name(int status);
 SPC3D_API int spc3d_device_count(int *count);
 

@@ -43,6 +43,7 @@ class PlanOpts(ctypes.Structure):
 SIGNATURES = {
     "spc3d_version": (ctypes.c_char_p, []),
     "spc3d_last_error": (ctypes.c_char_p, []),
+    "spc3d_kernel_variant": (ctypes.c_char_p, [ctypes.c_int, ctypes.c_uint32]),
     "spc3d_status_name": (ctypes.c_char_p, [c_int]),
     "spc3d_device_count": (c_int, [P(c_int)]),
     "spc3d_ctx_create": (c_int, [c_int, P(c_vp)]),

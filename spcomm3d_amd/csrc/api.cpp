@@ -231,6 +231,11 @@ const char *spc3d_version(void) { return "spcomm3d_hip 0.1 (gfx950)"; }
 
 const char *spc3d_last_error(void) { return g_err.c_str(); }
 
+const char *spc3d_kernel_variant(int dtype, uint32_t k)
+{
+    return dtype_ok(dtype) ? kernel_variant(dtype, k) : nullptr;
+}
+
 const char *spc3d_status_name(int status)
 {
     switch (status) {

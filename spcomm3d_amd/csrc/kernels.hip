@@ -1501,7 +1501,9 @@ const char *kernel_variant(int dtype, uint32_t K)
 {
     static thread_local char buf[64];
     const Shape sh = pick_shape(dtype == 1 ? 8 : 4, K);
-    if (sh.lpr == 0)
+    if (K == 0)
+        snprintf(buf, sizeof buf, "none (no columns)");
+    else if (sh.lpr == 0)
         snprintf(buf, sizeof buf, "seg<%s,LPR=64,VPL=4,odd> per 4 KiB slice",
                  dtype == 1 ? "f64" : "f32");
     else

@@ -250,3 +250,29 @@ def test_plan_build_host_rejects_bad_arguments():
     rc = lib.spc3d_plan_build_host(capi.F32, 2, 6, 3, vp(ii), vp(jj), ctypes.byref(o),
                                    ctypes.byref(info), None, None, None, 0, None, 0)
     assert rc == capi.ERR_INVALID_ARG
+
+
+def test_kernel_variant_for_every_kind_of_row_width():
+    lib = capi.load()
+    def v(dtype, k):
+        r = lib.spc3d_kernel_variant(dtype, k)
+        return r.decode() if r is not None else None
+    F32, F64 = 0, 1
+    # rows that fill a lane shape exactly: a power of two of 16-byte vectors, 1, 2 or 4 per lane
+    assert v(F32, 64) == "seg<f32,LPR=16,VPL=1>" and v(F64, 64) == "seg<f64,LPR=32,VPL=1>"
+    assert v(F32, 16) == "seg<f32,LPR=4,VPL=1>" and v(F64, 32) == "seg<f64,LPR=16,VPL=1>"
+    assert v(F32, 512) == "seg<f32,LPR=64,VPL=2>" and v(F64, 512) == "seg<f64,LPR=64,VPL=4>"
+    # whole vectors that leave lanes idle: clamped loads up to 16 vectors, masked loads above
+    assert v(F32, 4) == "seg<f32,LPR=4,VPL=1,odd>" and v(F32, 48) == "seg<f32,LPR=16,VPL=1,odd>"
+    assert v(F32, 100) == "seg<f32,LPR=32,VPL=1,ragged>" and v(F64, 100) == "seg<f64,LPR=64,VPL=1,ragged>"
+    assert v(F32, 300) == "seg<f32,LPR=64,VPL=2,ragged>" and v(F64, 300) == "seg<f64,LPR=64,VPL=4,ragged>"
+    # rows that end inside a vector
+    assert v(F32, 50) == "seg<f32,LPR=16,VPL=1,odd>" and v(F32, 65) == "seg<f32,LPR=32,VPL=1,odd>"
+    assert v(F64, 63) == "seg<f64,LPR=32,VPL=1,odd>" and v(F32, 1023) == "seg<f32,LPR=64,VPL=4,odd>"
+    # rows shorter than a vector, rows over 4 KiB
+    assert v(F32, 1) == v(F32, 3) == "seg<f32,LPR=4,VPL=1,thin>" and v(F64, 1) == "seg<f64,LPR=4,VPL=1,thin>"
+    assert v(F64, 2) == "seg<f64,LPR=4,VPL=1,odd>"
+    assert v(F32, 1024) == "seg<f32,LPR=64,VPL=4>" and "per 4 KiB slice" in v(F32, 1025)
+    assert "per 4 KiB slice" in v(F64, 513) and v(F32, 0) == "none (no columns)"
+    assert v(7, 64) is None
+
