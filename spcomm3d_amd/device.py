@@ -474,3 +474,12 @@ def plan_build_host(nrows: int, ncols: int, ii, jj, dtype="f32", **opts) -> dict
                                     info.nsplit_rows),
           "spc3d_plan_build_host")
     return {"info": info, "col": col, "perm": perm, "segs": segs, "splits": splits}
+
+
+def kernel_variant(dtype, k: int) -> str:
+    """Which kernel variant dense rows of k reals of `dtype` run (spc3d_kernel_variant)."""
+    r = capi.load().spc3d_kernel_variant(dtype_code(dtype), int(k))
+    if r is None:
+        raise ValueError("unknown dtype")
+    return r.decode()
+

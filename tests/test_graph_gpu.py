@@ -23,6 +23,9 @@ def operands(ctx, w, dtype):
     (lambda: W.erdos_renyi(16384, 16, 32), np.float64),          # one launch per call
     (lambda: W.rmat(15, 16, 64).shuffled(), np.float32),         # cut rows, fix-up, one launch
     (lambda: W.rmat(19, 16, 16), np.float32),                    # two launches on two streams
+    (lambda: W.rmat(15, 16, 50).shuffled(), np.float32),         # rows that end inside a vector
+    (lambda: W.rmat(13, 16, 1030).shuffled(), np.float64),       # rows over 4 KiB: three slices,
+                                                                 # SDDMM slices accumulate into C
 ])
 def test_replays_equal_eager_runs(ctx, maker, dtype):
     w = maker()
