@@ -44,10 +44,10 @@ METRIC = "SDDMM & SpMM GFLOP/s + % HBM roofline on 1 MI355X, RMAT-20 K=64"
 # on (default plan options) and left null for any other: long-segment launch +
 # short-segment launch (+ fix-up for spmm).
 MEASURED_TRAFFIC = {
-    ("rmat20_ef16", 64, "sorted", "f64"): {"sddmm": 4595.4e6 + 1169.0e6,
-                                           "spmm": 4090.5e6 + 1326.8e6 + 123.1e6},
-    ("rmat20_ef16", 64, "sorted", "f32"): {"sddmm": 2278.9e6 + 675.5e6,
-                                           "spmm": 1840.5e6 + 723.7e6 + 61.8e6},
+    ("rmat20_ef16", 64, "sorted", "f64"): {"sddmm": 4595.1e6 + 1169.0e6,
+                                           "spmm": 4090.1e6 + 1326.9e6 + 123.1e6},
+    ("rmat20_ef16", 64, "sorted", "f32"): {"sddmm": 2278.5e6 + 675.5e6,
+                                           "spmm": 1840.4e6 + 723.7e6 + 61.8e6},
 }
 
 
