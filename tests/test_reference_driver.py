@@ -1,8 +1,9 @@
 """The reference's own sequential checker (miniapp/numCheckSeq.cpp: read a
 MatrixMarket file, fill A and B with i/1000, run SpKernels::sddmm, print the sum
 of C), built twice by `make -C oracle ref`: entirely from the reference's sources
-(oracle/_ref/numCheckSeq_ref), and with the binding of INTEGRATION.md over the GPU
-library in place of the reference's core_ops.cpp (oracle/_ref/numCheckSeq_hip).
+(oracle/_ref/numCheckSeq_ref), and with the binding this library documents for a
+maintainer of the reference (oracle/ref_binding/core_ops_hip.cpp) over the GPU library
+in place of the reference's core_ops.cpp (oracle/_ref/numCheckSeq_hip).
 Same program, same arguments: the printed numbers must be the same."""
 import os
 import re
