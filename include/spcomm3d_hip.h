@@ -165,6 +165,14 @@ SPC3D_API int spc3d_timer_elapsed_ms(spc3d_ctx *ctx, int start, int stop, float 
 
 /* ---- dense panels: denseMatrix (src/basic.hpp:30-44) ------------------- */
 SPC3D_API int spc3d_panel_create(spc3d_ctx *ctx, int dtype, uint32_t m, uint32_t n, spc3d_panel **out);
+/* A panel over the caller's own device memory (m*n reals, row-major, 16-byte aligned,
+ * on the context's GPU): a receive buffer of a collective, a block of rows of a
+ * larger panel (dev + r0*n reals), a tensor of another library.  Nothing is copied
+ * and spc3d_panel_destroy leaves the memory alone; it must outlive the panel and
+ * every call queued on it.  No counterpart in the reference, whose panels are host
+ * vectors. */
+SPC3D_API int spc3d_panel_wrap(spc3d_ctx *ctx, int dtype, uint32_t m, uint32_t n, void *dev,
+                     spc3d_panel **out);
 SPC3D_API int spc3d_panel_destroy(spc3d_panel *p);
 SPC3D_API int spc3d_panel_upload(spc3d_panel *p, const void *host);   /* m*n reals, row-major */
 SPC3D_API int spc3d_panel_download(spc3d_panel *p, void *host);
@@ -176,6 +184,8 @@ SPC3D_API int spc3d_panel_shape(spc3d_panel *p, uint32_t *m, uint32_t *n, int *d
 
 /* ---- value vectors: cooMat::vv (src/SparseMatrix.hpp:36) --------------- */
 SPC3D_API int spc3d_vals_create(spc3d_ctx *ctx, int dtype, uint64_t n, spc3d_vals **out);
+/* The same for a value vector of n reals (see spc3d_panel_wrap). */
+SPC3D_API int spc3d_vals_wrap(spc3d_ctx *ctx, int dtype, uint64_t n, void *dev, spc3d_vals **out);
 SPC3D_API int spc3d_vals_destroy(spc3d_vals *v);
 SPC3D_API int spc3d_vals_upload(spc3d_vals *v, const void *host);
 SPC3D_API int spc3d_vals_download(spc3d_vals *v, void *host);

@@ -58,6 +58,7 @@ SIGNATURES = {
     "spc3d_graph_launch": (c_int, [c_vp]),
     "spc3d_graph_destroy": (c_int, [c_vp]),
     "spc3d_panel_create": (c_int, [c_vp, c_int, c_u32, c_u32, P(c_vp)]),
+    "spc3d_panel_wrap": (c_int, [c_vp, c_int, c_u32, c_u32, c_vp, P(c_vp)]),
     "spc3d_panel_destroy": (c_int, [c_vp]),
     "spc3d_panel_upload": (c_int, [c_vp, c_vp]),
     "spc3d_panel_download": (c_int, [c_vp, c_vp]),
@@ -66,6 +67,7 @@ SIGNATURES = {
     "spc3d_panel_device_ptr": (c_int, [c_vp, P(c_vp)]),
     "spc3d_panel_shape": (c_int, [c_vp, P(c_u32), P(c_u32), P(c_int)]),
     "spc3d_vals_create": (c_int, [c_vp, c_int, c_u64, P(c_vp)]),
+    "spc3d_vals_wrap": (c_int, [c_vp, c_int, c_u64, c_vp, P(c_vp)]),
     "spc3d_vals_destroy": (c_int, [c_vp]),
     "spc3d_vals_upload": (c_int, [c_vp, c_vp]),
     "spc3d_vals_download": (c_int, [c_vp, c_vp]),

@@ -77,6 +77,7 @@ struct spc3d_panel {
     int dtype;
     uint32_t m, n;
     void *dev;
+    bool owned = true; // false: the caller's device memory (spc3d_panel_wrap)
 };
 
 struct spc3d_vals {
@@ -85,6 +86,7 @@ struct spc3d_vals {
     int dtype;
     uint64_t n;
     void *dev;
+    bool owned = true; // false: the caller's device memory (spc3d_vals_wrap)
 };
 
 struct spc3d_rowmap {
@@ -559,6 +561,59 @@ int spc3d_panel_create(spc3d_ctx *ctx, int dtype, uint32_t m, uint32_t n, spc3d_
     return SPC3D_OK;
 }
 
+namespace {
+// `dev` must be `bytes` of device memory of ctx's GPU, 16-byte aligned (the copy and
+// pack kernels move 16-byte vectors from the start of a buffer).
+int check_wrapped(spc3d_ctx *ctx, const void *dev, size_t bytes)
+{
+    if (bytes == 0)
+        return SPC3D_OK;
+    if (!dev)
+        return fail(SPC3D_ERR_INVALID_ARG, "device pointer is NULL");
+    if (reinterpret_cast<uintptr_t>(dev) % 16)
+        return fail(SPC3D_ERR_INVALID_ARG, "device pointer is not 16-byte aligned");
+    hipPointerAttribute_t at;
+    std::memset(&at, 0, sizeof at);
+    if (hipPointerGetAttributes(&at, dev) != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(SPC3D_ERR_INVALID_ARG, "pointer is not known to the HIP runtime");
+    }
+    if (at.type != hipMemoryTypeDevice || at.device != ctx->device)
+        return fail(SPC3D_ERR_INVALID_ARG, "pointer is not device memory of the context's GPU");
+    return SPC3D_OK;
+}
+} // namespace
+
+int spc3d_panel_wrap(spc3d_ctx *ctx, int dtype, uint32_t m, uint32_t n, void *dev,
+                     spc3d_panel **out)
+{
+    if (!out)
+        return fail(SPC3D_ERR_INVALID_ARG, "out is NULL");
+    *out = nullptr;
+    if (!live(ctx))
+        return fail(SPC3D_ERR_INVALID_ARG, "context is NULL or destroyed");
+    if (!dtype_ok(dtype))
+        return fail(SPC3D_ERR_INVALID_ARG, "unknown dtype");
+    int rc = use_device(ctx);
+    if (rc)
+        return rc;
+    rc = check_wrapped(ctx, dev, (size_t)m * n * elem_size(dtype));
+    if (rc)
+        return rc;
+    spc3d_panel *p = new (std::nothrow) spc3d_panel();
+    if (!p)
+        return fail(SPC3D_ERR_ALLOC, "host allocation failed");
+    p->ctx = ctx;
+    p->dtype = dtype;
+    p->m = m;
+    p->n = n;
+    p->dev = (size_t)m * n ? dev : nullptr;
+    p->owned = false;
+    p->magic = kMagicPanel;
+    *out = p;
+    return SPC3D_OK;
+}
+
 int spc3d_panel_destroy(spc3d_panel *p)
 {
     if (!live(p))
@@ -567,7 +622,7 @@ int spc3d_panel_destroy(spc3d_panel *p)
         return rc;
     (void)hipSetDevice(p->ctx->device);
     (void)hipStreamSynchronize(p->ctx->stream);
-    if (p->dev)
+    if (p->dev && p->owned)
         (void)hipFree(p->dev);
     p->magic = 0;
     delete p;
@@ -674,6 +729,36 @@ int spc3d_vals_create(spc3d_ctx *ctx, int dtype, uint64_t n, spc3d_vals **out)
     return SPC3D_OK;
 }
 
+int spc3d_vals_wrap(spc3d_ctx *ctx, int dtype, uint64_t n, void *dev, spc3d_vals **out)
+{
+    if (!out)
+        return fail(SPC3D_ERR_INVALID_ARG, "out is NULL");
+    *out = nullptr;
+    if (!live(ctx))
+        return fail(SPC3D_ERR_INVALID_ARG, "context is NULL or destroyed");
+    if (!dtype_ok(dtype))
+        return fail(SPC3D_ERR_INVALID_ARG, "unknown dtype");
+    if (n >= (1ull << 32))
+        return fail(SPC3D_ERR_TOO_LARGE, "value vector longer than 2^32 - 1");
+    int rc = use_device(ctx);
+    if (rc)
+        return rc;
+    rc = check_wrapped(ctx, dev, (size_t)n * elem_size(dtype));
+    if (rc)
+        return rc;
+    spc3d_vals *v = new (std::nothrow) spc3d_vals();
+    if (!v)
+        return fail(SPC3D_ERR_ALLOC, "host allocation failed");
+    v->ctx = ctx;
+    v->dtype = dtype;
+    v->n = n;
+    v->dev = n ? dev : nullptr;
+    v->owned = false;
+    v->magic = kMagicVals;
+    *out = v;
+    return SPC3D_OK;
+}
+
 int spc3d_vals_destroy(spc3d_vals *v)
 {
     if (!live(v))
@@ -682,7 +767,7 @@ int spc3d_vals_destroy(spc3d_vals *v)
         return rc;
     (void)hipSetDevice(v->ctx->device);
     (void)hipStreamSynchronize(v->ctx->stream);
-    if (v->dev)
+    if (v->dev && v->owned)
         (void)hipFree(v->dev);
     v->magic = 0;
     delete v;

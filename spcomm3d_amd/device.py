@@ -179,13 +179,19 @@ class Context:
 class Panel:
     """Device-resident ``denseMatrix::data`` (``src/basic.hpp:30-36``)."""
 
-    def __init__(self, ctx: Context, m: int, n: int, dtype):
+    def __init__(self, ctx: Context, m: int, n: int, dtype, dev: int | None = None):
+        """``dev``: a device address to wrap (``spc3d_panel_wrap``) instead of allocating."""
         self.ctx, self.m, self.n = ctx, int(m), int(n)
         self.code = dtype_code(dtype)
         self.dtype = _NP[self.code]
         h = ctypes.c_void_p()
-        check(ctx._lib.spc3d_panel_create(ctx._h, self.code, self.m, self.n, ctypes.byref(h)),
-              "spc3d_panel_create")
+        if dev is None:
+            check(ctx._lib.spc3d_panel_create(ctx._h, self.code, self.m, self.n, ctypes.byref(h)),
+                  "spc3d_panel_create")
+        else:
+            check(ctx._lib.spc3d_panel_wrap(ctx._h, self.code, self.m, self.n,
+                                            ctypes.c_void_p(dev), ctypes.byref(h)),
+                  "spc3d_panel_wrap")
         self._h = h
 
     def upload(self, host: np.ndarray):
@@ -227,13 +233,18 @@ class Panel:
 class Vals:
     """Device-resident ``cooMat::vv`` (``src/SparseMatrix.hpp:36``)."""
 
-    def __init__(self, ctx: Context, n: int, dtype):
+    def __init__(self, ctx: Context, n: int, dtype, dev: int | None = None):
+        """``dev``: a device address to wrap (``spc3d_vals_wrap``) instead of allocating."""
         self.ctx, self.n = ctx, int(n)
         self.code = dtype_code(dtype)
         self.dtype = _NP[self.code]
         h = ctypes.c_void_p()
-        check(ctx._lib.spc3d_vals_create(ctx._h, self.code, self.n, ctypes.byref(h)),
-              "spc3d_vals_create")
+        if dev is None:
+            check(ctx._lib.spc3d_vals_create(ctx._h, self.code, self.n, ctypes.byref(h)),
+                  "spc3d_vals_create")
+        else:
+            check(ctx._lib.spc3d_vals_wrap(ctx._h, self.code, self.n, ctypes.c_void_p(dev),
+                                           ctypes.byref(h)), "spc3d_vals_wrap")
         self._h = h
 
     def upload(self, host: np.ndarray):

@@ -63,6 +63,12 @@ template <typename T> class Panel {
     {
         check(spc3d_panel_create(ctx.get(), dtype_of<T>(), m, n, &h_), "spc3d_panel_create");
     }
+    // Over the caller's device memory (spc3d_panel_wrap): nothing is copied or freed.
+    Panel(Context &ctx, uint32_t m, uint32_t n, T *device_memory) : m_(m), n_(n)
+    {
+        check(spc3d_panel_wrap(ctx.get(), dtype_of<T>(), m, n, device_memory, &h_),
+              "spc3d_panel_wrap");
+    }
     ~Panel()
     {
         if (h_)
@@ -88,6 +94,11 @@ template <typename T> class Vals {
     Vals(Context &ctx, uint64_t n) : n_(n)
     {
         check(spc3d_vals_create(ctx.get(), dtype_of<T>(), n, &h_), "spc3d_vals_create");
+    }
+    // Over the caller's device memory (spc3d_vals_wrap): nothing is copied or freed.
+    Vals(Context &ctx, uint64_t n, T *device_memory) : n_(n)
+    {
+        check(spc3d_vals_wrap(ctx.get(), dtype_of<T>(), n, device_memory, &h_), "spc3d_vals_wrap");
     }
     ~Vals()
     {
