@@ -9,9 +9,11 @@
 // holding VPL vectors each (nvec = LPR * VPL with the row stride a compile-time
 // constant, or nvec < LPR * VPL given at run time in the "ragged" variants, whose
 // spare lanes idle, or a row that ends inside its last vector in the "odd"
-// variants); one wavefront works on 64 / LPR segments at once and every
-// global load instruction moves 64 x 16 B.  Segments arrive sorted longest
-// first, so the lane groups of a wavefront run the same trip count.
+// variants, or one shorter than a vector in the "thin" variant; rows over 4 KiB
+// run as 4 KiB column slices, one launch each); one wavefront works on 64 / LPR
+// segments at once and every global load instruction moves 64 x 16 B.  Segments
+// arrive sorted longest first, so the lane groups of a wavefront run the same trip
+// count.
 //
 // A segment is walked in batches of UB entries; what remains is one masked
 // batch (the missing entries repeat the last one's loads and store nothing), or,
@@ -24,8 +26,9 @@
 //          across the group with a halving exchange (NB-1 exchanges for NB
 //          entries instead of NB*log2(LPR)); exchanges inside a 16-lane row
 //          are DPP moves, those across rows the gfx950 row swaps
-//          (v_permlane16_swap, v_permlane32_swap).  The lane that ends up with entry u's dot product
-//          scales it by S.vv and stores it at the caller's position.
+//          (v_permlane16_swap, v_permlane32_swap).  The lane that ends up
+//          with entry u's dot product scales it by S.vv and stores it at the
+//          caller's position.
 //   spmm : lane = slice of K, no cross-lane reduction; the group accumulates
 //          a * X[c,:] in registers and does one read-modify-write of the Y
 //          row slice.  Rows cut into several segments write partial sums that
