@@ -118,6 +118,51 @@ int main(int argc, char **argv)
         threw = true;
     }
     CHECK(threw);
+    // the block-buffered number reader against formatted stream extraction, token by
+    // token, on text with every kind of spacing and number spelling, read in blocks so
+    // small that tokens straddle them
+    {
+        const std::string path = "/tmp/spc3d_test_io_tokens.txt";
+        {
+            std::ofstream o(path);
+            o << "  12\t+7 \r\n\n3.25 -1e-3\t+2.5E+2 .5 7. 1.7976931348623157e308 4.9e-324\n";
+            unsigned long long x = 88172645463325252ull;
+            for (int i = 0; i < 5000; ++i) {
+                x ^= x << 13, x ^= x >> 7, x ^= x << 17;
+                char line[96];
+                std::snprintf(line, sizeof line, "%llu %llu %.17g%s", x % 100000 + 1, (x >> 20) % 100000 + 1,
+                              (double)(long long)(x >> 11) / 9007199254740992.0 - 0.5, i % 3 ? "\n" : " \r\n");
+                o << line;
+            }
+        }
+        for (std::size_t block : {(std::size_t)7, (std::size_t)64, (std::size_t)1000, (std::size_t)1 << 20}) {
+            std::ifstream a(path), b(path);
+            TokenReader tok(a, block);
+            std::uint64_t u = 0, v = 0;
+            double x = 0, y = 0;
+            CHECK(tok.next(u) && (b >> v) && u == v && u == 12);
+            CHECK(tok.next(u) && (b >> v) && u == v && u == 7);
+            std::size_t n = 0;
+            while (tok.next(x)) {
+                if (!(b >> y))
+                    break;
+                if (std::memcmp(&x, &y, 8) != 0)
+                    break;
+                ++n;
+            }
+            CHECK(n == 7 + 3 * 5000);
+            CHECK(!(b >> y)); // both at the end of the file
+        }
+        // what is no number is refused, not skipped
+        {
+            std::ofstream(path) << "12 abc 3";
+            std::ifstream a(path);
+            TokenReader tok(a);
+            std::uint64_t u = 0;
+            CHECK(tok.next(u) && u == 12);
+            CHECK(!tok.next(u));
+        }
+    }
     std::printf("%s (%d failures, real_t = %s)\n", g_fail ? "FAILED" : "PASSED", g_fail,
                 sizeof(real_t) == 8 ? "double" : "float");
     return g_fail ? 1 : 0;
