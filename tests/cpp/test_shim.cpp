@@ -317,6 +317,15 @@ static void test_random_against_oracle_and_remap()
     oracle_sddmm(A, B, S, ref);
     CHECK(max_rel(C.vv, ref, k * 1.0) < kTol);
 
+    // one index changed in place, the last one included (the tail of the key's last
+    // 32-byte block): a new pattern again
+    for (idx_large_t at : {(idx_large_t)7, S.nnz - 1}) {
+        S.jj[at] = (S.jj[at] + 1) % n;
+        sddmm(A, B, S, C);
+        oracle_sddmm(A, B, S, ref);
+        CHECK(max_rel(C.vv, ref, k * 1.0) < kTol);
+    }
+
     // new values on the same pattern
     for (auto &v : S.vv)
         v = (real_t)1 - v;
