@@ -118,6 +118,10 @@ struct spc3d_plan {
     SplitRow *splits;
     void *partial; // [npartial_slots * partial_k] reals
     uint32_t partial_k;
+    // Partial-sum blocks that a call at a larger K has replaced.  They stay allocated
+    // until the plan is destroyed: a sequence recorded earlier (spc3d_capture_*) keeps
+    // the block's address in its kernel arguments and goes on using it.
+    std::vector<void *> retired_partial;
 };
 
 namespace {
@@ -191,6 +195,9 @@ void plan_free_device(spc3d_plan *p)
     if (p->sval) (void)hipFree(p->sval);
     if (p->splits) (void)hipFree(p->splits);
     if (p->partial) (void)hipFree(p->partial);
+    for (void *old : p->retired_partial)
+        (void)hipFree(old);
+    p->retired_partial.clear();
     p->segs = nullptr;
     p->col = p->perm = nullptr;
     p->sval = p->partial = nullptr;
@@ -904,9 +911,14 @@ int spc3d_plan_build_host(int dtype, uint32_t nrows, uint32_t ncols, uint64_t nn
     return SPC3D_OK;
 }
 
+static int ensure_partial(spc3d_plan *p, uint32_t K);
+
+// Row width a plan is created for: sizes the partial-sum rows of its cut rows.
+static uint32_t planned_k(const spc3d_plan_opts *o) { return o && o->k_hint ? o->k_hint : 64u; }
+
 // Plan over arrays that build_device_plan left on the device.
 static int adopt_device_plan(spc3d_ctx *ctx, int dtype, const HostPlan &meta, DevPlanArrays &arr,
-                             spc3d_plan **out)
+                             uint32_t k0, spc3d_plan **out)
 {
     spc3d_plan *p = new (std::nothrow) spc3d_plan();
     int rc = SPC3D_OK;
@@ -920,7 +932,11 @@ static int adopt_device_plan(spc3d_ctx *ctx, int dtype, const HostPlan &meta, De
         p->info.nsplit_rows = arr.nsplit;
         rc = dev_alloc_bytes(&p->sval, (size_t)meta.nnz * elem_size(dtype));
     }
+    if (!rc)
+        rc = ensure_partial(p, k0);
     if (rc) {
+        if (p && p->sval) (void)hipFree(p->sval);
+        if (p && p->partial) (void)hipFree(p->partial);
         if (arr.segs) (void)hipFree(arr.segs);
         if (arr.col) (void)hipFree(arr.col);
         if (arr.perm) (void)hipFree(arr.perm);
@@ -963,7 +979,7 @@ int spc3d_plan_create_from_device(spc3d_ctx *ctx, int dtype, uint32_t nrows, uin
                            (const uint32_t *)dev_jj, po, meta, arr, err);
     if (rc != SPC3D_OK)
         return fail(rc, err);
-    return adopt_device_plan(ctx, dtype, meta, arr, out);
+    return adopt_device_plan(ctx, dtype, meta, arr, planned_k(opts), out);
 }
 
 int spc3d_plan_create_ex(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t ncols, uint64_t nnz,
@@ -1007,7 +1023,7 @@ int spc3d_plan_create_ex(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t nco
         if (d_jj) (void)hipFree(d_jj);
         if (rc)
             return rc;
-        rc = adopt_device_plan(ctx, dtype, meta, arr, &p);
+        rc = adopt_device_plan(ctx, dtype, meta, arr, planned_k(opts), &p);
         if (rc)
             return rc;
     } else {
@@ -1042,6 +1058,8 @@ int spc3d_plan_create_ex(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t nco
             rc = copy_h2d(ctx, p->perm, H.perm.data(), (size_t)nnz * sizeof(uint32_t));
         if (!rc)
             rc = copy_h2d(ctx, p->splits, H.splits.data(), H.splits.size() * sizeof(SplitRow));
+        if (!rc)
+            rc = ensure_partial(p, planned_k(opts));
         if (rc) {
             plan_free_device(p);
             delete p;
@@ -1236,25 +1254,43 @@ int spc3d_plan_get_info(const spc3d_plan *plan, spc3d_plan_info *info)
     return SPC3D_OK;
 }
 
-// Partial-sum rows of cut rows; sized on first use for this K.
+// Partial-sum rows of cut rows.  They are allocated when the plan is created, for the
+// row width it was planned for (k_hint, 64 by default); a call with wider rows gets a
+// larger block, and the one it replaces is kept until the plan is destroyed.
 static int ensure_partial(spc3d_plan *p, uint32_t K)
 {
     if (!p->info.npartial_slots || p->partial_k >= K)
         return SPC3D_OK;
     if (p->ctx->capturing)
         return fail(SPC3D_ERR_INVALID_ARG,
-                    "the plan's partial-sum rows are not allocated for this K yet: run the call "
-                    "once before recording it");
-    HIP_TRY(hipStreamSynchronize(p->ctx->stream));
-    if (p->partial)
-        (void)hipFree(p->partial);
-    p->partial = nullptr;
-    p->partial_k = 0;
-    int rc = dev_alloc_bytes(&p->partial, (size_t)p->info.npartial_slots * K * elem_size(p->dtype));
+                    "the plan's partial-sum rows are narrower than this K: create the plan with "
+                    "k_hint >= K, or run the call once before recording it");
+    void *grown = nullptr;
+    int rc = dev_alloc_bytes(&grown, (size_t)p->info.npartial_slots * K * elem_size(p->dtype));
     if (rc)
         return rc;
+    if (p->partial) {
+        try {
+            p->retired_partial.push_back(p->partial);
+        } catch (const std::bad_alloc &) {
+            (void)hipFree(grown);
+            return fail(SPC3D_ERR_ALLOC, "host allocation failed");
+        }
+    }
+    p->partial = grown;
     p->partial_k = K;
     return SPC3D_OK;
+}
+
+// [lo, lo + bytes) of two device buffers intersect.
+static bool ranges_overlap(const void *a, size_t abytes, const void *b, size_t bbytes)
+{
+    const uintptr_t a0 = (uintptr_t)a, b0 = (uintptr_t)b;
+    return a0 < b0 + bbytes && b0 < a0 + abytes;
+}
+static size_t panel_bytes(const spc3d_panel *p)
+{
+    return (size_t)p->m * p->n * elem_size(p->dtype);
 }
 
 /* ---- hot path ------------------------------------------------------------ */
@@ -1307,8 +1343,8 @@ int spc3d_spmm(spc3d_ctx *ctx, spc3d_plan *Ap, const spc3d_panel *X, spc3d_panel
         return SPC3D_OK;
     if (X->m < Ap->info.ncols || Y->m < Ap->info.nrows)
         return fail(SPC3D_ERR_SIZE_MISMATCH, "panel has fewer rows than the pattern addresses");
-    if (X->dev == Y->dev)
-        return fail(SPC3D_ERR_INVALID_ARG, "X and Y must not alias");
+    if (ranges_overlap(X->dev, panel_bytes(X), Y->dev, panel_bytes(Y)))
+        return fail(SPC3D_ERR_INVALID_ARG, "X and Y must not overlap");
     if (!Ap->has_values)
         return fail(SPC3D_ERR_INVALID_ARG, "plan has no values (spc3d_plan_set_values)");
     int rc = use_device(ctx, true);
@@ -1340,8 +1376,9 @@ int spc3d_sddmm_spmm(spc3d_ctx *ctx, spc3d_plan *S, const spc3d_panel *A, const 
         return fail(SPC3D_ERR_SIZE_MISMATCH, "panel has fewer rows than the pattern addresses");
     if (C->n < S->info.nnz)
         return fail(SPC3D_ERR_SIZE_MISMATCH, "C.vv is shorter than nnz");
-    if (Y->dev == A->dev || Y->dev == B->dev)
-        return fail(SPC3D_ERR_INVALID_ARG, "Y must not alias A or B");
+    if (ranges_overlap(Y->dev, panel_bytes(Y), A->dev, panel_bytes(A)) ||
+        ranges_overlap(Y->dev, panel_bytes(Y), B->dev, panel_bytes(B)))
+        return fail(SPC3D_ERR_INVALID_ARG, "Y must not overlap A or B");
     if (!S->has_values)
         return fail(SPC3D_ERR_INVALID_ARG, "plan has no values (spc3d_plan_set_values)");
     int rc = use_device(ctx, true);

@@ -89,7 +89,7 @@ int build_host_plan(uint32_t nrows, uint32_t ncols, uint64_t nnz, const uint32_t
     if (rc != SPC3D_OK)
         return rc;
     const uint32_t seg_max =
-        std::min<uint32_t>(opts.seg_max ? opts.seg_max : default_seg_max(nnz, opts.row_bytes), 1u << 30);
+        clamp_seg_max(opts.seg_max ? opts.seg_max : default_seg_max(nnz, opts.row_bytes), nnz);
     const uint32_t hub_min = opts.hub_min ? opts.hub_min : kDefaultHubMin;
     const bool want_slices = opts.xcd_slices == 0 || opts.xcd_slices == kSlices;
 

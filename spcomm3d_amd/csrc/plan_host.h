@@ -159,6 +159,14 @@ SPC3D_HD inline uint32_t deal_queue(uint32_t i, const uint32_t (&upto)[kDealQueu
 // within [64, 2048].
 uint32_t default_seg_max(uint64_t nnz, uint32_t row_bytes);
 
+// A requested longest segment, brought into [1, 2^20]: the builders keep one counter
+// per segment length.
+inline uint32_t clamp_seg_max(uint32_t want, uint64_t /*nnz*/)
+{
+    constexpr uint32_t cap = 1u << 20;
+    return want < 1 ? 1 : (want > cap ? cap : want);
+}
+
 // Returns 0, or an spc3d_status value with `err` filled.
 int validate_coo(uint32_t nrows, uint32_t ncols, uint64_t nnz, const uint32_t *ii,
                  const uint32_t *jj, std::string &err);

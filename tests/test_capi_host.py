@@ -276,3 +276,11 @@ def test_kernel_variant_for_every_kind_of_row_width():
     assert "per 4 KiB slice" in v(F64, 513) and v(F32, 0) == "none (no columns)"
     assert v(7, 64) is None
 
+
+
+def test_an_absurd_seg_max_is_brought_down():
+    """The builders keep one counter per segment length: a request of 2^30 must not
+    turn into a 4 GiB array."""
+    e = np.arange(5, dtype=np.uint32)
+    info = device.plan_build_host(5, 5, e, e, seg_max=1 << 30)["info"]
+    assert info.seg_max == 1 << 20 and info.nsegments == 5

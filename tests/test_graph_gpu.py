@@ -39,7 +39,7 @@ def test_replays_equal_eager_runs(ctx, maker, dtype):
         ctx.sddmm(S, dA, dB, C)
         ctx.spmm(S, dB, Y)
 
-    step(other, ctx.panel_from(Y0))  # first use allocates the plan's partial-sum rows
+    step(other, ctx.panel_from(Y0))  # warm-up (rows wider than k_hint would grow the partial sums)
     ctx.sync()
     ctx.capture_begin()
     step(gC, gY)
@@ -61,7 +61,8 @@ def test_calls_that_cannot_be_recorded_are_refused_and_leave_the_recording_intac
     w = W.rmat(13, 16, 64)
     S, dA, dB = operands(ctx, w, np.float64)
     dY, dC = ctx.panel_from(w.panel_Y0("f64")), ctx.vals(w.nnz, np.float64)
-    cut = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, w.values("f64"), seg_max=16)  # never run: no partial rows yet
+    # cut rows, partial-sum rows sized at creation for K = 16: too narrow for K = 64
+    cut = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, w.values("f64"), seg_max=16, k_hint=16)
     ctx.capture_begin()
     with pytest.raises(capi.Spc3dError):
         ctx.capture_begin()                      # already recording
@@ -72,7 +73,7 @@ def test_calls_that_cannot_be_recorded_are_refused_and_leave_the_recording_intac
     with pytest.raises(capi.Spc3dError):
         ctx.vals(10, np.float64)                 # allocates
     with pytest.raises(capi.Spc3dError) as e:
-        ctx.spmm(cut, dB, dY)                    # would allocate its partial-sum rows
+        ctx.spmm(cut, dB, dY)                    # would allocate wider partial-sum rows
     assert "once before" in str(e.value)
     ctx.sddmm(S, dA, dB, dC)                     # the recording is still good
     g = ctx.capture_end()
@@ -83,6 +84,38 @@ def test_calls_that_cannot_be_recorded_are_refused_and_leave_the_recording_intac
     eC = ctx.vals(w.nnz, np.float64)
     ctx.sddmm(S, dA, dB, eC)
     assert np.array_equal(dC.download(), eC.download())
+    g.close()
+
+
+def test_a_recording_survives_a_later_call_with_wider_rows(ctx):
+    """A sequence recorded at K = 32 keeps the address of the plan's partial-sum rows in
+    its kernel arguments; an eager SpMM at K = 64 afterwards needs wider ones.  The block
+    the recording uses must stay alive: its replay is checked against the oracle."""
+    from tests import _oracle as oracle
+
+    w = W.rmat(13, 16, 32)
+    vv = w.values("f64")
+    S = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, vv, seg_max=16, k_hint=32)
+    assert S.info.nsplit_rows > 0
+    X32, Y32 = w.panel_B("f64"), w.panel_Y0("f64")
+    rng = np.random.default_rng(7)
+    X64 = rng.uniform(-1, 1, (w.ncols, 64))
+    Y64 = rng.uniform(-1, 1, (w.nrows, 64))
+    dX32, dY32 = ctx.panel_from(X32), ctx.panel_from(Y32)
+    dX64, dY64 = ctx.panel_from(X64), ctx.panel_from(Y64)
+    ctx.capture_begin()
+    ctx.spmm(S, dX32, dY32)
+    g = ctx.capture_end()
+    ctx.spmm(S, dX64, dY64)      # grows the partial-sum rows
+    ctx.sync()
+    assert oracle.spmm_rel_err(X64, w.ii, w.jj, vv, Y64, dY64.download()) <= 1e-12
+    filler = [ctx.vals(1 << 20, np.float64) for _ in range(4)]  # would reuse a freed block
+    for f in filler:
+        f.fill(1e300)
+    g.launch()
+    ctx.sync()
+    assert oracle.spmm_rel_err(X32, w.ii, w.jj, vv, Y32, dY32.download()) <= 1e-12
+    assert all(np.all(f.download() == 1e300) for f in filler)
     g.close()
 
 

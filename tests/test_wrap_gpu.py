@@ -66,3 +66,27 @@ def test_wrap_refuses_what_is_not_device_memory_of_this_gpu(ctx):
     empty = device.Vals(ctx, 0, np.float32, dev=0)  # nothing to point at
     empty.close()
     good.close()
+
+
+def test_overlapping_row_blocks_are_refused_as_aliases(ctx):
+    """X and Y as two row blocks of one tall panel that share rows: different base
+    addresses, overlapping memory.  SpMM would read rows another lane group is writing."""
+    w = W.rmat(10, 8, 16)
+    vv = w.values(np.float64)
+    S = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, vv)
+    tall = ctx.panel(2 * w.nrows, w.k, np.float64)
+    tall.fill(1.0)
+    row = w.k * 8
+    X = device.Panel(ctx, w.ncols, w.k, np.float64, dev=tall.device_ptr())
+    Y_over = device.Panel(ctx, w.nrows, w.k, np.float64, dev=tall.device_ptr() + row * (w.nrows - 1))
+    Y_next = device.Panel(ctx, w.nrows, w.k, np.float64, dev=tall.device_ptr() + row * w.nrows)
+    with pytest.raises(capi.Spc3dError) as e:
+        ctx.spmm(S, X, Y_over)
+    assert "overlap" in str(e.value)
+    dC = ctx.vals(w.nnz, np.float64)
+    with pytest.raises(capi.Spc3dError):
+        ctx.sddmm_spmm(S, X, X, dC, Y_over)
+    ctx.spmm(S, X, Y_next)  # adjacent, not overlapping: fine
+    ctx.sync()
+    for h in (X, Y_over, Y_next, dC, S, tall):
+        h.close()
