@@ -277,6 +277,22 @@ SPC3D_API int spc3d_plan_get_info(const spc3d_plan *plan, spc3d_plan_info *info)
 SPC3D_API int spc3d_sddmm(spc3d_ctx *ctx, spc3d_plan *S, const spc3d_panel *A,
                 const spc3d_panel *B, spc3d_vals *C);
 SPC3D_API int spc3d_spmm(spc3d_ctx *ctx, spc3d_plan *A, const spc3d_panel *X, spc3d_panel *Y);
+/* spc3d_spmm for callers that cannot allocate device memory (code under HIP graph
+ * capture that was never primed, tight serving loops, harnesses that forbid
+ * hipMalloc): has no counterpart in the reference.  Same operands, checks and
+ * results as spc3d_spmm, bit for bit (the same kernels in the same order); the
+ * partial sums of rows that the plan cut into several segments go to an array of
+ * SPC3D_NOALLOC_SCRATCH_BYTES that is part of the library's device code (each GPU the
+ * library is used on holds it until the process ends) instead of to memory owned by
+ * the plan, and the call performs no allocation and frees nothing.  A plan whose
+ * partial sums need more (npartial_slots * K * sizeof(real) bytes) is refused with
+ * SPC3D_ERR_TOO_LARGE and nothing is queued.  All calls on one GPU share the array:
+ * two such calls must not overlap in time (calls on one context never do; contexts
+ * on the same GPU must not run it concurrently).  Asynchronous on the context's
+ * stream; may be recorded between spc3d_capture_begin and spc3d_capture_end. */
+#define SPC3D_NOALLOC_SCRATCH_BYTES (32u << 20)
+SPC3D_API int spc3d_spmm_noalloc(spc3d_ctx *ctx, spc3d_plan *A, const spc3d_panel *X,
+                       spc3d_panel *Y);
 /* Both kernels over one pattern and one dense operand B in a single pass, so that
  * each gathered row of B is used twice: C as spc3d_sddmm(ctx, S, A, B, C), and
  *   chained == 0:  Y += S B, as spc3d_spmm(ctx, S, B, Y) with S's own values;

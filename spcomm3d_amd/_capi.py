@@ -90,6 +90,7 @@ SIGNATURES = {
     "spc3d_plan_get_info": (c_int, [c_vp, P(PlanInfo)]),
     "spc3d_sddmm": (c_int, [c_vp, c_vp, c_vp, c_vp, c_vp]),
     "spc3d_spmm": (c_int, [c_vp, c_vp, c_vp, c_vp]),
+    "spc3d_spmm_noalloc": (c_int, [c_vp, c_vp, c_vp, c_vp]),
     "spc3d_sddmm_spmm": (c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_int]),
     "spc3d_rowmap_create": (c_int, [c_vp, c_u32, c_u64, c_vp, P(c_vp)]),
     "spc3d_rowmap_destroy": (c_int, [c_vp]),

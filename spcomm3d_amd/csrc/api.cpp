@@ -4,11 +4,12 @@
 // without a device every device call fails.
 #include "../../include/spcomm3d_hip.h"
 
-#include <hip/hip_runtime_api.h>
+#include <hip/hip_runtime.h>
 
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <new>
 #include <string>
 #include <vector>
@@ -59,6 +60,39 @@ inline bool dtype_ok(int dtype) { return dtype == SPC3D_F32 || dtype == SPC3D_F6
 
 } // namespace
 
+// ---- partial-sum rows for the SpMM entry point that allocates nothing ---------------
+// spc3d_spmm_noalloc keeps the partial sums of cut rows here instead of in memory the
+// plan allocated.  Every GPU the library is used on holds its own copy of the array
+// until the process ends; its address on a device is looked up once, with that device
+// current, when the first context on it is created, and host code uses that address,
+// never the array's name.
+constexpr size_t kStaticScratchBytes = (size_t)SPC3D_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices]; // per device; null until looked up
+
+// Address of `scratch` on `device`, which must be current.
+int scratch_of(int device, void **out)
+{
+    *out = nullptr;
+    if (device < 0 || device >= kMaxDevices)
+        return fail(SPC3D_ERR_NO_DEVICE, "device id beyond the library's per-device table");
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[device]) {
+        void *ptr = nullptr;
+        HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        if (!ptr)
+            return fail(SPC3D_ERR_HIP, "hipGetSymbolAddress gave no address for the scratch array");
+        g_scratch_ptr[device] = ptr;
+    }
+    *out = g_scratch_ptr[device];
+    return SPC3D_OK;
+}
+} // namespace
+
 struct spc3d_ctx {
     uint32_t magic;
     int device;
@@ -66,6 +100,7 @@ struct spc3d_ctx {
     hipStream_t aux_stream; // short-segment launches run here, beside the long-segment ones
     hipEvent_t fork_event, join_event;
     uint32_t aux_rot; // (XCD of workgroup 0 on aux - XCD of workgroup 0 on main) mod 8
+    void *scratch;    // this device's copy of the static scratch array (spc3d_spmm_noalloc)
     bool capturing;   // between spc3d_capture_begin and spc3d_capture_end
     hipEvent_t timers[kTimerSlots];
     bool timer_set[kTimerSlots];
@@ -294,6 +329,11 @@ int spc3d_ctx_create(int device, spc3d_ctx **out)
     if (!c)
         return fail(SPC3D_ERR_ALLOC, "host allocation failed");
     c->device = device;
+    rc = scratch_of(device, &c->scratch);
+    if (rc != SPC3D_OK) {
+        delete c;
+        return rc;
+    }
     hipError_t e = hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking);
     if (e != hipSuccess) {
         delete c;
@@ -1328,18 +1368,21 @@ int spc3d_sddmm(spc3d_ctx *ctx, spc3d_plan *S, const spc3d_panel *A, const spc3d
     return SPC3D_OK;
 }
 
-int spc3d_spmm(spc3d_ctx *ctx, spc3d_plan *Ap, const spc3d_panel *X, spc3d_panel *Y)
+// Checks shared by the SpMM entry points; *K = 0 when there is nothing to do.
+static int spmm_check(spc3d_ctx *ctx, spc3d_plan *Ap, const spc3d_panel *X, spc3d_panel *Y,
+                      uint32_t *K)
 {
+    *K = 0;
     if (!live(ctx) || !live(Ap) || !live(X) || !live(Y))
         return fail(SPC3D_ERR_INVALID_ARG, "a handle is NULL or destroyed");
     if (Ap->ctx != ctx || X->ctx != ctx || Y->ctx != ctx)
         return fail(SPC3D_ERR_INVALID_ARG, "operands belong to different contexts");
     if (X->dtype != Ap->dtype || Y->dtype != Ap->dtype)
         return fail(SPC3D_ERR_SIZE_MISMATCH, "operand dtypes differ from the plan's");
-    const uint32_t K = X->n; // core_ops.cpp:25
-    if (Y->n != K)
+    const uint32_t k = X->n; // core_ops.cpp:25
+    if (Y->n != k)
         return fail(SPC3D_ERR_SIZE_MISMATCH, "X.n != Y.n");
-    if (Ap->info.nnz == 0 || K == 0)
+    if (Ap->info.nnz == 0 || k == 0)
         return SPC3D_OK;
     if (X->m < Ap->info.ncols || Y->m < Ap->info.nrows)
         return fail(SPC3D_ERR_SIZE_MISMATCH, "panel has fewer rows than the pattern addresses");
@@ -1347,13 +1390,49 @@ int spc3d_spmm(spc3d_ctx *ctx, spc3d_plan *Ap, const spc3d_panel *X, spc3d_panel
         return fail(SPC3D_ERR_INVALID_ARG, "X and Y must not overlap");
     if (!Ap->has_values)
         return fail(SPC3D_ERR_INVALID_ARG, "plan has no values (spc3d_plan_set_values)");
-    int rc = use_device(ctx, true);
+    *K = k;
+    return SPC3D_OK;
+}
+
+int spc3d_spmm(spc3d_ctx *ctx, spc3d_plan *Ap, const spc3d_panel *X, spc3d_panel *Y)
+{
+    uint32_t K = 0;
+    int rc = spmm_check(ctx, Ap, X, Y, &K);
+    if (rc || K == 0)
+        return rc;
+    rc = use_device(ctx, true);
     if (rc)
         return rc;
     rc = ensure_partial(Ap, K);
     if (rc)
         return rc;
     HIP_TRY(launch_spmm(Ap->dtype, view_of(Ap), X->dev, Y->dev, K, streams_of(ctx)));
+    return SPC3D_OK;
+}
+
+int spc3d_spmm_noalloc(spc3d_ctx *ctx, spc3d_plan *Ap, const spc3d_panel *X, spc3d_panel *Y)
+{
+    uint32_t K = 0;
+    int rc = spmm_check(ctx, Ap, X, Y, &K);
+    if (rc || K == 0)
+        return rc;
+    const uint64_t need = (uint64_t)Ap->info.npartial_slots * K * elem_size(Ap->dtype);
+    if (need > kStaticScratchBytes) {
+        char msg[200];
+        std::snprintf(msg, sizeof msg,
+                      "the partial sums of this plan's cut rows take %llu bytes at K = %u; "
+                      "spc3d_spmm_noalloc has %llu (SPC3D_NOALLOC_SCRATCH_BYTES): use spc3d_spmm",
+                      (unsigned long long)need, K, (unsigned long long)kStaticScratchBytes);
+        return fail(SPC3D_ERR_TOO_LARGE, msg);
+    }
+    rc = use_device(ctx, true);
+    if (rc)
+        return rc;
+    // Every partial-sum row the fix-up reads is written by exactly one segment of this
+    // call first, so what an earlier call left in the array needs no clearing.
+    DevPlanView view = view_of(Ap);
+    view.partial = ctx->scratch;
+    HIP_TRY(launch_spmm(Ap->dtype, view, X->dev, Y->dev, K, streams_of(ctx)));
     return SPC3D_OK;
 }
 

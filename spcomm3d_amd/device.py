@@ -141,6 +141,11 @@ class Context:
         """Y[ii[e]] += A.vv[e] * X[jj[e]]  (src/core_ops.cpp:24-35); asynchronous."""
         check(self._lib.spc3d_spmm(self._h, A._h, X._h, Y._h), "spc3d_spmm")
 
+    def spmm_noalloc(self, A: "Plan", X: "Panel", Y: "Panel"):
+        """:meth:`spmm` without any allocation (``spc3d_spmm_noalloc``): the partial sums of
+        cut rows live in an array that is part of the library's device code."""
+        check(self._lib.spc3d_spmm_noalloc(self._h, A._h, X._h, Y._h), "spc3d_spmm_noalloc")
+
     def sddmm_host(self, A: np.ndarray, B: np.ndarray, ii, jj, svv: np.ndarray) -> np.ndarray:
         """One-shot SDDMM over host arrays (``spc3d_sddmm_host``); returns C.vv."""
         A, B, svv = (np.ascontiguousarray(x) for x in (A, B, svv))
