@@ -145,9 +145,10 @@ SPC3D_API int spc3d_ctx_probe_xcd(spc3d_ctx *ctx, uint32_t nblocks, uint32_t *xc
  * spc3d_panel_copy, spc3d_vals_fill, spc3d_plan_set_values_device - are recorded
  * instead of run; every other call on the context (anything that allocates,
  * copies to or from the host, waits or times) returns SPC3D_ERR_INVALID_ARG and
- * leaves the recording intact.  An SpMM over a plan with cut rows must have run
- * once with the same K before it is recorded (its partial-sum rows are
- * allocated on first use).  spc3d_graph_launch replays the sequence on the
+ * leaves the recording intact.  An SpMM over a plan with cut rows whose dense rows
+ * are wider than the plan was created for (k_hint, 64 by default) needs wider
+ * partial-sum rows than the plan holds: create the plan with k_hint >= K, or run
+ * the call once before recording it.  spc3d_graph_launch replays the sequence on the
  * context's stream, asynchronously, over the same operands; their contents at
  * launch time are what the kernels read.  Has no counterpart in the reference. */
 typedef struct spc3d_graph spc3d_graph;
