@@ -151,6 +151,7 @@ struct spc3d_plan {
     uint32_t *perm; // null when the caller's order is already the kernel order
     void *sval;     // values in kernel order
     SplitRow *splits;
+    uint32_t *first_cols; // [(nsegments_padded - nsegments_long) * kFirstCols], see kernels.h
     void *partial; // [npartial_slots * partial_k] reals
     uint32_t partial_k;
     // Partial-sum blocks that a call at a larger K has replaced.  They stay allocated
@@ -229,6 +230,7 @@ void plan_free_device(spc3d_plan *p)
     if (p->perm) (void)hipFree(p->perm);
     if (p->sval) (void)hipFree(p->sval);
     if (p->splits) (void)hipFree(p->splits);
+    if (p->first_cols) (void)hipFree(p->first_cols);
     if (p->partial) (void)hipFree(p->partial);
     for (void *old : p->retired_partial)
         (void)hipFree(old);
@@ -237,6 +239,7 @@ void plan_free_device(spc3d_plan *p)
     p->col = p->perm = nullptr;
     p->sval = p->partial = nullptr;
     p->splits = nullptr;
+    p->first_cols = nullptr;
 }
 
 Streams streams_of(const spc3d_ctx *c)
@@ -263,6 +266,7 @@ DevPlanView view_of(const spc3d_plan *p)
     v.splits = p->splits;
     v.nsplit = p->info.nsplit_rows;
     v.partial = p->partial;
+    v.first_cols = p->first_cols;
     v.nnz = p->info.nnz;
     return v;
 }
@@ -953,6 +957,20 @@ int spc3d_plan_build_host(int dtype, uint32_t nrows, uint32_t ncols, uint64_t nn
 
 static int ensure_partial(spc3d_plan *p, uint32_t K);
 
+// What a plan holds beside the builders' arrays: the table of first column indices of
+// its short segments (read by the short-segment launch next to the descriptors) and
+// the partial-sum rows of its cut rows for k0 columns.
+static int finish_plan(spc3d_plan *p, uint32_t k0)
+{
+    const uint32_t nshort = p->info.nsegments_padded - p->info.nsegments_long;
+    int rc = dev_alloc(&p->first_cols, (size_t)nshort * kFirstCols);
+    if (rc)
+        return rc;
+    HIP_TRY(launch_first_cols(p->segs + p->info.nsegments_long, nshort, p->col, p->first_cols,
+                              p->ctx->stream));
+    return ensure_partial(p, k0);
+}
+
 // Row width a plan is created for: sizes the partial-sum rows of its cut rows.
 static uint32_t planned_k(const spc3d_plan_opts *o) { return o && o->k_hint ? o->k_hint : 64u; }
 
@@ -972,11 +990,7 @@ static int adopt_device_plan(spc3d_ctx *ctx, int dtype, const HostPlan &meta, De
         p->info.nsplit_rows = arr.nsplit;
         rc = dev_alloc_bytes(&p->sval, (size_t)meta.nnz * elem_size(dtype));
     }
-    if (!rc)
-        rc = ensure_partial(p, k0);
     if (rc) {
-        if (p && p->sval) (void)hipFree(p->sval);
-        if (p && p->partial) (void)hipFree(p->partial);
         if (arr.segs) (void)hipFree(arr.segs);
         if (arr.col) (void)hipFree(arr.col);
         if (arr.perm) (void)hipFree(arr.perm);
@@ -989,6 +1003,12 @@ static int adopt_device_plan(spc3d_ctx *ctx, int dtype, const HostPlan &meta, De
     p->perm = arr.perm;
     p->splits = arr.splits;
     arr = DevPlanArrays{};
+    rc = finish_plan(p, k0);
+    if (rc) {
+        plan_free_device(p);
+        delete p;
+        return rc;
+    }
     p->magic = kMagicPlan;
     *out = p;
     return SPC3D_OK;
@@ -1099,7 +1119,7 @@ int spc3d_plan_create_ex(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t nco
         if (!rc)
             rc = copy_h2d(ctx, p->splits, H.splits.data(), H.splits.size() * sizeof(SplitRow));
         if (!rc)
-            rc = ensure_partial(p, planned_k(opts));
+            rc = finish_plan(p, planned_k(opts));
         if (rc) {
             plan_free_device(p);
             delete p;

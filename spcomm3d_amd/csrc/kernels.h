@@ -20,6 +20,9 @@ struct DevPlanView {
     const SplitRow *splits = nullptr;
     uint32_t nsplit = 0;
     void *partial = nullptr;          // [nslots * K] partial sums of cut rows (SpMM)
+    // [(nseg - nseg_long) * kFirstCols] the first column indices of every segment past
+    // the long ones (launch_first_cols); read by the short-segment launch
+    const uint32_t *first_cols = nullptr;
     uint64_t nnz = 0;
 };
 
@@ -46,6 +49,9 @@ hipError_t launch_spmm(int dtype, const DevPlanView &P, const void *X, void *Y, 
 // (dense rows over 4096 bytes).
 hipError_t launch_sddmm_spmm(int dtype, int chained, const DevPlanView &P, const void *A,
                              const void *B, void *C, void *Y, uint32_t K, const Streams &streams);
+// first_cols[s * kFirstCols + u] = column of entry min(u, len - 1) of segment segs[s], s < n
+hipError_t launch_first_cols(const Seg *segs, uint32_t n, const uint32_t *col, uint32_t *first_cols,
+                             hipStream_t stream);
 // out[p] = in[perm[p]] (perm == null: copy)
 hipError_t launch_gather_vals(int dtype, const void *in, const uint32_t *perm, void *out,
                               uint64_t n, hipStream_t stream);

@@ -243,6 +243,48 @@ template <int G> __device__ __forceinline__ uint64_t seg_index(uint32_t nq, uint
            (threadIdx.x & 63u) / (64 / G);
 }
 
+// The short-segment launch walks a dependency chain per segment: descriptor, then
+// column indices, then the gathers.  The plan keeps the first kFirstCols column indices
+// of every short segment in a table addressed by the segment's position (past the
+// segment's end they repeat its last column), so that they are fetched beside the
+// descriptor instead of after it: two memory latencies per segment instead of three.
+// Lane u of a group of LPR >= kFirstCols lanes gets the column of entry u % kFirstCols;
+// a group of 4 lanes gets those of entries u and 4 + u.
+struct FirstCols {
+    uint32_t c[2];
+};
+template <int LPR, bool WIDE>
+__device__ __forceinline__ FirstCols load_first_cols(const uint32_t *__restrict__ first_cols,
+                                                     uint64_t sid, uint32_t sub)
+{
+    FirstCols f{{0, 0}};
+    if constexpr (!WIDE) {
+        constexpr uint32_t GL = (uint32_t)LPR < kFirstCols ? (uint32_t)LPR : kFirstCols;
+        const uint32_t *at = first_cols + sid * kFirstCols + (sub & (GL - 1));
+        f.c[0] = nt_load(at);
+        if constexpr ((uint32_t)LPR < kFirstCols)
+            f.c[1] = nt_load(at + LPR);
+    }
+    return f;
+}
+
+// Fills the table above for `n` short segments.
+__global__ void __launch_bounds__(kBlock)
+first_cols_kernel(const Seg *__restrict__ segs, uint32_t n, const uint32_t *__restrict__ col,
+                  uint32_t *__restrict__ first_cols)
+{
+    const uint64_t t = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    const uint64_t s = t / kFirstCols;
+    const uint32_t u = (uint32_t)(t % kFirstCols);
+    if (s >= n)
+        return;
+    const Seg sg = segs[s];
+    uint32_t c = 0;
+    if (sg.len)
+        c = col[sg.start + (u < sg.len ? u : sg.len - 1)];
+    first_cols[t] = c;
+}
+
 // RG == 1 ("ragged"): a dense row is nvec 16-byte vectors with nvec < LPR * VPL,
 // given at run time; lanes whose vector index is >= nvec idle.  RG == 0: nvec ==
 // LPR * VPL exactly and the row stride is a compile-time constant.  RG == 2, 3: below.
@@ -450,13 +492,21 @@ __device__ __forceinline__ void odd_store(char *drow, bool whole,
 // acc += w_u * B[c_u,:] in kernel order, with w_u = S.vv (FZ == 1) or the SDDMM
 // result just computed (FZ == 2); the weight of entry u is broadcast from the lane
 // that stores it.
-template <typename T, int LPR, int VPL, int NB, int RG, bool MK, int FZ>
+//
+// PRE: the column indices of the batch were loaded ahead (lane u of the group holds that
+// of entry u in pre[0], or, where the group has fewer lanes than the batch has entries,
+// those of entries u and LPR + u in pre[0] and pre[1]); past the segment's end they
+// repeat its last column.
+//
+// NG <= NB: every lane group of the wavefront has at most NG entries in this batch, so
+// only the first NG gathers are issued.
+template <typename T, int LPR, int VPL, int NB, int RG, bool MK, int FZ, bool PRE, int NG>
 __device__ __forceinline__ void
 sddmm_batch_one(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type (&acc)[VPL],
             const uint32_t *__restrict__ col, const uint32_t *__restrict__ perm,
             const T *__restrict__ sval, const T *__restrict__ B, T *__restrict__ C, uint32_t p0,
             uint32_t n, uint32_t sub, uint32_t nvec,
-            const Odd<T, VPL, RG> &odd)
+            const Odd<T, VPL, RG> &odd, const uint32_t (&pre)[2])
 {
     using V = typename Vec<T>::type;
     static_assert(NB <= LPR, "batch must fit the lane group");
@@ -466,7 +516,7 @@ sddmm_batch_one(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type (&a
     uint32_t e = sub & (NB - 1);
     if (MK)
         e = e < n ? e : n - 1;
-    const uint32_t cme = nt_load(col + p0 + e);
+    const uint32_t cme = PRE ? pre[0] : nt_load(col + p0 + e);
     const uint32_t uo = entry_of<LPR, NB>(sub);
     const bool writer = is_writer<LPR, NB>(sub) && (!MK || uo < n);
     T sv = (T)0;
@@ -477,9 +527,10 @@ sddmm_batch_one(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type (&a
             dst = nt_load(perm + p0 + uo);
     }
 
-    V b[NB][VPL];
+    static_assert(NG >= 1 && NG <= NB && (MK || NG == NB), "NG < NB only in a masked batch");
+    V b[NG][VPL];
 #pragma unroll
-    for (int u = 0; u < NB; ++u) {
+    for (int u = 0; u < NG; ++u) {
         const uint32_t c = __shfl(cme, u, LPR);
         gather_row<T, LPR, VPL, RG>(b[u], B, c, sub, nvec, odd);
     }
@@ -488,7 +539,10 @@ sddmm_batch_one(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type (&a
     T part[NB];
 #pragma unroll
     for (int u = 0; u < NB; ++u) {
-        part[u] = lane_dot<T, VPL, RG>(a, b[u], odd);
+        if (u < NG)
+            part[u] = lane_dot<T, VPL, RG>(a, b[u], odd);
+        else
+            part[u] = (T)0;
     }
     group_reduce<T, LPR, NB>(part, sub);
     T result = part[0] * sv;
@@ -508,7 +562,7 @@ sddmm_batch_one(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type (&a
     if constexpr (FZ != 0) {
         const T mine = FZ == 2 ? result : sv; // valid on the writer lanes
 #pragma unroll
-        for (int u = 0; u < NB; ++u) {
+        for (int u = 0; u < NG; ++u) {
             const bool on = !MK || (uint32_t)u < n;
             const T w = on ? __shfl(mine, writer_lane<LPR, NB>(u), LPR) : (T)0;
 #pragma unroll
@@ -518,13 +572,13 @@ sddmm_batch_one(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type (&a
     }
 }
 
-template <typename T, int LPR, int VPL, int NB, int RG, bool MK, int FZ>
+template <typename T, int LPR, int VPL, int NB, int RG, bool MK, int FZ, bool PRE>
 __device__ __forceinline__ void
 sddmm_batch_rounds(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type (&acc)[VPL],
             const uint32_t *__restrict__ col, const uint32_t *__restrict__ perm,
             const T *__restrict__ sval, const T *__restrict__ B, T *__restrict__ C, uint32_t p0,
             uint32_t n, uint32_t sub, uint32_t nvec,
-            const Odd<T, VPL, RG> &odd)
+            const Odd<T, VPL, RG> &odd, const uint32_t (&pre)[2])
 {
     using V = typename Vec<T>::type;
     // A group of LPR lanes reduces at most LPR entries at a time: the NB entries of
@@ -533,6 +587,7 @@ sddmm_batch_rounds(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type 
     constexpr int G = NB < LPR ? NB : LPR;
     constexpr int R = NB / G;
     static_assert(R * G == NB, "a batch is a whole number of rounds");
+    static_assert(!PRE || R <= 2, "at most two rounds of columns are loaded ahead");
 
     // Lane u of the group fetches the column of entry u of each round; the writer
     // lanes fetch what they need for the store.  These head the dependency chain.
@@ -546,7 +601,7 @@ sddmm_batch_rounds(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type 
         uint32_t e = (uint32_t)r * G + (sub & (G - 1));
         if (MK)
             e = e < n ? e : n - 1;
-        cme[r] = nt_load(col + p0 + e);
+        cme[r] = PRE ? pre[r & 1] : nt_load(col + p0 + e);
         const uint32_t mine = (uint32_t)r * G + uo;
         writer[r] = wlane && (!MK || mine < n);
         sv[r] = (T)0;
@@ -607,56 +662,81 @@ sddmm_batch_rounds(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type 
 // R = 1 case of the rounds form, the single round compiles to 24 more VGPRs
 // (100 -> 124 in the wide launch, 62 -> 74 and two wavefronts per SIMD fewer in
 // the short one), which cost the 5-entry rows of a stencil 20 %.
-template <typename T, int LPR, int VPL, int NB, int RG, bool MK, int FZ>
+template <typename T, int LPR, int VPL, int NB, int RG, bool MK, int FZ, bool PRE = false,
+          int NG = NB>
 __device__ __forceinline__ void
 sddmm_batch(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type (&acc)[VPL],
             const uint32_t *__restrict__ col, const uint32_t *__restrict__ perm,
             const T *__restrict__ sval, const T *__restrict__ B, T *__restrict__ C, uint32_t p0,
             uint32_t n, uint32_t sub, uint32_t nvec,
-            const Odd<T, VPL, RG> &odd)
+            const Odd<T, VPL, RG> &odd, const uint32_t (&pre)[2])
 {
     if constexpr (NB <= LPR)
-        sddmm_batch_one<T, LPR, VPL, NB, RG, MK, FZ>(a, acc, col, perm, sval, B, C, p0, n, sub,
-                                                     nvec, odd);
+        sddmm_batch_one<T, LPR, VPL, NB, RG, MK, FZ, PRE, NG>(a, acc, col, perm, sval, B, C, p0, n,
+                                                              sub, nvec, odd, pre);
     else
-        sddmm_batch_rounds<T, LPR, VPL, NB, RG, MK, FZ>(a, acc, col, perm, sval, B, C, p0, n, sub,
-                                                        nvec, odd);
+        sddmm_batch_rounds<T, LPR, VPL, NB, RG, MK, FZ, PRE>(a, acc, col, perm, sval, B, C, p0, n,
+                                                             sub, nvec, odd, pre);
 }
 
 // n consecutive entries from p.  WIDE: full batches of UB, then one masked batch
 // of the smallest size in {4, 8, 16} that holds the rest.  !WIDE (segments known
-// to be short, run at twice the occupancy): masked batches of UB throughout.
+// to be short, run at twice the occupancy): masked batches of UB throughout, the
+// first of them on the column indices in `pre` (loaded ahead, beside the segment's
+// descriptor, from the plan's table of first columns: kFirstCols per short segment).
 template <typename T, int LPR, int VPL, int UB, int RG, bool WIDE, int FZ>
 __device__ __forceinline__ void
 sddmm_walk(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type (&acc)[VPL],
            const uint32_t *__restrict__ col, const uint32_t *__restrict__ perm,
            const T *__restrict__ sval, const T *__restrict__ B, T *__restrict__ C, uint32_t p,
            uint32_t n, uint32_t sub, uint32_t nvec,
-            const Odd<T, VPL, RG> &odd)
+            const Odd<T, VPL, RG> &odd, const uint32_t (&pre)[2])
 {
     if constexpr (WIDE) {
         for (; n >= UB; n -= UB, p += UB)
-            sddmm_batch<T, LPR, VPL, UB, RG, false, FZ>(a, acc, col, perm, sval, B, C, p, UB, sub, nvec, odd);
+            sddmm_batch<T, LPR, VPL, UB, RG, false, FZ>(a, acc, col, perm, sval, B, C, p, UB, sub, nvec, odd, pre);
         if (n == 0)
             return;
         if constexpr (UB > 8) {
             if (n > 8) {
-                sddmm_batch<T, LPR, VPL, UB, RG, true, FZ>(a, acc, col, perm, sval, B, C, p, n, sub, nvec, odd);
+                sddmm_batch<T, LPR, VPL, UB, RG, true, FZ>(a, acc, col, perm, sval, B, C, p, n, sub, nvec, odd, pre);
                 return;
             }
         }
         if constexpr (UB > 4) {
             if (n > 4) {
-                sddmm_batch<T, LPR, VPL, 8, RG, true, FZ>(a, acc, col, perm, sval, B, C, p, n, sub, nvec, odd);
+                sddmm_batch<T, LPR, VPL, 8, RG, true, FZ>(a, acc, col, perm, sval, B, C, p, n, sub, nvec, odd, pre);
                 return;
             }
         }
-        sddmm_batch<T, LPR, VPL, (UB < 4 ? UB : 4), RG, true, FZ>(a, acc, col, perm, sval, B, C, p, n, sub, nvec, odd);
+        sddmm_batch<T, LPR, VPL, (UB < 4 ? UB : 4), RG, true, FZ>(a, acc, col, perm, sval, B, C, p, n, sub, nvec, odd, pre);
     } else {
+        static_assert(WIDE || UB <= (int)kFirstCols, "the first batch runs on the columns loaded ahead");
+        {
+            // Segments arrive sorted by length, so the groups of a wavefront mostly hold
+            // the same number of entries: the batch is cut to what the longest of them
+            // needs (a condition uniform over the wavefront), which spares the memory
+            // pipeline the repeated gathers of a full masked batch.
+            const uint32_t m = n < (uint32_t)UB ? n : (uint32_t)UB;
+            if constexpr (UB == 8 && LPR >= 8) {
+                if (__ballot(m > 2) == 0)
+                    sddmm_batch<T, LPR, VPL, 2, RG, true, FZ, true>(a, acc, col, perm, sval, B, C, p, m, sub, nvec, odd, pre);
+                else if (__ballot(m > 4) == 0)
+                    sddmm_batch<T, LPR, VPL, 4, RG, true, FZ, true>(a, acc, col, perm, sval, B, C, p, m, sub, nvec, odd, pre);
+                else if (__ballot(m > 5) == 0)
+                    sddmm_batch<T, LPR, VPL, 8, RG, true, FZ, true, 5>(a, acc, col, perm, sval, B, C, p, m, sub, nvec, odd, pre);
+                else
+                    sddmm_batch<T, LPR, VPL, 8, RG, true, FZ, true>(a, acc, col, perm, sval, B, C, p, m, sub, nvec, odd, pre);
+            } else {
+                sddmm_batch<T, LPR, VPL, UB, RG, true, FZ, true>(a, acc, col, perm, sval, B, C, p, m, sub, nvec, odd, pre);
+            }
+            n -= m;
+            p += m;
+        }
 #pragma nounroll
         while (n > 0) {
             const uint32_t m = n < (uint32_t)UB ? n : (uint32_t)UB;
-            sddmm_batch<T, LPR, VPL, UB, RG, true, FZ>(a, acc, col, perm, sval, B, C, p, m, sub, nvec, odd);
+            sddmm_batch<T, LPR, VPL, UB, RG, true, FZ>(a, acc, col, perm, sval, B, C, p, m, sub, nvec, odd, pre);
             n -= m;
             p += m;
         }
@@ -671,7 +751,7 @@ sddmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint3
                  const uint32_t *__restrict__ col, const uint32_t *__restrict__ perm,
                  const T *__restrict__ sval, const T *__restrict__ A, const T *__restrict__ B,
                  T *__restrict__ C, T *__restrict__ Y, T *__restrict__ partial, uint32_t nvec,
-                 uint32_t stride, uint32_t accum)
+                 uint32_t stride, uint32_t accum, const uint32_t *__restrict__ first_cols)
 {
     static_assert(UB <= 16 && LPR <= 64, "at most 16 entries in flight per lane");
     using V = typename Vec<T>::type;
@@ -679,6 +759,7 @@ sddmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint3
     const uint64_t sid = seg_index<64 / LPR>(nq, rot);
     if (sid >= nseg)
         return;
+    const FirstCols pre = load_first_cols<LPR, WIDE>(first_cols, sid, sub);
     const u32x4 sg = nt_load(reinterpret_cast<const u32x4 *>(segs) + sid); // row, start, len, slot
     if (sg[2] == 0)
         return;
@@ -704,7 +785,7 @@ sddmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint3
         }
     }
     sddmm_walk<T, LPR, VPL, UB, RG, WIDE, FZ>(a, acc, col, perm, sval, B, C, sg[1], sg[2], sub,
-                                              nvec, odd);
+                                              nvec, odd, pre.c);
     if constexpr (FZ != 0 && RG >= 2) {
         const bool whole = sg[3] == kWholeRow;
         char *drow = const_cast<char *>(whole ? odd_row<T, RG>(Y, sg[0], stride)
@@ -733,26 +814,41 @@ sddmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint3
 // ----------------------------------------------------------------- SpMM ----
 // MK: only the first n of the NB entries exist; the others repeat the loads of
 // entry n - 1 and add zero times zero.
-template <typename T, int LPR, int VPL, int NB, int RG, bool MK>
+// Column of entry j < kFirstCols of a short segment out of the indices loaded ahead:
+// lane u of the group holds that of entry u in pre[0] (groups of 4 lanes: of entries u
+// and 4 + u in pre[0] and pre[1]).
+template <int LPR> __device__ __forceinline__ uint32_t first_col(const uint32_t (&pre)[2], uint32_t j)
+{
+    if constexpr (LPR >= (int)kFirstCols)
+        return __shfl(pre[0], j, LPR);
+    else
+        return __shfl((j & LPR) ? pre[1] : pre[0], j & (LPR - 1), LPR);
+}
+
+// PRE: the batch is entries off .. off + NB - 1 of a short segment, off + NB <=
+// kFirstCols, and takes its column indices from `pre` (first_col).
+template <typename T, int LPR, int VPL, int NB, int RG, bool MK, bool PRE>
 __device__ __forceinline__ void
 spmm_batch_one(typename Vec<T>::type (&acc)[VPL], const uint32_t *__restrict__ col,
            const T *__restrict__ sval, const T *__restrict__ X, uint32_t p0, uint32_t n,
            uint32_t sub, uint32_t nvec,
-            const Odd<T, VPL, RG> &odd)
+            const Odd<T, VPL, RG> &odd, const uint32_t (&pre)[2], uint32_t off)
 {
     using V = typename Vec<T>::type;
     static_assert(NB <= LPR, "batch must fit the lane group");
     uint32_t e = sub & (NB - 1);
     if (MK)
         e = e < n ? e : n - 1;
-    const uint32_t cme = nt_load(col + p0 + e);
+    uint32_t cme = 0;
+    if constexpr (!PRE)
+        cme = nt_load(col + p0 + e);
     const T vme = nt_load(sval + p0 + e);
 
     V x[NB][VPL];
     T av[NB];
 #pragma unroll
     for (int u = 0; u < NB; ++u) {
-        const uint32_t c = __shfl(cme, u, LPR);
+        const uint32_t c = PRE ? first_col<LPR>(pre, off + u) : __shfl(cme, u, LPR);
         av[u] = __shfl(vme, u, LPR);
         gather_row<T, LPR, VPL, RG>(x[u], X, c, sub, nvec, odd);
     }
@@ -819,8 +915,10 @@ spmm_batch(typename Vec<T>::type (&acc)[VPL], const uint32_t *__restrict__ col,
            uint32_t sub, uint32_t nvec,
             const Odd<T, VPL, RG> &odd)
 {
+    const uint32_t none[2] = {0, 0};
     if constexpr (NB <= LPR)
-        spmm_batch_one<T, LPR, VPL, NB, RG, MK>(acc, col, sval, X, p0, n, sub, nvec, odd);
+        spmm_batch_one<T, LPR, VPL, NB, RG, MK, false>(acc, col, sval, X, p0, n, sub, nvec, odd,
+                                                       none, 0u);
     else
         spmm_batch_rounds<T, LPR, VPL, NB, RG, MK>(acc, col, sval, X, p0, n, sub, nvec, odd);
 }
@@ -830,13 +928,35 @@ __device__ __forceinline__ void
 spmm_walk(typename Vec<T>::type (&acc)[VPL], const uint32_t *__restrict__ col,
           const T *__restrict__ sval, const T *__restrict__ X, uint32_t p, uint32_t n,
           uint32_t sub, uint32_t nvec,
-            const Odd<T, VPL, RG> &odd)
+            const Odd<T, VPL, RG> &odd, const uint32_t (&pre)[2])
 {
     // Short segments: exact batches of UB, then UB/2 ... 1 as n requires.  Measured
     // against masked batches here (which cost registers, hence occupancy): 3 % faster
     // on 5-entry rows, level elsewhere.  SpMM's short rows are bound by the Y
-    // read-modify-write stream, not by rounds of gathers.
+    // read-modify-write stream, not by rounds of gathers.  The first kFirstCols
+    // entries take their column indices from `pre`, which was loaded ahead, beside the
+    // segment's descriptor.
     if constexpr (!WIDE) {
+        static_assert(WIDE || (UB <= 4 && UB <= LPR), "short batches fit the lane group");
+        {
+            const uint32_t m = n < kFirstCols ? n : kFirstCols;
+            uint32_t off = 0;
+            for (; off + UB <= m; off += UB)
+                spmm_batch_one<T, LPR, VPL, UB, RG, false, true>(acc, col, sval, X, p + off, UB,
+                                                                 sub, nvec, odd, pre, off);
+            if constexpr (UB > 2)
+                if ((m - off) & 2) {
+                    spmm_batch_one<T, LPR, VPL, 2, RG, false, true>(acc, col, sval, X, p + off, 2,
+                                                                    sub, nvec, odd, pre, off);
+                    off += 2;
+                }
+            if constexpr (UB > 1)
+                if ((m - off) & 1)
+                    spmm_batch_one<T, LPR, VPL, 1, RG, false, true>(acc, col, sval, X, p + off, 1,
+                                                                    sub, nvec, odd, pre, off);
+            n -= m;
+            p += m;
+        }
         for (; n >= UB; n -= UB, p += UB)
             spmm_batch<T, LPR, VPL, UB, RG, false>(acc, col, sval, X, p, UB, sub, nvec, odd);
         if constexpr (UB > 8)
@@ -883,7 +1003,7 @@ __global__ void __launch_bounds__(kBlock)
 spmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint32_t rot,
                 const uint32_t *__restrict__ col, const T *__restrict__ sval,
                 const T *__restrict__ X, T *__restrict__ Y, T *__restrict__ partial,
-                uint32_t nvec, uint32_t stride)
+                uint32_t nvec, uint32_t stride, const uint32_t *__restrict__ first_cols)
 {
     static_assert(UB <= 16 && LPR <= 64, "at most 16 entries in flight per lane");
     using V = typename Vec<T>::type;
@@ -891,6 +1011,7 @@ spmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint32
     const uint64_t sid = seg_index<64 / LPR>(nq, rot);
     if (sid >= nseg)
         return;
+    const FirstCols pre = load_first_cols<LPR, WIDE>(first_cols, sid, sub);
     const u32x4 sg = nt_load(reinterpret_cast<const u32x4 *>(segs) + sid); // row, start, len, slot
     if (sg[2] == 0)
         return;
@@ -911,7 +1032,7 @@ spmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint32
             for (int v = 0; v < VPL; ++v)
                 y0[v] = odd_load<T, RG, VPL, true>(drow, v, nvec, odd);
         }
-        spmm_walk<T, LPR, VPL, UB, RG, WIDE>(acc, col, sval, X, sg[1], sg[2], sub, nvec, odd);
+        spmm_walk<T, LPR, VPL, UB, RG, WIDE>(acc, col, sval, X, sg[1], sg[2], sub, nvec, odd, pre.c);
         odd_store<T, VPL>(drow, whole, y0, acc, odd);
     } else {
         V *dst = const_cast<V *>(whole ? row_ptr<T, LPR, VPL, RG>(Y, sg[0], sub, nvec)
@@ -922,7 +1043,7 @@ spmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint32
                 if (lane_on<LPR, RG>(sub, v, nvec))
                     y0[v] = nt_load(dst + v * LPR);
         }
-        spmm_walk<T, LPR, VPL, UB, RG, WIDE>(acc, col, sval, X, sg[1], sg[2], sub, nvec, odd);
+        spmm_walk<T, LPR, VPL, UB, RG, WIDE>(acc, col, sval, X, sg[1], sg[2], sub, nvec, odd, pre.c);
 #pragma unroll
         for (int v = 0; v < VPL; ++v) {
             if (!lane_on<LPR, RG>(sub, v, nvec))
@@ -1172,13 +1293,14 @@ hipError_t run_sddmm(const DevPlanView &P, const T *A, const T *B, T *C, T *Y, c
         hipLaunchKernelGGL((sddmm_seg_kernel<T, LPR, VPL, UB, RG, true, FZ>),
                            dim3(blocks_for_groups(nl, P.nqueues, 64 / LPR)), dim3(kBlock), 0,
                            S.main, P.segs, nl, P.nqueues, 0u, P.col, P.perm, (const T *)P.sval,
-                           A, B, C, Y, (T *)P.partial, nvec, stride ? stride : nvec, accum);
+                           A, B, C, Y, (T *)P.partial, nvec, stride ? stride : nvec, accum,
+                           (const uint32_t *)nullptr);
     if (ns)
         hipLaunchKernelGGL((sddmm_seg_kernel<T, LPR, VPL, US, RG, false, FZ>),
                            dim3(blocks_for_groups(ns, P.nqueues, 64 / LPR)), dim3(kBlock), 0,
                            both ? S.aux : S.main, P.segs + nl, ns, P.nqueues,
                            both ? S.aux_rot : 0u, P.col, P.perm, (const T *)P.sval, A, B, C, Y,
-                           (T *)P.partial, nvec, stride ? stride : nvec, accum);
+                           (T *)P.partial, nvec, stride ? stride : nvec, accum, P.first_cols);
     const hipError_t launched = hipGetLastError();
     const hipError_t joined = both ? join_aux(S) : hipSuccess;
     return launched != hipSuccess ? launched : joined;
@@ -1196,13 +1318,14 @@ hipError_t run_spmm(const DevPlanView &P, const T *X, T *Y, const Streams &S, ui
         hipLaunchKernelGGL((spmm_seg_kernel<T, LPR, VPL, UB, RG, true>),
                            dim3(blocks_for_groups(nl, P.nqueues, 64 / LPR)), dim3(kBlock), 0,
                            S.main, P.segs, nl, P.nqueues, 0u, P.col, (const T *)P.sval, X, Y,
-                           (T *)P.partial + slice_off, nvec, stride ? stride : nvec);
+                           (T *)P.partial + slice_off, nvec, stride ? stride : nvec,
+                           (const uint32_t *)nullptr);
     if (ns)
         hipLaunchKernelGGL((spmm_seg_kernel<T, LPR, VPL, US, RG, false>),
                            dim3(blocks_for_groups(ns, P.nqueues, 64 / LPR)), dim3(kBlock), 0,
                            both ? S.aux : S.main, P.segs + nl, ns, P.nqueues,
                            both ? S.aux_rot : 0u, P.col, (const T *)P.sval, X, Y,
-                           (T *)P.partial + slice_off, nvec, stride ? stride : nvec);
+                           (T *)P.partial + slice_off, nvec, stride ? stride : nvec, P.first_cols);
     const hipError_t launched = hipGetLastError();
     const hipError_t joined = both ? join_aux(S) : hipSuccess;
     return launched != hipSuccess ? launched : joined;
@@ -1414,6 +1537,17 @@ hipError_t launch_spmm(int dtype, const DevPlanView &P, const void *X, void *Y, 
 {
     return dtype == 1 ? spmm_typed<double>(P, X, Y, K, stream)
                       : spmm_typed<float>(P, X, Y, K, stream);
+}
+
+hipError_t launch_first_cols(const Seg *segs, uint32_t n, const uint32_t *col, uint32_t *first_cols,
+                             hipStream_t stream)
+{
+    if (n == 0)
+        return hipSuccess;
+    const uint64_t threads = (uint64_t)n * kFirstCols;
+    hipLaunchKernelGGL(first_cols_kernel, dim3((uint32_t)((threads + kBlock - 1) / kBlock)),
+                       dim3(kBlock), 0, stream, segs, n, col, first_cols);
+    return hipGetLastError();
 }
 
 hipError_t launch_gather_vals(int dtype, const void *in, const uint32_t *perm, void *out,

@@ -26,6 +26,7 @@ struct Seg {
 constexpr uint32_t kWholeRow = 0xFFFFFFFFu;
 constexpr uint32_t kChunk = 64; // segments per chunk; one chunk is dealt to one XCD
 constexpr uint32_t kLongSegment = 16; // segments this long fill the wide kernel's batches
+constexpr uint32_t kFirstCols = 8;    // column indices kept per short segment beside its descriptor
 
 // A row cut into several segments: its partial sums are slots
 // [first_slot, first_slot + nslots).
