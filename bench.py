@@ -19,7 +19,10 @@ point spc3d_sddmm_spmm (an extension without counterpart in the reference); it i
 reported beside `value`, which always comes from the two separate calls.
 `row_copies` times the pack and sum-unpack copies of a sparse exchange over the
 touched rows of Y (algorithmic bytes: rows read + buffer written; buffer read +
-rows read and written).
+rows read and written).  `also` holds the other real type, the same workload
+handed over in shuffled COO order (the reference never sorts its entries) in
+both types, and `configs`: one compact row per other benchmark configuration
+(time per kernel, strict-model fraction of the HBM peak).
 """
 from __future__ import annotations
 
@@ -37,18 +40,31 @@ if ROOT not in sys.path:
 
 METRIC = "SDDMM & SpMM GFLOP/s + % HBM roofline on 1 MI355X, RMAT-20 K=64"
 
-# HBM-side bytes per launch (L2 fills + write-backs) measured with rocprofv3
-# --pmc FETCH_SIZE / WRITE_SIZE, calibrated on a plain copy; they cannot be
-# collected from inside this process, so they are quoted from
-# profiles/sddmm_spmm_rmat20_k64_hbm_traffic.md for the workload they were taken
-# on (default plan options) and left null for any other: long-segment launch +
-# short-segment launch (+ fix-up for spmm).
-MEASURED_TRAFFIC = {
-    ("rmat20_ef16", 64, "sorted", "f64"): {"sddmm": 4595.1e6 + 1169.0e6,
-                                           "spmm": 4090.1e6 + 1326.9e6 + 123.1e6},
-    ("rmat20_ef16", 64, "sorted", "f32"): {"sddmm": 2278.5e6 + 675.5e6,
-                                           "spmm": 1840.4e6 + 723.7e6 + 61.8e6},
-}
+# Bytes that cross between the eight L2s and the fabric (Infinity Cache / HBM) per call,
+# measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and calibrated on a plain copy.
+# They cannot be collected from inside this process, so they are read from the profile
+# summary they were recorded in, for the workload and plan options it was taken on, and
+# are null for any other.
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "sddmm_spmm_rmat20_k64_hbm_traffic.md")
+TRAFFIC_LEVEL = "l2_fabric (FETCH_SIZE x 2 + WRITE_SIZE: fills and write-backs of the L2s; " \
+                "hits in the Infinity Cache are included, no HBM-side counter is exposed)"
+TRAFFIC_WORKLOAD = ("rmat20_ef16", 64, "sorted")
+
+
+def measured_traffic(path=TRAFFIC_PROFILE):
+    """{(dtype, call): bytes} from the 'Per call' table of the traffic profile."""
+    import re
+
+    out = {}
+    try:
+        text = open(path).read()
+    except OSError:
+        return out
+    row = re.compile(r"^\|\s*(f32|f64)\s*\|\s*(sddmm_spmm|sddmm|spmm)[^|]*\|\s*([\d,]+\.?\d*)\s*\|",
+                     re.M)
+    for dtype, call, mb in row.findall(text.split("Per call", 1)[-1]):
+        out[(dtype, call)] = float(mb.replace(",", "")) * 1e6
+    return out
 
 
 def log(*a):
@@ -157,7 +173,7 @@ def run_gpu(w, dtype, steps, warmup, seg_max=None, max_timed=1300, copies=0, ven
         vendor_out = None
         if vendor and w.order == "sorted":
             try:
-                from spcomm3d_amd import vendor_baseline
+                import vendor_baseline
 
                 vendor_out = vendor_baseline.time_rocsparse(ctx, w, dtype, dA, dB, dY)
             except Exception as e:  # a measurement aid: never fails the bench
@@ -198,6 +214,59 @@ def run_gpu(w, dtype, steps, warmup, seg_max=None, max_timed=1300, copies=0, ven
             "strict_frac": strict / avg / 1e6 / roofline.HBM_PEAK_GBS,
             "gather_frac": gather / avg / 1e6 / roofline.HBM_PEAK_GBS}
     return out
+
+
+def run_compact(w, dtype, steps, warmup):
+    """One compact row for a workload: mean time per kernel over `steps` passes on
+    resident operands, strict-model fraction of the HBM peak."""
+    from spcomm3d_amd import device, roofline
+    from spcomm3d_amd import workloads as W
+
+    wbytes = np.dtype(W.np_dtype(dtype)).itemsize
+    vv = w.values(dtype)
+    with device.Context(0) as ctx:
+        hint = {} if w.k == 64 else {"k_hint": w.k}
+        t0 = time.perf_counter()
+        S = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, vv, **hint)
+        ctx.sync()
+        plan_s = time.perf_counter() - t0
+        del vv
+        info = S.info
+        dA, dB = ctx.panel_from(w.panel_A(dtype)), ctx.panel_from(w.panel_B(dtype))
+        dY = ctx.panel_from(w.panel_Y0(dtype))
+        dC = ctx.vals(w.nnz, dtype)
+        for _ in range(warmup):
+            ctx.sddmm(S, dA, dB, dC)
+            ctx.spmm(S, dB, dY)
+        ctx.sync()
+        ctx.mark(0)
+        for _ in range(steps):
+            ctx.sddmm(S, dA, dB, dC)
+        ctx.mark(1)
+        for _ in range(steps):
+            ctx.spmm(S, dB, dY)
+        ctx.mark(2)
+        sd_ms = ctx.elapsed_ms(0, 1) / steps
+        sp_ms = ctx.elapsed_ms(1, 2) / steps
+        for h in (S, dA, dB, dY, dC):
+            h.close()
+    m_t, n_t = info.rows_touched, info.cols_touched
+    with_perm = not info.order_is_identity
+    fl = roofline.flops(w.nnz, w.k)
+    sd_b = roofline.sddmm_bytes(w.nrows, w.nnz, w.k, wbytes, m_t, n_t, with_perm)
+    sp_b = roofline.spmm_bytes(w.nrows, w.nnz, w.k, wbytes, m_t, n_t)
+    return {"workload": f"{w.name} K={w.k} ({w.order} COO)", "dtype": dtype, "nnz": w.nnz,
+            "nrows": w.nrows, "ncols": w.ncols, "k": w.k, "steps": steps,
+            "sddmm_ms": sd_ms, "spmm_ms": sp_ms,
+            "sddmm_frac": sd_b / sd_ms / 1e6 / roofline.HBM_PEAK_GBS,
+            "spmm_frac": sp_b / sp_ms / 1e6 / roofline.HBM_PEAK_GBS,
+            "gflops": 2 * fl / (sd_ms + sp_ms) / 1e6, "plan_build_s": plan_s}
+
+
+# The other benchmark configurations as (name, real type, timed passes): the reference's own
+# CPU-runnable case in its real type, the three larger ones in fp32 as they are specified.
+OTHER_CONFIGS = (("er16k", "f64", 50), ("rmat24_block", "f32", 10), ("stencil4096", "f32", 10),
+                 ("hypergraph", "f32", 3))
 
 
 def run_reference_baseline(w):
@@ -290,6 +359,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-vendor", action="store_true",
                     help="skip the rocSPARSE timings on the same operands")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="skip the shuffled-order runs and the rows of the other configurations")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path; run with --gpus 1")
@@ -313,6 +384,25 @@ def main():
         also[other] = run_gpu(w, other, args.steps, args.warmup, args.seg_max,
                               vendor=not args.no_vendor)
         log(json.dumps(also[other]))
+    if not (args.only or args.no_configs):
+        ws = w.shuffled() if w.order == "sorted" else None
+        if ws is not None:
+            also["shuffled"] = {dt: run_compact(ws, dt, max(5, args.steps // 2), args.warmup)
+                                for dt in ("f64", "f32")}
+            log(json.dumps(also["shuffled"]))
+            del ws
+        rows = []
+        for name, dt, steps in OTHER_CONFIGS:
+            if name == args.config:
+                continue
+            t0 = time.perf_counter()
+            wo = W.make(name)
+            row = run_compact(wo, dt, steps, 2)
+            row["wall_s"] = time.perf_counter() - t0
+            del wo
+            rows.append(row)
+            log(json.dumps(row))
+        also["configs"] = rows
     cpu = None
     if not args.no_cpu:
         port = run_cpu_baseline(w, args.dtype)
@@ -324,8 +414,9 @@ def main():
     from spcomm3d_amd import roofline
 
     traffic = None
-    if args.seg_max is None and not any(k.startswith("SPC3D_") for k in os.environ):
-        traffic = MEASURED_TRAFFIC.get((w.name, w.k, w.order, args.dtype), {}).get(dom)
+    if (args.seg_max is None and not any(k.startswith("SPC3D_") for k in os.environ)
+            and (w.name, w.k, w.order) == TRAFFIC_WORKLOAD):
+        traffic = measured_traffic().get((args.dtype, dom))
 
     line = {
         "metric": METRIC, "value": main_r["gflops"], "unit": "GFLOP/s", "n_gpus": 1,
@@ -337,7 +428,8 @@ def main():
                    "rows_touched": main_r["rows_touched"], "cols_touched": main_r["cols_touched"]},
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": kd["strict_gbs"],
                      "peak": roofline.HBM_PEAK_GBS, "unit": "GB/s", "frac": kd["strict_frac"],
-                     "traffic": traffic,
+                     "traffic": traffic, "traffic_level": TRAFFIC_LEVEL,
+                     "traffic_source": os.path.relpath(TRAFFIC_PROFILE, ROOT),
                      "traffic_gbs": None if traffic is None else traffic / kd["ms_avg"] / 1e6,
                      "bytes_per_launch": kd["strict_bytes"],
                      "ms_per_launch": kd["ms_avg"], "model": "strict (each operand once)"},

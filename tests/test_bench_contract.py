@@ -39,10 +39,48 @@ def test_byte_models_of_the_roofline():
     assert roofline.flops(nnz, 64) == 2 * nnz * 64
 
 
+def test_traffic_in_the_bench_line_is_what_the_profile_summary_holds():
+    """bench.py quotes the measured L2 <-> fabric traffic from the committed profile
+    summary: the 'Per call' table must parse, add up from the per-launch table of the same
+    file, and lie between the strict and the gather model."""
+    import re
+
+    sys.path.insert(0, ROOT)
+    import bench
+    from spcomm3d_amd import roofline
+
+    got = bench.measured_traffic()
+    assert set(got) == {(d, c) for d in ("f32", "f64") for c in ("sddmm", "spmm", "sddmm_spmm")}
+    text = open(bench.TRAFFIC_PROFILE).read()
+    per_launch = text.split("Per call", 1)[0]
+    rows = re.findall(r"^\|\s*(f32|f64)\s*\|\s*`(\w+)<([^`]*)>`\s*\|[^|]*\|[^|]*\|[^|]*\|[^|]*\|"
+                      r"\s*([\d,\.]+)\s*\|", per_launch, re.M)
+    assert len(rows) >= 14
+    total = {}
+    for dtype, kernel, targs, mb in rows:
+        mb = float(mb.replace(",", ""))
+        fused = kernel.startswith("sddmm") and targs.strip().endswith("1")
+        call = "sddmm_spmm" if fused else ("sddmm" if kernel.startswith("sddmm") else "spmm")
+        total[(dtype, call)] = total.get((dtype, call), 0.0) + mb * 1e6
+        if kernel == "spmm_fixup_kernel":  # the one-pass call ends with the same fix-up
+            total[(dtype, "sddmm_spmm")] = total.get((dtype, "sddmm_spmm"), 0.0) + mb * 1e6
+    nnz, m, mt, nt = 16086740, 1048576, 547169, 547037
+    for (dtype, call), traffic in got.items():
+        assert abs(total[(dtype, call)] - traffic) <= 0.002 * traffic, (dtype, call)
+        w = 8 if dtype == "f64" else 4
+        strict = {"sddmm": roofline.sddmm_bytes(m, nnz, 64, w, mt, nt, True),
+                  "spmm": roofline.spmm_bytes(m, nnz, 64, w, mt, nt),
+                  "sddmm_spmm": roofline.fused_bytes(m, nnz, 64, w, mt, nt, True)}[call]
+        gather = roofline.fused_bytes(m, nnz, 64, w, mt, nt, True, gather=True)
+        assert strict < traffic < gather, (dtype, call)
+    assert "l2_fabric" in bench.TRAFFIC_LEVEL
+
+
 @pytest.mark.gpu
 def test_bench_line_has_the_contract_fields():
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--config", "er16k",
-                        "--steps", "5", "--warmup", "1"], capture_output=True, text=True,
+                        "--steps", "5", "--warmup", "1", "--no-configs"], capture_output=True,
+                       text=True,
                        timeout=600)
     assert r.returncode == 0, r.stderr[-2000:]
     lines = [ln for ln in r.stdout.splitlines() if ln.strip()]
@@ -54,7 +92,8 @@ def test_bench_line_has_the_contract_fields():
         assert k in d, k
     assert d["n_gpus"] == 1 and d["steps"] == 5 and d["vs_baseline"] is None
     assert d["dtype"] == "f64" and "workload" in d["config"]
-    assert set(("bound", "achieved", "peak", "unit", "frac", "traffic")) <= set(d["roofline"])
+    assert set(("bound", "achieved", "peak", "unit", "frac", "traffic", "traffic_level")) <= \
+        set(d["roofline"])
     assert d["roofline"]["bound"] == "hbm" and d["roofline"]["peak"] == 8000.0
     assert abs(d["roofline"]["frac"] - d["roofline"]["achieved"] / 8000.0) < 1e-12
     assert set(("value", "unit", "cores", "kind", "sample")) <= set(d["cpu_baseline"])

@@ -39,7 +39,7 @@ def time_rocsparse(ctx, w, dtype, dA, dB, dY, reps=10):
     """Times rocSPARSE on workload `w` with this context's resident panels dA (m x K),
     dB (n x K) and dY (m x K); w must be sorted by row.  Returns a dict of
     microseconds per call.  dY is overwritten."""
-    from . import device
+    from spcomm3d_amd import device
 
     rs, hip = _load()
     p = ctypes.c_void_p
