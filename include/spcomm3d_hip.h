@@ -89,7 +89,9 @@ typedef struct {
     uint64_t hot_entries;      /* XCD slicing: entries in those columns */
     uint32_t nsegments_long;   /* leading stored segments (all of >= 16 entries) that run in the
                                   wide-batch launch; the rest run in the high-occupancy one */
-    uint32_t reserved;
+    uint32_t ncol_blocks;      /* 1, or the number of column blocks the plan is kept in: the
+                                  segment counts above are then sums over the blocks,
+                                  npartial_slots the largest block's */
 } spc3d_plan_info;
 
 /* Plan tuning; a zero field selects the default.  Only speed depends on these. */
@@ -109,7 +111,15 @@ typedef struct {
     uint32_t builder;      /* where spc3d_plan_create[_ex] builds the plan: 0 (default) or 2:
                               on the GPU; 1: on the host, then uploaded.  Both give the same
                               arrays bit for bit. */
-    uint32_t reserved[2];  /* must be 0 */
+    uint32_t col_blocks;   /* 0 (default): the pattern is kept in blocks of columns, run one
+                              after the other so that one block of dense rows (about 5 MiB)
+                              is what the L2s see at a time, when its columns are not skewed,
+                              the dense rows it gathers exceed 64 MiB at k_hint columns and
+                              its rows are long enough (entry-weighted mean length at least
+                              16 times the block count); 1: never; n > 1: in n blocks (at
+                              most 4096).  Built on the GPU only; results are those of the
+                              whole plan up to summation order (SpMM adds block after block) */
+    uint32_t reserved[1];  /* must be 0 */
 } spc3d_plan_opts;
 
 /* ---- library / errors ------------------------------------------------- */

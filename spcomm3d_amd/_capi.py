@@ -30,13 +30,13 @@ class PlanInfo(ctypes.Structure):
                 ("max_row_nnz", c_u32), ("seg_max", c_u32),
                 ("order_is_identity", ctypes.c_int32), ("nqueues", c_u32),
                 ("hot_cols", c_u32), ("hub_rows", c_u32), ("hot_entries", c_u64),
-                ("nsegments_long", c_u32), ("reserved", c_u32)]
+                ("nsegments_long", c_u32), ("ncol_blocks", c_u32)]
 
 
 class PlanOpts(ctypes.Structure):
     _fields_ = [("seg_max", c_u32), ("k_hint", c_u32), ("l2_hot_bytes", c_u32),
                 ("hub_min", c_u32), ("xcd_slices", c_u32), ("builder", c_u32),
-                ("reserved", c_u32 * 2)]
+                ("col_blocks", c_u32), ("reserved", c_u32 * 1)]
 
 
 # name -> (restype, argtypes); one entry for every function the header declares.

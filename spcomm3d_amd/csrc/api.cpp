@@ -54,6 +54,7 @@ constexpr uint32_t kMagicPlan = 0x5343334c;
 constexpr uint32_t kMagicRowMap = 0x5343334d;
 constexpr uint32_t kMagicGraph = 0x53433347;
 constexpr int kTimerSlots = 4096;
+constexpr uint32_t kMaxColBlocks = 4096;
 
 inline size_t elem_size(int dtype) { return dtype == SPC3D_F64 ? 8 : 4; }
 inline bool dtype_ok(int dtype) { return dtype == SPC3D_F32 || dtype == SPC3D_F64; }
@@ -158,6 +159,26 @@ struct spc3d_plan {
     // until the plan is destroyed: a sequence recorded earlier (spc3d_capture_*) keeps
     // the block's address in its kernel arguments and goes on using it.
     std::vector<void *> retired_partial;
+    // A pattern kept in column blocks: one complete plan per block of columns, each over
+    // the entries of its block with `perm` giving the caller's positions; this plan then
+    // holds no arrays of its own, only `info` for the whole pattern.  The calls run the
+    // blocks one after the other, so that one block of dense rows is what the L2s see at
+    // a time.
+    std::vector<spc3d_plan *> blocks;
+    // SDDMM over blocks.  Stored straight at the caller's positions, the results of one
+    // block are short runs between those of the other blocks, written at different times
+    // (36 against 24 ms for the kernels on the 572 M-entry pattern the blocks are meant
+    // for).  So the blocks write into a staging vector, and one pass brings the results
+    // to the caller's positions, C[e] = c_stage[stage_pos[e]].  The staging order is by
+    // tile of rows (about 2 MiB of results), inside a tile by block, inside a block the
+    // block's kernel order: a block's stores are long runs, and the final pass reads one
+    // tile's worth of staged results (L2-sized) while it writes that tile's C in order.
+    // stage_of[g] = staging position of entry g of the blocks' concatenated kernel
+    // orders; block b's part starts at stage_off.
+    void *c_stage = nullptr;       // [nnz] reals
+    uint32_t *stage_pos = nullptr; // [nnz] caller's position -> staging position
+    uint32_t *stage_of = nullptr;  // [nnz]
+    uint64_t stage_off = 0;
 };
 
 namespace {
@@ -892,7 +913,7 @@ static void fill_info(spc3d_plan_info &info, const HostPlan &H)
     info.hub_rows = H.hub_rows;
     info.hot_entries = H.hot_entries;
     info.nsegments_long = H.nseg_long;
-    info.reserved = 0;
+    info.ncol_blocks = 1;
 }
 
 // Library defaults, overridable field by field.  With XCD slicing, 2 MiB of
@@ -903,8 +924,13 @@ static int resolve_opts(int dtype, const spc3d_plan_opts *o, PlanOpts &out)
     std::memset(&z, 0, sizeof z);
     if (o)
         z = *o;
-    if (z.reserved[0] || z.reserved[1])
+    if (z.reserved[0])
         return fail(SPC3D_ERR_INVALID_ARG, "spc3d_plan_opts.reserved must be 0");
+    if (z.col_blocks > kMaxColBlocks)
+        return fail(SPC3D_ERR_INVALID_ARG, "spc3d_plan_opts.col_blocks must be at most 4096");
+    if (z.col_blocks > 1 && z.builder == 1)
+        return fail(SPC3D_ERR_INVALID_ARG,
+                    "column blocks are built on the GPU: builder must be 0 or 2 with col_blocks > 1");
     if (z.builder > 2)
         return fail(SPC3D_ERR_INVALID_ARG, "spc3d_plan_opts.builder must be 0, 1 or 2");
     if (z.xcd_slices != 0 && z.xcd_slices != 1 && z.xcd_slices != 8)
@@ -1014,6 +1040,203 @@ static int adopt_device_plan(spc3d_ctx *ctx, int dtype, const HostPlan &meta, De
     return SPC3D_OK;
 }
 
+static void destroy_blocks(spc3d_plan *p)
+{
+    for (spc3d_plan *b : p->blocks) {
+        plan_free_device(b);
+        b->magic = 0;
+        delete b;
+    }
+    p->blocks.clear();
+    if (p->c_stage) (void)hipFree(p->c_stage);
+    if (p->stage_pos) (void)hipFree(p->stage_pos);
+    if (p->stage_of) (void)hipFree(p->stage_of);
+    p->c_stage = nullptr;
+    p->stage_pos = p->stage_of = nullptr;
+}
+
+// How many column blocks a finished single plan should be rebuilt in (1: keep it).
+// Blocks pay when the dense rows the pattern gathers do not fit the L2s, the columns
+// are not skewed (then a few hot rows carry the reuse, and the plan deals them to the
+// XCDs instead), and the rows are long enough that a row's piece in one block still
+// amortises reading its A row / updating its Y row: the entry-weighted mean segment
+// length divided by the block count must stay at 16 or more.  Measured on a 2 M x 500 k
+// pattern with 286 entries per row on average (capped Zipf, weighted mean 890) at 512-byte
+// dense rows: 43 -> 24 ms SDDMM, 42 -> 27 ms SpMM in 48 blocks of 5 MiB; a uniform
+// pattern of 256 entries per row gains 10 % in SDDMM and loses in SpMM, and stays whole.
+static int choose_col_blocks(spc3d_plan *p, const spc3d_plan_opts *opts, uint32_t *nblocks)
+{
+    *nblocks = 1;
+    const uint32_t want = opts ? opts->col_blocks : 0;
+    const spc3d_plan_info &I = p->info;
+    if (want == 1 || I.nnz == 0 || I.ncols < 2)
+        return SPC3D_OK;
+    if (want > 1) {
+        *nblocks = std::min<uint32_t>(want, I.ncols);
+        return SPC3D_OK;
+    }
+    if (I.nqueues != 1)
+        return SPC3D_OK;
+    const uint64_t row_bytes = (uint64_t)planned_k(opts) * elem_size(p->dtype);
+    const uint64_t panel = (uint64_t)I.cols_touched * row_bytes;
+    constexpr uint64_t kBlockBytes = (uint64_t)21 << 18; // 5.25 MiB of dense rows per block
+    if (panel < ((uint64_t)64 << 20))
+        return SPC3D_OK;
+    const uint64_t nb = std::min<uint64_t>((panel + kBlockBytes - 1) / kBlockBytes, 256);
+    uint64_t sumsq = 0;
+    std::string err;
+    int rc = sum_sq_seg_len_device(p->ctx->stream, p->segs, I.nsegments_padded, &sumsq, err);
+    if (rc != SPC3D_OK)
+        return fail(rc, err);
+    const double wmean = (double)sumsq / (double)I.nnz;
+    if (wmean / (double)nb >= 16.0)
+        *nblocks = (uint32_t)nb;
+    return SPC3D_OK;
+}
+
+// Plan of a pattern that lies on the device: the single plan first (validation, the
+// whole pattern's figures), then, where choose_col_blocks says so, one plan per block
+// of columns in its place.
+static int build_from_device(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t ncols,
+                             uint64_t nnz, const uint32_t *d_ii, const uint32_t *d_jj,
+                             const PlanOpts &po, const spc3d_plan_opts *opts, spc3d_plan **out)
+{
+    HostPlan meta;
+    DevPlanArrays arr;
+    std::string err;
+    int rc = build_device_plan(ctx->stream, nrows, ncols, nnz, d_ii, d_jj, po, meta, arr, err);
+    if (rc != SPC3D_OK)
+        return fail(rc, err);
+    spc3d_plan *p = nullptr;
+    rc = adopt_device_plan(ctx, dtype, meta, arr, planned_k(opts), &p);
+    if (rc)
+        return rc;
+    uint32_t nb = 1;
+    rc = choose_col_blocks(p, opts, &nb);
+    if (rc || nb <= 1) {
+        if (rc)
+            spc3d_plan_destroy(p);
+        else
+            *out = p;
+        return rc;
+    }
+    // ---- in column blocks ----
+    uint32_t *b_ii = nullptr, *b_jj = nullptr, *order = nullptr;
+    std::vector<uint32_t> first;
+    try {
+        first.resize((size_t)nb + 1);
+        p->blocks.reserve(nb);
+    } catch (const std::bad_alloc &) {
+        spc3d_plan_destroy(p);
+        return fail(SPC3D_ERR_ALLOC, "host allocation failed");
+    }
+    rc = dev_alloc(&b_ii, (size_t)nnz);
+    if (!rc) rc = dev_alloc(&b_jj, (size_t)nnz);
+    if (!rc) rc = dev_alloc(&order, (size_t)nnz);
+    if (!rc) {
+        rc = partition_by_col_block(ctx->stream, nnz, d_ii, d_jj, ncols, nb, b_ii, b_jj, order,
+                                    first.data(), err);
+        if (rc)
+            fail(rc, err);
+    }
+    // rows per tile of the staging order: about 2 MiB of results
+    const uint64_t per_row = std::max<uint64_t>(1, nnz / std::max<uint32_t>(1, p->info.rows_touched));
+    const uint32_t rows_per_tile = (uint32_t)std::max<uint64_t>(
+        1, ((uint64_t)2 << 20) / (per_row * elem_size(dtype)));
+    uint32_t *tile_key = nullptr;
+    if (!rc) rc = dev_alloc(&tile_key, (size_t)nnz);
+    spc3d_plan_info total = p->info;
+    total.nsegments = total.nsegments_padded = total.nsplit_rows = total.npartial_slots = 0;
+    total.nsegments_long = 0;
+    total.order_is_identity = 0;
+    for (uint32_t b = 0; !rc && b < nb; ++b) {
+        const uint64_t cnt = (uint64_t)first[b + 1] - first[b];
+        if (cnt == 0)
+            continue;
+        HostPlan bmeta;
+        DevPlanArrays barr;
+        rc = build_device_plan(ctx->stream, nrows, ncols, cnt, b_ii + first[b], b_jj + first[b], po,
+                               bmeta, barr, err);
+        if (rc) {
+            fail(rc, err);
+            break;
+        }
+        spc3d_plan *child = nullptr;
+        rc = adopt_device_plan(ctx, dtype, bmeta, barr, planned_k(opts), &child);
+        if (rc)
+            break;
+        p->blocks.push_back(child);
+        rc = tile_keys_device(ctx->stream, b_ii + first[b], child->perm, cnt, rows_per_tile,
+                              tile_key + first[b], err);
+        if (rc) {
+            fail(rc, err);
+            break;
+        }
+        uint32_t *gperm = nullptr;
+        rc = dev_alloc(&gperm, (size_t)cnt);
+        if (!rc) {
+            rc = compose_perm_device(ctx->stream, order + first[b], child->perm, cnt, gperm, err);
+            if (rc)
+                fail(rc, err);
+        }
+        if (rc) {
+            if (gperm) (void)hipFree(gperm);
+            break;
+        }
+        hipError_t e = hipStreamSynchronize(ctx->stream); // child->perm is read until here
+        if (e != hipSuccess) {
+            (void)hipFree(gperm);
+            rc = fail_hip(e, "hipStreamSynchronize");
+            break;
+        }
+        if (child->perm) (void)hipFree(child->perm);
+        child->perm = gperm;
+        child->stage_off = first[b];
+        child->info.order_is_identity = 0;
+        total.nsegments += child->info.nsegments;
+        total.nsegments_padded += child->info.nsegments_padded;
+        total.nsegments_long += child->info.nsegments_long;
+        total.nsplit_rows += child->info.nsplit_rows;
+        total.npartial_slots = std::max(total.npartial_slots, child->info.npartial_slots);
+        total.nqueues = std::max(total.nqueues, child->info.nqueues);
+    }
+    if (!rc) rc = dev_alloc_bytes(&p->c_stage, (size_t)nnz * elem_size(dtype));
+    if (!rc) rc = dev_alloc(&p->stage_pos, (size_t)nnz);
+    if (!rc) rc = dev_alloc(&p->stage_of, (size_t)nnz);
+    if (!rc) {
+        rc = stable_ranks_device(ctx->stream, tile_key, nnz, (nrows - 1) / rows_per_tile,
+                                 p->stage_of, err);
+        if (rc)
+            fail(rc, err);
+    }
+    for (spc3d_plan *child : p->blocks) {
+        if (rc)
+            break;
+        // stage_pos[caller's position of entry q] = its staging position
+        rc = scatter_device(ctx->stream, child->perm, p->stage_of + child->stage_off,
+                            child->info.nnz, p->stage_pos, err);
+        if (rc)
+            fail(rc, err);
+    }
+    if (tile_key) (void)hipFree(tile_key);
+    if (b_ii) (void)hipFree(b_ii);
+    if (b_jj) (void)hipFree(b_jj);
+    if (order) (void)hipFree(order);
+    if (rc) {
+        std::string keep = g_err;
+        spc3d_plan_destroy(p);
+        return fail(rc, keep);
+    }
+    // the whole pattern's arrays give way to the blocks'
+    (void)hipStreamSynchronize(ctx->stream);
+    plan_free_device(p);
+    p->partial_k = 0;
+    p->info = total;
+    p->info.ncol_blocks = (uint32_t)p->blocks.size();
+    *out = p;
+    return SPC3D_OK;
+}
+
 int spc3d_plan_create_from_device(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t ncols,
                                   uint64_t nnz, const void *dev_ii, const void *dev_jj,
                                   const spc3d_plan_opts *opts, spc3d_plan **out)
@@ -1032,14 +1255,8 @@ int spc3d_plan_create_from_device(spc3d_ctx *ctx, int dtype, uint32_t nrows, uin
     rc = use_device(ctx);
     if (rc)
         return rc;
-    HostPlan meta;
-    DevPlanArrays arr;
-    std::string err;
-    rc = build_device_plan(ctx->stream, nrows, ncols, nnz, (const uint32_t *)dev_ii,
-                           (const uint32_t *)dev_jj, po, meta, arr, err);
-    if (rc != SPC3D_OK)
-        return fail(rc, err);
-    return adopt_device_plan(ctx, dtype, meta, arr, planned_k(opts), out);
+    return build_from_device(ctx, dtype, nrows, ncols, nnz, (const uint32_t *)dev_ii,
+                             (const uint32_t *)dev_jj, po, opts, out);
 }
 
 int spc3d_plan_create_ex(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t ncols, uint64_t nnz,
@@ -1071,19 +1288,10 @@ int spc3d_plan_create_ex(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t nco
         if (!rc) rc = dev_alloc(&d_jj, (size_t)nnz);
         if (!rc) rc = copy_h2d(ctx, d_ii, ii, (size_t)nnz * sizeof(uint32_t));
         if (!rc) rc = copy_h2d(ctx, d_jj, jj, (size_t)nnz * sizeof(uint32_t));
-        HostPlan meta;
-        DevPlanArrays arr;
-        if (!rc) {
-            std::string err;
-            rc = build_device_plan(ctx->stream, nrows, ncols, nnz, d_ii, d_jj, po, meta, arr, err);
-            if (rc != SPC3D_OK)
-                fail(rc, err);
-        }
+        if (!rc)
+            rc = build_from_device(ctx, dtype, nrows, ncols, nnz, d_ii, d_jj, po, opts, &p);
         if (d_ii) (void)hipFree(d_ii);
         if (d_jj) (void)hipFree(d_jj);
-        if (rc)
-            return rc;
-        rc = adopt_device_plan(ctx, dtype, meta, arr, planned_k(opts), &p);
         if (rc)
             return rc;
     } else {
@@ -1177,6 +1385,10 @@ int spc3d_plan_download(spc3d_plan *plan, uint32_t *col, uint32_t *perm, uint32_
     if (!live(plan))
         return fail(SPC3D_ERR_INVALID_ARG, "plan is NULL or destroyed");
     const spc3d_plan_info &I = plan->info;
+    if (!plan->blocks.empty())
+        return fail(SPC3D_ERR_INVALID_ARG,
+                    "the plan is kept in column blocks (spc3d_plan_info.ncol_blocks > 1): there "
+                    "is one set of arrays per block, not one for the pattern");
     if ((segs && seg_cap < I.nsegments_padded) || (splits && split_cap < I.nsplit_rows))
         return fail(SPC3D_ERR_SIZE_MISMATCH, "output capacity is smaller than the plan");
     int rc = use_device(plan->ctx);
@@ -1223,7 +1435,8 @@ static spc3d_plan_opts opts_from_env()
                {"SPC3D_K_HINT", &o.k_hint},
                {"SPC3D_L2_HOT_BYTES", &o.l2_hot_bytes},
                {"SPC3D_HUB_MIN", &o.hub_min},
-               {"SPC3D_XCD_SLICES", &o.xcd_slices}};
+               {"SPC3D_XCD_SLICES", &o.xcd_slices},
+               {"SPC3D_COL_BLOCKS", &o.col_blocks}};
     for (auto &e : env)
         if (const char *s = std::getenv(e.name)) {
             const long long v = std::atoll(s);
@@ -1250,10 +1463,43 @@ int spc3d_plan_destroy(spc3d_plan *plan)
         return rc;
     (void)hipSetDevice(plan->ctx->device);
     (void)hipStreamSynchronize(plan->ctx->stream);
+    destroy_blocks(plan);
     plan_free_device(plan);
     plan->magic = 0;
     delete plan;
     return SPC3D_OK;
+}
+
+// The parts a call works on: the plan itself, or its column blocks.
+static std::vector<spc3d_plan *> &parts_of(spc3d_plan *plan, std::vector<spc3d_plan *> &self)
+{
+    if (!plan->blocks.empty())
+        return plan->blocks;
+    self.assign(1, plan);
+    return self;
+}
+
+// A block's view for SDDMM: results at their places in the parent's staging vector.
+static DevPlanView staged_view(const spc3d_plan *parent, const spc3d_plan *block)
+{
+    DevPlanView v = view_of(block);
+    v.perm = parent->stage_of + block->stage_off;
+    v.stream_c = true;
+    return v;
+}
+// C[e] = c_stage[stage_pos[e]]; a caller's C that is not 16-byte aligned (a wrapped
+// vector) goes the element-wise way.
+static hipError_t unstage(const spc3d_plan *S, spc3d_vals *C)
+{
+    if (((uintptr_t)C->dev & 15u) == 0)
+        return launch_unstage(S->dtype, S->c_stage, S->stage_pos, C->dev, S->info.nnz,
+                              S->ctx->stream);
+    return launch_gather_vals(S->dtype, S->c_stage, S->stage_pos, C->dev, S->info.nnz,
+                              S->ctx->stream);
+}
+static void *staged_out(const spc3d_plan *parent, const spc3d_plan *)
+{
+    return parent->c_stage;
 }
 
 int spc3d_plan_set_values(spc3d_plan *plan, const void *vv_host)
@@ -1267,7 +1513,7 @@ int spc3d_plan_set_values(spc3d_plan *plan, const void *vv_host)
     if (rc)
         return rc;
     const size_t bytes = (size_t)nnz * elem_size(plan->dtype);
-    if (!plan->perm) {
+    if (plan->blocks.empty() && !plan->perm) {
         rc = copy_h2d(plan->ctx, plan->sval, vv_host, bytes);
     } else {
         void *tmp = nullptr;
@@ -1275,11 +1521,17 @@ int spc3d_plan_set_values(spc3d_plan *plan, const void *vv_host)
         if (rc)
             return rc;
         rc = copy_h2d(plan->ctx, tmp, vv_host, bytes);
+        std::vector<spc3d_plan *> self;
+        for (spc3d_plan *part : parts_of(plan, self)) {
+            if (rc)
+                break;
+            hipError_t e = launch_gather_vals(plan->dtype, tmp, part->perm, part->sval,
+                                              part->info.nnz, plan->ctx->stream);
+            if (e != hipSuccess)
+                rc = fail_hip(e, "gather of sparse values");
+        }
         if (!rc) {
-            hipError_t e = launch_gather_vals(plan->dtype, tmp, plan->perm, plan->sval, nnz,
-                                              plan->ctx->stream);
-            if (e == hipSuccess)
-                e = hipStreamSynchronize(plan->ctx->stream);
+            hipError_t e = hipStreamSynchronize(plan->ctx->stream);
             if (e != hipSuccess)
                 rc = fail_hip(e, "gather of sparse values");
         }
@@ -1300,8 +1552,10 @@ int spc3d_plan_set_values_device(spc3d_plan *plan, const spc3d_vals *vv)
     int rc = use_device(plan->ctx, true);
     if (rc)
         return rc;
-    HIP_TRY(launch_gather_vals(plan->dtype, vv->dev, plan->perm, plan->sval, plan->info.nnz,
-                               plan->ctx->stream));
+    std::vector<spc3d_plan *> self;
+    for (spc3d_plan *part : parts_of(plan, self))
+        HIP_TRY(launch_gather_vals(plan->dtype, vv->dev, part->perm, part->sval, part->info.nnz,
+                                   plan->ctx->stream));
     plan->has_values = true;
     return SPC3D_OK;
 }
@@ -1384,7 +1638,14 @@ int spc3d_sddmm(spc3d_ctx *ctx, spc3d_plan *S, const spc3d_panel *A, const spc3d
     int rc = use_device(ctx, true);
     if (rc)
         return rc;
-    HIP_TRY(launch_sddmm(S->dtype, view_of(S), A->dev, B->dev, C->dev, K, streams_of(ctx)));
+    if (S->blocks.empty()) {
+        HIP_TRY(launch_sddmm(S->dtype, view_of(S), A->dev, B->dev, C->dev, K, streams_of(ctx)));
+        return SPC3D_OK;
+    }
+    for (spc3d_plan *part : S->blocks)
+        HIP_TRY(launch_sddmm(S->dtype, staged_view(S, part), A->dev, B->dev, staged_out(S, part), K,
+                             streams_of(ctx)));
+    HIP_TRY(unstage(S, C));
     return SPC3D_OK;
 }
 
@@ -1423,10 +1684,15 @@ int spc3d_spmm(spc3d_ctx *ctx, spc3d_plan *Ap, const spc3d_panel *X, spc3d_panel
     rc = use_device(ctx, true);
     if (rc)
         return rc;
-    rc = ensure_partial(Ap, K);
-    if (rc)
-        return rc;
-    HIP_TRY(launch_spmm(Ap->dtype, view_of(Ap), X->dev, Y->dev, K, streams_of(ctx)));
+    std::vector<spc3d_plan *> self;
+    for (spc3d_plan *part : parts_of(Ap, self)) {
+        rc = ensure_partial(part, K);
+        if (rc)
+            return rc;
+    }
+    // The blocks add into Y one after the other on the stream: a fixed order.
+    for (spc3d_plan *part : parts_of(Ap, self))
+        HIP_TRY(launch_spmm(Ap->dtype, view_of(part), X->dev, Y->dev, K, streams_of(ctx)));
     return SPC3D_OK;
 }
 
@@ -1449,10 +1715,15 @@ int spc3d_spmm_noalloc(spc3d_ctx *ctx, spc3d_plan *Ap, const spc3d_panel *X, spc
     if (rc)
         return rc;
     // Every partial-sum row the fix-up reads is written by exactly one segment of this
-    // call first, so what an earlier call left in the array needs no clearing.
-    DevPlanView view = view_of(Ap);
-    view.partial = ctx->scratch;
-    HIP_TRY(launch_spmm(Ap->dtype, view, X->dev, Y->dev, K, streams_of(ctx)));
+    // call first, so what an earlier call left in the array needs no clearing.  (The
+    // blocks of a plan kept in column blocks use the array one after the other;
+    // npartial_slots is the largest block's.)
+    std::vector<spc3d_plan *> self;
+    for (spc3d_plan *part : parts_of(Ap, self)) {
+        DevPlanView view = view_of(part);
+        view.partial = ctx->scratch;
+        HIP_TRY(launch_spmm(Ap->dtype, view, X->dev, Y->dev, K, streams_of(ctx)));
+    }
     return SPC3D_OK;
 }
 
@@ -1487,23 +1758,33 @@ int spc3d_sddmm_spmm(spc3d_ctx *ctx, spc3d_plan *S, const spc3d_panel *A, const 
         HIP_TRY(launch_fill(C->dtype, C->dev, S->info.nnz, 0.0, ctx->stream));
         return SPC3D_OK;
     }
-    rc = ensure_partial(S, K);
-    if (rc)
-        return rc;
-    hipError_t e = launch_sddmm_spmm(S->dtype, chained != 0, view_of(S), A->dev, B->dev, C->dev,
-                                     Y->dev, K, streams_of(ctx));
-    if (e == hipErrorNotSupported) {
-        (void)hipGetLastError();
-        if (chained)
-            return fail(SPC3D_ERR_INVALID_ARG,
-                        "the chained form needs dense rows of at most 4096 bytes "
-                        "(K * sizeof(real))");
-        // No vector kernel for this K: the two calls one after the other.
-        HIP_TRY(launch_sddmm(S->dtype, view_of(S), A->dev, B->dev, C->dev, K, streams_of(ctx)));
-        HIP_TRY(launch_spmm(S->dtype, view_of(S), B->dev, Y->dev, K, streams_of(ctx)));
-        return SPC3D_OK;
+    std::vector<spc3d_plan *> self;
+    for (spc3d_plan *part : parts_of(S, self)) {
+        rc = ensure_partial(part, K);
+        if (rc)
+            return rc;
     }
-    HIP_TRY(e);
+    const bool staged = !S->blocks.empty();
+    for (spc3d_plan *part : parts_of(S, self)) {
+        const DevPlanView view = staged ? staged_view(S, part) : view_of(part);
+        void *out = staged ? staged_out(S, part) : C->dev;
+        hipError_t e = launch_sddmm_spmm(S->dtype, chained != 0, view, A->dev, B->dev, out, Y->dev,
+                                         K, streams_of(ctx));
+        if (e == hipErrorNotSupported) {
+            (void)hipGetLastError();
+            if (chained)
+                return fail(SPC3D_ERR_INVALID_ARG,
+                            "the chained form needs dense rows of at most 4096 bytes "
+                            "(K * sizeof(real))");
+            // No vector kernel for this K: the two calls one after the other.
+            HIP_TRY(launch_sddmm(S->dtype, view, A->dev, B->dev, out, K, streams_of(ctx)));
+            HIP_TRY(launch_spmm(S->dtype, view, B->dev, Y->dev, K, streams_of(ctx)));
+            continue;
+        }
+        HIP_TRY(e);
+    }
+    if (staged)
+        HIP_TRY(unstage(S, C));
     return SPC3D_OK;
 }
 

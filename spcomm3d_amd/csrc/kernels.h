@@ -24,6 +24,7 @@ struct DevPlanView {
     // the long ones (launch_first_cols); read by the short-segment launch
     const uint32_t *first_cols = nullptr;
     uint64_t nnz = 0;
+    bool stream_c = false;            // SDDMM: streaming stores also at permuted positions
 };
 
 // The context's stream, plus an auxiliary stream of the same (default) priority
@@ -52,6 +53,9 @@ hipError_t launch_sddmm_spmm(int dtype, int chained, const DevPlanView &P, const
 // first_cols[s * kFirstCols + u] = column of entry min(u, len - 1) of segment segs[s], s < n
 hipError_t launch_first_cols(const Seg *segs, uint32_t n, const uint32_t *col, uint32_t *first_cols,
                              hipStream_t stream);
+// out[i] = in[pos[i]], i < n; pos and out 16-byte aligned
+hipError_t launch_unstage(int dtype, const void *in, const uint32_t *pos, void *out, uint64_t n,
+                          hipStream_t stream);
 // out[p] = in[perm[p]] (perm == null: copy)
 hipError_t launch_gather_vals(int dtype, const void *in, const uint32_t *perm, void *out,
                               uint64_t n, hipStream_t stream);

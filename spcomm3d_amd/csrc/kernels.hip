@@ -250,20 +250,25 @@ template <int G> __device__ __forceinline__ uint64_t seg_index(uint32_t nq, uint
 // descriptor instead of after it: two memory latencies per segment instead of three.
 // Lane u of a group of LPR >= kFirstCols lanes gets the column of entry u % kFirstCols;
 // a group of 4 lanes gets those of entries u and 4 + u.
-struct FirstCols {
-    uint32_t c[2];
+// stream_c: SDDMM stores its results at permuted positions past the L2 (streaming)
+// instead of with plain stores that the L2 can merge: for the blocks of a plan kept in
+// column blocks, whose positions are long runs in a staging vector and whose block of
+// dense rows is meant to stay in the L2s.
+struct Ahead {
+    uint32_t first[2] = {0, 0};
+    bool stream_c = false;
 };
 template <int LPR, bool WIDE>
-__device__ __forceinline__ FirstCols load_first_cols(const uint32_t *__restrict__ first_cols,
-                                                     uint64_t sid, uint32_t sub)
+__device__ __forceinline__ Ahead load_first_cols(const uint32_t *__restrict__ first_cols,
+                                                 uint64_t sid, uint32_t sub)
 {
-    FirstCols f{{0, 0}};
+    Ahead f;
     if constexpr (!WIDE) {
         constexpr uint32_t GL = (uint32_t)LPR < kFirstCols ? (uint32_t)LPR : kFirstCols;
         const uint32_t *at = first_cols + sid * kFirstCols + (sub & (GL - 1));
-        f.c[0] = nt_load(at);
+        f.first[0] = nt_load(at);
         if constexpr ((uint32_t)LPR < kFirstCols)
-            f.c[1] = nt_load(at + LPR);
+            f.first[1] = nt_load(at + LPR);
     }
     return f;
 }
@@ -494,8 +499,8 @@ __device__ __forceinline__ void odd_store(char *drow, bool whole,
 // that stores it.
 //
 // PRE: the column indices of the batch were loaded ahead (lane u of the group holds that
-// of entry u in pre[0], or, where the group has fewer lanes than the batch has entries,
-// those of entries u and LPR + u in pre[0] and pre[1]); past the segment's end they
+// of entry u in ex.first[0], or, where the group has fewer lanes than the batch has entries,
+// those of entries u and LPR + u in ex.first[0] and ex.first[1]); past the segment's end they
 // repeat its last column.
 //
 // NG <= NB: every lane group of the wavefront has at most NG entries in this batch, so
@@ -506,7 +511,7 @@ sddmm_batch_one(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type (&a
             const uint32_t *__restrict__ col, const uint32_t *__restrict__ perm,
             const T *__restrict__ sval, const T *__restrict__ B, T *__restrict__ C, uint32_t p0,
             uint32_t n, uint32_t sub, uint32_t nvec,
-            const Odd<T, VPL, RG> &odd, const uint32_t (&pre)[2])
+            const Odd<T, VPL, RG> &odd, const Ahead &ex)
 {
     using V = typename Vec<T>::type;
     static_assert(NB <= LPR, "batch must fit the lane group");
@@ -516,7 +521,7 @@ sddmm_batch_one(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type (&a
     uint32_t e = sub & (NB - 1);
     if (MK)
         e = e < n ? e : n - 1;
-    const uint32_t cme = PRE ? pre[0] : nt_load(col + p0 + e);
+    const uint32_t cme = PRE ? ex.first[0] : nt_load(col + p0 + e);
     const uint32_t uo = entry_of<LPR, NB>(sub);
     const bool writer = is_writer<LPR, NB>(sub) && (!MK || uo < n);
     T sv = (T)0;
@@ -554,7 +559,7 @@ sddmm_batch_one(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type (&a
             if (odd.accum)
                 result += C[dst];
         }
-        if (perm)
+        if (perm && !ex.stream_c)
             C[dst] = result;
         else
             nt_store(result, C + dst);
@@ -578,7 +583,7 @@ sddmm_batch_rounds(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type 
             const uint32_t *__restrict__ col, const uint32_t *__restrict__ perm,
             const T *__restrict__ sval, const T *__restrict__ B, T *__restrict__ C, uint32_t p0,
             uint32_t n, uint32_t sub, uint32_t nvec,
-            const Odd<T, VPL, RG> &odd, const uint32_t (&pre)[2])
+            const Odd<T, VPL, RG> &odd, const Ahead &ex)
 {
     using V = typename Vec<T>::type;
     // A group of LPR lanes reduces at most LPR entries at a time: the NB entries of
@@ -601,7 +606,7 @@ sddmm_batch_rounds(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type 
         uint32_t e = (uint32_t)r * G + (sub & (G - 1));
         if (MK)
             e = e < n ? e : n - 1;
-        cme[r] = PRE ? pre[r & 1] : nt_load(col + p0 + e);
+        cme[r] = PRE ? ex.first[r & 1] : nt_load(col + p0 + e);
         const uint32_t mine = (uint32_t)r * G + uo;
         writer[r] = wlane && (!MK || mine < n);
         sv[r] = (T)0;
@@ -638,7 +643,7 @@ sddmm_batch_rounds(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type 
                 if (odd.accum)
                     result += C[dst[r]];
             }
-            if (perm)
+            if (perm && !ex.stream_c)
                 C[dst[r]] = result;
             else
                 nt_store(result, C + dst[r]);
@@ -669,20 +674,20 @@ sddmm_batch(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type (&acc)[
             const uint32_t *__restrict__ col, const uint32_t *__restrict__ perm,
             const T *__restrict__ sval, const T *__restrict__ B, T *__restrict__ C, uint32_t p0,
             uint32_t n, uint32_t sub, uint32_t nvec,
-            const Odd<T, VPL, RG> &odd, const uint32_t (&pre)[2])
+            const Odd<T, VPL, RG> &odd, const Ahead &ex)
 {
     if constexpr (NB <= LPR)
         sddmm_batch_one<T, LPR, VPL, NB, RG, MK, FZ, PRE, NG>(a, acc, col, perm, sval, B, C, p0, n,
-                                                              sub, nvec, odd, pre);
+                                                              sub, nvec, odd, ex);
     else
         sddmm_batch_rounds<T, LPR, VPL, NB, RG, MK, FZ, PRE>(a, acc, col, perm, sval, B, C, p0, n,
-                                                             sub, nvec, odd, pre);
+                                                             sub, nvec, odd, ex);
 }
 
 // n consecutive entries from p.  WIDE: full batches of UB, then one masked batch
 // of the smallest size in {4, 8, 16} that holds the rest.  !WIDE (segments known
 // to be short, run at twice the occupancy): masked batches of UB throughout, the
-// first of them on the column indices in `pre` (loaded ahead, beside the segment's
+// first of them on the column indices in `ex.first` (loaded ahead, beside the segment's
 // descriptor, from the plan's table of first columns: kFirstCols per short segment).
 template <typename T, int LPR, int VPL, int UB, int RG, bool WIDE, int FZ>
 __device__ __forceinline__ void
@@ -690,26 +695,26 @@ sddmm_walk(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type (&acc)[V
            const uint32_t *__restrict__ col, const uint32_t *__restrict__ perm,
            const T *__restrict__ sval, const T *__restrict__ B, T *__restrict__ C, uint32_t p,
            uint32_t n, uint32_t sub, uint32_t nvec,
-            const Odd<T, VPL, RG> &odd, const uint32_t (&pre)[2])
+            const Odd<T, VPL, RG> &odd, const Ahead &ex)
 {
     if constexpr (WIDE) {
         for (; n >= UB; n -= UB, p += UB)
-            sddmm_batch<T, LPR, VPL, UB, RG, false, FZ>(a, acc, col, perm, sval, B, C, p, UB, sub, nvec, odd, pre);
+            sddmm_batch<T, LPR, VPL, UB, RG, false, FZ>(a, acc, col, perm, sval, B, C, p, UB, sub, nvec, odd, ex);
         if (n == 0)
             return;
         if constexpr (UB > 8) {
             if (n > 8) {
-                sddmm_batch<T, LPR, VPL, UB, RG, true, FZ>(a, acc, col, perm, sval, B, C, p, n, sub, nvec, odd, pre);
+                sddmm_batch<T, LPR, VPL, UB, RG, true, FZ>(a, acc, col, perm, sval, B, C, p, n, sub, nvec, odd, ex);
                 return;
             }
         }
         if constexpr (UB > 4) {
             if (n > 4) {
-                sddmm_batch<T, LPR, VPL, 8, RG, true, FZ>(a, acc, col, perm, sval, B, C, p, n, sub, nvec, odd, pre);
+                sddmm_batch<T, LPR, VPL, 8, RG, true, FZ>(a, acc, col, perm, sval, B, C, p, n, sub, nvec, odd, ex);
                 return;
             }
         }
-        sddmm_batch<T, LPR, VPL, (UB < 4 ? UB : 4), RG, true, FZ>(a, acc, col, perm, sval, B, C, p, n, sub, nvec, odd, pre);
+        sddmm_batch<T, LPR, VPL, (UB < 4 ? UB : 4), RG, true, FZ>(a, acc, col, perm, sval, B, C, p, n, sub, nvec, odd, ex);
     } else {
         static_assert(WIDE || UB <= (int)kFirstCols, "the first batch runs on the columns loaded ahead");
         {
@@ -720,15 +725,15 @@ sddmm_walk(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type (&acc)[V
             const uint32_t m = n < (uint32_t)UB ? n : (uint32_t)UB;
             if constexpr (UB == 8 && LPR >= 8) {
                 if (__ballot(m > 2) == 0)
-                    sddmm_batch<T, LPR, VPL, 2, RG, true, FZ, true>(a, acc, col, perm, sval, B, C, p, m, sub, nvec, odd, pre);
+                    sddmm_batch<T, LPR, VPL, 2, RG, true, FZ, true>(a, acc, col, perm, sval, B, C, p, m, sub, nvec, odd, ex);
                 else if (__ballot(m > 4) == 0)
-                    sddmm_batch<T, LPR, VPL, 4, RG, true, FZ, true>(a, acc, col, perm, sval, B, C, p, m, sub, nvec, odd, pre);
+                    sddmm_batch<T, LPR, VPL, 4, RG, true, FZ, true>(a, acc, col, perm, sval, B, C, p, m, sub, nvec, odd, ex);
                 else if (__ballot(m > 5) == 0)
-                    sddmm_batch<T, LPR, VPL, 8, RG, true, FZ, true, 5>(a, acc, col, perm, sval, B, C, p, m, sub, nvec, odd, pre);
+                    sddmm_batch<T, LPR, VPL, 8, RG, true, FZ, true, 5>(a, acc, col, perm, sval, B, C, p, m, sub, nvec, odd, ex);
                 else
-                    sddmm_batch<T, LPR, VPL, 8, RG, true, FZ, true>(a, acc, col, perm, sval, B, C, p, m, sub, nvec, odd, pre);
+                    sddmm_batch<T, LPR, VPL, 8, RG, true, FZ, true>(a, acc, col, perm, sval, B, C, p, m, sub, nvec, odd, ex);
             } else {
-                sddmm_batch<T, LPR, VPL, UB, RG, true, FZ, true>(a, acc, col, perm, sval, B, C, p, m, sub, nvec, odd, pre);
+                sddmm_batch<T, LPR, VPL, UB, RG, true, FZ, true>(a, acc, col, perm, sval, B, C, p, m, sub, nvec, odd, ex);
             }
             n -= m;
             p += m;
@@ -736,7 +741,7 @@ sddmm_walk(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type (&acc)[V
 #pragma nounroll
         while (n > 0) {
             const uint32_t m = n < (uint32_t)UB ? n : (uint32_t)UB;
-            sddmm_batch<T, LPR, VPL, UB, RG, true, FZ>(a, acc, col, perm, sval, B, C, p, m, sub, nvec, odd, pre);
+            sddmm_batch<T, LPR, VPL, UB, RG, true, FZ>(a, acc, col, perm, sval, B, C, p, m, sub, nvec, odd, ex);
             n -= m;
             p += m;
         }
@@ -751,7 +756,8 @@ sddmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint3
                  const uint32_t *__restrict__ col, const uint32_t *__restrict__ perm,
                  const T *__restrict__ sval, const T *__restrict__ A, const T *__restrict__ B,
                  T *__restrict__ C, T *__restrict__ Y, T *__restrict__ partial, uint32_t nvec,
-                 uint32_t stride, uint32_t accum, const uint32_t *__restrict__ first_cols)
+                 uint32_t stride, uint32_t accum, const uint32_t *__restrict__ first_cols,
+                 uint32_t stream_c)
 {
     static_assert(UB <= 16 && LPR <= 64, "at most 16 entries in flight per lane");
     using V = typename Vec<T>::type;
@@ -759,7 +765,8 @@ sddmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint3
     const uint64_t sid = seg_index<64 / LPR>(nq, rot);
     if (sid >= nseg)
         return;
-    const FirstCols pre = load_first_cols<LPR, WIDE>(first_cols, sid, sub);
+    Ahead ex = load_first_cols<LPR, WIDE>(first_cols, sid, sub);
+    ex.stream_c = stream_c != 0;
     const u32x4 sg = nt_load(reinterpret_cast<const u32x4 *>(segs) + sid); // row, start, len, slot
     if (sg[2] == 0)
         return;
@@ -785,7 +792,7 @@ sddmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint3
         }
     }
     sddmm_walk<T, LPR, VPL, UB, RG, WIDE, FZ>(a, acc, col, perm, sval, B, C, sg[1], sg[2], sub,
-                                              nvec, odd, pre.c);
+                                              nvec, odd, ex);
     if constexpr (FZ != 0 && RG >= 2) {
         const bool whole = sg[3] == kWholeRow;
         char *drow = const_cast<char *>(whole ? odd_row<T, RG>(Y, sg[0], stride)
@@ -815,24 +822,24 @@ sddmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint3
 // MK: only the first n of the NB entries exist; the others repeat the loads of
 // entry n - 1 and add zero times zero.
 // Column of entry j < kFirstCols of a short segment out of the indices loaded ahead:
-// lane u of the group holds that of entry u in pre[0] (groups of 4 lanes: of entries u
-// and 4 + u in pre[0] and pre[1]).
-template <int LPR> __device__ __forceinline__ uint32_t first_col(const uint32_t (&pre)[2], uint32_t j)
+// lane u of the group holds that of entry u in FC[0] (groups of 4 lanes: of entries u
+// and 4 + u in FC[0] and FC[1]).
+template <int LPR> __device__ __forceinline__ uint32_t first_col(const uint32_t (&FC)[2], uint32_t j)
 {
     if constexpr (LPR >= (int)kFirstCols)
-        return __shfl(pre[0], j, LPR);
+        return __shfl(FC[0], j, LPR);
     else
-        return __shfl((j & LPR) ? pre[1] : pre[0], j & (LPR - 1), LPR);
+        return __shfl((j & LPR) ? FC[1] : FC[0], j & (LPR - 1), LPR);
 }
 
 // PRE: the batch is entries off .. off + NB - 1 of a short segment, off + NB <=
-// kFirstCols, and takes its column indices from `pre` (first_col).
+// kFirstCols, and takes its column indices from `ex.first` (first_col).
 template <typename T, int LPR, int VPL, int NB, int RG, bool MK, bool PRE>
 __device__ __forceinline__ void
 spmm_batch_one(typename Vec<T>::type (&acc)[VPL], const uint32_t *__restrict__ col,
            const T *__restrict__ sval, const T *__restrict__ X, uint32_t p0, uint32_t n,
            uint32_t sub, uint32_t nvec,
-            const Odd<T, VPL, RG> &odd, const uint32_t (&pre)[2], uint32_t off)
+            const Odd<T, VPL, RG> &odd, const Ahead &ex, uint32_t off)
 {
     using V = typename Vec<T>::type;
     static_assert(NB <= LPR, "batch must fit the lane group");
@@ -848,7 +855,7 @@ spmm_batch_one(typename Vec<T>::type (&acc)[VPL], const uint32_t *__restrict__ c
     T av[NB];
 #pragma unroll
     for (int u = 0; u < NB; ++u) {
-        const uint32_t c = PRE ? first_col<LPR>(pre, off + u) : __shfl(cme, u, LPR);
+        const uint32_t c = PRE ? first_col<LPR>(ex.first, off + u) : __shfl(cme, u, LPR);
         av[u] = __shfl(vme, u, LPR);
         gather_row<T, LPR, VPL, RG>(x[u], X, c, sub, nvec, odd);
     }
@@ -915,7 +922,7 @@ spmm_batch(typename Vec<T>::type (&acc)[VPL], const uint32_t *__restrict__ col,
            uint32_t sub, uint32_t nvec,
             const Odd<T, VPL, RG> &odd)
 {
-    const uint32_t none[2] = {0, 0};
+    const Ahead none{};
     if constexpr (NB <= LPR)
         spmm_batch_one<T, LPR, VPL, NB, RG, MK, false>(acc, col, sval, X, p0, n, sub, nvec, odd,
                                                        none, 0u);
@@ -928,13 +935,13 @@ __device__ __forceinline__ void
 spmm_walk(typename Vec<T>::type (&acc)[VPL], const uint32_t *__restrict__ col,
           const T *__restrict__ sval, const T *__restrict__ X, uint32_t p, uint32_t n,
           uint32_t sub, uint32_t nvec,
-            const Odd<T, VPL, RG> &odd, const uint32_t (&pre)[2])
+            const Odd<T, VPL, RG> &odd, const Ahead &ex)
 {
     // Short segments: exact batches of UB, then UB/2 ... 1 as n requires.  Measured
     // against masked batches here (which cost registers, hence occupancy): 3 % faster
     // on 5-entry rows, level elsewhere.  SpMM's short rows are bound by the Y
     // read-modify-write stream, not by rounds of gathers.  The first kFirstCols
-    // entries take their column indices from `pre`, which was loaded ahead, beside the
+    // entries take their column indices from `ex.first`, which was loaded ahead, beside the
     // segment's descriptor.
     if constexpr (!WIDE) {
         static_assert(WIDE || (UB <= 4 && UB <= LPR), "short batches fit the lane group");
@@ -943,17 +950,17 @@ spmm_walk(typename Vec<T>::type (&acc)[VPL], const uint32_t *__restrict__ col,
             uint32_t off = 0;
             for (; off + UB <= m; off += UB)
                 spmm_batch_one<T, LPR, VPL, UB, RG, false, true>(acc, col, sval, X, p + off, UB,
-                                                                 sub, nvec, odd, pre, off);
+                                                                 sub, nvec, odd, ex, off);
             if constexpr (UB > 2)
                 if ((m - off) & 2) {
                     spmm_batch_one<T, LPR, VPL, 2, RG, false, true>(acc, col, sval, X, p + off, 2,
-                                                                    sub, nvec, odd, pre, off);
+                                                                    sub, nvec, odd, ex, off);
                     off += 2;
                 }
             if constexpr (UB > 1)
                 if ((m - off) & 1)
                     spmm_batch_one<T, LPR, VPL, 1, RG, false, true>(acc, col, sval, X, p + off, 1,
-                                                                    sub, nvec, odd, pre, off);
+                                                                    sub, nvec, odd, ex, off);
             n -= m;
             p += m;
         }
@@ -1011,7 +1018,7 @@ spmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint32
     const uint64_t sid = seg_index<64 / LPR>(nq, rot);
     if (sid >= nseg)
         return;
-    const FirstCols pre = load_first_cols<LPR, WIDE>(first_cols, sid, sub);
+    const Ahead ex = load_first_cols<LPR, WIDE>(first_cols, sid, sub);
     const u32x4 sg = nt_load(reinterpret_cast<const u32x4 *>(segs) + sid); // row, start, len, slot
     if (sg[2] == 0)
         return;
@@ -1032,7 +1039,7 @@ spmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint32
             for (int v = 0; v < VPL; ++v)
                 y0[v] = odd_load<T, RG, VPL, true>(drow, v, nvec, odd);
         }
-        spmm_walk<T, LPR, VPL, UB, RG, WIDE>(acc, col, sval, X, sg[1], sg[2], sub, nvec, odd, pre.c);
+        spmm_walk<T, LPR, VPL, UB, RG, WIDE>(acc, col, sval, X, sg[1], sg[2], sub, nvec, odd, ex);
         odd_store<T, VPL>(drow, whole, y0, acc, odd);
     } else {
         V *dst = const_cast<V *>(whole ? row_ptr<T, LPR, VPL, RG>(Y, sg[0], sub, nvec)
@@ -1043,7 +1050,7 @@ spmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint32
                 if (lane_on<LPR, RG>(sub, v, nvec))
                     y0[v] = nt_load(dst + v * LPR);
         }
-        spmm_walk<T, LPR, VPL, UB, RG, WIDE>(acc, col, sval, X, sg[1], sg[2], sub, nvec, odd, pre.c);
+        spmm_walk<T, LPR, VPL, UB, RG, WIDE>(acc, col, sval, X, sg[1], sg[2], sub, nvec, odd, ex);
 #pragma unroll
         for (int v = 0; v < VPL; ++v) {
             if (!lane_on<LPR, RG>(sub, v, nvec))
@@ -1148,6 +1155,32 @@ gather_kernel(const T *__restrict__ in, const uint32_t *__restrict__ perm, T *__
     const uint64_t stride = (uint64_t)gridDim.x * kBlock;
     for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride)
         out[i] = perm ? in[perm[i]] : in[i];
+}
+
+// out[i] = in[pos[i]], four results per lane: positions and results move as 16-byte
+// vectors, streaming; the reads in between are whatever `pos` makes them (runs, for the
+// staged results of a plan kept in column blocks).
+template <typename T>
+__global__ void __launch_bounds__(kBlock)
+gather4_kernel(const T *__restrict__ in, const uint32_t *__restrict__ pos, T *__restrict__ out,
+               uint64_t n)
+{
+    const uint64_t stride = (uint64_t)gridDim.x * kBlock * 4;
+    const uint64_t nfull = n / 4 * 4;
+    for (uint64_t i = ((uint64_t)blockIdx.x * kBlock + threadIdx.x) * 4; i < nfull; i += stride) {
+        const u32x4 p = nt_load(reinterpret_cast<const u32x4 *>(pos + i));
+        using V = typename Vec<T>::type; // 16 bytes: 4 floats or 2 doubles
+        V v[4 / Vec<T>::N];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            v[u / Vec<T>::N][u % Vec<T>::N] = in[p[u]];
+#pragma unroll
+        for (int u = 0; u < 4 / Vec<T>::N; ++u)
+            nt_store(v[u], reinterpret_cast<V *>(out + i) + u);
+    }
+    const uint64_t t = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (t < n - nfull)
+        out[nfull + t] = in[pos[nfull + t]];
 }
 
 template <typename T>
@@ -1294,13 +1327,14 @@ hipError_t run_sddmm(const DevPlanView &P, const T *A, const T *B, T *C, T *Y, c
                            dim3(blocks_for_groups(nl, P.nqueues, 64 / LPR)), dim3(kBlock), 0,
                            S.main, P.segs, nl, P.nqueues, 0u, P.col, P.perm, (const T *)P.sval,
                            A, B, C, Y, (T *)P.partial, nvec, stride ? stride : nvec, accum,
-                           (const uint32_t *)nullptr);
+                           (const uint32_t *)nullptr, P.stream_c ? 1u : 0u);
     if (ns)
         hipLaunchKernelGGL((sddmm_seg_kernel<T, LPR, VPL, US, RG, false, FZ>),
                            dim3(blocks_for_groups(ns, P.nqueues, 64 / LPR)), dim3(kBlock), 0,
                            both ? S.aux : S.main, P.segs + nl, ns, P.nqueues,
                            both ? S.aux_rot : 0u, P.col, P.perm, (const T *)P.sval, A, B, C, Y,
-                           (T *)P.partial, nvec, stride ? stride : nvec, accum, P.first_cols);
+                           (T *)P.partial, nvec, stride ? stride : nvec, accum, P.first_cols,
+                           P.stream_c ? 1u : 0u);
     const hipError_t launched = hipGetLastError();
     const hipError_t joined = both ? join_aux(S) : hipSuccess;
     return launched != hipSuccess ? launched : joined;
@@ -1547,6 +1581,21 @@ hipError_t launch_first_cols(const Seg *segs, uint32_t n, const uint32_t *col, u
     const uint64_t threads = (uint64_t)n * kFirstCols;
     hipLaunchKernelGGL(first_cols_kernel, dim3((uint32_t)((threads + kBlock - 1) / kBlock)),
                        dim3(kBlock), 0, stream, segs, n, col, first_cols);
+    return hipGetLastError();
+}
+
+hipError_t launch_unstage(int dtype, const void *in, const uint32_t *pos, void *out, uint64_t n,
+                          hipStream_t stream)
+{
+    if (n == 0)
+        return hipSuccess;
+    const uint32_t grid = stream_grid((n + 3) / 4);
+    if (dtype == 1)
+        hipLaunchKernelGGL((gather4_kernel<double>), dim3(grid), dim3(kBlock), 0, stream,
+                           (const double *)in, pos, (double *)out, n);
+    else
+        hipLaunchKernelGGL((gather4_kernel<float>), dim3(grid), dim3(kBlock), 0, stream,
+                           (const float *)in, pos, (float *)out, n);
     return hipGetLastError();
 }
 

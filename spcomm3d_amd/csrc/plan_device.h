@@ -41,4 +41,32 @@ int localize_device(hipStream_t stream, uint64_t n, uint32_t *d_idx, uint32_t *d
 int remap_device(hipStream_t stream, uint64_t n, uint32_t *d_idx, const uint32_t *d_map,
                  uint32_t map_len, std::string &err);
 
+// ---- column blocks -----------------------------------------------------------------
+// Stable partition of a device COO by column block (block b = columns [b * w, (b + 1) * w),
+// w = ceil(ncols / nblocks)): d_order[q] = caller's position of partitioned entry q (the
+// caller's order kept inside a block), d_ii_out / d_jj_out the entries in that order,
+// first[b] (host, nblocks + 1 words) where block b starts.  The indices must have been
+// validated (jj < ncols).
+int partition_by_col_block(hipStream_t stream, uint64_t nnz, const uint32_t *d_ii,
+                           const uint32_t *d_jj, uint32_t ncols, uint32_t nblocks,
+                           uint32_t *d_ii_out, uint32_t *d_jj_out, uint32_t *d_order,
+                           uint32_t *first, std::string &err);
+// d_out[q] = d_order[d_perm ? d_perm[q] : q], q < n (a block's kernel order -> the caller's
+// positions).  Asynchronous on `stream`.
+int compose_perm_device(hipStream_t stream, const uint32_t *d_order, const uint32_t *d_perm,
+                        uint64_t n, uint32_t *d_out, std::string &err);
+// d_out[d_perm[q]] = d_vals[q], q < n.  Asynchronous on `stream`.
+int scatter_device(hipStream_t stream, const uint32_t *d_perm, const uint32_t *d_vals, uint64_t n,
+                   uint32_t *d_out, std::string &err);
+// d_key[q] = d_rows[d_perm ? d_perm[q] : q] / rows_per_tile, q < n.  Asynchronous.
+int tile_keys_device(hipStream_t stream, const uint32_t *d_rows, const uint32_t *d_perm, uint64_t n,
+                     uint32_t rows_per_tile, uint32_t *d_key, std::string &err);
+// d_rank[i] = position of element i in the stable ascending order of d_key (keys <=
+// max_key).  Synchronous.
+int stable_ranks_device(hipStream_t stream, const uint32_t *d_key, uint64_t n, uint32_t max_key,
+                        uint32_t *d_rank, std::string &err);
+// Sum of len^2 over a plan's segments (device array); synchronous.
+int sum_sq_seg_len_device(hipStream_t stream, const Seg *d_segs, uint64_t nseg, uint64_t *out,
+                          std::string &err);
+
 } // namespace spc3d

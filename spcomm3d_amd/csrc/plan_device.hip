@@ -767,6 +767,65 @@ int order_entries(Arena &arena, Temp &tmp, hipStream_t st, uint64_t nnz, int key
     return SPC3D_OK;
 }
 
+// ---- column blocks ---------------------------------------------------------------
+__global__ void block_keys_k(const uint32_t *__restrict__ jj, uint64_t nnz, uint32_t block_cols,
+                             uint32_t *key)
+{
+    GRID_STRIDE(e, nnz) key[e] = jj[e] / block_cols;
+}
+__global__ void gather_u32_k(const uint32_t *__restrict__ in, const uint32_t *__restrict__ idx,
+                             uint64_t n, uint32_t *out)
+{
+    GRID_STRIDE(e, n) out[e] = in[idx[e]];
+}
+// first[b] = position of the first entry of block b in the sorted keys (first[nblocks] = n)
+__global__ void block_firsts_k(const uint32_t *__restrict__ sorted, uint64_t n, uint32_t nblocks,
+                               uint32_t *first)
+{
+    GRID_STRIDE(i, n + 1)
+    {
+        const uint32_t lo = i == 0 ? 0u : sorted[i - 1] + 1;
+        const uint32_t hi = i == n ? nblocks : sorted[i];
+        for (uint32_t b = lo; b <= hi && b <= nblocks; ++b)
+            first[b] = (uint32_t)i;
+    }
+}
+// perm[q] = order[off + (perm ? perm[q] : q)]
+__global__ void compose_perm_k(const uint32_t *__restrict__ order, const uint32_t *__restrict__ perm,
+                               uint64_t n, uint32_t *out)
+{
+    GRID_STRIDE(q, n) out[q] = order[perm ? perm[q] : (uint32_t)q];
+}
+// out[perm[q]] = vals[q]
+__global__ void scatter_u32_k(const uint32_t *__restrict__ perm, const uint32_t *__restrict__ vals,
+                              uint64_t n, uint32_t *out)
+{
+    GRID_STRIDE(q, n) out[perm[q]] = vals[q];
+}
+// key[q] = rows[perm ? perm[q] : q] / rows_per_tile
+__global__ void tile_keys_k(const uint32_t *__restrict__ rows, const uint32_t *__restrict__ perm,
+                            uint64_t n, uint32_t rows_per_tile, uint32_t *key)
+{
+    GRID_STRIDE(q, n) key[q] = rows[perm ? perm[q] : (uint32_t)q] / rows_per_tile;
+}
+// rank[sorted[i]] = i
+__global__ void ranks_k(const uint32_t *__restrict__ sorted, uint64_t n, uint32_t *rank)
+{
+    GRID_STRIDE(i, n) rank[sorted[i]] = (uint32_t)i;
+}
+__global__ void sum_sq_len_k(const Seg *__restrict__ segs, uint64_t n, unsigned long long *out)
+{
+    unsigned long long s = 0;
+    GRID_STRIDE(i, n)
+    {
+        const unsigned long long l = segs[i].len;
+        s += l * l;
+    }
+    s = block_sum(s);
+    if (threadIdx.x == 0 && s)
+        atomicAdd(out, s);
+}
+
 } // namespace
 
 int build_device_plan(hipStream_t st, uint32_t nrows, uint32_t ncols, uint64_t nnz,
@@ -1119,6 +1178,105 @@ int remap_device(hipStream_t st, uint64_t n, uint32_t *d_idx, const uint32_t *d_
     LAUNCH(remap_apply_k, n, d_idx, n, d_map);
     HIP_OK(hipGetLastError());
     HIP_OK(hipStreamSynchronize(st));
+    return SPC3D_OK;
+}
+
+} // namespace spc3d
+
+namespace spc3d {
+
+int partition_by_col_block(hipStream_t st, uint64_t nnz, const uint32_t *d_ii, const uint32_t *d_jj,
+                           uint32_t ncols, uint32_t nblocks, uint32_t *d_ii_out, uint32_t *d_jj_out,
+                           uint32_t *d_order, uint32_t *first, std::string &err)
+{
+    for (uint32_t b = 0; b <= nblocks; ++b)
+        first[b] = 0;
+    if (nnz == 0 || nblocks == 0)
+        return SPC3D_OK;
+    const uint32_t block_cols = (ncols + nblocks - 1) / nblocks;
+    Arena arena;
+    HIP_OK(arena.reserve((size_t)nnz * 12 + (size_t)nblocks * 4 + ((size_t)8 << 20)));
+    Temp tmp(arena);
+    SBuf<uint32_t> key, key_out, ident, dfirst;
+    HIP_OK(key.alloc(arena, nnz));
+    HIP_OK(key_out.alloc(arena, nnz));
+    HIP_OK(ident.alloc(arena, nnz));
+    HIP_OK(dfirst.alloc(arena, (size_t)nblocks + 1));
+    LAUNCH(block_keys_k, nnz, d_jj, nnz, block_cols, key.p);
+    LAUNCH(iota_k, nnz, ident.p, nnz);
+    TRY(sort_pairs<uint32_t>(tmp, key.p, key_out.p, ident.p, d_order, (uint32_t)nnz,
+                             bits_for(nblocks), false, st, err));
+    LAUNCH(gather_u32_k, nnz, d_ii, d_order, nnz, d_ii_out);
+    LAUNCH(gather_u32_k, nnz, d_jj, d_order, nnz, d_jj_out);
+    LAUNCH(block_firsts_k, nnz + 1, key_out.p, nnz, nblocks, dfirst.p);
+    TRY(fetch(st, first, dfirst.p, ((size_t)nblocks + 1) * sizeof(uint32_t), err));
+    return SPC3D_OK;
+}
+
+int compose_perm_device(hipStream_t st, const uint32_t *d_order, const uint32_t *d_perm, uint64_t n,
+                        uint32_t *d_out, std::string &err)
+{
+    if (n == 0)
+        return SPC3D_OK;
+    LAUNCH(compose_perm_k, n, d_order, d_perm, n, d_out);
+    HIP_OK(hipGetLastError());
+    return SPC3D_OK;
+}
+
+int scatter_device(hipStream_t st, const uint32_t *d_perm, const uint32_t *d_vals, uint64_t n,
+                   uint32_t *d_out, std::string &err)
+{
+    if (n == 0)
+        return SPC3D_OK;
+    LAUNCH(scatter_u32_k, n, d_perm, d_vals, n, d_out);
+    HIP_OK(hipGetLastError());
+    return SPC3D_OK;
+}
+
+int tile_keys_device(hipStream_t st, const uint32_t *d_rows, const uint32_t *d_perm, uint64_t n,
+                     uint32_t rows_per_tile, uint32_t *d_key, std::string &err)
+{
+    if (n == 0)
+        return SPC3D_OK;
+    LAUNCH(tile_keys_k, n, d_rows, d_perm, n, rows_per_tile, d_key);
+    HIP_OK(hipGetLastError());
+    return SPC3D_OK;
+}
+
+int stable_ranks_device(hipStream_t st, const uint32_t *d_key, uint64_t n, uint32_t max_key,
+                        uint32_t *d_rank, std::string &err)
+{
+    if (n == 0)
+        return SPC3D_OK;
+    Arena arena;
+    HIP_OK(arena.reserve((size_t)n * 12 + ((size_t)8 << 20)));
+    Temp tmp(arena);
+    SBuf<uint32_t> key_out, ident, sorted;
+    HIP_OK(key_out.alloc(arena, n));
+    HIP_OK(ident.alloc(arena, n));
+    HIP_OK(sorted.alloc(arena, n));
+    LAUNCH(iota_k, n, ident.p, n);
+    TRY(sort_pairs<uint32_t>(tmp, d_key, key_out.p, ident.p, sorted.p, (uint32_t)n,
+                             bits_for(max_key), false, st, err));
+    LAUNCH(ranks_k, n, sorted.p, n, d_rank);
+    HIP_OK(hipGetLastError());
+    HIP_OK(hipStreamSynchronize(st)); // the arena goes away with this call
+    return SPC3D_OK;
+}
+
+int sum_sq_seg_len_device(hipStream_t st, const Seg *d_segs, uint64_t nseg, uint64_t *out,
+                          std::string &err)
+{
+    *out = 0;
+    if (nseg == 0)
+        return SPC3D_OK;
+    DBuf<unsigned long long> acc;
+    HIP_OK(acc.alloc(1));
+    HIP_OK(hipMemsetAsync(acc.p, 0, sizeof(unsigned long long), st));
+    LAUNCH_SMALL(sum_sq_len_k, nseg, d_segs, nseg, acc.p);
+    unsigned long long h = 0;
+    TRY(fetch(st, &h, acc.p, sizeof h, err));
+    *out = h;
     return SPC3D_OK;
 }
 

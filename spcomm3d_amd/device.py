@@ -32,7 +32,7 @@ _BUILDERS = {None: 0, "device": 2, "host": 1}
 
 
 def make_opts(seg_max=None, k_hint=None, l2_hot_bytes=None, hub_min=None,
-              xcd_slices=None, builder=None) -> PlanOpts:
+              xcd_slices=None, builder=None, col_blocks=None) -> PlanOpts:
     """``spc3d_plan_opts``; ``None`` keeps the library default.  ``builder``:
     ``"device"`` or ``"host"`` (where ``spc3d_plan_create_ex`` builds the plan)."""
     o = PlanOpts()
@@ -42,6 +42,7 @@ def make_opts(seg_max=None, k_hint=None, l2_hot_bytes=None, hub_min=None,
     o.l2_hot_bytes = int(l2_hot_bytes or 0)
     o.hub_min = int(hub_min or 0)
     o.xcd_slices = int(xcd_slices or 0)
+    o.col_blocks = int(col_blocks or 0)
     return o
 
 

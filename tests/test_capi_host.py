@@ -246,7 +246,7 @@ def test_plan_build_host_rejects_bad_arguments():
     with pytest.raises(capi.Spc3dError):
         device.plan_build_host(2, 6, ii, jj, xcd_slices=4)
     o = capi.PlanOpts()
-    o.reserved[1] = 7
+    o.reserved[0] = 7
     rc = lib.spc3d_plan_build_host(capi.F32, 2, 6, 3, vp(ii), vp(jj), ctypes.byref(o),
                                    ctypes.byref(info), None, None, None, 0, None, 0)
     assert rc == capi.ERR_INVALID_ARG

@@ -17,11 +17,17 @@ from tests import _oracle as oracle
 pytestmark = pytest.mark.gpu
 
 
-def _check_sampled(ctx, w, dtype, n_entries=200_000, n_rows=3000, seed=9):
+def _check_sampled(ctx, w, dtype, n_entries=200_000, n_rows=3000, seed=9, col_blocks=None):
+    """col_blocks: None = a plan with every option at its default; "auto" = the plan must
+    have chosen column blocks by itself (k_hint given, as bench.py does)."""
     tol = oracle.TOL[np.dtype(W.np_dtype(dtype))]
     rng = np.random.default_rng(seed)
     A, B, Y0, vv = w.panel_A(dtype), w.panel_B(dtype), w.panel_Y0(dtype), w.values(dtype)
-    S = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, vv)
+    if col_blocks == "auto":
+        S = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, vv, k_hint=w.k)
+        assert S.info.ncol_blocks > 1
+    else:
+        S = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, vv)
     info = S.info
     assert info.nnz == w.nnz and info.nsegments >= info.rows_touched
     dA, dB, dY = ctx.panel_from(A), ctx.panel_from(B), ctx.panel_from(Y0)
@@ -91,4 +97,4 @@ def test_config4_stencil_full(ctx):
 def test_config5_hypergraph_full(ctx):
     w = W.hypergraph_zipf(2_000_000, 500_000, 128, 1.2, 1024)
     assert w.nrows == 2_000_000 and w.ncols == 500_000 and w.k == 128
-    _check_sampled(ctx, w, "f32", n_entries=200_000, n_rows=2000)
+    _check_sampled(ctx, w, "f32", n_entries=200_000, n_rows=2000, col_blocks="auto")

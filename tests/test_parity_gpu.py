@@ -463,6 +463,71 @@ def test_xcd_sliced_plan_matches_oracle(ctx, dtype):
     check_spmm(B, w.ii, w.jj, vv, Y0, dY.download())
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nblocks", [2, 7, 300])
+def test_plan_in_column_blocks_matches_oracle(ctx, dtype, nblocks):
+    """A pattern kept in column blocks (one plan per block, run one after the other):
+    same results as the whole plan up to summation order, in the caller's order."""
+    w = W.rmat(12, 24, 40).shuffled()
+    A, B, Y0, vv = w.panel_A(dtype), w.panel_B(dtype), w.panel_Y0(dtype), w.values(dtype)
+    S = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, vv, col_blocks=nblocks, seg_max=32, k_hint=w.k)
+    info = S.info
+    assert 1 < info.ncol_blocks <= nblocks and info.nnz == w.nnz
+    assert info.nsegments >= info.rows_touched and not info.order_is_identity
+    with pytest.raises(capi.Spc3dError):
+        S.download()  # one set of arrays per block, none for the pattern
+    dA, dB, dY = ctx.panel_from(A), ctx.panel_from(B), ctx.panel_from(Y0)
+    dC = ctx.vals(w.nnz, dtype)
+    dC.fill(float("nan"))
+    ctx.sddmm(S, dA, dB, dC)
+    ctx.spmm(S, dB, dY)
+    check_sddmm(A, B, w.ii, w.jj, vv, dC.download())
+    check_spmm(B, w.ii, w.jj, vv, Y0, dY.download())
+    # the one-pass call and the call that allocates nothing go block by block as well
+    dY2, dY3, dC2 = ctx.panel_from(Y0), ctx.panel_from(Y0), ctx.vals(w.nnz, dtype)
+    ctx.sddmm_spmm(S, dA, dB, dC2, dY2)
+    ctx.spmm_noalloc(S, dB, dY3)
+    check_sddmm(A, B, w.ii, w.jj, vv, dC2.download())
+    check_spmm(B, w.ii, w.jj, vv, Y0, dY2.download())
+    assert np.array_equal(dY3.download(), dY.download())
+    # new values, from the host and from the device
+    vv2 = (vv * 3 + 1).astype(vv.dtype)
+    S.set_values(vv2)
+    ctx.sddmm(S, dA, dB, dC)
+    check_sddmm(A, B, w.ii, w.jj, vv2, dC.download())
+    dv = ctx.vals(w.nnz, dtype)
+    dv.upload(vv)
+    S.set_values_device(dv)
+    ctx.sddmm(S, dA, dB, dC)
+    check_sddmm(A, B, w.ii, w.jj, vv, dC.download())
+    for h in (S, dA, dB, dY, dY2, dY3, dC, dC2, dv):
+        h.close()
+
+
+def test_column_blocks_are_chosen_for_long_rows_over_a_wide_unskewed_panel(ctx):
+    # 140 k columns of 512 bytes (68 MiB, uniform), rows of 890 entries in the weighted
+    # mean: the rule picks blocks; R-MAT (skewed columns) and short rows stay whole
+    w = W.hypergraph_zipf(3000, 140_000, 128)
+    vv = w.values("f32")
+    S = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, vv, k_hint=w.k)
+    assert 12 <= S.info.ncol_blocks <= 14 and S.info.nqueues == 1, S.info.ncol_blocks
+    whole = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, vv, k_hint=w.k, col_blocks=1)
+    assert whole.info.ncol_blocks == 1
+    A, B, Y0 = w.panel_A("f32"), w.panel_B("f32"), w.panel_Y0("f32")
+    dA, dB, dY, dC = ctx.panel_from(A), ctx.panel_from(B), ctx.panel_from(Y0), ctx.vals(w.nnz, "f32")
+    ctx.sddmm(S, dA, dB, dC)
+    ctx.spmm(S, dB, dY)
+    check_sddmm(A, B, w.ii, w.jj, vv, dC.download())
+    check_spmm(B, w.ii, w.jj, vv, Y0, dY.download())
+    for h in (S, whole, dA, dB, dY, dC):
+        h.close()
+    for other in (W.rmat(16, 16, 64), W.stencil5(256, 256, 32), W.erdos_renyi(16384, 16, 32)):
+        P = ctx.plan(other.nrows, other.ncols, other.ii, other.jj, other.values("f32"),
+                     k_hint=other.k)
+        assert P.info.ncol_blocks == 1
+        P.close()
+
+
 def test_workgroups_are_dealt_to_xcds_round_robin(ctx):
     # what the XCD-sliced plan layout relies on for its speed (not for its results)
     # round-robin by workgroup id, from a starting XCD that is fixed per hardware queue
