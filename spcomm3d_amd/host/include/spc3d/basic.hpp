@@ -7,8 +7,6 @@
 // (denseMatrix).  Differences, all deliberate:
 //   - the scalar types are real typedefs, not #defines, and real_t can be
 //     switched to float with -DSPC3D_REAL=float (the reference is double only);
-//   - parallelTiming carries an extra microsecond field for the compute phase:
-//     a GPU kernel here lasts well under the reference's 1 ms resolution;
 //   - denseMatrix::at computes its offset in 64 bits (the reference's 32-bit
 //     x*n+y wraps for m*n >= 2^32).
 #pragma once
@@ -30,11 +28,10 @@ using idx_large_t = std::uint64_t;
 
 static_assert(sizeof(real_t) == 4 || sizeof(real_t) == 8, "real_t must be float or double");
 
-// Per-call phase times in whole milliseconds, as the reference reports them;
-// compTimeUs is the compute phase again, in microseconds.
+// Per-call phase times in whole milliseconds, as the reference reports them
+// (five idx_t, the reference's layout).
 struct parallelTiming {
     idx_t comm1Time = 0, comm2Time = 0, commcpyTime = 0, compTime = 0, totalTime = 0;
-    idx_large_t compTimeUs = 0;
 };
 
 struct triplet {

@@ -1,17 +1,21 @@
 // The reference's distributed kernel wrappers (src/distributed_comp.hpp:11-64),
 // for ONE rank on ONE GPU: pre-communication, the local kernel, post-
 // communication, and the reference's statistics line, with the reference's
-// names and parameter order.  With a single rank every exchange is empty
-// (inDegree = outDegree = 0, src/comm.hpp:66-70) and the Z reduction of SDDMM is
-// a copy of C.vv into C.ownedVals (MPI_Reduce_scatter over one rank,
-// src/denseComm.hpp:39 with the buffers of src/comm_setup.cpp:678-679), so
-// this header carries single-rank stand-ins for SparseComm / DenseComm instead
+// names, parameter order and return type (void).  With a single rank every
+// exchange is empty (inDegree = outDegree = 0, src/comm.hpp:66-70) and the Z
+// reduction of SDDMM is a copy of C.vv into C.ownedVals (MPI_Reduce_scatter over
+// one rank, src/denseComm.hpp:39 with the buffers of src/comm_setup.cpp:678-679),
+// so this header carries single-rank stand-ins for SparseComm / DenseComm instead
 // of MPI: the MPI communication layer itself is outside this library.
 //
-// The last parameter of every wrapper is the process mesh (the reference passes
-// the Cartesian communicator and reads its dimensions back, e.g.
-// src/distributed_comp.cpp:25-27); here it is the dimensions themselves and
-// must be 1 x 1 x 1.
+// The last parameter of every wrapper is the process mesh.  The reference passes
+// the Cartesian communicator and reads its dimensions back
+// (src/distributed_comp.cpp:25-27): compiled with -DSPC3D_WITH_MPI (and an mpi.h
+// on the include path) this header declares exactly those signatures,
+// `void dist_*(..., MPI_Comm comm)`, which read the dimensions with MPI_Cart_get
+// and refuse anything but 1 x 1 x 1.  Without MPI the same wrappers take the
+// dimensions themselves (`const Mesh &`).  The phase times the reference keeps in
+// a local and only prints are also kept for the caller: dist_last_timing().
 #pragma once
 
 #include <cstdio>
@@ -21,6 +25,10 @@
 
 #include "SparseMatrix.hpp"
 #include "basic.hpp"
+
+#ifdef SPC3D_WITH_MPI
+#include <mpi.h>
+#endif
 
 namespace SpKernels {
 
@@ -97,37 +105,113 @@ struct DenseComm {
 void setup_sddmm_reduce_single_rank(SpKernels::cooMat &C, DComm::DenseComm &comm_post);
 
 // src/distributed_comp.hpp:11-64.  Each prints the reference's statistics lines
-// (src/comm_stats.cpp:33-36,53) and returns the phase times of the call.
-SpKernels::parallelTiming dist_spmm_spcomm(SpKernels::denseMatrix &X, SpKernels::cooMat &A,
-                                           SpKernels::denseMatrix &Y,
-                                           SpKernels::SparseComm<SpKernels::real_t> &comm_pre,
-                                           SpKernels::SparseComm<SpKernels::real_t> &comm_post,
-                                           const SpKernels::Mesh &mesh);
-SpKernels::parallelTiming dist_spmm_dcomm(SpKernels::denseMatrix &X, SpKernels::denseMatrix &Y,
-                                          SpKernels::cooMat &A, DComm::DenseComm &comm_pre,
-                                          DComm::DenseComm &comm_post,
-                                          const SpKernels::Mesh &mesh);
-SpKernels::parallelTiming dist_sddmm_spcomm(SpKernels::denseMatrix &A, SpKernels::denseMatrix &B,
-                                            SpKernels::cooMat &S,
-                                            SpKernels::SparseComm<SpKernels::real_t> &comm_pre,
-                                            DComm::DenseComm &comm_post, SpKernels::cooMat &C,
-                                            const SpKernels::Mesh &mesh);
-SpKernels::parallelTiming dist_sddmm_spcomm2(SpKernels::denseMatrix &A, SpKernels::denseMatrix &B,
-                                             SpKernels::cooMat &S,
-                                             SpKernels::SparseComm<SpKernels::real_t> &comm_preA,
-                                             SpKernels::SparseComm<SpKernels::real_t> &comm_preB,
-                                             DComm::DenseComm &comm_post, SpKernels::cooMat &C,
-                                             const SpKernels::Mesh &mesh);
-SpKernels::parallelTiming dist_sddmm_spcomm3(SpKernels::denseMatrix &A, SpKernels::denseMatrix &B,
-                                             SpKernels::cooMat &S,
-                                             SpKernels::SparseComm<SpKernels::real_t> &comm_preA,
-                                             SpKernels::SparseComm<SpKernels::real_t> &comm_preB,
-                                             DComm::DenseComm &comm_post, SpKernels::cooMat &C,
-                                             const SpKernels::Mesh &mesh);
-SpKernels::parallelTiming dist_sddmm_dcomm(SpKernels::denseMatrix &A, SpKernels::denseMatrix &B,
-                                           SpKernels::cooMat &S, DComm::DenseComm &comm_pre,
-                                           DComm::DenseComm &comm_post, SpKernels::cooMat &C,
-                                           const SpKernels::Mesh &mesh);
+// (src/comm_stats.cpp:33-36,53).
+void dist_spmm_spcomm(SpKernels::denseMatrix &X, SpKernels::cooMat &A,
+                      SpKernels::denseMatrix &Y,
+                      SpKernels::SparseComm<SpKernels::real_t> &comm_pre,
+                      SpKernels::SparseComm<SpKernels::real_t> &comm_post,
+                      const SpKernels::Mesh &mesh);
+void dist_spmm_dcomm(SpKernels::denseMatrix &X, SpKernels::denseMatrix &Y,
+                     SpKernels::cooMat &A, DComm::DenseComm &comm_pre,
+                     DComm::DenseComm &comm_post,
+                     const SpKernels::Mesh &mesh);
+void dist_sddmm_spcomm(SpKernels::denseMatrix &A, SpKernels::denseMatrix &B,
+                       SpKernels::cooMat &S,
+                       SpKernels::SparseComm<SpKernels::real_t> &comm_pre,
+                       DComm::DenseComm &comm_post, SpKernels::cooMat &C,
+                       const SpKernels::Mesh &mesh);
+void dist_sddmm_spcomm2(SpKernels::denseMatrix &A, SpKernels::denseMatrix &B,
+                        SpKernels::cooMat &S,
+                        SpKernels::SparseComm<SpKernels::real_t> &comm_preA,
+                        SpKernels::SparseComm<SpKernels::real_t> &comm_preB,
+                        DComm::DenseComm &comm_post, SpKernels::cooMat &C,
+                        const SpKernels::Mesh &mesh);
+void dist_sddmm_spcomm3(SpKernels::denseMatrix &A, SpKernels::denseMatrix &B,
+                        SpKernels::cooMat &S,
+                        SpKernels::SparseComm<SpKernels::real_t> &comm_preA,
+                        SpKernels::SparseComm<SpKernels::real_t> &comm_preB,
+                        DComm::DenseComm &comm_post, SpKernels::cooMat &C,
+                        const SpKernels::Mesh &mesh);
+void dist_sddmm_dcomm(SpKernels::denseMatrix &A, SpKernels::denseMatrix &B,
+                      SpKernels::cooMat &S, DComm::DenseComm &comm_pre,
+                      DComm::DenseComm &comm_post, SpKernels::cooMat &C,
+                      const SpKernels::Mesh &mesh);
 
 // Where the statistics lines go (default stdout); nullptr silences them.
 void dist_set_stats_stream(std::FILE *f);
+
+// Phase times of the last dist_* call on this thread: the reference's five
+// millisecond counters, and the compute phase again as the device measured it, in
+// microseconds (a GPU kernel lasts well under the reference's 1 ms resolution).
+struct distTiming {
+    SpKernels::parallelTiming pt;
+    SpKernels::idx_large_t compTimeUs = 0;
+};
+const distTiming &dist_last_timing();
+
+#ifdef SPC3D_WITH_MPI
+// The reference's own signatures (src/distributed_comp.hpp:11-64).  Inline, so
+// that the library itself needs no MPI: the caller's translation unit, which has
+// the communicator, links the MPI library it was made with.
+namespace spc3d_detail {
+inline SpKernels::Mesh mesh_of(MPI_Comm comm)
+{
+    int dims[3] = {0, 0, 0}, periods[3], coords[3], nd = 0, topo = MPI_UNDEFINED;
+    MPI_Topo_test(comm, &topo);
+    if (topo == MPI_CART)
+        MPI_Cartdim_get(comm, &nd);
+    if (topo != MPI_CART || nd != 3)
+        throw std::runtime_error("dist_*: the communicator must be the 3D Cartesian one "
+                                 "(src/distributed_comp.cpp:25-27)");
+    MPI_Cart_get(comm, 3, dims, periods, coords);
+    SpKernels::Mesh m;
+    m.X = dims[0];
+    m.Y = dims[1];
+    m.Z = dims[2];
+    return m;
+}
+} // namespace spc3d_detail
+
+inline void dist_spmm_spcomm(SpKernels::denseMatrix &X, SpKernels::cooMat &A,
+                             SpKernels::denseMatrix &Y,
+                             SpKernels::SparseComm<SpKernels::real_t> &comm_pre,
+                             SpKernels::SparseComm<SpKernels::real_t> &comm_post, MPI_Comm comm)
+{
+    dist_spmm_spcomm(X, A, Y, comm_pre, comm_post, spc3d_detail::mesh_of(comm));
+}
+inline void dist_spmm_dcomm(SpKernels::denseMatrix &X, SpKernels::denseMatrix &Y,
+                            SpKernels::cooMat &A, DComm::DenseComm &comm_pre,
+                            DComm::DenseComm &comm_post, MPI_Comm comm)
+{
+    dist_spmm_dcomm(X, Y, A, comm_pre, comm_post, spc3d_detail::mesh_of(comm));
+}
+inline void dist_sddmm_spcomm(SpKernels::denseMatrix &A, SpKernels::denseMatrix &B,
+                              SpKernels::cooMat &S,
+                              SpKernels::SparseComm<SpKernels::real_t> &comm_pre,
+                              DComm::DenseComm &comm_post, SpKernels::cooMat &C, MPI_Comm comm)
+{
+    dist_sddmm_spcomm(A, B, S, comm_pre, comm_post, C, spc3d_detail::mesh_of(comm));
+}
+inline void dist_sddmm_spcomm2(SpKernels::denseMatrix &A, SpKernels::denseMatrix &B,
+                               SpKernels::cooMat &S,
+                               SpKernels::SparseComm<SpKernels::real_t> &comm_preA,
+                               SpKernels::SparseComm<SpKernels::real_t> &comm_preB,
+                               DComm::DenseComm &comm_post, SpKernels::cooMat &C, MPI_Comm comm)
+{
+    dist_sddmm_spcomm2(A, B, S, comm_preA, comm_preB, comm_post, C, spc3d_detail::mesh_of(comm));
+}
+inline void dist_sddmm_spcomm3(SpKernels::denseMatrix &A, SpKernels::denseMatrix &B,
+                               SpKernels::cooMat &S,
+                               SpKernels::SparseComm<SpKernels::real_t> &comm_preA,
+                               SpKernels::SparseComm<SpKernels::real_t> &comm_preB,
+                               DComm::DenseComm &comm_post, SpKernels::cooMat &C, MPI_Comm comm)
+{
+    dist_sddmm_spcomm3(A, B, S, comm_preA, comm_preB, comm_post, C, spc3d_detail::mesh_of(comm));
+}
+inline void dist_sddmm_dcomm(SpKernels::denseMatrix &A, SpKernels::denseMatrix &B,
+                             SpKernels::cooMat &S, DComm::DenseComm &comm_pre,
+                             DComm::DenseComm &comm_post, SpKernels::cooMat &C, MPI_Comm comm)
+{
+    dist_sddmm_dcomm(A, B, S, comm_pre, comm_post, C, spc3d_detail::mesh_of(comm));
+}
+#endif // SPC3D_WITH_MPI

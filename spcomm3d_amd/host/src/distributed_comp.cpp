@@ -15,6 +15,7 @@ using DComm::DenseComm;
 namespace {
 
 std::FILE *g_stats = stdout;
+thread_local distTiming g_last;
 
 using clk = std::chrono::high_resolution_clock;
 
@@ -102,12 +103,14 @@ template <typename F> void timed_kernel(parallelTiming &pt, F fn)
     const auto t0 = clk::now();
     fn();
     pt.compTime = ms_since(t0);
-    pt.compTimeUs = (idx_large_t)hip::last_kernel_us();
+    g_last.compTimeUs = (idx_large_t)hip::last_kernel_us();
 }
 
 } // namespace
 
 void dist_set_stats_stream(std::FILE *f) { g_stats = f; }
+
+const distTiming &dist_last_timing() { return g_last; }
 
 void setup_sddmm_reduce_single_rank(cooMat &C, DenseComm &comm_post)
 {
@@ -125,7 +128,7 @@ void setup_sddmm_reduce_single_rank(cooMat &C, DenseComm &comm_post)
 // src/distributed_comp.cpp:17-76.  The reference's post phase calls
 // comm_pre.copy_from_recvbuff() where comm_post.copy_to_sendbuff() is evidently
 // meant (:59); the call is kept as it is there.  With one rank both are empty.
-parallelTiming dist_spmm_spcomm(denseMatrix &X, cooMat &A, denseMatrix &Y,
+void dist_spmm_spcomm(denseMatrix &X, cooMat &A, denseMatrix &Y,
                                 SparseComm<real_t> &comm_pre, SparseComm<real_t> &comm_post,
                                 const Mesh &mesh)
 {
@@ -158,11 +161,11 @@ parallelTiming dist_spmm_spcomm(denseMatrix &X, cooMat &A, denseMatrix &Y,
     pt.totalTime = ms_since(tot);
     stats_sparse(A.mtxName, "sparse spmm PRE", comm_pre, X.n, pt, mesh);
     stats_sparse(A.mtxName, "sparse spmm POST", comm_post, X.n, pt, mesh);
-    return pt;
+    g_last.pt = pt;
 }
 
 // src/distributed_comp.cpp:285-348
-parallelTiming dist_spmm_dcomm(denseMatrix &X, denseMatrix &Y, cooMat &A, DenseComm &comm_pre,
+void dist_spmm_dcomm(denseMatrix &X, denseMatrix &Y, cooMat &A, DenseComm &comm_pre,
                                DenseComm &comm_post, const Mesh &mesh)
 {
     require_single(mesh);
@@ -178,11 +181,11 @@ parallelTiming dist_spmm_dcomm(denseMatrix &X, denseMatrix &Y, cooMat &A, DenseC
     pt.totalTime = ms_since(tot);
     stats_dense(A.mtxName, "dense spmm PRE", comm_pre, X.n, pt, mesh);
     stats_dense(A.mtxName, "dense spmm POST", comm_post, X.n, pt, mesh);
-    return pt;
+    g_last.pt = pt;
 }
 
 // src/distributed_comp.cpp:141-193
-parallelTiming dist_sddmm_spcomm(denseMatrix &A, denseMatrix &B, cooMat &S,
+void dist_sddmm_spcomm(denseMatrix &A, denseMatrix &B, cooMat &S,
                                  SparseComm<real_t> &comm_pre, DenseComm &comm_post, cooMat &C,
                                  const Mesh &mesh)
 {
@@ -207,14 +210,14 @@ parallelTiming dist_sddmm_spcomm(denseMatrix &A, denseMatrix &B, cooMat &S,
     pt.totalTime = ms_since(tot);
     stats_sparse(C.mtxName, "sparse sddmm PRE", comm_pre, A.n, pt, mesh);
     stats_dense(C.mtxName, "sparse sddmm POST", comm_post, A.n, pt, mesh);
-    return pt;
+    g_last.pt = pt;
 }
 
 namespace {
 // Shared body of spcomm2 / spcomm3 (src/distributed_comp.cpp:194-284): the two
 // differ in how the expand is sent (derived datatypes vs. no receive buffer),
 // which has no single-rank counterpart.
-parallelTiming sddmm_two_sided(denseMatrix &A, denseMatrix &B, cooMat &S,
+void sddmm_two_sided(denseMatrix &A, denseMatrix &B, cooMat &S,
                                SparseComm<real_t> &preA, SparseComm<real_t> &preB,
                                DenseComm &comm_post, cooMat &C, const Mesh &mesh,
                                const char *pre_name, const char *post_name, bool with_dt)
@@ -237,30 +240,30 @@ parallelTiming sddmm_two_sided(denseMatrix &A, denseMatrix &B, cooMat &S,
     pt.totalTime = ms_since(tot);
     stats_sparse2(C.mtxName, pre_name, preA, preB, A.n, pt, mesh);
     stats_dense(C.mtxName, post_name, comm_post, A.n, pt, mesh);
-    return pt;
+    g_last.pt = pt;
 }
 } // namespace
 
 // src/distributed_comp.cpp:237-284
-parallelTiming dist_sddmm_spcomm2(denseMatrix &A, denseMatrix &B, cooMat &S,
+void dist_sddmm_spcomm2(denseMatrix &A, denseMatrix &B, cooMat &S,
                                   SparseComm<real_t> &comm_preA, SparseComm<real_t> &comm_preB,
                                   DenseComm &comm_post, cooMat &C, const Mesh &mesh)
 {
-    return sddmm_two_sided(A, B, S, comm_preA, comm_preB, comm_post, C, mesh,
+    sddmm_two_sided(A, B, S, comm_preA, comm_preB, comm_post, C, mesh,
                            "sparseNRB sddmm PRE", "sparseNRB sddmm POST", false);
 }
 
 // src/distributed_comp.cpp:194-236
-parallelTiming dist_sddmm_spcomm3(denseMatrix &A, denseMatrix &B, cooMat &S,
+void dist_sddmm_spcomm3(denseMatrix &A, denseMatrix &B, cooMat &S,
                                   SparseComm<real_t> &comm_preA, SparseComm<real_t> &comm_preB,
                                   DenseComm &comm_post, cooMat &C, const Mesh &mesh)
 {
-    return sddmm_two_sided(A, B, S, comm_preA, comm_preB, comm_post, C, mesh,
+    sddmm_two_sided(A, B, S, comm_preA, comm_preB, comm_post, C, mesh,
                            "sparseNB sddmm PRE", "sparseNB sddmm POST", true);
 }
 
 // src/distributed_comp.cpp:349-413
-parallelTiming dist_sddmm_dcomm(denseMatrix &A, denseMatrix &B, cooMat &S, DenseComm &comm_pre,
+void dist_sddmm_dcomm(denseMatrix &A, denseMatrix &B, cooMat &S, DenseComm &comm_pre,
                                 DenseComm &comm_post, cooMat &C, const Mesh &mesh)
 {
     require_single(mesh);
@@ -276,5 +279,5 @@ parallelTiming dist_sddmm_dcomm(denseMatrix &A, denseMatrix &B, cooMat &S, Dense
     pt.totalTime = ms_since(tot);
     stats_dense(C.mtxName, "dense sddmm PRE", comm_pre, A.n, pt, mesh);
     stats_dense(C.mtxName, "dense sddmm POST", comm_post, A.n, pt, mesh);
-    return pt;
+    g_last.pt = pt;
 }

@@ -54,3 +54,25 @@ def test_binary_file_layout_with_numpy():
 @pytest.mark.parametrize("name", ["test_shim_f64", "test_shim_f32"])
 def test_shim_on_gpu(name):
     _run(name)
+
+
+def _mpi_env():
+    """Environment in which a program linked with the image's MPI library starts: the
+    system's libstdc++ ahead of the MPI library's own directory."""
+    env = dict(os.environ)
+    env["LD_LIBRARY_PATH"] = "/usr/lib/x86_64-linux-gnu:/opt/conda/lib:" + env.get("LD_LIBRARY_PATH", "")
+    return env
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["test_dist_mpi_f64", "test_dist_mpi_f32"])
+def test_dist_wrappers_under_the_reference_signatures(name):
+    # void dist_*(..., MPI_Comm) on a 1 x 1 x 1 Cartesian communicator
+    # (src/distributed_comp.hpp:11-64); built only where the image has an MPI
+    path = os.path.join(CPP, name)
+    if not os.path.exists(path):
+        pytest.skip("no MPI installation where the tests were built")
+    r = subprocess.run([path], capture_output=True, text=True, timeout=300, env=_mpi_env())
+    if r.returncode == 127 or "error while loading shared libraries" in r.stderr:
+        pytest.skip("the MPI library the test was linked with does not load here: " + r.stderr[-300:])
+    assert r.returncode == 0 and "PASSED" in r.stdout, r.stdout[-3000:] + r.stderr[-3000:]

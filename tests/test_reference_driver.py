@@ -67,3 +67,67 @@ def test_gpu_build_of_the_reference_driver_on_a_generated_matrix(tmp_path, k):
         for r, c, v in zip(ii, jj, vv):
             f.write(f"{r} {c} {v:.17g}\n")
     assert run(HIP, k, str(path)) == run(REF, k, str(path))
+
+
+# The reference's own six distributed wrappers (src/distributed_comp.cpp with
+# src/comm_stats.cpp, compiled from where they lie) under oracle/ref_dist_driver.cpp, one
+# MPI rank: linked with the reference's core_ops.cpp (distDriver_ref), and with the binding
+# in its place (distDriver_hip), so that all six call sites of SpKernels::sddmm / spmm
+# (src/distributed_comp.cpp:53,177,220,268,314,379) run on the GPU library.
+DREF = os.path.join(ROOT, "oracle", "_ref", "distDriver_ref")
+DHIP = os.path.join(ROOT, "oracle", "_ref", "distDriver_hip")
+needs_dist = pytest.mark.skipif(not (os.path.exists(DREF) and os.path.exists(DHIP)),
+                                reason="built only where the reference and an MPI are present")
+
+
+def run_dist(binary, *args):
+    env = dict(os.environ)
+    env["LD_LIBRARY_PATH"] = "/usr/lib/x86_64-linux-gnu:/opt/conda/lib:" + env.get("LD_LIBRARY_PATH", "")
+    r = subprocess.run([binary, *map(str, args)], capture_output=True, text=True, timeout=300, env=env)
+    if r.returncode == 127 or "error while loading shared libraries" in r.stderr:
+        pytest.skip("the MPI library does not load here: " + r.stderr[-300:])
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+    return r.stdout.splitlines()
+
+
+def strip_times(lines):
+    """CHK lines whole; statistics lines without their five trailing phase times."""
+    return [ln if ln.startswith("CHK") else " ".join(ln.split()[:-5]) for ln in lines]
+
+
+@needs_dist
+def test_reference_dist_wrappers_print_what_serial_loops_give():
+    # K=4, 30 x 20, 200 entries: checked against numpy on the driver's own seeded inputs
+    lines = run_dist(DREF, 4, 30, 20, 200)
+    chk = {ln.split()[1]: [float(x) for x in ln.split()[2:]] for ln in lines if ln.startswith("CHK")}
+    assert set(chk) == {"sddmm_spcomm", "sddmm_spcomm2", "sddmm_spcomm3", "sddmm_dcomm",
+                        "spmm_spcomm", "spmm_dcomm"}
+    s = 12345
+
+    def lcg():
+        nonlocal s
+        s = (s * 6364136223846793005 + 1442695040888963407) % 2**64
+        return s >> 33
+
+    m, n, k, nnz = 30, 20, 4, 200
+    ii, jj, vv = [], [], []
+    for _ in range(nnz):
+        r = lcg() % 3 if lcg() % 4 == 0 else lcg() % m
+        ii.append(r); jj.append(lcg() % n); vv.append((lcg() % 9) / 4.0)
+    fill = lambda rows, a, b: np.array([[((i * a + j * b) % 11 - 5) / 8.0 for j in range(k)] for i in range(rows)])
+    A, B, Y = fill(m, 7, 3), fill(n, 5, 2), fill(m, 3, 1)
+    C = np.array([v * (A[i] @ B[j]) for i, j, v in zip(ii, jj, vv)])
+    w = np.arange(nnz) % 13 + 1
+    assert chk["sddmm_spcomm"] == [C.sum(), (C * w).sum()]
+    for i, j, v in zip(ii, jj, vv):
+        Y[i] += v * B[j]
+    wy = np.arange(m * k) % 13 + 1
+    assert chk["spmm_spcomm"] == [Y.sum(), (Y.ravel() * wy).sum()]
+
+
+@pytest.mark.gpu
+@needs_dist
+@pytest.mark.parametrize("k,m,n,nnz", [(16, 300, 200, 5000), (64, 5000, 3000, 200000), (5, 40, 40, 100)])
+def test_reference_dist_wrappers_over_the_gpu_binding_print_the_same(k, m, n, nnz):
+    # exact operands (multiples of 1/8 and 1/4): the sums are the same in any order
+    assert strip_times(run_dist(DHIP, k, m, n, nnz)) == strip_times(run_dist(DREF, k, m, n, nnz))
