@@ -9,11 +9,14 @@
 // indices 0-based.  Values are float64 on disk whatever real_t is in memory.
 #pragma once
 
+#include <algorithm>
 #include <charconv>
+#include <cmath>
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
 #include <fstream>
+#include <random>
 #include <stdexcept>
 #include <string>
 #include <vector>
@@ -56,7 +59,8 @@ class TokenReader {
         if (b != e && *b == '+')
             ++b;
         const auto r = std::from_chars(b, e, v);
-        return r.ec == std::errc() && r.ptr == e;
+        // "inf" and "nan" are no numbers to stream extraction; from_chars would take them
+        return r.ec == std::errc() && r.ptr == e && std::isfinite(v);
     }
 
   private:
@@ -263,6 +267,95 @@ inline void read_binary(const std::string &inFN, cooMat &C, bool single_rank = t
         C.ncols = c;
         C.ownedNnz = (idx_t)n;
     }
+}
+
+// The 2D block of one rank, from a binary file, in a single process: what
+// read_bin_parallel_distribute_coo (src/parallel_io.hpp:132-190) leaves in Sloc on the rank
+// with coordinates (gx, gy, gz) of an X x Y x Z mesh, ready for localizeIndices()
+// (miniapp/bench_both.cpp:156-158).  The rule (src/parallel_io.hpp:64-76,98-105): the row
+// ids are permuted at random and dealt to the X row groups round-robin, the i-th row of the
+// permuted order to group i mod X; the column ids likewise to the Y column groups; entry
+// (r, c) belongs to the rank at (rpvec2D[r], cpvec2D[c]).  A rank ends up with its entries
+// in file order: every reader forwards its contiguous share of the file in order, and the
+// shares arrive in reader order (:86-94,107-123).  All Z ranks of a fibre hold the same block
+// (:150-163) and own lnnz / Z of its values, the first lnnz mod Z of them one more (:166-169).
+//
+// The reference shuffles with std::random_shuffle and no seed, so its partition differs from
+// run to run; here the permutation is a Fisher-Yates shuffle driven by std::mt19937_64(seed)
+// (position i swapped with position rng() mod (i + 1), from the back), the same on every
+// platform.  rpvec2D / cpvec2D return the group of every row and column as the reference's
+// reader does; the partitioner that runs next reads them (src/distribute.cpp:152,197,204).
+//
+// The file is streamed: memory is the two group vectors plus the block.
+inline void read_binary_block(const std::string &inFN, cooMat &C, int X, int Y, int gx, int gy,
+                              std::uint64_t seed, std::vector<int> &rpvec2D,
+                              std::vector<int> &cpvec2D, int Z = 1, int gz = 0)
+{
+    if (X < 1 || Y < 1 || Z < 1 || gx < 0 || gx >= X || gy < 0 || gy >= Y || gz < 0 || gz >= Z)
+        throw std::out_of_range("read_binary_block: no such rank in the mesh");
+    std::ifstream f(inFN, std::ios::binary);
+    if (!f)
+        throw std::runtime_error("read_binary_block: cannot open " + inFN);
+    std::uint32_t r = 0, c = 0;
+    std::uint64_t n = 0;
+    f.read(reinterpret_cast<char *>(&r), 4);
+    f.read(reinterpret_cast<char *>(&c), 4);
+    f.read(reinterpret_cast<char *>(&n), 8);
+    if (!f)
+        throw std::runtime_error("read_binary_block: " + inFN + " has no header");
+    f.seekg(0, std::ios::end);
+    const std::uint64_t file_bytes = (std::uint64_t)f.tellg();
+    f.seekg(16, std::ios::beg);
+    if (n > (file_bytes - 16) / 16)
+        throw std::runtime_error("read_binary_block: " + inFN + " ends before its last entry");
+
+    std::mt19937_64 rng(seed);
+    auto deal = [&rng](std::uint32_t count, int groups, std::vector<int> &group_of) {
+        std::vector<idx_t> order(count);
+        for (std::uint32_t i = 0; i < count; ++i)
+            order[i] = i;
+        for (std::uint32_t i = count; i > 1; --i)
+            std::swap(order[i - 1], order[rng() % i]);
+        group_of.assign(count, 0);
+        for (std::uint32_t i = 0; i < count; ++i)
+            group_of[order[i]] = (int)(i % (std::uint32_t)groups);
+    };
+    deal(r, X, rpvec2D); // rows first, then columns, as the reference draws them
+    deal(c, Y, cpvec2D);
+
+    C.gnrows = r;
+    C.gncols = c;
+    C.gnnz = n;
+    C.ii.clear();
+    C.jj.clear();
+    C.vv.clear();
+    std::vector<char> block;
+    const idx_large_t kChunk = 1 << 16;
+    for (idx_large_t at = 0; at < n; at += kChunk) {
+        const idx_large_t m = std::min<idx_large_t>(kChunk, n - at);
+        block.resize(m * 16);
+        f.read(block.data(), (std::streamsize)block.size());
+        if (!f)
+            throw std::runtime_error("read_binary_block: " + inFN + " ends before its last entry");
+        for (idx_large_t i = 0; i < m; ++i) {
+            std::uint32_t ri, ci;
+            double v;
+            std::memcpy(&ri, &block[i * 16], 4);
+            std::memcpy(&ci, &block[i * 16 + 4], 4);
+            if (ri >= r || ci >= c)
+                throw std::out_of_range("read_binary_block: entry outside the matrix in " + inFN);
+            if (rpvec2D[ri] != gx || cpvec2D[ci] != gy)
+                continue;
+            std::memcpy(&v, &block[i * 16 + 8], 8);
+            C.ii.push_back(ri);
+            C.jj.push_back(ci);
+            C.vv.push_back((real_t)v);
+        }
+    }
+    const idx_large_t lnnz = C.ii.size();
+    C.nnz = lnnz;
+    C.ownedNnz = (idx_t)(lnnz / (idx_large_t)Z + ((idx_large_t)gz < lnnz % (idx_large_t)Z ? 1 : 0));
+    C.ownedVals.assign(C.ownedNnz, (real_t)0);
 }
 
 } // namespace SpKernels

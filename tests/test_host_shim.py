@@ -76,3 +76,23 @@ def test_dist_wrappers_under_the_reference_signatures(name):
     if r.returncode == 127 or "error while loading shared libraries" in r.stderr:
         pytest.skip("the MPI library the test was linked with does not load here: " + r.stderr[-300:])
     assert r.returncode == 0 and "PASSED" in r.stdout, r.stdout[-3000:] + r.stderr[-3000:]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["test_file_gpu_f64", "test_file_gpu_f32"])
+@pytest.mark.parametrize("k", [4, 64])
+def test_files_through_this_builds_readers_onto_the_gpu(name, k):
+    # .mtx / .bin -> spc3d/io.hpp -> (2D block of a mesh) -> localizeIndices -> SDDMM + SpMM on
+    # the GPU -> oracle; and, for the reference's real type, the printed SDDMM sum against
+    # what the reference's own sequential checker prints for the same file
+    io = os.path.join(ROOT, "tests", "golden", "io")
+    r = subprocess.run([_binary(name), io, str(k)], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and "PASSED" in r.stdout, r.stdout[-3000:] + r.stderr[-3000:]
+    sums = {ln.split()[1]: ln.split()[2] for ln in r.stdout.splitlines() if ln.startswith("SUM ")}
+    assert set(sums) == {"general", "symmetric", "integer", "pattern_symmetric", "complex"}
+    ref = os.path.join(ROOT, "oracle", "_ref", "numCheckSeq_ref")
+    if name.endswith("f64") and os.path.exists(ref):
+        for stem, got in sums.items():
+            want = subprocess.run([ref, "-k", str(k), os.path.join(io, stem + ".mtx")],
+                                  capture_output=True, text=True, timeout=60)
+            assert want.returncode == 0 and got == want.stdout.strip(), (stem, got, want.stdout)
