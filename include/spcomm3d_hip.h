@@ -345,14 +345,44 @@ SPC3D_API int spc3d_rows_unpack(spc3d_ctx *ctx, spc3d_panel *P, const spc3d_rowm
 SPC3D_API int spc3d_rows_unpack_sum(spc3d_ctx *ctx, spc3d_panel *P, const spc3d_rowmap *map,
                           const spc3d_vals *buf);
 
-/* One-shot forms over host memory with exactly the reference's operands:
- * plan, upload, run, download, free.  Synchronous. */
+/* One-shot forms over host memory with exactly the reference's operands
+ * (SpKernels::sddmm / spmm, src/core_ops.hpp:9-12, on the data() of the caller's
+ * vectors).  Synchronous: the results are in cvv / Y when the call returns.
+ *
+ * The reference's drivers call the kernel five times over one pattern and the same
+ * panels (miniapp/bench_both.cpp:202-203, bench_spmm.cpp:185-186), so the context keeps
+ * what a call built for the next one, decided by CONTENT, never by address (ReMapIndices
+ * rewrites ii / jj in place between groups of calls, bench_both.cpp:200-205):
+ *   - up to four plans, reused when every 4 MiB block of ii and of jj has the key it had
+ *     when the plan was made (four CRC-32C streams, a sum and a fold over every word),
+ *     nnz, sizes, type and k agree, and a sample of the indices compares equal; a new
+ *     pattern is planned, and validated, as before;
+ *   - up to four device panels with the keys of the host memory they mirror: blocks of
+ *     A, B, X whose key is unchanged are not sent again, changed blocks are; Y is sent
+ *     and fetched in full on every call, the values svv / avv are sent on every call;
+ *   - the result vector of SDDMM.
+ * Reading an unchanged operand for its keys (several threads) takes about half the time
+ * of sending it.  The cache holds device memory until spc3d_host_cache_clear or
+ * spc3d_ctx_destroy; SPC3D_HOST_CACHE=0 in the environment gives plan, upload, run,
+ * download, free on every call instead.  One-shot calls on one context run one at a time
+ * (they take a lock).  The kernels of the last one-shot call lie between the timer slots
+ * SPC3D_TIMER_HOST_CALL_BEGIN and _END. */
+#define SPC3D_TIMER_HOST_CALL_BEGIN 4094
+#define SPC3D_TIMER_HOST_CALL_END 4095
 SPC3D_API int spc3d_sddmm_host(spc3d_ctx *ctx, int dtype, uint32_t m, uint32_t n, uint32_t k,
                      const void *A, const void *B, uint64_t nnz, const uint32_t *ii,
                      const uint32_t *jj, const void *svv, void *cvv);
 SPC3D_API int spc3d_spmm_host(spc3d_ctx *ctx, int dtype, uint32_t ncols, uint32_t nrows, uint32_t k,
                     const void *X, uint64_t nnz, const uint32_t *ii, const uint32_t *jj,
                     const void *avv, void *Y);
+/* Frees what the one-shot calls keep (no counterpart in the reference, whose operands
+ * live in host vectors). */
+SPC3D_API int spc3d_host_cache_clear(spc3d_ctx *ctx);
+/* What the last one-shot call on this context moved: bytes sent to the device, bytes of
+ * dense operands left in place because their content had not changed, and whether the
+ * plan was reused (1) or made (0).  Any pointer may be NULL. */
+SPC3D_API int spc3d_host_call_stats(spc3d_ctx *ctx, uint64_t *bytes_sent, uint64_t *bytes_kept,
+                          int *plan_reused);
 
 #ifdef __cplusplus
 }

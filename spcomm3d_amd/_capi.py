@@ -101,6 +101,8 @@ SIGNATURES = {
                                  c_vp, c_vp]),
     "spc3d_spmm_host": (c_int, [c_vp, c_int, c_u32, c_u32, c_u32, c_vp, c_u64, c_vp, c_vp, c_vp,
                                 c_vp]),
+    "spc3d_host_cache_clear": (c_int, [c_vp]),
+    "spc3d_host_call_stats": (c_int, [c_vp, c_vp, c_vp, c_vp]),
 }
 
 _lib = None

@@ -9,11 +9,13 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <memory>
 #include <mutex>
 #include <new>
 #include <string>
 #include <vector>
 
+#include "host_cache.h"
 #include "kernels.h"
 #include "plan_device.h"
 #include "plan_host.h"
@@ -94,6 +96,11 @@ int scratch_of(int device, void **out)
 }
 } // namespace
 
+// What the one-shot entry points over host memory keep between calls: plans by the
+// content of the pattern, device panels with the keys of the host memory they mirror,
+// and the result vector.  Defined after the handle types.
+struct HostCallCache;
+
 struct spc3d_ctx {
     uint32_t magic;
     int device;
@@ -105,6 +112,8 @@ struct spc3d_ctx {
     bool capturing;   // between spc3d_capture_begin and spc3d_capture_end
     hipEvent_t timers[kTimerSlots];
     bool timer_set[kTimerSlots];
+    HostCallCache *host_cache; // made by the first spc3d_*_host call
+    std::mutex host_mutex;     // the one-shot calls of a context run one at a time
 };
 
 struct spc3d_panel {
@@ -179,6 +188,38 @@ struct spc3d_plan {
     uint32_t *stage_pos = nullptr; // [nnz] caller's position -> staging position
     uint32_t *stage_of = nullptr;  // [nnz]
     uint64_t stage_off = 0;
+};
+
+// A cached plan answers for a pattern when the keys of every block of ii and jj, the
+// sizes, the type and the row width agree, and a sample of the indices read back equal.
+struct CachedHostPlan {
+    spc3d_plan *plan = nullptr;
+    int dtype = 0;
+    uint32_t nrows = 0, ncols = 0, k = 0;
+    uint64_t nnz = 0;
+    std::vector<BlockKey> key_ii, key_jj;
+    std::vector<uint32_t> sample; // ii, jj at kSamples evenly spaced entries
+    uint64_t last_use = 0;
+};
+
+// A device panel and the keys of the host memory it was filled from, block by block.
+// No keys: the panel's content is not known to equal any host memory (an output).
+struct CachedHostPanel {
+    spc3d_panel *panel = nullptr;
+    std::vector<BlockKey> keys;
+    const void *host = nullptr; // where it came from last: a preference among equals, never a proof
+    uint64_t last_use = 0;
+};
+
+struct HostCallCache {
+    static constexpr size_t kMaxPlans = 4, kMaxPanels = 4, kSamples = 64;
+    std::vector<CachedHostPlan> plans;
+    std::vector<CachedHostPanel> panels;
+    spc3d_vals *c = nullptr;
+    uint64_t clock = 0;
+    // what the last call did, for spc3d_host_call_stats
+    uint64_t bytes_sent = 0, bytes_kept = 0;
+    int plan_reused = 0;
 };
 
 namespace {
@@ -412,6 +453,7 @@ int spc3d_ctx_create(int device, spc3d_ctx **out)
         c->timers[i] = nullptr;
         c->timer_set[i] = false;
     }
+    c->host_cache = nullptr;
     c->magic = kMagicCtx;
     *out = c;
     return SPC3D_OK;
@@ -431,6 +473,7 @@ int spc3d_ctx_destroy(spc3d_ctx *ctx)
     }
     (void)hipSetDevice(ctx->device);
     (void)hipStreamSynchronize(ctx->stream);
+    (void)spc3d_host_cache_clear(ctx);
     for (int i = 0; i < kTimerSlots; ++i)
         if (ctx->timers[i])
             (void)hipEventDestroy(ctx->timers[i]);
@@ -1923,12 +1966,236 @@ int spc3d_rows_unpack_sum(spc3d_ctx *ctx, spc3d_panel *P, const spc3d_rowmap *ma
     return rows_op(2, ctx, P, map, buf);
 }
 
-int spc3d_sddmm_host(spc3d_ctx *ctx, int dtype, uint32_t m, uint32_t n, uint32_t k, const void *A,
-                     const void *B, uint64_t nnz, const uint32_t *ii, const uint32_t *jj,
-                     const void *svv, void *cvv)
+namespace {
+
+bool host_cache_enabled()
 {
-    if (nnz && (!svv || !cvv))
-        return fail(SPC3D_ERR_INVALID_ARG, "svv or cvv is NULL");
+    const char *e = std::getenv("SPC3D_HOST_CACHE");
+    return !e || std::atoi(e) != 0;
+}
+
+HostCallCache *cache_of(spc3d_ctx *ctx)
+{
+    if (!ctx->host_cache)
+        ctx->host_cache = new (std::nothrow) HostCallCache();
+    return ctx->host_cache;
+}
+
+void sample_indices(const uint32_t *ii, const uint32_t *jj, uint64_t nnz, std::vector<uint32_t> &out)
+{
+    out.clear();
+    for (size_t s = 0; s < HostCallCache::kSamples && nnz; ++s) {
+        const uint64_t e = (uint64_t)((unsigned __int128)s * nnz / HostCallCache::kSamples);
+        out.push_back(ii[e]);
+        out.push_back(jj[e]);
+    }
+}
+
+// The plan for this pattern at this row width: the cached one when the pattern's
+// content is what it was planned from, else a new one (which validates every index, so
+// a bad one is reported as the one-shot calls always reported it).  The values are
+// sent on every call: that costs less than reading them to see whether they changed.
+int host_plan(spc3d_ctx *ctx, HostCallCache *hc, int dtype, uint32_t nrows, uint32_t ncols,
+              uint32_t k, uint64_t nnz, const uint32_t *ii, const uint32_t *jj, const void *vv,
+              spc3d_plan **out)
+{
+    *out = nullptr;
+    if (nnz && (!ii || !jj))
+        return fail(SPC3D_ERR_INVALID_ARG, "ii or jj is NULL");
+    std::vector<BlockKey> kii, kjj;
+    std::vector<uint32_t> sample;
+    keys_of(ii, (size_t)nnz * 4, kii);
+    keys_of(jj, (size_t)nnz * 4, kjj);
+    sample_indices(ii, jj, nnz, sample);
+    ++hc->clock;
+    for (CachedHostPlan &e : hc->plans) {
+        if (e.dtype == dtype && e.nrows == nrows && e.ncols == ncols && e.k == k && e.nnz == nnz &&
+            e.key_ii == kii && e.key_jj == kjj && e.sample == sample) {
+            int rc = spc3d_plan_set_values(e.plan, vv);
+            if (rc)
+                return rc;
+            e.last_use = hc->clock;
+            hc->plan_reused = 1;
+            hc->bytes_sent += (uint64_t)nnz * elem_size(dtype);
+            *out = e.plan;
+            return SPC3D_OK;
+        }
+    }
+    hc->plan_reused = 0;
+    if (hc->plans.size() >= HostCallCache::kMaxPlans) {
+        size_t oldest = 0;
+        for (size_t i = 1; i < hc->plans.size(); ++i)
+            if (hc->plans[i].last_use < hc->plans[oldest].last_use)
+                oldest = i;
+        (void)spc3d_plan_destroy(hc->plans[oldest].plan);
+        hc->plans.erase(hc->plans.begin() + (std::ptrdiff_t)oldest);
+    }
+    spc3d_plan_opts o = opts_from_env();
+    if (!o.k_hint)
+        o.k_hint = k; // the one width this plan will run with; sizes the partial-sum rows too
+    spc3d_plan *plan = nullptr;
+    int rc = spc3d_plan_create_ex(ctx, dtype, nrows, ncols, nnz, ii, jj, vv, &o, &plan);
+    if (rc)
+        return rc;
+    hc->bytes_sent += (uint64_t)nnz * (8 + elem_size(dtype));
+    CachedHostPlan e;
+    e.plan = plan;
+    e.dtype = dtype;
+    e.nrows = nrows;
+    e.ncols = ncols;
+    e.k = k;
+    e.nnz = nnz;
+    e.key_ii.swap(kii);
+    e.key_jj.swap(kjj);
+    e.sample.swap(sample);
+    e.last_use = hc->clock;
+    hc->plans.push_back(std::move(e));
+    *out = plan;
+    return SPC3D_OK;
+}
+
+// A device panel of this shape holding what `host` holds.  input = true: the blocks whose
+// keys are those of the cached panel's source stay as they are, the others are sent.
+// input = false: a panel of this shape whose content is about to be overwritten from
+// `host` in full (an operand the kernel changes, so the device copy equals no host memory
+// afterwards).  `stamp` marks the panels this call already uses.
+int host_panel(spc3d_ctx *ctx, HostCallCache *hc, int dtype, uint32_t m, uint32_t n,
+               const void *host, bool input, uint64_t stamp, spc3d_panel **out)
+{
+    *out = nullptr;
+    const size_t bytes = (size_t)m * n * elem_size(dtype);
+    if (bytes && !host)
+        return fail(SPC3D_ERR_INVALID_ARG, "a dense operand is NULL");
+    std::vector<BlockKey> keys;
+    if (input)
+        keys_of(host, bytes, keys);
+    CachedHostPanel *hit = nullptr;
+    size_t best = 0; // number of blocks that would stay
+    for (CachedHostPanel &e : hc->panels) {
+        if (e.last_use == stamp || e.panel->dtype != dtype || e.panel->m != m || e.panel->n != n)
+            continue;
+        if (!input && !e.keys.empty())
+            continue; // an output does not take over a panel that mirrors an input
+        size_t same = 0;
+        if (input && e.keys.size() == keys.size())
+            for (size_t b = 0; b < keys.size(); ++b)
+                same += e.keys[b] == keys[b];
+        if (!hit || same > best || (same == best && e.host == host)) {
+            hit = &e;
+            best = same;
+        }
+    }
+    if (!hit) {
+        if (hc->panels.size() >= HostCallCache::kMaxPanels) {
+            size_t oldest = hc->panels.size();
+            for (size_t i = 0; i < hc->panels.size(); ++i)
+                if (hc->panels[i].last_use != stamp &&
+                    (oldest == hc->panels.size() || hc->panels[i].last_use < hc->panels[oldest].last_use))
+                    oldest = i;
+            if (oldest < hc->panels.size()) {
+                (void)spc3d_panel_destroy(hc->panels[oldest].panel);
+                hc->panels.erase(hc->panels.begin() + (std::ptrdiff_t)oldest);
+            }
+        }
+        CachedHostPanel e;
+        int rc = spc3d_panel_create(ctx, dtype, m, n, &e.panel);
+        if (rc)
+            return rc;
+        hc->panels.push_back(std::move(e));
+        hit = &hc->panels.back();
+    }
+    // send the blocks that differ, neighbouring ones in one copy
+    const bool known = input && hit->keys.size() == keys.size();
+    const size_t nblocks = (bytes + kKeyBlockBytes - 1) / kKeyBlockBytes;
+    const char *src = static_cast<const char *>(host);
+    char *dst = static_cast<char *>(hit->panel->dev);
+    for (size_t b = 0; b < nblocks;) {
+        if (known && hit->keys[b] == keys[b]) {
+            hc->bytes_kept += std::min(kKeyBlockBytes, bytes - b * kKeyBlockBytes);
+            ++b;
+            continue;
+        }
+        size_t e = b + 1;
+        while (e < nblocks && !(known && hit->keys[e] == keys[e]))
+            ++e;
+        const size_t off = b * kKeyBlockBytes, len = std::min(bytes, e * kKeyBlockBytes) - off;
+        hipError_t err = hipMemcpyAsync(dst + off, src + off, len, hipMemcpyHostToDevice, ctx->stream);
+        if (err != hipSuccess) {
+            hit->keys.clear(); // the panel's content is no longer known
+            return fail_hip(err, "upload of a dense operand");
+        }
+        hc->bytes_sent += len;
+        b = e;
+    }
+    hipError_t err = hipStreamSynchronize(ctx->stream);
+    if (err != hipSuccess) {
+        hit->keys.clear();
+        return fail_hip(err, "upload of a dense operand");
+    }
+    if (input)
+        hit->keys.swap(keys);
+    else
+        hit->keys.clear();
+    hit->host = host;
+    hit->last_use = stamp;
+    *out = hit->panel;
+    return SPC3D_OK;
+}
+
+int host_call_begin(spc3d_ctx *ctx, HostCallCache **hc)
+{
+    if (!live(ctx))
+        return fail(SPC3D_ERR_INVALID_ARG, "context is NULL or destroyed");
+    if (int rc = use_device(ctx))
+        return rc;
+    *hc = cache_of(ctx);
+    if (!*hc)
+        return fail(SPC3D_ERR_ALLOC, "host allocation failed");
+    (*hc)->bytes_sent = (*hc)->bytes_kept = 0;
+    (*hc)->plan_reused = 0;
+    return SPC3D_OK;
+}
+
+} // namespace
+
+int spc3d_host_cache_clear(spc3d_ctx *ctx)
+{
+    if (!live(ctx))
+        return fail(SPC3D_ERR_INVALID_ARG, "context is NULL or destroyed");
+    std::lock_guard<std::mutex> lock(ctx->host_mutex);
+    HostCallCache *hc = ctx->host_cache;
+    if (!hc)
+        return SPC3D_OK;
+    (void)hipSetDevice(ctx->device);
+    for (CachedHostPlan &e : hc->plans)
+        (void)spc3d_plan_destroy(e.plan);
+    for (CachedHostPanel &e : hc->panels)
+        (void)spc3d_panel_destroy(e.panel);
+    if (hc->c)
+        (void)spc3d_vals_destroy(hc->c);
+    delete hc;
+    ctx->host_cache = nullptr;
+    return SPC3D_OK;
+}
+
+int spc3d_host_call_stats(spc3d_ctx *ctx, uint64_t *bytes_sent, uint64_t *bytes_kept,
+                          int *plan_reused)
+{
+    if (!live(ctx))
+        return fail(SPC3D_ERR_INVALID_ARG, "context is NULL or destroyed");
+    std::lock_guard<std::mutex> lock(ctx->host_mutex);
+    const HostCallCache *hc = ctx->host_cache;
+    if (bytes_sent) *bytes_sent = hc ? hc->bytes_sent : 0;
+    if (bytes_kept) *bytes_kept = hc ? hc->bytes_kept : 0;
+    if (plan_reused) *plan_reused = hc ? hc->plan_reused : 0;
+    return SPC3D_OK;
+}
+
+// One-shot SDDMM without the cache (SPC3D_HOST_CACHE=0): plan, upload, run, download, free.
+static int sddmm_host_uncached(spc3d_ctx *ctx, int dtype, uint32_t m, uint32_t n, uint32_t k,
+                               const void *A, const void *B, uint64_t nnz, const uint32_t *ii,
+                               const uint32_t *jj, const void *svv, void *cvv)
+{
     spc3d_plan *S = nullptr;
     spc3d_panel *a = nullptr, *b = nullptr;
     spc3d_vals *c = nullptr;
@@ -1941,7 +2208,9 @@ int spc3d_sddmm_host(spc3d_ctx *ctx, int dtype, uint32_t m, uint32_t n, uint32_t
     if (!rc) rc = spc3d_vals_create(ctx, dtype, nnz, &c);
     if (!rc) rc = spc3d_panel_upload(a, A);
     if (!rc) rc = spc3d_panel_upload(b, B);
+    if (!rc) rc = spc3d_timer_mark(ctx, SPC3D_TIMER_HOST_CALL_BEGIN);
     if (!rc) rc = spc3d_sddmm(ctx, S, a, b, c);
+    if (!rc) rc = spc3d_timer_mark(ctx, SPC3D_TIMER_HOST_CALL_END);
     if (!rc) rc = spc3d_vals_download(c, cvv);
     const std::string keep = g_err;
     if (c) spc3d_vals_destroy(c);
@@ -1951,12 +2220,44 @@ int spc3d_sddmm_host(spc3d_ctx *ctx, int dtype, uint32_t m, uint32_t n, uint32_t
     return rc ? fail(rc, keep) : SPC3D_OK;
 }
 
-int spc3d_spmm_host(spc3d_ctx *ctx, int dtype, uint32_t ncols, uint32_t nrows, uint32_t k,
-                    const void *X, uint64_t nnz, const uint32_t *ii, const uint32_t *jj,
-                    const void *avv, void *Y)
+int spc3d_sddmm_host(spc3d_ctx *ctx, int dtype, uint32_t m, uint32_t n, uint32_t k, const void *A,
+                     const void *B, uint64_t nnz, const uint32_t *ii, const uint32_t *jj,
+                     const void *svv, void *cvv)
 {
-    if (nnz && !avv)
-        return fail(SPC3D_ERR_INVALID_ARG, "avv is NULL");
+    if (nnz && (!svv || !cvv))
+        return fail(SPC3D_ERR_INVALID_ARG, "svv or cvv is NULL");
+    if (!live(ctx) || !dtype_ok(dtype)) // reported as plan creation reports it (bad pattern first)
+        return sddmm_host_uncached(ctx, dtype, m, n, k, A, B, nnz, ii, jj, svv, cvv);
+    std::lock_guard<std::mutex> lock(ctx->host_mutex);
+    if (!host_cache_enabled())
+        return sddmm_host_uncached(ctx, dtype, m, n, k, A, B, nnz, ii, jj, svv, cvv);
+    HostCallCache *hc = nullptr;
+    int rc = host_call_begin(ctx, &hc);
+    if (rc)
+        return rc;
+    spc3d_plan *S = nullptr;
+    spc3d_panel *a = nullptr, *b = nullptr;
+    rc = host_plan(ctx, hc, dtype, m, n, k, nnz, ii, jj, svv, &S);
+    const uint64_t stamp = hc->clock; // host_plan advanced it: unique to this call
+    if (!rc) rc = host_panel(ctx, hc, dtype, m, k, A, true, stamp, &a);
+    if (!rc) rc = host_panel(ctx, hc, dtype, n, k, B, true, stamp, &b);
+    if (!rc && (!hc->c || hc->c->dtype != dtype || hc->c->n != nnz)) {
+        if (hc->c)
+            (void)spc3d_vals_destroy(hc->c);
+        hc->c = nullptr;
+        rc = spc3d_vals_create(ctx, dtype, nnz, &hc->c);
+    }
+    if (!rc) rc = spc3d_timer_mark(ctx, SPC3D_TIMER_HOST_CALL_BEGIN);
+    if (!rc) rc = spc3d_sddmm(ctx, S, a, b, hc->c);
+    if (!rc) rc = spc3d_timer_mark(ctx, SPC3D_TIMER_HOST_CALL_END);
+    if (!rc) rc = spc3d_vals_download(hc->c, cvv);
+    return rc;
+}
+
+static int spmm_host_uncached(spc3d_ctx *ctx, int dtype, uint32_t ncols, uint32_t nrows, uint32_t k,
+                              const void *X, uint64_t nnz, const uint32_t *ii, const uint32_t *jj,
+                              const void *avv, void *Y)
+{
     spc3d_plan *S = nullptr;
     spc3d_panel *x = nullptr, *y = nullptr;
     spc3d_plan_opts o = opts_from_env();
@@ -1967,13 +2268,45 @@ int spc3d_spmm_host(spc3d_ctx *ctx, int dtype, uint32_t ncols, uint32_t nrows, u
     if (!rc) rc = spc3d_panel_create(ctx, dtype, nrows, k, &y);
     if (!rc) rc = spc3d_panel_upload(x, X);
     if (!rc) rc = spc3d_panel_upload(y, Y);
+    if (!rc) rc = spc3d_timer_mark(ctx, SPC3D_TIMER_HOST_CALL_BEGIN);
     if (!rc) rc = spc3d_spmm(ctx, S, x, y);
+    if (!rc) rc = spc3d_timer_mark(ctx, SPC3D_TIMER_HOST_CALL_END);
     if (!rc) rc = spc3d_panel_download(y, Y);
     const std::string keep = g_err;
     if (y) spc3d_panel_destroy(y);
     if (x) spc3d_panel_destroy(x);
     if (S) spc3d_plan_destroy(S);
     return rc ? fail(rc, keep) : SPC3D_OK;
+}
+
+int spc3d_spmm_host(spc3d_ctx *ctx, int dtype, uint32_t ncols, uint32_t nrows, uint32_t k,
+                    const void *X, uint64_t nnz, const uint32_t *ii, const uint32_t *jj,
+                    const void *avv, void *Y)
+{
+    if (nnz && !avv)
+        return fail(SPC3D_ERR_INVALID_ARG, "avv is NULL");
+    if (!live(ctx) || !dtype_ok(dtype))
+        return spmm_host_uncached(ctx, dtype, ncols, nrows, k, X, nnz, ii, jj, avv, Y);
+    std::lock_guard<std::mutex> lock(ctx->host_mutex);
+    if (!host_cache_enabled())
+        return spmm_host_uncached(ctx, dtype, ncols, nrows, k, X, nnz, ii, jj, avv, Y);
+    HostCallCache *hc = nullptr;
+    int rc = host_call_begin(ctx, &hc);
+    if (rc)
+        return rc;
+    spc3d_plan *S = nullptr;
+    spc3d_panel *x = nullptr, *y = nullptr;
+    rc = host_plan(ctx, hc, dtype, nrows, ncols, k, nnz, ii, jj, avv, &S);
+    const uint64_t stamp = hc->clock;
+    if (!rc) rc = host_panel(ctx, hc, dtype, ncols, k, X, true, stamp, &x);
+    // Y comes back changed, so its device copy never equals the caller's memory when the
+    // next call starts: it is sent in full every time
+    if (!rc) rc = host_panel(ctx, hc, dtype, nrows, k, Y, false, stamp, &y);
+    if (!rc) rc = spc3d_timer_mark(ctx, SPC3D_TIMER_HOST_CALL_BEGIN);
+    if (!rc) rc = spc3d_spmm(ctx, S, x, y);
+    if (!rc) rc = spc3d_timer_mark(ctx, SPC3D_TIMER_HOST_CALL_END);
+    if (!rc) rc = spc3d_panel_download(y, Y);
+    return rc;
 }
 
 } // extern "C"

@@ -7,9 +7,11 @@
 // std::vectors, as in the reference; each call uploads the dense panels, runs
 // the kernel and downloads the result, so C.vv / Y.data are valid on return
 // (the reference's comm plans keep raw pointers into them, src/comm.hpp:41,49).
-// The sparse pattern is planned once and cached: the benches call the kernels
-// five times on the same pattern (miniapp/bench_both.cpp:202-203,
-// bench_spmm.cpp:185-186).
+// The benches call the kernels five times on one pattern and the same panels
+// (miniapp/bench_both.cpp:202-203, bench_spmm.cpp:185-186): the library keeps the
+// plan and the device panels between calls and reuses what still holds the
+// operands' content (spc3d_sddmm_host / spc3d_spmm_host); calls may come from
+// several threads, they run one at a time.
 //
 // Failures: the reference fails by std::out_of_range from .at()
 // (core_ops.cpp:16,18,32).  Here a bad index or a too-short C.vv throws
@@ -34,9 +36,8 @@ namespace hip {
 // Device the shim runs on (default 0); call before the first kernel.
 void set_device(int device);
 
-// Forget the cached plan of this matrix (or of all, with nullptr).  Needed only
-// if ii / jj are changed in a way the pattern fingerprint cannot see; the
-// fingerprint covers every index, so by default never.
+// Drop everything kept between calls (plans, device panels).  Never needed for
+// correctness, the keys cover every byte of the operands; it frees device memory.
 void invalidate(const cooMat *S = nullptr);
 
 // Device time of the last sddmm / spmm kernel (without transfers), microseconds.

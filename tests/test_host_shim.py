@@ -96,3 +96,13 @@ def test_files_through_this_builds_readers_onto_the_gpu(name, k):
             want = subprocess.run([ref, "-k", str(k), os.path.join(io, stem + ".mtx")],
                                   capture_output=True, text=True, timeout=60)
             assert want.returncode == 0 and got == want.stdout.strip(), (stem, got, want.stdout)
+
+
+@pytest.mark.gpu
+def test_one_shot_host_calls_reuse_only_what_still_holds():
+    # spc3d_sddmm_host / spc3d_spmm_host called five times over one pattern as the reference's
+    # drivers call the kernels (miniapp/bench_both.cpp:202-203), then with every operand
+    # changed in the smallest way: plan and panels are reused by content, results against the oracle
+    r = subprocess.run([_binary("test_host_calls")], capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0 and "PASSED" in r.stdout, r.stdout[-3000:] + r.stderr[-3000:]
+    print("\n".join(ln for ln in r.stdout.splitlines() if ln.startswith("TIMING")))
