@@ -1761,9 +1761,9 @@ int spc3d_spmm_noalloc(spc3d_ctx *ctx, spc3d_plan *Ap, const spc3d_panel *X, spc
     // call first, so what an earlier call left in the array needs no clearing.  (The
     // blocks of a plan kept in column blocks use the array one after the other;
     // npartial_slots is the largest block's.)
-    std::vector<spc3d_plan *> self;
-    for (spc3d_plan *part : parts_of(Ap, self)) {
-        DevPlanView view = view_of(part);
+    const size_t nparts = Ap->blocks.empty() ? 1 : Ap->blocks.size(); // no container: no host heap either
+    for (size_t i = 0; i < nparts; ++i) {
+        DevPlanView view = view_of(Ap->blocks.empty() ? Ap : Ap->blocks[i]);
         view.partial = ctx->scratch;
         HIP_TRY(launch_spmm(Ap->dtype, view, X->dev, Y->dev, K, streams_of(ctx)));
     }
