@@ -77,6 +77,13 @@ __attribute__((target("sse4.2"))) void key_crc(const unsigned char *p, size_t by
 
 } // namespace
 
+BlockKey key_of_block_portable(const void *data, size_t bytes)
+{
+    BlockKey k;
+    key_plain(static_cast<const unsigned char *>(data), bytes, k);
+    return k;
+}
+
 BlockKey key_of_block(const void *data, size_t bytes)
 {
     BlockKey k;

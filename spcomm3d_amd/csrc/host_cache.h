@@ -31,6 +31,9 @@ struct BlockKey {
 constexpr size_t kKeyBlockBytes = (size_t)4 << 20;
 
 BlockKey key_of_block(const void *data, size_t bytes);
+// The form used on hosts without the CRC-32C instruction (multiply-xorshift chains in place
+// of the CRC streams); exposed so that it is tested on hosts that have the instruction.
+BlockKey key_of_block_portable(const void *data, size_t bytes);
 
 // Keys of every kKeyBlockBytes block of `data` (the last one may be short), computed on up
 // to `threads` threads (0: a default from the machine, at most 8).

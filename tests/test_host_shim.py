@@ -106,3 +106,9 @@ def test_one_shot_host_calls_reuse_only_what_still_holds():
     r = subprocess.run([_binary("test_host_calls")], capture_output=True, text=True, timeout=600)
     assert r.returncode == 0 and "PASSED" in r.stdout, r.stdout[-3000:] + r.stderr[-3000:]
     print("\n".join(ln for ln in r.stdout.splitlines() if ln.startswith("TIMING")))
+
+
+def test_content_keys_of_the_one_shot_host_calls():
+    # what decides whether a plan or a device panel is reused: every byte, the order of the
+    # words and the length go into a key; any number of threads gives the same keys
+    _run("test_keys")
