@@ -131,3 +131,44 @@ def test_reference_dist_wrappers_print_what_serial_loops_give():
 def test_reference_dist_wrappers_over_the_gpu_binding_print_the_same(k, m, n, nnz):
     # exact operands (multiples of 1/8 and 1/4): the sums are the same in any order
     assert strip_times(run_dist(DHIP, k, m, n, nnz)) == strip_times(run_dist(DREF, k, m, n, nnz))
+
+
+# The reference's two live bench programs whole (miniapp/bench_both.cpp, bench_spmm.cpp with all
+# of its src/, as its Makefile links them), one MPI rank, once as they are and once with the
+# binding in place of src/core_ops.cpp: reader, localizeIndices, the partitioner, the comm
+# set-up, ReMapIndices, then five calls of every dist_* variant per K.  They print the
+# statistics lines only (their checksum calls are commented out, bench_both.cpp:206,224,254),
+# so what is held is that the GPU build runs the whole program to its end and prints the
+# same lines; the numbers of the kernels are held by the other tests of this file.
+BENCH = {name: (os.path.join(ROOT, "oracle", "_ref", name + "_ref"),
+                os.path.join(ROOT, "oracle", "_ref", name + "_hip")) for name in ("benchBoth", "benchSpMM")}
+needs_bench = pytest.mark.skipif(not all(os.path.exists(p) for pair in BENCH.values() for p in pair),
+                                 reason="built only where the reference and an MPI are present")
+
+
+def write_bin(path, m, n, ii, jj, vv):
+    """uint32 rows, uint32 cols, uint64 nnz, then {uint32, uint32, float64} triplets
+    (tools/read_convert_mm.cpp:81-94)."""
+    rec = np.empty(len(ii), dtype=np.dtype([("r", "<u4"), ("c", "<u4"), ("v", "<f8")]))
+    rec["r"], rec["c"], rec["v"] = ii, jj, vv
+    with open(path, "wb") as f:
+        f.write(np.array([m, n], dtype="<u4").tobytes())
+        f.write(np.array([len(ii)], dtype="<u8").tobytes())
+        f.write(rec.tobytes())
+
+
+@pytest.mark.gpu
+@needs_bench
+@pytest.mark.parametrize("app", ["benchBoth", "benchSpMM"])
+def test_reference_bench_programs_run_whole_over_the_gpu_binding(app, tmp_path):
+    ref, hip = BENCH[app]
+    small = os.path.join(IO, "symmetric.bin")
+    rng = np.random.default_rng(11)
+    m, n, nnz = 40000, 30000, 300000
+    ii = np.where(rng.random(nnz) < 0.1, rng.integers(0, 4, nnz), rng.integers(0, m, nnz))  # hub rows
+    big = str(tmp_path / "generated.bin")
+    write_bin(big, m, n, ii, rng.integers(0, n, nnz), rng.uniform(-1, 1, nnz))
+    for path, ks in ((small, "8"), (big, "16,64")):
+        want = strip_times(run_dist(ref, "-k", ks, "-c", "1", path))
+        got = strip_times(run_dist(hip, "-k", ks, "-c", "1", path))
+        assert got == want and len(got) >= 20 * len(ks.split(","))
