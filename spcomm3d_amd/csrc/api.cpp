@@ -2069,32 +2069,48 @@ int host_panel(spc3d_ctx *ctx, HostCallCache *hc, int dtype, uint32_t m, uint32_
     std::vector<BlockKey> keys;
     if (input)
         keys_of(host, bytes, keys);
-    CachedHostPanel *hit = nullptr;
-    size_t best = 0; // number of blocks that would stay
+    // Among the kept panels of this shape that this call does not use yet: the one that
+    // holds most of this operand already; failing that, one that mirrors nothing (an
+    // output's); failing that a new one while there is room, so that a second operand of
+    // the same shape (A and B of a square pattern, two panels used in turn) does not push
+    // the first one out; only then the one unused for longest.
+    CachedHostPanel *hit = nullptr, *blank = nullptr, *oldest = nullptr;
+    size_t best = 0; // blocks that would stay
     for (CachedHostPanel &e : hc->panels) {
         if (e.last_use == stamp || e.panel->dtype != dtype || e.panel->m != m || e.panel->n != n)
             continue;
-        if (!input && !e.keys.empty())
+        if (e.keys.empty()) {
+            if (!blank || e.host == host)
+                blank = &e;
+            continue;
+        }
+        if (!input)
             continue; // an output does not take over a panel that mirrors an input
         size_t same = 0;
-        if (input && e.keys.size() == keys.size())
+        if (e.keys.size() == keys.size())
             for (size_t b = 0; b < keys.size(); ++b)
                 same += e.keys[b] == keys[b];
-        if (!hit || same > best || (same == best && e.host == host)) {
+        if (same > best || (same == best && same > 0 && e.host == host)) {
             hit = &e;
             best = same;
         }
+        if (!oldest || e.last_use < oldest->last_use)
+            oldest = &e;
     }
+    if (!hit)
+        hit = blank;
+    if (!hit && hc->panels.size() >= HostCallCache::kMaxPanels && input)
+        hit = oldest; // same shape, other content: overwritten in full below
     if (!hit) {
         if (hc->panels.size() >= HostCallCache::kMaxPanels) {
-            size_t oldest = hc->panels.size();
+            size_t lru = hc->panels.size();
             for (size_t i = 0; i < hc->panels.size(); ++i)
                 if (hc->panels[i].last_use != stamp &&
-                    (oldest == hc->panels.size() || hc->panels[i].last_use < hc->panels[oldest].last_use))
-                    oldest = i;
-            if (oldest < hc->panels.size()) {
-                (void)spc3d_panel_destroy(hc->panels[oldest].panel);
-                hc->panels.erase(hc->panels.begin() + (std::ptrdiff_t)oldest);
+                    (lru == hc->panels.size() || hc->panels[i].last_use < hc->panels[lru].last_use))
+                    lru = i;
+            if (lru < hc->panels.size()) {
+                (void)spc3d_panel_destroy(hc->panels[lru].panel);
+                hc->panels.erase(hc->panels.begin() + (std::ptrdiff_t)lru);
             }
         }
         CachedHostPanel e;

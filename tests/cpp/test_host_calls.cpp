@@ -139,6 +139,24 @@ int main(int argc, char **argv)
     CHECK(reused == 1 && kept == 2 * panel_bytes);
     CHECK(sddmm_matches(p, c));
 
+    // ---- two panels used in turn for one operand: both stay ----------------------------
+    {
+        std::vector<double> other(p.A.size());
+        for (auto &x : other)
+            x = (double)(g() % 2001) / 1000.0 - 1.0;
+        p.A.swap(other);
+        sddmm();
+        CHECK(reused == 1 && kept == panel_bytes && sent == val_bytes + panel_bytes); // B stays, the new A goes up
+        CHECK(sddmm_matches(p, c));
+        p.A.swap(other);
+        sddmm();
+        CHECK(kept == 2 * panel_bytes && sddmm_matches(p, c)); // the first A was not pushed out
+        p.A.swap(other);
+        sddmm();
+        CHECK(kept == 2 * panel_bytes && sddmm_matches(p, c)); // nor the second
+        p.A.swap(other);
+    }
+
     // ---- values change: always sent ---------------------------------------------------
     p.vv[p.nnz / 2] = 7.25;
     sddmm();
