@@ -357,9 +357,14 @@ SPC3D_API int spc3d_rows_unpack_sum(spc3d_ctx *ctx, spc3d_panel *P, const spc3d_
  *     when the plan was made (four CRC-32C streams, a sum and a fold over every word),
  *     nnz, sizes, type and k agree, and a sample of the indices compares equal; a new
  *     pattern is planned, and validated, as before;
- *   - up to four device panels with the keys of the host memory they mirror: blocks of
- *     A, B, X whose key is unchanged are not sent again, changed blocks are; Y is sent
- *     and fetched in full on every call, the values svv / avv are sent on every call;
+ *   - up to six device panels with the keys of the host memory they equal: blocks of
+ *     A, B, X whose key is unchanged are not sent again, changed blocks are.  Y, which the
+ *     kernel changes, is fetched into the caller's memory in pieces that are keyed while
+ *     the next piece is on its way, so the next call sends only what the caller touched
+ *     since (a caller that rewrites most of Y between calls is noticed, and Y then goes
+ *     up unread for a stretch of calls that doubles, up to 16, each time that proves
+ *     right); Y goes up on a thread of its own while X is read for its keys.  The values
+ *     svv / avv are sent on every call;
  *   - the result vector of SDDMM.
  * Reading an unchanged operand for its keys (several threads) takes about half the time
  * of sending it.  The cache holds device memory until spc3d_host_cache_clear or

@@ -8,9 +8,12 @@
 
 #include <cstdio>
 #include <cstdlib>
+#include <atomic>
 #include <cstring>
+#include <functional>
 #include <memory>
 #include <mutex>
+#include <thread>
 #include <new>
 #include <string>
 #include <vector>
@@ -202,19 +205,28 @@ struct CachedHostPlan {
     uint64_t last_use = 0;
 };
 
-// A device panel and the keys of the host memory it was filled from, block by block.
-// No keys: the panel's content is not known to equal any host memory (an output).
+// A device panel and the keys of the host memory it equals, block by block (the memory it
+// was filled from, or the memory its content was fetched into).  No keys: the panel's
+// content is not known to equal any host memory.
 struct CachedHostPanel {
     spc3d_panel *panel = nullptr;
     std::vector<BlockKey> keys;
     const void *host = nullptr; // where it came from last: a preference among equals, never a proof
     uint64_t last_use = 0;
+    // An operand the kernel changes (SpMM's Y): its result is fetched into the caller's
+    // memory, so the two are equal again when the call returns, and the keys of what was
+    // fetched let the next call leave in place what the caller did not touch.  When the
+    // caller rewrites most of it between calls anyway, reading it for keys first is wasted:
+    // the next `skip` calls send it unread, and each time that turns out right the stretch
+    // doubles (to at most 16 calls).
+    bool output = false;
+    uint32_t skip = 0, backoff = 0;
 };
 
 struct HostCallCache {
-    static constexpr size_t kMaxPlans = 4, kMaxPanels = 4, kSamples = 64;
+    static constexpr size_t kMaxPlans = 4, kMaxPanels = 6, kSamples = 64;
     std::vector<CachedHostPlan> plans;
-    std::vector<CachedHostPanel> panels;
+    std::vector<std::unique_ptr<CachedHostPanel>> panels; // the objects stay where they are
     spc3d_vals *c = nullptr;
     uint64_t clock = 0;
     // what the last call did, for spc3d_host_call_stats
@@ -2054,107 +2066,224 @@ int host_plan(spc3d_ctx *ctx, HostCallCache *hc, int dtype, uint32_t nrows, uint
     return SPC3D_OK;
 }
 
-// A device panel of this shape holding what `host` holds.  input = true: the blocks whose
-// keys are those of the cached panel's source stay as they are, the others are sent.
-// input = false: a panel of this shape whose content is about to be overwritten from
-// `host` in full (an operand the kernel changes, so the device copy equals no host memory
-// afterwards).  `stamp` marks the panels this call already uses.
-int host_panel(spc3d_ctx *ctx, HostCallCache *hc, int dtype, uint32_t m, uint32_t n,
-               const void *host, bool input, uint64_t stamp, spc3d_panel **out)
+// A kept device panel of this shape for the operand at `host`, or a new one.  keys: those
+// of the operand's blocks, or empty when they were not computed.  Among the panels that this
+// call does not use yet: the one that holds most of the operand already; failing that, for
+// an output, the one this memory's last result was fetched from; failing that one that
+// mirrors nothing;
+// failing that a new one while there is room, so that a second operand of the same shape
+// (A and B of a square pattern, two panels used in turn) does not push the first one out;
+// only then the one unused for longest.
+int pick_panel(spc3d_ctx *ctx, HostCallCache *hc, int dtype, uint32_t m, uint32_t n,
+               const std::vector<BlockKey> &keys, bool output, const void *host, uint64_t stamp,
+               CachedHostPanel **out)
 {
     *out = nullptr;
-    const size_t bytes = (size_t)m * n * elem_size(dtype);
-    if (bytes && !host)
-        return fail(SPC3D_ERR_INVALID_ARG, "a dense operand is NULL");
-    std::vector<BlockKey> keys;
-    if (input)
-        keys_of(host, bytes, keys);
-    // Among the kept panels of this shape that this call does not use yet: the one that
-    // holds most of this operand already; failing that, one that mirrors nothing (an
-    // output's); failing that a new one while there is room, so that a second operand of
-    // the same shape (A and B of a square pattern, two panels used in turn) does not push
-    // the first one out; only then the one unused for longest.
-    CachedHostPanel *hit = nullptr, *blank = nullptr, *oldest = nullptr;
+    CachedHostPanel *hit = nullptr, *was_output = nullptr, *other_output = nullptr, *blank = nullptr,
+                    *oldest = nullptr;
     size_t best = 0; // blocks that would stay
-    for (CachedHostPanel &e : hc->panels) {
+    for (auto &up : hc->panels) {
+        CachedHostPanel &e = *up;
         if (e.last_use == stamp || e.panel->dtype != dtype || e.panel->m != m || e.panel->n != n)
             continue;
+        if (output && e.output) {
+            if (e.host == host)
+                was_output = &e; // this memory's own result panel
+            else if (!other_output || e.last_use < other_output->last_use)
+                other_output = &e; // another result, which a later call may want as an input
+        }
         if (e.keys.empty()) {
             if (!blank || e.host == host)
                 blank = &e;
             continue;
         }
-        if (!input)
-            continue; // an output does not take over a panel that mirrors an input
         size_t same = 0;
-        if (e.keys.size() == keys.size())
+        if (!keys.empty() && e.keys.size() == keys.size())
             for (size_t b = 0; b < keys.size(); ++b)
                 same += e.keys[b] == keys[b];
         if (same > best || (same == best && same > 0 && e.host == host)) {
             hit = &e;
             best = same;
         }
-        if (!oldest || e.last_use < oldest->last_use)
+        if (!e.output && (!oldest || e.last_use < oldest->last_use))
             oldest = &e;
     }
     if (!hit)
+        hit = was_output;
+    if (!hit)
         hit = blank;
-    if (!hit && hc->panels.size() >= HostCallCache::kMaxPanels && input)
-        hit = oldest; // same shape, other content: overwritten in full below
+    if (!hit && hc->panels.size() >= HostCallCache::kMaxPanels)
+        hit = output ? other_output : oldest; // same shape, other content: sent in full
     if (!hit) {
         if (hc->panels.size() >= HostCallCache::kMaxPanels) {
             size_t lru = hc->panels.size();
             for (size_t i = 0; i < hc->panels.size(); ++i)
-                if (hc->panels[i].last_use != stamp &&
-                    (lru == hc->panels.size() || hc->panels[i].last_use < hc->panels[lru].last_use))
+                if (hc->panels[i]->last_use != stamp &&
+                    (lru == hc->panels.size() || hc->panels[i]->last_use < hc->panels[lru]->last_use))
                     lru = i;
             if (lru < hc->panels.size()) {
-                (void)spc3d_panel_destroy(hc->panels[lru].panel);
+                (void)spc3d_panel_destroy(hc->panels[lru]->panel);
                 hc->panels.erase(hc->panels.begin() + (std::ptrdiff_t)lru);
             }
         }
-        CachedHostPanel e;
-        int rc = spc3d_panel_create(ctx, dtype, m, n, &e.panel);
+        std::unique_ptr<CachedHostPanel> e(new (std::nothrow) CachedHostPanel());
+        if (!e)
+            return fail(SPC3D_ERR_ALLOC, "host allocation failed");
+        int rc = spc3d_panel_create(ctx, dtype, m, n, &e->panel);
         if (rc)
             return rc;
         hc->panels.push_back(std::move(e));
-        hit = &hc->panels.back();
+        hit = hc->panels.back().get();
     }
-    // send the blocks that differ, neighbouring ones in one copy
-    const bool known = input && hit->keys.size() == keys.size();
+    hit->last_use = stamp;
+    *out = hit;
+    return SPC3D_OK;
+}
+
+// What one operand's transfer did; merged into the cache's figures by the calling thread.
+struct Moved {
+    uint64_t sent = 0, kept = 0;
+    int rc = SPC3D_OK;
+    std::string err; // the failing thread's message (the error text is per thread)
+};
+
+// Brings `slot`'s panel to the content of `host`.  keys (of host's blocks): the blocks whose
+// key is the slot's stay as they are, the others are sent, neighbouring ones in one copy;
+// no keys: everything is sent and the slot mirrors nothing known afterwards.  May run on a
+// thread of its own (it touches this slot only).
+void send_panel(spc3d_ctx *ctx, CachedHostPanel *slot, const void *host,
+                std::vector<BlockKey> &keys, Moved &mv)
+{
+    const spc3d_panel *P = slot->panel;
+    const size_t bytes = (size_t)P->m * P->n * elem_size(P->dtype);
+    const bool known = !keys.empty() && slot->keys.size() == keys.size();
     const size_t nblocks = (bytes + kKeyBlockBytes - 1) / kKeyBlockBytes;
     const char *src = static_cast<const char *>(host);
-    char *dst = static_cast<char *>(hit->panel->dev);
-    for (size_t b = 0; b < nblocks;) {
-        if (known && hit->keys[b] == keys[b]) {
-            hc->bytes_kept += std::min(kKeyBlockBytes, bytes - b * kKeyBlockBytes);
+    char *dst = static_cast<char *>(P->dev);
+    hipError_t err = hipSetDevice(ctx->device);
+    for (size_t b = 0; err == hipSuccess && b < nblocks;) {
+        if (known && slot->keys[b] == keys[b]) {
+            mv.kept += std::min(kKeyBlockBytes, bytes - b * kKeyBlockBytes);
             ++b;
             continue;
         }
         size_t e = b + 1;
-        while (e < nblocks && !(known && hit->keys[e] == keys[e]))
+        while (e < nblocks && !(known && slot->keys[e] == keys[e]))
             ++e;
         const size_t off = b * kKeyBlockBytes, len = std::min(bytes, e * kKeyBlockBytes) - off;
-        hipError_t err = hipMemcpyAsync(dst + off, src + off, len, hipMemcpyHostToDevice, ctx->stream);
-        if (err != hipSuccess) {
-            hit->keys.clear(); // the panel's content is no longer known
-            return fail_hip(err, "upload of a dense operand");
-        }
-        hc->bytes_sent += len;
+        err = hipMemcpyAsync(dst + off, src + off, len, hipMemcpyHostToDevice, ctx->stream);
+        mv.sent += len;
         b = e;
     }
-    hipError_t err = hipStreamSynchronize(ctx->stream);
+    if (err == hipSuccess)
+        err = hipStreamSynchronize(ctx->stream);
     if (err != hipSuccess) {
-        hit->keys.clear();
-        return fail_hip(err, "upload of a dense operand");
+        slot->keys.clear(); // the panel's content is no longer known
+        mv.rc = fail_hip(err, "upload of a dense operand");
+        mv.err = g_err;
+        return;
     }
-    if (input)
-        hit->keys.swap(keys);
-    else
-        hit->keys.clear();
-    hit->host = host;
-    hit->last_use = stamp;
-    *out = hit->panel;
+    slot->keys.swap(keys); // empty when none were given
+    slot->host = host;
+}
+
+// An input operand: keys of every block (threads), the kept panel that matches best, the
+// changed blocks sent.
+int host_input(spc3d_ctx *ctx, HostCallCache *hc, int dtype, uint32_t m, uint32_t n,
+               const void *host, uint64_t stamp, spc3d_panel **out)
+{
+    *out = nullptr;
+    const size_t bytes = (size_t)m * n * elem_size(dtype);
+    if (bytes && !host)
+        return fail(SPC3D_ERR_INVALID_ARG, "a dense operand is NULL");
+    std::vector<BlockKey> keys;
+    keys_of(host, bytes, keys);
+    CachedHostPanel *slot = nullptr;
+    int rc = pick_panel(ctx, hc, dtype, m, n, keys, false, host, stamp, &slot);
+    if (rc)
+        return rc;
+    slot->output = false;
+    Moved mv;
+    send_panel(ctx, slot, host, keys, mv);
+    hc->bytes_sent += mv.sent;
+    hc->bytes_kept += mv.kept;
+    if (mv.rc)
+        return fail(mv.rc, mv.err);
+    *out = slot->panel;
+    return SPC3D_OK;
+}
+
+// The operand the kernel changes, before the call: what the caller left untouched since the
+// last result was fetched into this memory stays on the device (see CachedHostPanel).
+// Runs beside the inputs' transfers, on a thread of its own.
+void send_output_operand(spc3d_ctx *ctx, CachedHostPanel *slot, const void *host, Moved &mv)
+{
+    const size_t bytes = (size_t)slot->panel->m * slot->panel->n * elem_size(slot->panel->dtype);
+    std::vector<BlockKey> keys;
+    const bool read_first = !slot->keys.empty() && slot->skip == 0;
+    if (read_first)
+        keys_of(host, bytes, keys, 4);
+    else if (slot->skip)
+        --slot->skip;
+    send_panel(ctx, slot, host, keys, mv);
+    if (mv.rc || !read_first)
+        return;
+    if (mv.sent > mv.kept) { // mostly rewritten: do not read it first for a while
+        slot->backoff = std::min<uint32_t>(16, slot->backoff ? 2 * slot->backoff : 1);
+        slot->skip = slot->backoff;
+    } else {
+        slot->backoff = 0;
+    }
+}
+
+// The changed operand, after the call: fetched into the caller's memory in pieces, each
+// piece keyed by worker threads while the next one is on its way.
+int fetch_output_operand(spc3d_ctx *ctx, CachedHostPanel *slot, void *host)
+{
+    const spc3d_panel *P = slot->panel;
+    const size_t bytes = (size_t)P->m * P->n * elem_size(P->dtype);
+    const size_t nblocks = (bytes + kKeyBlockBytes - 1) / kKeyBlockBytes;
+    std::vector<BlockKey> keys(nblocks);
+    std::atomic<size_t> ready{0}, next{0};
+    char *dst = static_cast<char *>(host);
+    auto work = [&]() {
+        for (;;) {
+            const size_t b = next.fetch_add(1, std::memory_order_relaxed);
+            if (b >= nblocks)
+                return;
+            while (ready.load(std::memory_order_acquire) <= b)
+                std::this_thread::yield();
+            const size_t off = b * kKeyBlockBytes;
+            keys[b] = key_of_block(dst + off, std::min(kKeyBlockBytes, bytes - off));
+        }
+    };
+    const unsigned hw = std::thread::hardware_concurrency();
+    const unsigned nthreads = (unsigned)std::min<size_t>(std::min(4u, hw ? hw : 1u), nblocks);
+    std::vector<std::thread> pool;
+    for (unsigned t = 0; t < nthreads; ++t)
+        pool.emplace_back(work);
+    constexpr size_t kPiece = 4; // blocks per copy: 16 MiB
+    hipError_t err = hipSuccess;
+    const char *src = static_cast<const char *>(P->dev);
+    for (size_t b = 0; b < nblocks && err == hipSuccess; b += kPiece) {
+        const size_t off = b * kKeyBlockBytes;
+        const size_t len = std::min(bytes, (b + kPiece) * kKeyBlockBytes) - off;
+        err = hipMemcpyAsync(dst + off, src + off, len, hipMemcpyDeviceToHost, ctx->stream);
+        if (err == hipSuccess)
+            err = hipStreamSynchronize(ctx->stream);
+        if (err == hipSuccess)
+            ready.store(std::min(nblocks, b + kPiece), std::memory_order_release);
+    }
+    ready.store(nblocks, std::memory_order_release); // lets the workers run out also after a failure
+    for (std::thread &t : pool)
+        t.join();
+    if (err != hipSuccess) {
+        slot->keys.clear();
+        return fail_hip(err, "download of a dense operand");
+    }
+    slot->keys.swap(keys);
+    slot->host = host;
+    slot->output = true;
     return SPC3D_OK;
 }
 
@@ -2185,8 +2314,8 @@ int spc3d_host_cache_clear(spc3d_ctx *ctx)
     (void)hipSetDevice(ctx->device);
     for (CachedHostPlan &e : hc->plans)
         (void)spc3d_plan_destroy(e.plan);
-    for (CachedHostPanel &e : hc->panels)
-        (void)spc3d_panel_destroy(e.panel);
+    for (auto &e : hc->panels)
+        (void)spc3d_panel_destroy(e->panel);
     if (hc->c)
         (void)spc3d_vals_destroy(hc->c);
     delete hc;
@@ -2255,8 +2384,8 @@ int spc3d_sddmm_host(spc3d_ctx *ctx, int dtype, uint32_t m, uint32_t n, uint32_t
     spc3d_panel *a = nullptr, *b = nullptr;
     rc = host_plan(ctx, hc, dtype, m, n, k, nnz, ii, jj, svv, &S);
     const uint64_t stamp = hc->clock; // host_plan advanced it: unique to this call
-    if (!rc) rc = host_panel(ctx, hc, dtype, m, k, A, true, stamp, &a);
-    if (!rc) rc = host_panel(ctx, hc, dtype, n, k, B, true, stamp, &b);
+    if (!rc) rc = host_input(ctx, hc, dtype, m, k, A, stamp, &a);
+    if (!rc) rc = host_input(ctx, hc, dtype, n, k, B, stamp, &b);
     if (!rc && (!hc->c || hc->c->dtype != dtype || hc->c->n != nnz)) {
         if (hc->c)
             (void)spc3d_vals_destroy(hc->c);
@@ -2310,18 +2439,44 @@ int spc3d_spmm_host(spc3d_ctx *ctx, int dtype, uint32_t ncols, uint32_t nrows, u
     int rc = host_call_begin(ctx, &hc);
     if (rc)
         return rc;
+    const size_t ybytes = (size_t)nrows * k * elem_size(dtype);
+    if (ybytes && !Y)
+        return fail(SPC3D_ERR_INVALID_ARG, "Y is NULL");
     spc3d_plan *S = nullptr;
-    spc3d_panel *x = nullptr, *y = nullptr;
+    spc3d_panel *x = nullptr;
     rc = host_plan(ctx, hc, dtype, nrows, ncols, k, nnz, ii, jj, avv, &S);
+    if (rc)
+        return rc;
     const uint64_t stamp = hc->clock;
-    if (!rc) rc = host_panel(ctx, hc, dtype, ncols, k, X, true, stamp, &x);
-    // Y comes back changed, so its device copy never equals the caller's memory when the
-    // next call starts: it is sent in full every time
-    if (!rc) rc = host_panel(ctx, hc, dtype, nrows, k, Y, false, stamp, &y);
+    // Y first: its panel is chosen here, then brought up to date on a thread of its own
+    // while this one reads X for its keys and sends what changed of it.
+    CachedHostPanel *yslot = nullptr;
+    {
+        std::vector<BlockKey> none;
+        rc = pick_panel(ctx, hc, dtype, nrows, k, none, true, Y, stamp, &yslot);
+        if (rc)
+            return rc;
+        if (!yslot->output || yslot->host != Y) { // another operand's panel, or other memory:
+            yslot->keys.clear();                  // nothing of it is known to be Y's
+            yslot->skip = yslot->backoff = 0;
+        }
+        yslot->output = true;
+    }
+    Moved ymv;
+    std::thread ythread(send_output_operand, ctx, yslot, (const void *)Y, std::ref(ymv));
+    rc = host_input(ctx, hc, dtype, ncols, k, X, stamp, &x);
+    ythread.join();
+    hc->bytes_sent += ymv.sent;
+    hc->bytes_kept += ymv.kept;
+    if (!rc && ymv.rc)
+        rc = fail(ymv.rc, ymv.err);
     if (!rc) rc = spc3d_timer_mark(ctx, SPC3D_TIMER_HOST_CALL_BEGIN);
-    if (!rc) rc = spc3d_spmm(ctx, S, x, y);
+    if (!rc) rc = spc3d_spmm(ctx, S, x, yslot->panel);
     if (!rc) rc = spc3d_timer_mark(ctx, SPC3D_TIMER_HOST_CALL_END);
-    if (!rc) rc = spc3d_panel_download(y, Y);
+    if (!rc)
+        rc = fetch_output_operand(ctx, yslot, Y);
+    else
+        yslot->keys.clear(); // whatever the panel holds now, it is not known to be Y
     return rc;
 }
 

@@ -214,30 +214,71 @@ int main(int argc, char **argv)
         }
     }
 
-    // ---- SpMM: X kept, Y accumulates over the calls ---------------------------------------
+    // ---- SpMM: X kept; Y accumulates over the calls and goes up again only where the caller
+    //      touched it since the last result came back ------------------------------------------
     {
         std::vector<double> y_ref = p.Y;
         double t_first = 0, t_later = 0;
-        for (int rep = 0; rep < 5; ++rep) {
+        auto spmm = [&]() {
             const auto t0 = clk::now();
             OK(spc3d_spmm_host(ctx, SPC3D_F64, p.n, p.m, p.k, p.B.data(), p.nnz, p.ii.data(),
                                p.jj.data(), p.vv.data(), p.Y.data()));
-            (rep ? t_later : t_first) += ms_since(t0) / (rep ? 4 : 1);
+            const double ms = ms_since(t0);
             OK(spc3d_host_call_stats(ctx, &sent, &kept, &reused));
-            CHECK(reused == 1);                    // the SDDMM calls planned this pattern at this k
-            CHECK(kept == panel_bytes);            // X is SDDMM's B, already there
-            CHECK(sent == val_bytes + panel_bytes); // the values and Y
             CHECK(oracle_spmm_f64(p.n, p.m, p.k, p.B.data(), p.nnz, p.ii.data(), p.jj.data(),
                                   p.vv.data(), y_ref.data()) == 0);
+            return ms;
+        };
+        auto y_matches = [&]() {
+            double worst = 0;
+            for (size_t i = 0; i < y_ref.size(); ++i)
+                worst = std::fmax(worst, std::fabs(p.Y[i] - y_ref[i]) / std::fmax(std::fabs(y_ref[i]), 100.0));
+            return worst < 1e-12;
+        };
+        for (int rep = 0; rep < 5; ++rep) {
+            (rep ? t_later : t_first) += spmm() / (rep ? 4 : 1);
+            CHECK(reused == 1); // the SDDMM calls planned this pattern at this k
+            if (rep == 0)       // X is SDDMM's B, already there; Y goes up whole the first time
+                CHECK(kept == panel_bytes && sent == val_bytes + panel_bytes);
+            else                // then the result that came back is what the device holds
+                CHECK(kept == 2 * panel_bytes && sent == val_bytes);
         }
-        double worst = 0;
-        for (size_t i = 0; i < y_ref.size(); ++i)
-            worst = std::fmax(worst, std::fabs(p.Y[i] - y_ref[i]) / std::fmax(std::fabs(y_ref[i]), 100.0));
-        CHECK(worst < 1e-12);
+        CHECK(y_matches());
         std::printf("TIMING spmm_host: first call %.1f ms, calls 2..5 %.1f ms each\n", t_first, t_later);
-        // SDDMM still finds A and B after SpMM used a panel for Y
+        // one element of Y changes on the host: its block goes up, the rest stays
+        p.Y[p.Y.size() / 2] += 3.0;
+        y_ref[p.Y.size() / 2] += 3.0;
+        spmm();
+        CHECK(sent > val_bytes && sent <= val_bytes + ((uint64_t)4 << 20) && y_matches());
+        // the caller rewrites all of Y before every call: the first time it is read in vain,
+        // then it goes up unread for a stretch, and the results are right throughout
+        for (int rep = 0; rep < 5; ++rep) {
+            for (size_t i = 0; i < p.Y.size(); ++i)
+                p.Y[i] = y_ref[i] = 0.5 + (double)((i + rep) % 7);
+            spmm();
+            CHECK(sent == val_bytes + panel_bytes && kept == panel_bytes && y_matches());
+        }
+        // and a Y left alone again is found again (after the stretch has run out)
+        for (int rep = 0; rep < 4; ++rep)
+            spmm();
+        CHECK(kept == 2 * panel_bytes && sent == val_bytes && y_matches());
+        // the result of one call as the dense operand of the next: found by content
+        {
+            std::vector<double> x2 = p.Y, y2((size_t)p.m * p.k, 0.0), y2_ref = y2;
+            OK(spc3d_spmm_host(ctx, SPC3D_F64, p.n, p.m, p.k, x2.data(), p.nnz, p.ii.data(),
+                               p.jj.data(), p.vv.data(), y2.data()));
+            OK(spc3d_host_call_stats(ctx, &sent, &kept, &reused));
+            CHECK(kept >= panel_bytes); // x2 is a copy of the Y that was just fetched
+            CHECK(oracle_spmm_f64(p.n, p.m, p.k, x2.data(), p.nnz, p.ii.data(), p.jj.data(),
+                                  p.vv.data(), y2_ref.data()) == 0);
+            double worst = 0;
+            for (size_t i = 0; i < y2.size(); ++i)
+                worst = std::fmax(worst, std::fabs(y2[i] - y2_ref[i]) / std::fmax(std::fabs(y2_ref[i]), 1e4));
+            CHECK(worst < 1e-12);
+        }
+        // SDDMM still finds A and B after SpMM used panels for Y
         sddmm();
-        CHECK(reused == 1 && kept == 2 * panel_bytes && sddmm_matches(p, c));
+        CHECK(reused == 1 && sddmm_matches(p, c));
     }
 
     // ---- dropping what is kept changes nothing but the work ------------------------------
