@@ -112,3 +112,11 @@ def test_content_keys_of_the_one_shot_host_calls():
     # what decides whether a plan or a device panel is reused: every byte, the order of the
     # words and the length go into a key; any number of threads gives the same keys
     _run("test_keys")
+
+
+@pytest.mark.gpu
+def test_shim_without_the_cache_of_the_one_shot_calls():
+    # SPC3D_HOST_CACHE=0: plan, upload, run, download, free on every call; same results
+    env = dict(os.environ, SPC3D_HOST_CACHE="0")
+    r = subprocess.run([_binary("test_shim_f64")], capture_output=True, text=True, timeout=300, env=env)
+    assert r.returncode == 0 and "PASSED" in r.stdout, r.stdout[-3000:] + r.stderr[-3000:]

@@ -366,6 +366,32 @@ def test_one_shot_host_entry_points(ctx, dtype):
     check_spmm(B, ii, jj, vv, Y0, Y)
 
 
+def test_one_shot_host_calls_at_the_edges(ctx):
+    """Repeated one-shot calls that alternate types, widths and shapes over one context:
+    whatever the context keeps between calls, every result is the oracle's.  Also an empty
+    pattern, a single entry, and a dense operand of one column."""
+    rng = np.random.default_rng(5)
+    for rep in range(2):
+        for dtype, k, m, n, nnz in ((np.float64, 1, 9, 7, 20), (np.float32, 3, 9, 7, 20),
+                                    (np.float64, 64, 300, 200, 5000), (np.float32, 64, 300, 200, 5000),
+                                    (np.float64, 33, 300, 200, 1), (np.float32, 50, 1, 1, 1)):
+            ii, jj, vv, A, B, Y0 = rand_case(40 + rep, m, n, k, nnz, dtype)
+            check_sddmm(A, B, ii, jj, vv, ctx.sddmm_host(A, B, ii, jj, vv))
+            Y = Y0.copy()
+            ctx.spmm_host(B, ii, jj, vv, Y)
+            check_spmm(B, ii, jj, vv, Y0, Y)
+            Y1 = Y.copy()
+            ctx.spmm_host(B, ii, jj, vv, Y)  # accumulates over calls (core_ops.cpp:32)
+            check_spmm(B, ii, jj, vv, Y1, Y)
+    # an empty pattern: nothing is written
+    A, B = rng.uniform(-1, 1, (5, 8)), rng.uniform(-1, 1, (6, 8))
+    none = np.zeros(0, dtype=np.uint32)
+    assert ctx.sddmm_host(A, B, none, none, np.zeros(0)).size == 0
+    Y = np.ones((5, 8))
+    ctx.spmm_host(B, none, none, np.zeros(0), Y)
+    assert np.array_equal(Y, np.ones((5, 8)))
+
+
 def test_values_can_be_replaced_from_host_and_device(ctx):
     ii, jj, vv, A, B, _ = rand_case(32, 40, 40, 32, 1500, np.float64)
     S = ctx.plan(40, 40, ii, jj, dtype=np.float64)  # pattern only
