@@ -17,7 +17,9 @@ oracle (a serial restatement of the reference's loops), timed on one host core
 on the same workload.  `fused_step` is the same step through the one-pass entry
 point spc3d_sddmm_spmm (an extension without counterpart in the reference); it is
 reported beside `value`, which always comes from the two separate calls.
-`row_copies` times the pack and sum-unpack copies of a sparse exchange over the
+`roofline.device_copy_gbs` is a plain device copy of one panel timed in the same run
+(read + write), with the kernel's strict-model rate and its measured traffic as fractions
+of it.  `row_copies` times the pack and sum-unpack copies of a sparse exchange over the
 touched rows of Y (algorithmic bytes: rows read + buffer written; buffer read +
 rows read and written).  `also` holds the other real type, the same workload
 handed over in shuffled COO order (the reference never sorts its entries) in
@@ -169,6 +171,17 @@ def run_gpu(w, dtype, steps, warmup, seg_max=None, max_timed=1300, copies=0, ven
             v["frac"] = v["gbs"] / roofline.HBM_PEAK_GBS
         rmap.close()
         dbuf.close()
+        # A plain device copy of one panel (read + write), the rate this machine moves bytes
+        # at when nothing is gathered: the second yardstick beside the 8 TB/s peak.
+        dT = ctx.panel(w.nrows, w.k, dtype)
+        for _ in range(warmup):
+            dT.copy_from(dA)
+        ctx.mark(4003)
+        for _ in range(steps):
+            dT.copy_from(dA)
+        ctx.mark(4004)
+        copy_gbs = 2 * w.nrows * w.k * wbytes / (ctx.elapsed_ms(4003, 4004) / steps) / 1e6
+        dT.close()
         # The vendor's library on the same resident operands, last (it overwrites Y).
         vendor_out = None
         if vendor and w.order == "sorted":
@@ -193,6 +206,7 @@ def run_gpu(w, dtype, steps, warmup, seg_max=None, max_timed=1300, copies=0, ven
                          "gflops": 2 * fl / (fused_wall / steps) / 1e9, "strict_bytes": int(fb),
                          "strict_frac": fb / (fused_wall / steps) / 1e9 / roofline.HBM_PEAK_GBS}
     out["row_copies"] = rows
+    out["device_copy_gbs"] = copy_gbs
     if vendor_out:
         sd_ms, sp_ms = float(sd.mean()), float(sp.mean())
         vendor_out["sddmm_ratio"] = vendor_out["sddmm_us"] / (sd_ms * 1e3)
@@ -434,6 +448,10 @@ def main():
                      "traffic": traffic, "traffic_level": TRAFFIC_LEVEL,
                      "traffic_source": os.path.relpath(TRAFFIC_PROFILE, ROOT),
                      "traffic_gbs": None if traffic is None else traffic / kd["ms_avg"] / 1e6,
+                     "device_copy_gbs": main_r["device_copy_gbs"],
+                     "frac_of_device_copy": kd["strict_gbs"] / main_r["device_copy_gbs"],
+                     "traffic_frac_of_device_copy": None if traffic is None else
+                     traffic / kd["ms_avg"] / 1e6 / main_r["device_copy_gbs"],
                      "bytes_per_launch": kd["strict_bytes"],
                      "ms_per_launch": kd["ms_avg"], "model": "strict (each operand once)"},
         "cpu_baseline": cpu,
