@@ -16,6 +16,7 @@
 #include <thread>
 #include <new>
 #include <string>
+#include <system_error>
 #include <vector>
 
 #include "host_cache.h"
@@ -2260,8 +2261,12 @@ int fetch_output_operand(spc3d_ctx *ctx, CachedHostPanel *slot, void *host)
     const unsigned hw = std::thread::hardware_concurrency();
     const unsigned nthreads = (unsigned)std::min<size_t>(std::min(4u, hw ? hw : 1u), nblocks);
     std::vector<std::thread> pool;
-    for (unsigned t = 0; t < nthreads; ++t)
-        pool.emplace_back(work);
+    try {
+        for (unsigned t = 0; t < nthreads; ++t)
+            pool.emplace_back(work);
+    } catch (const std::system_error &) {
+        // fewer workers, or none: what is left over is keyed by this thread at the end
+    }
     constexpr size_t kPiece = 4; // blocks per copy: 16 MiB
     hipError_t err = hipSuccess;
     const char *src = static_cast<const char *>(P->dev);
@@ -2275,6 +2280,7 @@ int fetch_output_operand(spc3d_ctx *ctx, CachedHostPanel *slot, void *host)
             ready.store(std::min(nblocks, b + kPiece), std::memory_order_release);
     }
     ready.store(nblocks, std::memory_order_release); // lets the workers run out also after a failure
+    work(); // whatever no worker has taken
     for (std::thread &t : pool)
         t.join();
     if (err != hipSuccess) {
@@ -2463,9 +2469,15 @@ int spc3d_spmm_host(spc3d_ctx *ctx, int dtype, uint32_t ncols, uint32_t nrows, u
         yslot->output = true;
     }
     Moved ymv;
-    std::thread ythread(send_output_operand, ctx, yslot, (const void *)Y, std::ref(ymv));
+    std::thread ythread;
+    try {
+        ythread = std::thread(send_output_operand, ctx, yslot, (const void *)Y, std::ref(ymv));
+    } catch (const std::system_error &) {
+        send_output_operand(ctx, yslot, Y, ymv); // no thread to be had: one after the other
+    }
     rc = host_input(ctx, hc, dtype, ncols, k, X, stamp, &x);
-    ythread.join();
+    if (ythread.joinable())
+        ythread.join();
     hc->bytes_sent += ymv.sent;
     hc->bytes_kept += ymv.kept;
     if (!rc && ymv.rc)

@@ -4,6 +4,7 @@
 #include <algorithm>
 #include <atomic>
 #include <cstring>
+#include <system_error>
 #include <thread>
 
 #if defined(__x86_64__)
@@ -127,8 +128,12 @@ void keys_of(const void *data, size_t bytes, std::vector<BlockKey> &out, unsigne
     }
     std::vector<std::thread> pool;
     pool.reserve(threads - 1);
-    for (unsigned t = 1; t < threads; ++t)
-        pool.emplace_back(work);
+    try {
+        for (unsigned t = 1; t < threads; ++t)
+            pool.emplace_back(work);
+    } catch (const std::system_error &) {
+        // no more threads to be had: those that started and this one share the blocks
+    }
     work();
     for (std::thread &t : pool)
         t.join();
