@@ -92,6 +92,15 @@ typedef struct {
     uint32_t ncol_blocks;      /* 1, or the number of column blocks the plan is kept in: the
                                   segment counts above are then sums over the blocks,
                                   npartial_slots the largest block's */
+    uint64_t staged_entries;   /* entries of segments whose caller's positions are not
+                                  consecutive (hub rows cut by column slice): spc3d_sddmm
+                                  writes their results in kernel order to a staging vector
+                                  and brings them to C in one ordered pass; 0: none, or a
+                                  pattern whose order makes that pass no better */
+    uint32_t positions_by_segment; /* 1: every segment's results go to consecutive positions
+                                  (of C or of the staging vector), so spc3d_sddmm reads one
+                                  position per segment; 0: one per entry, or none (identity) */
+    uint32_t reserved0;
 } spc3d_plan_info;
 
 /* Plan tuning; a zero field selects the default.  Only speed depends on these. */

@@ -30,7 +30,9 @@ class PlanInfo(ctypes.Structure):
                 ("max_row_nnz", c_u32), ("seg_max", c_u32),
                 ("order_is_identity", ctypes.c_int32), ("nqueues", c_u32),
                 ("hot_cols", c_u32), ("hub_rows", c_u32), ("hot_entries", c_u64),
-                ("nsegments_long", c_u32), ("ncol_blocks", c_u32)]
+                ("nsegments_long", c_u32), ("ncol_blocks", c_u32),
+                ("staged_entries", c_u64), ("positions_by_segment", c_u32),
+                ("reserved0", c_u32)]
 
 
 class PlanOpts(ctypes.Structure):

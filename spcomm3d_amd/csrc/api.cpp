@@ -188,7 +188,11 @@ struct spc3d_plan {
     // tile's worth of staged results (L2-sized) while it writes that tile's C in order.
     // stage_of[g] = staging position of entry g of the blocks' concatenated kernel
     // orders; block b's part starts at stage_off.
-    void *c_stage = nullptr;       // [nnz] reals
+    // A single plan whose kernel order regroups entries inside rows (hub rows cut by column
+    // slice) stages the SDDMM results of those segments (build_store_staging): `store`
+    // holds the positions, c_stage the store.n results.
+    StoreStaging store;
+    void *c_stage = nullptr;       // [nnz] reals (column blocks), [store.n] (staged segments)
     uint32_t *stage_pos = nullptr; // [nnz] caller's position -> staging position
     uint32_t *stage_of = nullptr;  // [nnz]
     uint64_t stage_off = 0;
@@ -306,6 +310,14 @@ void plan_free_device(spc3d_plan *p)
     if (p->sval) (void)hipFree(p->sval);
     if (p->splits) (void)hipFree(p->splits);
     if (p->first_cols) (void)hipFree(p->first_cols);
+    if (p->store.perm2) (void)hipFree(p->store.perm2);
+    if (p->store.dst) (void)hipFree(p->store.dst);
+    if (p->store.src) (void)hipFree(p->store.src);
+    if (p->store.n && p->c_stage) {
+        (void)hipFree(p->c_stage);
+        p->c_stage = nullptr;
+    }
+    p->store = StoreStaging();
     if (p->partial) (void)hipFree(p->partial);
     for (void *old : p->retired_partial)
         (void)hipFree(old);
@@ -343,6 +355,12 @@ DevPlanView view_of(const spc3d_plan *p)
     v.partial = p->partial;
     v.first_cols = p->first_cols;
     v.nnz = p->info.nnz;
+    v.seg_base = p->store.consecutive;
+    if (p->store.n) {
+        v.perm = p->store.perm2;
+        v.stage = p->c_stage;
+        v.stage_from = (uint32_t)p->info.nnz;
+    }
     return v;
 }
 
@@ -970,6 +988,9 @@ static void fill_info(spc3d_plan_info &info, const HostPlan &H)
     info.hot_entries = H.hot_entries;
     info.nsegments_long = H.nseg_long;
     info.ncol_blocks = 1;
+    info.staged_entries = 0;
+    info.positions_by_segment = 0;
+    info.reserved0 = 0;
 }
 
 // Library defaults, overridable field by field.  With XCD slicing, 2 MiB of
@@ -1051,6 +1072,50 @@ static int finish_plan(spc3d_plan *p, uint32_t k0)
     HIP_TRY(launch_first_cols(p->segs + p->info.nsegments_long, nshort, p->col, p->first_cols,
                               p->ctx->stream));
     return ensure_partial(p, k0);
+}
+
+// A finished single plan (not a block of a plan kept in column blocks) whose kernel order
+// regroups entries inside rows gets the staging of its SDDMM results (see StoreStaging).
+// SPC3D_STAGE_STORES=0 in the environment keeps every result on its way straight to C.
+static int add_store_staging(spc3d_plan *p)
+{
+    static const bool off = [] {
+        const char *e = std::getenv("SPC3D_STAGE_STORES");
+        return e && std::atoi(e) == 0;
+    }();
+    if (off || !p->perm || !p->blocks.empty())
+        return SPC3D_OK;
+    std::string err;
+    StoreStaging st;
+    int rc = build_store_staging(p->ctx->stream, p->segs, p->info.nsegments_padded, p->perm,
+                                 p->info.nnz, st, err);
+    if (rc)
+        return fail(rc, err);
+    p->store.consecutive = st.consecutive;
+    p->info.positions_by_segment = st.consecutive ? 1 : 0;
+    if (!st.n)
+        return SPC3D_OK;
+    rc = dev_alloc_bytes(&p->c_stage, (size_t)st.n * elem_size(p->dtype));
+    if (rc) {
+        (void)hipFree(st.perm2);
+        (void)hipFree(st.dst);
+        (void)hipFree(st.src);
+        p->store = StoreStaging();
+        p->info.positions_by_segment = 0;
+        return rc;
+    }
+    p->store = st;
+    p->info.staged_entries = st.n;
+    return SPC3D_OK;
+}
+
+// The staged results of a single plan to their places in C; queued after the launches.
+static hipError_t unstage_stores(const spc3d_plan *S, void *C)
+{
+    if (!S->store.n)
+        return hipSuccess;
+    return launch_unstage_pairs(S->dtype, S->c_stage, S->store.src, S->store.dst, C, S->store.n,
+                                S->ctx->stream);
 }
 
 // Row width a plan is created for: sizes the partial-sum rows of its cut rows.
@@ -1169,11 +1234,15 @@ static int build_from_device(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t
         return rc;
     uint32_t nb = 1;
     rc = choose_col_blocks(p, opts, &nb);
+    if (!rc && nb <= 1)
+        rc = add_store_staging(p);
     if (rc || nb <= 1) {
-        if (rc)
+        if (rc) {
+            const std::string keep = g_err;
             spc3d_plan_destroy(p);
-        else
-            *out = p;
+            return fail(rc, keep);
+        }
+        *out = p;
         return rc;
     }
     // ---- in column blocks ----
@@ -1384,6 +1453,8 @@ int spc3d_plan_create_ex(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t nco
             rc = copy_h2d(ctx, p->splits, H.splits.data(), H.splits.size() * sizeof(SplitRow));
         if (!rc)
             rc = finish_plan(p, planned_k(opts));
+        if (!rc)
+            rc = add_store_staging(p);
         if (rc) {
             plan_free_device(p);
             delete p;
@@ -1696,6 +1767,7 @@ int spc3d_sddmm(spc3d_ctx *ctx, spc3d_plan *S, const spc3d_panel *A, const spc3d
         return rc;
     if (S->blocks.empty()) {
         HIP_TRY(launch_sddmm(S->dtype, view_of(S), A->dev, B->dev, C->dev, K, streams_of(ctx)));
+        HIP_TRY(unstage_stores(S, C->dev));
         return SPC3D_OK;
     }
     for (spc3d_plan *part : S->blocks)
@@ -1841,6 +1913,8 @@ int spc3d_sddmm_spmm(spc3d_ctx *ctx, spc3d_plan *S, const spc3d_panel *A, const 
     }
     if (staged)
         HIP_TRY(unstage(S, C));
+    else
+        HIP_TRY(unstage_stores(S, C->dev));
     return SPC3D_OK;
 }
 

@@ -25,6 +25,14 @@ struct DevPlanView {
     const uint32_t *first_cols = nullptr;
     uint64_t nnz = 0;
     bool stream_c = false;            // SDDMM: streaming stores also at permuted positions
+    // SDDMM results whose position in `perm` is stage_from or more go to place (position -
+    // stage_from) of `stage` (see build_store_staging in plan_device.h); launch_unstage_pairs
+    // brings them to the caller's positions afterwards
+    void *stage = nullptr;
+    uint32_t stage_from = 0xFFFFFFFFu;
+    // every segment's positions in `perm` are perm[start], perm[start] + 1, ...: SDDMM
+    // reads one position per segment
+    bool seg_base = false;
 };
 
 // The context's stream, plus an auxiliary stream of the same (default) priority
@@ -56,6 +64,9 @@ hipError_t launch_first_cols(const Seg *segs, uint32_t n, const uint32_t *col, u
 // out[i] = in[pos[i]], i < n; pos and out 16-byte aligned
 hipError_t launch_unstage(int dtype, const void *in, const uint32_t *pos, void *out, uint64_t n,
                           hipStream_t stream);
+// out[dst[h]] = stage[src[h]], h < n (dst ascending, mostly consecutive)
+hipError_t launch_unstage_pairs(int dtype, const void *stage, const uint32_t *src,
+                                const uint32_t *dst, void *out, uint64_t n, hipStream_t stream);
 // out[p] = in[perm[p]] (perm == null: copy)
 hipError_t launch_gather_vals(int dtype, const void *in, const uint32_t *perm, void *out,
                               uint64_t n, hipStream_t stream);

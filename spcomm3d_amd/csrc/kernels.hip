@@ -254,10 +254,20 @@ template <int G> __device__ __forceinline__ uint64_t seg_index(uint32_t nq, uint
 // instead of with plain stores that the L2 can merge: for the blocks of a plan kept in
 // column blocks, whose positions are long runs in a staging vector and whose block of
 // dense rows is meant to stay in the L2s.
+// stage / stage_from: SDDMM results whose position (perm) is stage_from or more go to
+// place (position - stage_from) of the staging vector instead of into C (segments whose
+// caller's positions are not consecutive; unstage_pairs_kernel brings them home).
+// shift: added to the kernel position of an entry when no `perm` is read (a plan whose
+// segments all have consecutive positions: perm[start] - start of the segment).
 struct Ahead {
     uint32_t first[2] = {0, 0};
     bool stream_c = false;
+    uint32_t stage_from = 0xFFFFFFFFu;
+    void *stage = nullptr;
+    uint32_t shift = 0;
 };
+constexpr uint32_t kStoreStream = 1u;  // sddmm_seg_kernel flags: Ahead::stream_c
+constexpr uint32_t kStoreSegBase = 2u; // positions are perm[segment start] + offset
 template <int LPR, bool WIDE>
 __device__ __forceinline__ Ahead load_first_cols(const uint32_t *__restrict__ first_cols,
                                                  uint64_t sid, uint32_t sub)
@@ -525,7 +535,7 @@ sddmm_batch_one(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type (&a
     const uint32_t uo = entry_of<LPR, NB>(sub);
     const bool writer = is_writer<LPR, NB>(sub) && (!MK || uo < n);
     T sv = (T)0;
-    uint32_t dst = p0 + uo;
+    uint32_t dst = p0 + uo + ex.shift;
     if (writer) {
         sv = nt_load(sval + p0 + uo);
         if (perm)
@@ -555,14 +565,16 @@ sddmm_batch_one(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type (&a
     // batch fill whole lines and stream out; when it is not they are scattered, and
     // plain stores let the L2 merge neighbours into lines before writing back.
     if (writer) {
+        const bool staged = dst >= ex.stage_from;
+        T *out = staged ? static_cast<T *>(ex.stage) + (dst - ex.stage_from) : C + dst;
         if constexpr (RG >= 2) {
             if (odd.accum)
-                result += C[dst];
+                result += *out;
         }
-        if (perm && !ex.stream_c)
-            C[dst] = result;
+        if (perm && !ex.stream_c && !staged)
+            *out = result;
         else
-            nt_store(result, C + dst);
+            nt_store(result, out);
     }
     if constexpr (FZ != 0) {
         const T mine = FZ == 2 ? result : sv; // valid on the writer lanes
@@ -610,7 +622,7 @@ sddmm_batch_rounds(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type 
         const uint32_t mine = (uint32_t)r * G + uo;
         writer[r] = wlane && (!MK || mine < n);
         sv[r] = (T)0;
-        dst[r] = p0 + mine;
+        dst[r] = p0 + mine + ex.shift;
         if (writer[r]) {
             sv[r] = nt_load(sval + p0 + mine);
             if (perm)
@@ -639,14 +651,16 @@ sddmm_batch_rounds(const typename Vec<T>::type (&a)[VPL], typename Vec<T>::type 
         // batch fill whole lines and stream out; when it is not they are scattered, and
         // plain stores let the L2 merge neighbours into lines before writing back.
         if (writer[r]) {
+            const bool staged = dst[r] >= ex.stage_from;
+            T *out = staged ? static_cast<T *>(ex.stage) + (dst[r] - ex.stage_from) : C + dst[r];
             if constexpr (RG >= 2) {
                 if (odd.accum)
-                    result += C[dst[r]];
+                    result += *out;
             }
-            if (perm && !ex.stream_c)
-                C[dst[r]] = result;
+            if (perm && !ex.stream_c && !staged)
+                *out = result;
             else
-                nt_store(result, C + dst[r]);
+                nt_store(result, out);
         }
         if constexpr (FZ != 0) {
             const T mine = FZ == 2 ? result : sv[r]; // valid on the writer lanes
@@ -757,7 +771,7 @@ sddmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint3
                  const T *__restrict__ sval, const T *__restrict__ A, const T *__restrict__ B,
                  T *__restrict__ C, T *__restrict__ Y, T *__restrict__ partial, uint32_t nvec,
                  uint32_t stride, uint32_t accum, const uint32_t *__restrict__ first_cols,
-                 uint32_t stream_c)
+                 uint32_t flags, T *__restrict__ stage, uint32_t stage_from)
 {
     static_assert(UB <= 16 && LPR <= 64, "at most 16 entries in flight per lane");
     using V = typename Vec<T>::type;
@@ -766,10 +780,16 @@ sddmm_seg_kernel(const Seg *__restrict__ segs, uint32_t nseg, uint32_t nq, uint3
     if (sid >= nseg)
         return;
     Ahead ex = load_first_cols<LPR, WIDE>(first_cols, sid, sub);
-    ex.stream_c = stream_c != 0;
+    ex.stream_c = (flags & kStoreStream) != 0;
+    ex.stage = stage;
+    ex.stage_from = stage_from;
     const u32x4 sg = nt_load(reinterpret_cast<const u32x4 *>(segs) + sid); // row, start, len, slot
     if (sg[2] == 0)
         return;
+    if (flags & kStoreSegBase) { // one position per segment instead of one per entry
+        ex.shift = nt_load(perm + sg[1]) - sg[1];
+        perm = nullptr;
+    }
 
     const Odd<T, VPL, RG> odd = odd_lanes<T, LPR, VPL, RG>(sub, nvec, stride, accum);
     V a[VPL], acc[VPL];
@@ -1183,6 +1203,36 @@ gather4_kernel(const T *__restrict__ in, const uint32_t *__restrict__ pos, T *__
         out[nfull + t] = in[pos[nfull + t]];
 }
 
+// out[dst[h]] = stage[src[h]], h < n, dst ascending and mostly consecutive: four results in
+// flight per lane, consecutive lanes on consecutive h.
+template <typename T>
+__global__ void __launch_bounds__(kBlock)
+unstage_pairs_kernel(const T *__restrict__ stage, const uint32_t *__restrict__ src,
+                     const uint32_t *__restrict__ dst, T *__restrict__ out, uint64_t n)
+{
+    constexpr uint64_t U = 4;
+    const uint64_t span = (uint64_t)kBlock * U;
+    uint64_t base = (uint64_t)blockIdx.x * span;
+    for (; base + span <= n; base += (uint64_t)gridDim.x * span) {
+        uint32_t s[U], d[U];
+        T v[U];
+#pragma unroll
+        for (uint64_t u = 0; u < U; ++u) {
+            s[u] = nt_load(src + base + u * kBlock + threadIdx.x);
+            d[u] = nt_load(dst + base + u * kBlock + threadIdx.x);
+        }
+#pragma unroll
+        for (uint64_t u = 0; u < U; ++u)
+            v[u] = nt_load(stage + s[u]);
+#pragma unroll
+        for (uint64_t u = 0; u < U; ++u)
+            nt_store(v[u], out + d[u]);
+    }
+    // what is left is less than one span, and one workgroup's `base` lies in it
+    for (uint64_t h = base + threadIdx.x; h < n; h += kBlock)
+        out[dst[h]] = stage[src[h]];
+}
+
 template <typename T>
 __global__ void __launch_bounds__(kBlock) fill_kernel(T *__restrict__ p, uint64_t n, T value)
 {
@@ -1314,6 +1364,11 @@ inline hipError_t join_aux(const Streams &S)
     return hipStreamSynchronize(S.aux);
 }
 
+inline uint32_t store_flags(const DevPlanView &P)
+{
+    return (P.stream_c ? kStoreStream : 0u) | (P.perm && P.seg_base ? kStoreSegBase : 0u);
+}
+
 template <typename T, int LPR, int VPL, int UB, int US, int RG, int FZ>
 hipError_t run_sddmm(const DevPlanView &P, const T *A, const T *B, T *C, T *Y, const Streams &S,
                      uint32_t nvec, uint32_t stride = 0, uint32_t accum = 0)
@@ -1327,14 +1382,15 @@ hipError_t run_sddmm(const DevPlanView &P, const T *A, const T *B, T *C, T *Y, c
                            dim3(blocks_for_groups(nl, P.nqueues, 64 / LPR)), dim3(kBlock), 0,
                            S.main, P.segs, nl, P.nqueues, 0u, P.col, P.perm, (const T *)P.sval,
                            A, B, C, Y, (T *)P.partial, nvec, stride ? stride : nvec, accum,
-                           (const uint32_t *)nullptr, P.stream_c ? 1u : 0u);
+                           (const uint32_t *)nullptr, store_flags(P), (T *)P.stage,
+                           P.stage_from);
     if (ns)
         hipLaunchKernelGGL((sddmm_seg_kernel<T, LPR, VPL, US, RG, false, FZ>),
                            dim3(blocks_for_groups(ns, P.nqueues, 64 / LPR)), dim3(kBlock), 0,
                            both ? S.aux : S.main, P.segs + nl, ns, P.nqueues,
                            both ? S.aux_rot : 0u, P.col, P.perm, (const T *)P.sval, A, B, C, Y,
                            (T *)P.partial, nvec, stride ? stride : nvec, accum, P.first_cols,
-                           P.stream_c ? 1u : 0u);
+                           store_flags(P), (T *)P.stage, P.stage_from);
     const hipError_t launched = hipGetLastError();
     const hipError_t joined = both ? join_aux(S) : hipSuccess;
     return launched != hipSuccess ? launched : joined;
@@ -1596,6 +1652,22 @@ hipError_t launch_unstage(int dtype, const void *in, const uint32_t *pos, void *
     else
         hipLaunchKernelGGL((gather4_kernel<float>), dim3(grid), dim3(kBlock), 0, stream,
                            (const float *)in, pos, (float *)out, n);
+    return hipGetLastError();
+}
+
+hipError_t launch_unstage_pairs(int dtype, const void *stage, const uint32_t *src,
+                                const uint32_t *dst, void *out, uint64_t n, hipStream_t stream)
+{
+    if (n == 0)
+        return hipSuccess;
+    const uint64_t want = (n + (uint64_t)kBlock * 4 - 1) / ((uint64_t)kBlock * 4);
+    const uint32_t grid = (uint32_t)(want > 65536 ? 65536 : want);
+    if (dtype == 1)
+        hipLaunchKernelGGL((unstage_pairs_kernel<double>), dim3(grid), dim3(kBlock), 0, stream,
+                           (const double *)stage, src, dst, (double *)out, n);
+    else
+        hipLaunchKernelGGL((unstage_pairs_kernel<float>), dim3(grid), dim3(kBlock), 0, stream,
+                           (const float *)stage, src, dst, (float *)out, n);
     return hipGetLastError();
 }
 

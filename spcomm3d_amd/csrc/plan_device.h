@@ -65,6 +65,34 @@ int tile_keys_device(hipStream_t stream, const uint32_t *d_rows, const uint32_t 
 // max_key).  Synchronous.
 int stable_ranks_device(hipStream_t stream, const uint32_t *d_key, uint64_t n, uint32_t max_key,
                         uint32_t *d_rank, std::string &err);
+// ---- staged SDDMM results ---------------------------------------------------------
+// Where the kernel order regroups the entries of a row (the pieces a hub row is cut into
+// by column slice), SDDMM's results leave a segment for caller's positions that are not
+// consecutive: one 4- or 8-byte store per entry, each into a line of its own.  Such
+// segments are "staged": their results go to consecutive places of a staging vector, as
+// the segment holds them, and one pass afterwards brings them to the caller's positions
+// in ascending order of those (so that its stores are the consecutive ones).
+//   perm2[p]  = perm[p] for an entry whose segment stores to consecutive positions,
+//               else nnz + the entry's place in the staging vector
+//   dst, src  = for staged entry h in ascending order of caller's position: that
+//               position, and its place in the staging vector
+// n == 0 (and null arrays) when no segment needs it, or when staging does not pay: the
+// staged entries' positions are not mostly consecutive, or the final pass would not read
+// near what its neighbours read (a shuffled pattern, where that pass would scatter just as
+// the kernel does), or nnz + n does not fit 32 bits.
+// consecutive: with `perm2` in place of `perm` (n != 0), or with `perm` as it is (n == 0),
+// every segment's positions are perm[start], perm[start] + 1, ...: the kernel can read one
+// position per segment.  The arrays belong to the receiver (hipFree).  Synchronous.
+struct StoreStaging {
+    uint32_t *perm2 = nullptr; // [nnz]
+    uint32_t *dst = nullptr;   // [n]
+    uint32_t *src = nullptr;   // [n]
+    uint64_t n = 0;
+    bool consecutive = false;
+};
+int build_store_staging(hipStream_t stream, const Seg *d_segs, uint32_t nseg, const uint32_t *d_perm,
+                        uint64_t nnz, StoreStaging &out, std::string &err);
+
 // Sum of len^2 over a plan's segments (device array); synchronous.
 int sum_sq_seg_len_device(hipStream_t stream, const Seg *d_segs, uint64_t nseg, uint64_t *out,
                           std::string &err);

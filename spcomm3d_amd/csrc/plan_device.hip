@@ -1264,6 +1264,129 @@ int stable_ranks_device(hipStream_t st, const uint32_t *d_key, uint64_t n, uint3
     return SPC3D_OK;
 }
 
+// One wavefront per segment: flag[p] = 1 for every entry of a segment whose caller's
+// positions are not perm[start], perm[start] + 1, ...
+__global__ void staged_flags_k(const Seg *__restrict__ segs, uint32_t nseg,
+                               const uint32_t *__restrict__ perm, uint32_t *__restrict__ flag)
+{
+    const uint32_t lane = threadIdx.x & 63u;
+    for (uint64_t s = ((uint64_t)blockIdx.x * kTB + threadIdx.x) / 64; s < nseg;
+         s += (uint64_t)gridDim.x * (kTB / 64)) {
+        const Seg sg = segs[s];
+        if (sg.len == 0)
+            continue;
+        const uint32_t base = perm[sg.start];
+        bool bad = false;
+        for (uint32_t u = lane; u < sg.len; u += 64)
+            bad |= perm[sg.start + u] != base + u;
+        const uint32_t any = __any(bad) ? 1u : 0u;
+        for (uint32_t u = lane; u < sg.len; u += 64)
+            flag[sg.start + u] = any;
+    }
+}
+
+__global__ void staged_fill_k(const uint32_t *__restrict__ perm, const uint32_t *__restrict__ flag,
+                              const uint32_t *__restrict__ idx, uint64_t nnz, uint32_t *perm2,
+                              uint32_t *key, uint32_t *val)
+{
+    GRID_STRIDE(p, nnz)
+    {
+        if (flag[p]) {
+            perm2[p] = (uint32_t)nnz + idx[p];
+            key[idx[p]] = perm[p];
+            val[idx[p]] = idx[p];
+        } else {
+            perm2[p] = perm[p];
+        }
+    }
+}
+
+__global__ void adjacent_k(const uint32_t *__restrict__ sorted, uint64_t n, unsigned long long *acc)
+{
+    unsigned long long c = 0;
+    GRID_STRIDE(i, n)
+    if (i + 1 < n && sorted[i + 1] == sorted[i] + 1)
+        ++c;
+    c = wave_sum(c);
+    if ((threadIdx.x & 63u) == 0 && c)
+        atomicAdd(acc, c);
+}
+
+// How many of the n staged results are read next to another one of the same wavefront of
+// the final pass (64 consecutive h): src[h] - 1 is the src of another lane.
+__global__ void src_neighbours_k(const uint32_t *__restrict__ src, uint64_t n, unsigned long long *acc)
+{
+    unsigned long long c = 0;
+    const uint64_t nround = (n + 63) / 64 * 64;
+    GRID_STRIDE(h, nround)
+    {
+        const uint32_t mine = h < n ? src[h] : 0xFFFFFFFFu;
+        bool near = false;
+        for (int j = 0; j < 64; ++j)
+            near |= __shfl(mine, j) + 1 == mine;
+        if (h < n && near)
+            ++c;
+    }
+    c = wave_sum(c);
+    if ((threadIdx.x & 63u) == 0 && c)
+        atomicAdd(acc, c);
+}
+
+int build_store_staging(hipStream_t st, const Seg *d_segs, uint32_t nseg, const uint32_t *d_perm,
+                        uint64_t nnz, StoreStaging &out, std::string &err)
+{
+    out = StoreStaging();
+    if (!d_perm || nnz == 0 || nseg == 0 || nnz >= (1ull << 31))
+        return SPC3D_OK;
+    Arena arena;
+    HIP_OK(arena.reserve((size_t)nnz * 8 + ((size_t)8 << 20)));
+    Temp tmp(arena);
+    SBuf<uint32_t> flag, idx;
+    HIP_OK(flag.alloc(arena, nnz));
+    HIP_OK(idx.alloc(arena, nnz));
+    HIP_OK(hipMemsetAsync(flag.p, 0, (size_t)nnz * 4, st));
+    hipLaunchKernelGGL(staged_flags_k, dim3(grid_for((uint64_t)nseg * 64)), dim3(kTB), 0, st, d_segs,
+                       nseg, d_perm, flag.p);
+    TRY(exclusive_sum<uint32_t>(tmp, flag.p, idx.p, (size_t)nnz, st, err));
+    uint32_t last[2] = {0, 0};
+    TRY(fetch(st, &last[0], idx.p + (nnz - 1), 4, err));
+    TRY(fetch(st, &last[1], flag.p + (nnz - 1), 4, err));
+    const uint64_t n = (uint64_t)last[0] + last[1];
+    if (n == 0) {
+        out.consecutive = true;
+        return SPC3D_OK;
+    }
+    if (nnz + n >= (1ull << 32))
+        return SPC3D_OK;
+    DBuf<uint32_t> perm2, dst, src;
+    HIP_OK(perm2.alloc(nnz));
+    HIP_OK(dst.alloc(n));
+    HIP_OK(src.alloc(n));
+    SBuf<uint32_t> key, val;
+    HIP_OK(key.alloc(arena, n));
+    HIP_OK(val.alloc(arena, n));
+    LAUNCH(staged_fill_k, nnz, d_perm, flag.p, idx.p, nnz, perm2.p, key.p, val.p);
+    TRY(sort_pairs<uint32_t>(tmp, key.p, dst.p, val.p, src.p, (uint32_t)n, bits_for(nnz - 1), false,
+                             st, err));
+    // The final pass pays when it writes runs and reads near what its neighbours read; an
+    // arbitrary order of the entries gives neither, and keeps its scattered stores.
+    DBuf<unsigned long long> acc;
+    HIP_OK(acc.alloc(2));
+    HIP_OK(hipMemsetAsync(acc.p, 0, 2 * sizeof(unsigned long long), st));
+    LAUNCH_SMALL(adjacent_k, n, dst.p, n, acc.p);
+    LAUNCH_SMALL(src_neighbours_k, n, src.p, n, acc.p + 1);
+    unsigned long long seen[2] = {0, 0};
+    TRY(fetch(st, seen, acc.p, sizeof seen, err));
+    if (seen[0] * 2 < n || seen[1] * 2 < n)
+        return SPC3D_OK; // (the DBufs free themselves)
+    out.perm2 = perm2.release();
+    out.dst = dst.release();
+    out.src = src.release();
+    out.n = n;
+    out.consecutive = true;
+    return SPC3D_OK;
+}
+
 int sum_sq_seg_len_device(hipStream_t st, const Seg *d_segs, uint64_t nseg, uint64_t *out,
                           std::string &err)
 {

@@ -490,6 +490,55 @@ def test_xcd_sliced_plan_matches_oracle(ctx, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("k", [64, 50, 3, 1030])
+def test_staged_results_of_hub_row_pieces_reach_the_callers_positions(ctx, dtype, k):
+    """Sorted input whose hub rows are cut by column slice: the pieces' results are written
+    in kernel order to a staging vector and brought to C by one ordered pass (plan info
+    staged_entries > 0), the other segments read one position each.  Every entry of C must be
+    overwritten, through spc3d_sddmm and both forms of spc3d_sddmm_spmm, call after call,
+    also for dense rows over 4 KiB (several launches that accumulate in place)."""
+    w = W.rmat(14, 16, k)
+    A, B, Y0, vv = w.panel_A(dtype), w.panel_B(dtype), w.panel_Y0(dtype), w.values(dtype)
+    S = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, vv, xcd_slices=8, l2_hot_bytes=64 * 1024,
+                 hub_min=32, seg_max=256)
+    I = S.info
+    assert I.nqueues == 8 and I.hub_rows > 0 and I.order_is_identity == 0
+    assert 0 < I.staged_entries < w.nnz, I.staged_entries
+    dA, dB, dY, dC = ctx.panel_from(A), ctx.panel_from(B), ctx.panel_from(Y0), ctx.vals(w.nnz, dtype)
+    for _ in range(2):
+        dC.fill(np.nan)
+        ctx.sddmm(S, dA, dB, dC)
+        check_sddmm(A, B, w.ii, w.jj, vv, dC.download())
+    first = dC.download()
+    if k * np.dtype(dtype).itemsize <= 4096:
+        dC.fill(np.nan)
+        ctx.sddmm_spmm(S, dA, dB, dC, dY)
+        assert np.array_equal(dC.download(), first)
+        check_spmm(B, w.ii, w.jj, vv, Y0, dY.download())
+        dC.fill(np.nan)
+        dY.upload(Y0)
+        ctx.sddmm_spmm(S, dA, dB, dC, dY, chained=True)
+        assert np.array_equal(dC.download(), first)
+        check_spmm(B, w.ii, w.jj, first, Y0, dY.download())
+    # new values through the original order, then the same plan again
+    vv2 = (vv * 0.5 + 1).astype(dtype)
+    S.set_values(vv2)
+    dC.fill(np.nan)
+    ctx.sddmm(S, dA, dB, dC)
+    check_sddmm(A, B, w.ii, w.jj, vv2, dC.download())
+    for h in (S, dA, dB, dY, dC):
+        h.close()
+
+
+def test_a_shuffled_pattern_keeps_its_stores_unstaged(ctx):
+    # every segment's positions are scattered and so would be the final pass: no staging
+    w = W.rmat(14, 16, 64).shuffled()
+    S = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, w.values(np.float32))
+    assert S.info.order_is_identity == 0 and S.info.staged_entries == 0
+    S.close()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("nblocks", [2, 7, 300])
 def test_plan_in_column_blocks_matches_oracle(ctx, dtype, nblocks):
     """A pattern kept in column blocks (one plan per block, run one after the other):

@@ -16,7 +16,10 @@ pytestmark = pytest.mark.gpu
 GOLDEN_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden",
                            "core_ops_golden.npz")
 
-INFO_FIELDS = [name for name, _ in capi.PlanInfo._fields_ if name != "reserved"]
+# how SDDMM's results are stored is decided on the device, after either builder: the
+# host-only build leaves these 0
+INFO_FIELDS = [name for name, _ in capi.PlanInfo._fields_
+               if name not in ("reserved0", "staged_entries", "positions_by_segment")]
 
 
 def assert_same_plan(dev: dict, host: dict):
