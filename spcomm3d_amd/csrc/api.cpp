@@ -2296,10 +2296,14 @@ void send_output_operand(spc3d_ctx *ctx, CachedHostPanel *slot, const void *host
     const size_t bytes = (size_t)slot->panel->m * slot->panel->n * elem_size(slot->panel->dtype);
     std::vector<BlockKey> keys;
     const bool read_first = !slot->keys.empty() && slot->skip == 0;
-    if (read_first)
-        keys_of(host, bytes, keys, 4);
-    else if (slot->skip)
-        --slot->skip;
+    try { // runs as a thread's function: nothing may leave it
+        if (read_first)
+            keys_of(host, bytes, keys, 4);
+        else if (slot->skip)
+            --slot->skip;
+    } catch (const std::exception &) {
+        keys.clear(); // no keys: everything is sent
+    }
     send_panel(ctx, slot, host, keys, mv);
     if (mv.rc || !read_first)
         return;
@@ -2334,11 +2338,25 @@ int fetch_output_operand(spc3d_ctx *ctx, CachedHostPanel *slot, void *host)
     };
     const unsigned hw = std::thread::hardware_concurrency();
     const unsigned nthreads = (unsigned)std::min<size_t>(std::min(4u, hw ? hw : 1u), nblocks);
-    std::vector<std::thread> pool;
+    // Joined on every way out, after the workers have been let run out.
+    struct Pool {
+        std::vector<std::thread> threads;
+        std::atomic<size_t> &ready;
+        size_t nblocks;
+        ~Pool()
+        {
+            ready.store(nblocks, std::memory_order_release);
+            for (std::thread &t : threads)
+                if (t.joinable())
+                    t.join();
+        }
+    } workers{{}, ready, nblocks};
+    std::vector<std::thread> &pool = workers.threads;
     try {
+        pool.reserve(nthreads);
         for (unsigned t = 0; t < nthreads; ++t)
             pool.emplace_back(work);
-    } catch (const std::system_error &) {
+    } catch (const std::exception &) {
         // fewer workers, or none: what is left over is keyed by this thread at the end
     }
     constexpr size_t kPiece = 4; // blocks per copy: 16 MiB
@@ -2445,9 +2463,9 @@ static int sddmm_host_uncached(spc3d_ctx *ctx, int dtype, uint32_t m, uint32_t n
     return rc ? fail(rc, keep) : SPC3D_OK;
 }
 
-int spc3d_sddmm_host(spc3d_ctx *ctx, int dtype, uint32_t m, uint32_t n, uint32_t k, const void *A,
-                     const void *B, uint64_t nnz, const uint32_t *ii, const uint32_t *jj,
-                     const void *svv, void *cvv)
+static int sddmm_host_call(spc3d_ctx *ctx, int dtype, uint32_t m, uint32_t n, uint32_t k,
+                           const void *A, const void *B, uint64_t nnz, const uint32_t *ii,
+                           const uint32_t *jj, const void *svv, void *cvv)
 {
     if (nnz && (!svv || !cvv))
         return fail(SPC3D_ERR_INVALID_ARG, "svv or cvv is NULL");
@@ -2479,6 +2497,17 @@ int spc3d_sddmm_host(spc3d_ctx *ctx, int dtype, uint32_t m, uint32_t n, uint32_t
     return rc;
 }
 
+int spc3d_sddmm_host(spc3d_ctx *ctx, int dtype, uint32_t m, uint32_t n, uint32_t k, const void *A,
+                     const void *B, uint64_t nnz, const uint32_t *ii, const uint32_t *jj,
+                     const void *svv, void *cvv)
+{
+    try {
+        return sddmm_host_call(ctx, dtype, m, n, k, A, B, nnz, ii, jj, svv, cvv);
+    } catch (const std::bad_alloc &) {
+        return fail(SPC3D_ERR_ALLOC, "host allocation failed");
+    }
+}
+
 static int spmm_host_uncached(spc3d_ctx *ctx, int dtype, uint32_t ncols, uint32_t nrows, uint32_t k,
                               const void *X, uint64_t nnz, const uint32_t *ii, const uint32_t *jj,
                               const void *avv, void *Y)
@@ -2504,9 +2533,9 @@ static int spmm_host_uncached(spc3d_ctx *ctx, int dtype, uint32_t ncols, uint32_
     return rc ? fail(rc, keep) : SPC3D_OK;
 }
 
-int spc3d_spmm_host(spc3d_ctx *ctx, int dtype, uint32_t ncols, uint32_t nrows, uint32_t k,
-                    const void *X, uint64_t nnz, const uint32_t *ii, const uint32_t *jj,
-                    const void *avv, void *Y)
+static int spmm_host_call(spc3d_ctx *ctx, int dtype, uint32_t ncols, uint32_t nrows, uint32_t k,
+                          const void *X, uint64_t nnz, const uint32_t *ii, const uint32_t *jj,
+                          const void *avv, void *Y)
 {
     if (nnz && !avv)
         return fail(SPC3D_ERR_INVALID_ARG, "avv is NULL");
@@ -2544,6 +2573,14 @@ int spc3d_spmm_host(spc3d_ctx *ctx, int dtype, uint32_t ncols, uint32_t nrows, u
     }
     Moved ymv;
     std::thread ythread;
+    struct Joined { // on every way out
+        std::thread &t;
+        ~Joined()
+        {
+            if (t.joinable())
+                t.join();
+        }
+    } joined{ythread};
     try {
         ythread = std::thread(send_output_operand, ctx, yslot, (const void *)Y, std::ref(ymv));
     } catch (const std::system_error &) {
@@ -2564,6 +2601,17 @@ int spc3d_spmm_host(spc3d_ctx *ctx, int dtype, uint32_t ncols, uint32_t nrows, u
     else
         yslot->keys.clear(); // whatever the panel holds now, it is not known to be Y
     return rc;
+}
+
+int spc3d_spmm_host(spc3d_ctx *ctx, int dtype, uint32_t ncols, uint32_t nrows, uint32_t k,
+                    const void *X, uint64_t nnz, const uint32_t *ii, const uint32_t *jj,
+                    const void *avv, void *Y)
+{
+    try {
+        return spmm_host_call(ctx, dtype, ncols, nrows, k, X, nnz, ii, jj, avv, Y);
+    } catch (const std::bad_alloc &) {
+        return fail(SPC3D_ERR_ALLOC, "host allocation failed");
+    }
 }
 
 } // extern "C"
