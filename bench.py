@@ -22,9 +22,10 @@ reported beside `value`, which always comes from the two separate calls.
 of it.  `row_copies` times the pack and sum-unpack copies of a sparse exchange over the
 touched rows of Y (algorithmic bytes: rows read + buffer written; buffer read +
 rows read and written).  `also` holds the other real type, the same workload
-handed over in shuffled COO order (the reference never sorts its entries) in
-both types, and `configs`: one compact row per other benchmark configuration
-(time per kernel, strict-model fraction of the HBM peak).
+handed over in shuffled COO order (the reference never sorts its entries) and in
+column-major order (the order of the MatrixMarket files it reads) in both types,
+and `configs`: one compact row per other benchmark configuration (time per kernel,
+strict-model fraction of the HBM peak).
 """
 from __future__ import annotations
 
@@ -406,6 +407,11 @@ def main():
                                 for dt in ("f64", "f32")}
             log(json.dumps(also["shuffled"]))
             del ws
+            wc = w.column_major()
+            also["column_major"] = {dt: run_compact(wc, dt, max(5, args.steps // 2), args.warmup)
+                                    for dt in ("f64", "f32")}
+            log(json.dumps(also["column_major"]))
+            del wc
         rows = []
         for name, dtypes, steps in OTHER_CONFIGS:
             if name == args.config:

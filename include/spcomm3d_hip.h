@@ -100,7 +100,11 @@ typedef struct {
     uint32_t positions_by_segment; /* 1: every segment's results go to consecutive positions
                                   (of C or of the staging vector), so spc3d_sddmm reads one
                                   position per segment; 0: one per entry, or none (identity) */
-    uint32_t reserved0;
+    uint32_t sddmm_by_column;  /* 1: the pattern came sorted by column, and spc3d_sddmm runs a
+                                  second plan of the same entries with rows and columns (and
+                                  so A and B) exchanged, whose kernel order is the caller's:
+                                  the same bits, stored in runs instead of one by one; the
+                                  plan then holds its arrays twice (GPU builder only) */
 } spc3d_plan_info;
 
 /* Plan tuning; a zero field selects the default.  Only speed depends on these. */
@@ -224,7 +228,10 @@ SPC3D_API int spc3d_coo_validate(uint32_t nrows, uint32_t ncols, uint64_t nnz,
  * uploaded as it is and all of this happens on the GPU (histograms, scans and
  * stable radix sorts; milliseconds for 16 M entries); spc3d_plan_opts.builder or
  * SPC3D_PLAN_BUILDER=host in the environment (spc3d_plan_create only) selects
- * the single-threaded host builder instead.  `vv` (nnz reals of
+ * the single-threaded host builder instead.  How spc3d_sddmm brings its results to
+ * the caller's positions is settled here as well (spc3d_plan_info: staged_entries,
+ * positions_by_segment, sddmm_by_column; the environment variables SPC3D_STAGE_STORES=0
+ * and SPC3D_SDDMM_BY_COLUMN=0 keep the plain form, for comparisons).  `vv` (nnz reals of
  * `dtype`, caller's order) may be NULL and set later.  The pattern is copied:
  * the caller's arrays are not referenced afterwards.  Replaces nothing in the
  * reference (it walks the unsorted COO directly, core_ops.cpp:7-10); it is the

@@ -192,6 +192,13 @@ struct spc3d_plan {
     // slice) stages the SDDMM results of those segments (build_store_staging): `store`
     // holds the positions, c_stage the store.n results.
     StoreStaging store;
+    // SDDMM is symmetric in its two dense operands.  For a pattern handed over sorted by
+    // column (the order of a MatrixMarket file), whose results in this plan's row-major
+    // kernel order would each be stored to a place of its own, `by_col` is the plan of the
+    // same entries with rows and columns exchanged: its kernel order is the caller's, and
+    // spc3d_sddmm runs it with A and B exchanged (the same products summed in the same
+    // order: the same bits).  SpMM and the one-pass call run this plan.
+    spc3d_plan *by_col = nullptr;
     void *c_stage = nullptr;       // [nnz] reals (column blocks), [store.n] (staged segments)
     uint32_t *stage_pos = nullptr; // [nnz] caller's position -> staging position
     uint32_t *stage_of = nullptr;  // [nnz]
@@ -990,7 +997,7 @@ static void fill_info(spc3d_plan_info &info, const HostPlan &H)
     info.ncol_blocks = 1;
     info.staged_entries = 0;
     info.positions_by_segment = 0;
-    info.reserved0 = 0;
+    info.sddmm_by_column = 0;
 }
 
 // Library defaults, overridable field by field.  With XCD slicing, 2 MiB of
@@ -1215,6 +1222,50 @@ static int choose_col_blocks(spc3d_plan *p, const spc3d_plan_opts *opts, uint32_
     return SPC3D_OK;
 }
 
+// The companion plan for SDDMM (spc3d_plan::by_col) of a finished single plan whose results
+// would be stored one by one, when the pattern is sorted by column and the exchanged plan
+// does store in runs.  SPC3D_SDDMM_BY_COLUMN=0 in the environment switches it off.
+static int add_sddmm_companion(spc3d_plan *p, uint32_t nrows, uint32_t ncols, uint64_t nnz,
+                               const uint32_t *d_ii, const uint32_t *d_jj, const PlanOpts &po)
+{
+    static const bool off = [] {
+        const char *e = std::getenv("SPC3D_SDDMM_BY_COLUMN");
+        return e && std::atoi(e) == 0;
+    }();
+    if (off || nnz < 2 || !p->perm || p->store.consecutive || !p->blocks.empty())
+        return SPC3D_OK;
+    std::string err;
+    bool sorted = false;
+    int rc = is_nondecreasing_device(p->ctx->stream, d_jj, nnz, &sorted, err);
+    if (rc)
+        return fail(rc, err);
+    if (!sorted)
+        return SPC3D_OK;
+    HostPlan meta;
+    DevPlanArrays arr;
+    rc = build_device_plan(p->ctx->stream, ncols, nrows, nnz, d_jj, d_ii, po, meta, arr, err);
+    if (rc)
+        return fail(rc, err);
+    spc3d_plan *q = nullptr;
+    rc = adopt_device_plan(p->ctx, p->dtype, meta, arr, 0 /* never runs SpMM */, &q);
+    if (!rc)
+        rc = add_store_staging(q);
+    if (rc || (q->perm && !q->store.consecutive)) { // no better than what there is
+        if (q) {
+            const std::string keep = g_err;
+            plan_free_device(q);
+            q->magic = 0;
+            delete q;
+            if (rc)
+                return fail(rc, keep);
+        }
+        return rc;
+    }
+    p->by_col = q;
+    p->info.sddmm_by_column = 1;
+    return SPC3D_OK;
+}
+
 // Plan of a pattern that lies on the device: the single plan first (validation, the
 // whole pattern's figures), then, where choose_col_blocks says so, one plan per block
 // of columns in its place.
@@ -1236,6 +1287,8 @@ static int build_from_device(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t
     rc = choose_col_blocks(p, opts, &nb);
     if (!rc && nb <= 1)
         rc = add_store_staging(p);
+    if (!rc && nb <= 1)
+        rc = add_sddmm_companion(p, nrows, ncols, nnz, d_ii, d_jj, po);
     if (rc || nb <= 1) {
         if (rc) {
             const std::string keep = g_err;
@@ -1591,6 +1644,12 @@ int spc3d_plan_destroy(spc3d_plan *plan)
     (void)hipSetDevice(plan->ctx->device);
     (void)hipStreamSynchronize(plan->ctx->stream);
     destroy_blocks(plan);
+    if (plan->by_col) {
+        plan_free_device(plan->by_col);
+        plan->by_col->magic = 0;
+        delete plan->by_col;
+        plan->by_col = nullptr;
+    }
     plan_free_device(plan);
     plan->magic = 0;
     delete plan;
@@ -1640,7 +1699,7 @@ int spc3d_plan_set_values(spc3d_plan *plan, const void *vv_host)
     if (rc)
         return rc;
     const size_t bytes = (size_t)nnz * elem_size(plan->dtype);
-    if (plan->blocks.empty() && !plan->perm) {
+    if (plan->blocks.empty() && !plan->perm && !plan->by_col) {
         rc = copy_h2d(plan->ctx, plan->sval, vv_host, bytes);
     } else {
         void *tmp = nullptr;
@@ -1656,6 +1715,13 @@ int spc3d_plan_set_values(spc3d_plan *plan, const void *vv_host)
                                               part->info.nnz, plan->ctx->stream);
             if (e != hipSuccess)
                 rc = fail_hip(e, "gather of sparse values");
+        }
+        if (!rc && plan->by_col) {
+            hipError_t e = launch_gather_vals(plan->dtype, tmp, plan->by_col->perm,
+                                              plan->by_col->sval, nnz, plan->ctx->stream);
+            if (e != hipSuccess)
+                rc = fail_hip(e, "gather of sparse values");
+            plan->by_col->has_values = true;
         }
         if (!rc) {
             hipError_t e = hipStreamSynchronize(plan->ctx->stream);
@@ -1683,6 +1749,11 @@ int spc3d_plan_set_values_device(spc3d_plan *plan, const spc3d_vals *vv)
     for (spc3d_plan *part : parts_of(plan, self))
         HIP_TRY(launch_gather_vals(plan->dtype, vv->dev, part->perm, part->sval, part->info.nnz,
                                    plan->ctx->stream));
+    if (plan->by_col) {
+        HIP_TRY(launch_gather_vals(plan->dtype, vv->dev, plan->by_col->perm, plan->by_col->sval,
+                                   plan->info.nnz, plan->ctx->stream));
+        plan->by_col->has_values = true;
+    }
     plan->has_values = true;
     return SPC3D_OK;
 }
@@ -1765,6 +1836,12 @@ int spc3d_sddmm(spc3d_ctx *ctx, spc3d_plan *S, const spc3d_panel *A, const spc3d
     int rc = use_device(ctx, true);
     if (rc)
         return rc;
+    if (S->by_col) { // the same entries with rows and columns, and so A and B, exchanged
+        const spc3d_plan *T = S->by_col;
+        HIP_TRY(launch_sddmm(S->dtype, view_of(T), B->dev, A->dev, C->dev, K, streams_of(ctx)));
+        HIP_TRY(unstage_stores(T, C->dev));
+        return SPC3D_OK;
+    }
     if (S->blocks.empty()) {
         HIP_TRY(launch_sddmm(S->dtype, view_of(S), A->dev, B->dev, C->dev, K, streams_of(ctx)));
         HIP_TRY(unstage_stores(S, C->dev));

@@ -93,6 +93,10 @@ struct StoreStaging {
 int build_store_staging(hipStream_t stream, const Seg *d_segs, uint32_t nseg, const uint32_t *d_perm,
                         uint64_t nnz, StoreStaging &out, std::string &err);
 
+// *out = d[0] <= d[1] <= ... <= d[n - 1] (device array); synchronous.
+int is_nondecreasing_device(hipStream_t stream, const uint32_t *d, uint64_t n, bool *out,
+                            std::string &err);
+
 // Sum of len^2 over a plan's segments (device array); synchronous.
 int sum_sq_seg_len_device(hipStream_t stream, const Seg *d_segs, uint64_t nseg, uint64_t *out,
                           std::string &err);

@@ -1387,6 +1387,33 @@ int build_store_staging(hipStream_t st, const Seg *d_segs, uint32_t nseg, const 
     return SPC3D_OK;
 }
 
+__global__ void descents_k(const uint32_t *__restrict__ d, uint64_t n, unsigned long long *acc)
+{
+    unsigned long long c = 0;
+    GRID_STRIDE(i, n)
+    if (i + 1 < n && d[i + 1] < d[i])
+        ++c;
+    c = wave_sum(c);
+    if ((threadIdx.x & 63u) == 0 && c)
+        atomicAdd(acc, c);
+}
+
+int is_nondecreasing_device(hipStream_t st, const uint32_t *d, uint64_t n, bool *out,
+                            std::string &err)
+{
+    *out = true;
+    if (n < 2)
+        return SPC3D_OK;
+    DBuf<unsigned long long> acc;
+    HIP_OK(acc.alloc(1));
+    HIP_OK(hipMemsetAsync(acc.p, 0, sizeof(unsigned long long), st));
+    LAUNCH_SMALL(descents_k, n, d, n, acc.p);
+    unsigned long long descents = 0;
+    TRY(fetch(st, &descents, acc.p, sizeof descents, err));
+    *out = descents == 0;
+    return SPC3D_OK;
+}
+
 int sum_sq_seg_len_device(hipStream_t st, const Seg *d_segs, uint64_t nseg, uint64_t *out,
                           std::string &err)
 {

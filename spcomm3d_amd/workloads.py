@@ -153,6 +153,15 @@ class Workload:
                         np.ascontiguousarray(self.ii[p]), np.ascontiguousarray(self.jj[p]),
                         np.ascontiguousarray(self.vv64[p]), "shuffled", dict(self.notes))
 
+    def column_major(self) -> "Workload":
+        """Same matrix, entries sorted by column and by row inside a column: the order
+        of a MatrixMarket file, which the reference's converter and readers keep
+        (tools/read_convert_mm.cpp:81-94, src/parallel_io.hpp:132-190)."""
+        p = np.lexsort((self.ii, self.jj))
+        return Workload(self.name, self.nrows, self.ncols, self.k,
+                        np.ascontiguousarray(self.ii[p]), np.ascontiguousarray(self.jj[p]),
+                        np.ascontiguousarray(self.vv64[p]), "column-major", dict(self.notes))
+
 
 def _sort_unique(rows: np.ndarray, cols: np.ndarray):
     key = (rows.astype(np.uint64) << np.uint64(32)) | cols.astype(np.uint64)

@@ -530,11 +530,65 @@ def test_staged_results_of_hub_row_pieces_reach_the_callers_positions(ctx, dtype
         h.close()
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("k", [64, 7, 1030])
+def test_column_sorted_input_runs_sddmm_through_the_exchanged_plan(ctx, dtype, k):
+    """A pattern sorted by column (the order of a MatrixMarket file): spc3d_sddmm runs the plan
+    of the same entries with rows and columns exchanged, A and B exchanged with them (plan info
+    sddmm_by_column).  The results are those of the row-major plan bit for bit (the one-pass
+    call still runs that one), SpMM is untouched, new values reach both plans."""
+    w = W.rmat(14, 16, k)
+    o = np.lexsort((w.ii, w.jj))
+    ii, jj = np.ascontiguousarray(w.ii[o]), np.ascontiguousarray(w.jj[o])
+    A, B, Y0 = w.panel_A(dtype), w.panel_B(dtype), w.panel_Y0(dtype)
+    vv = np.ascontiguousarray(w.values(dtype)[o])
+    S = ctx.plan(w.nrows, w.ncols, ii, jj, vv, xcd_slices=8, l2_hot_bytes=64 * 1024, hub_min=32,
+                 seg_max=256)
+    assert S.info.sddmm_by_column == 1 and S.info.order_is_identity == 0
+    dA, dB, dY, dC = ctx.panel_from(A), ctx.panel_from(B), ctx.panel_from(Y0), ctx.vals(w.nnz, dtype)
+    for _ in range(2):
+        dC.fill(np.nan)
+        ctx.sddmm(S, dA, dB, dC)
+        check_sddmm(A, B, ii, jj, vv, dC.download())
+    by_col = dC.download()
+    ctx.spmm(S, dB, dY)
+    check_spmm(B, ii, jj, vv, Y0, dY.download())
+    if k * np.dtype(dtype).itemsize <= 4096:
+        dC.fill(np.nan)
+        dY.upload(Y0)
+        ctx.sddmm_spmm(S, dA, dB, dC, dY)
+        assert np.array_equal(dC.download(), by_col)
+        check_spmm(B, ii, jj, vv, Y0, dY.download())
+    vv2 = (vv * 0.25 - 1).astype(dtype)
+    S.set_values(vv2)
+    dC.fill(np.nan)
+    ctx.sddmm(S, dA, dB, dC)
+    check_sddmm(A, B, ii, jj, vv2, dC.download())
+    dv = ctx.vals(w.nnz, dtype)
+    dv.upload(vv)
+    S.set_values_device(dv)
+    ctx.sddmm(S, dA, dB, dC)
+    assert np.array_equal(dC.download(), by_col)
+    # rectangular, and sorted by column only (rows inside a column in any order)
+    ii2, jj2, vv3, A2, B2, _ = rand_case(11, 300, 90, k, 5000, dtype, hub=900)
+    o2 = np.argsort(jj2, kind="stable")
+    ii2, jj2, vv3 = (np.ascontiguousarray(x[o2]) for x in (ii2, jj2, vv3))
+    S2 = ctx.plan(300, 90, ii2, jj2, vv3)
+    assert S2.info.sddmm_by_column == 1
+    dA2, dB2, dC2 = ctx.panel_from(A2), ctx.panel_from(B2), ctx.vals(5000, dtype)
+    dC2.fill(np.nan)
+    ctx.sddmm(S2, dA2, dB2, dC2)
+    check_sddmm(A2, B2, ii2, jj2, vv3, dC2.download())
+    for h in (S, S2, dA, dB, dY, dC, dv, dA2, dB2, dC2):
+        h.close()
+
+
 def test_a_shuffled_pattern_keeps_its_stores_unstaged(ctx):
     # every segment's positions are scattered and so would be the final pass: no staging
     w = W.rmat(14, 16, 64).shuffled()
     S = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, w.values(np.float32))
     assert S.info.order_is_identity == 0 and S.info.staged_entries == 0
+    assert S.info.sddmm_by_column == 0
     S.close()
 
 
