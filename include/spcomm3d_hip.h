@@ -105,6 +105,12 @@ typedef struct {
                                   so A and B) exchanged, whose kernel order is the caller's:
                                   the same bits, stored in runs instead of one by one; the
                                   plan then holds its arrays twice (GPU builder only) */
+    uint32_t two_pass_results; /* 1: an arbitrary entry order of 2^22 entries or more: the
+                                  SDDMM kernels write their results in kernel order to a
+                                  vector of the plan, and two passes of tile-local moves
+                                  through LDS bring them to the caller's positions (24 more
+                                  bytes per entry in fp64, 16 in fp32) */
+    uint32_t reserved1;
 } spc3d_plan_info;
 
 /* Plan tuning; a zero field selects the default.  Only speed depends on these. */
@@ -230,8 +236,9 @@ SPC3D_API int spc3d_coo_validate(uint32_t nrows, uint32_t ncols, uint64_t nnz,
  * SPC3D_PLAN_BUILDER=host in the environment (spc3d_plan_create only) selects
  * the single-threaded host builder instead.  How spc3d_sddmm brings its results to
  * the caller's positions is settled here as well (spc3d_plan_info: staged_entries,
- * positions_by_segment, sddmm_by_column; the environment variables SPC3D_STAGE_STORES=0
- * and SPC3D_SDDMM_BY_COLUMN=0 keep the plain form, for comparisons).  `vv` (nnz reals of
+ * positions_by_segment, sddmm_by_column, two_pass_results; the environment variables
+ * SPC3D_STAGE_STORES=0, SPC3D_SDDMM_BY_COLUMN=0 and SPC3D_TWO_PASS=0 keep the plain form,
+ * for comparisons).  `vv` (nnz reals of
  * `dtype`, caller's order) may be NULL and set later.  The pattern is copied:
  * the caller's arrays are not referenced afterwards.  Replaces nothing in the
  * reference (it walks the unsorted COO directly, core_ops.cpp:7-10); it is the

@@ -32,7 +32,8 @@ class PlanInfo(ctypes.Structure):
                 ("hot_cols", c_u32), ("hub_rows", c_u32), ("hot_entries", c_u64),
                 ("nsegments_long", c_u32), ("ncol_blocks", c_u32),
                 ("staged_entries", c_u64), ("positions_by_segment", c_u32),
-                ("sddmm_by_column", c_u32)]
+                ("sddmm_by_column", c_u32), ("two_pass_results", c_u32),
+                ("reserved1", c_u32)]
 
 
 class PlanOpts(ctypes.Structure):

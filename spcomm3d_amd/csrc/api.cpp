@@ -199,7 +199,12 @@ struct spc3d_plan {
     // spc3d_sddmm runs it with A and B exchanged (the same products summed in the same
     // order: the same bits).  SpMM and the one-pass call run this plan.
     spc3d_plan *by_col = nullptr;
-    void *c_stage = nullptr;       // [nnz] reals (column blocks), [store.n] (staged segments)
+    // An arbitrary entry order (neither of the above applies): the kernels write their results
+    // in kernel order into c_stage, and two tile-local passes through c_mid bring them to the
+    // caller's positions (TwoPass in plan_device.h).
+    TwoPass two;
+    void *c_mid = nullptr; // [nnz] reals
+    void *c_stage = nullptr;       // [nnz] reals (column blocks, two passes), [store.n] (staged segments)
     uint32_t *stage_pos = nullptr; // [nnz] caller's position -> staging position
     uint32_t *stage_of = nullptr;  // [nnz]
     uint64_t stage_off = 0;
@@ -320,11 +325,17 @@ void plan_free_device(spc3d_plan *p)
     if (p->store.perm2) (void)hipFree(p->store.perm2);
     if (p->store.dst) (void)hipFree(p->store.dst);
     if (p->store.src) (void)hipFree(p->store.src);
-    if (p->store.n && p->c_stage) {
+    if ((p->store.n || p->two.n) && p->c_stage) {
         (void)hipFree(p->c_stage);
         p->c_stage = nullptr;
     }
     p->store = StoreStaging();
+    if (p->two.l1) (void)hipFree(p->two.l1);
+    if (p->two.dst1) (void)hipFree(p->two.dst1);
+    if (p->two.l2) (void)hipFree(p->two.l2);
+    if (p->c_mid) (void)hipFree(p->c_mid);
+    p->two = TwoPass();
+    p->c_mid = nullptr;
     if (p->partial) (void)hipFree(p->partial);
     for (void *old : p->retired_partial)
         (void)hipFree(old);
@@ -363,6 +374,8 @@ DevPlanView view_of(const spc3d_plan *p)
     v.first_cols = p->first_cols;
     v.nnz = p->info.nnz;
     v.seg_base = p->store.consecutive;
+    if (p->two.n)
+        v.perm = nullptr; // results in kernel order (into c_stage, see sddmm_out)
     if (p->store.n) {
         v.perm = p->store.perm2;
         v.stage = p->c_stage;
@@ -998,6 +1011,8 @@ static void fill_info(spc3d_plan_info &info, const HostPlan &H)
     info.staged_entries = 0;
     info.positions_by_segment = 0;
     info.sddmm_by_column = 0;
+    info.two_pass_results = 0;
+    info.reserved1 = 0;
 }
 
 // Library defaults, overridable field by field.  With XCD slicing, 2 MiB of
@@ -1081,15 +1096,19 @@ static int finish_plan(spc3d_plan *p, uint32_t k0)
     return ensure_partial(p, k0);
 }
 
+// A switch in the environment, read at every plan creation: set to 0 it keeps the plain form.
+static bool env_off(const char *name)
+{
+    const char *e = std::getenv(name);
+    return e && *e && std::atoi(e) == 0;
+}
+
 // A finished single plan (not a block of a plan kept in column blocks) whose kernel order
 // regroups entries inside rows gets the staging of its SDDMM results (see StoreStaging).
 // SPC3D_STAGE_STORES=0 in the environment keeps every result on its way straight to C.
 static int add_store_staging(spc3d_plan *p)
 {
-    static const bool off = [] {
-        const char *e = std::getenv("SPC3D_STAGE_STORES");
-        return e && std::atoi(e) == 0;
-    }();
+    const bool off = env_off("SPC3D_STAGE_STORES");
     if (off || !p->perm || !p->blocks.empty())
         return SPC3D_OK;
     std::string err;
@@ -1123,6 +1142,59 @@ static hipError_t unstage_stores(const spc3d_plan *S, void *C)
         return hipSuccess;
     return launch_unstage_pairs(S->dtype, S->c_stage, S->store.src, S->store.dst, C, S->store.n,
                                 S->ctx->stream);
+}
+
+// Where a single plan's SDDMM kernels write: C, or the plan's staging vector when the two
+// passes bring the results home afterwards.
+static void *sddmm_out(const spc3d_plan *S, void *C) { return S->two.n ? S->c_stage : C; }
+static hipError_t finish_sddmm(const spc3d_plan *S, void *C)
+{
+    if (S->two.n)
+        return launch_unpermute_two_pass(S->dtype, S->c_stage, S->c_mid, S->two.l1, S->two.dst1,
+                                         S->two.l2, C, S->two.n, S->ctx->stream);
+    return unstage_stores(S, C);
+}
+
+// The two-pass tables of a finished single plan whose results would each be a store of its
+// own (an arbitrary entry order), from 2^22 entries on (SPC3D_TWO_PASS_MIN in the environment
+// gives another bound): below that the scattered stores mostly meet in the L2s.
+// SPC3D_TWO_PASS=0 in the environment switches it off.
+static int add_two_pass(spc3d_plan *p)
+{
+    const bool off = env_off("SPC3D_TWO_PASS");
+    uint64_t least = 1ull << 22;
+    if (const char *e = std::getenv("SPC3D_TWO_PASS_MIN")) // for tests on small patterns
+        least = std::strtoull(e, nullptr, 10);
+    if (off || !p->perm || p->store.consecutive || p->by_col || !p->blocks.empty() ||
+        p->info.nnz < least)
+        return SPC3D_OK;
+    int lds = 0;
+    if (hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerBlock, p->ctx->device) !=
+            hipSuccess ||
+        lds < (int)two_pass_lds_bytes())
+        return SPC3D_OK;
+    std::string err;
+    TwoPass tp;
+    int rc = build_two_pass(p->ctx->stream, p->perm, p->info.nnz, two_pass_tile_elems(p->dtype), tp,
+                            err);
+    if (rc)
+        return fail(rc, err);
+    if (!tp.n)
+        return SPC3D_OK;
+    const size_t bytes = (size_t)p->info.nnz * elem_size(p->dtype);
+    rc = dev_alloc_bytes(&p->c_stage, bytes);
+    if (!rc) rc = dev_alloc_bytes(&p->c_mid, bytes);
+    if (rc) {
+        (void)hipFree(tp.l1);
+        (void)hipFree(tp.dst1);
+        (void)hipFree(tp.l2);
+        if (p->c_stage) (void)hipFree(p->c_stage);
+        p->c_stage = nullptr;
+        return rc;
+    }
+    p->two = tp;
+    p->info.two_pass_results = 1;
+    return SPC3D_OK;
 }
 
 // Row width a plan is created for: sizes the partial-sum rows of its cut rows.
@@ -1228,10 +1300,7 @@ static int choose_col_blocks(spc3d_plan *p, const spc3d_plan_opts *opts, uint32_
 static int add_sddmm_companion(spc3d_plan *p, uint32_t nrows, uint32_t ncols, uint64_t nnz,
                                const uint32_t *d_ii, const uint32_t *d_jj, const PlanOpts &po)
 {
-    static const bool off = [] {
-        const char *e = std::getenv("SPC3D_SDDMM_BY_COLUMN");
-        return e && std::atoi(e) == 0;
-    }();
+    const bool off = env_off("SPC3D_SDDMM_BY_COLUMN");
     if (off || nnz < 2 || !p->perm || p->store.consecutive || !p->blocks.empty())
         return SPC3D_OK;
     std::string err;
@@ -1289,6 +1358,8 @@ static int build_from_device(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t
         rc = add_store_staging(p);
     if (!rc && nb <= 1)
         rc = add_sddmm_companion(p, nrows, ncols, nnz, d_ii, d_jj, po);
+    if (!rc && nb <= 1)
+        rc = add_two_pass(p);
     if (rc || nb <= 1) {
         if (rc) {
             const std::string keep = g_err;
@@ -1508,6 +1579,8 @@ int spc3d_plan_create_ex(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t nco
             rc = finish_plan(p, planned_k(opts));
         if (!rc)
             rc = add_store_staging(p);
+        if (!rc)
+            rc = add_two_pass(p);
         if (rc) {
             plan_free_device(p);
             delete p;
@@ -1843,8 +1916,9 @@ int spc3d_sddmm(spc3d_ctx *ctx, spc3d_plan *S, const spc3d_panel *A, const spc3d
         return SPC3D_OK;
     }
     if (S->blocks.empty()) {
-        HIP_TRY(launch_sddmm(S->dtype, view_of(S), A->dev, B->dev, C->dev, K, streams_of(ctx)));
-        HIP_TRY(unstage_stores(S, C->dev));
+        HIP_TRY(launch_sddmm(S->dtype, view_of(S), A->dev, B->dev, sddmm_out(S, C->dev), K,
+                             streams_of(ctx)));
+        HIP_TRY(finish_sddmm(S, C->dev));
         return SPC3D_OK;
     }
     for (spc3d_plan *part : S->blocks)
@@ -1972,7 +2046,7 @@ int spc3d_sddmm_spmm(spc3d_ctx *ctx, spc3d_plan *S, const spc3d_panel *A, const 
     const bool staged = !S->blocks.empty();
     for (spc3d_plan *part : parts_of(S, self)) {
         const DevPlanView view = staged ? staged_view(S, part) : view_of(part);
-        void *out = staged ? staged_out(S, part) : C->dev;
+        void *out = staged ? staged_out(S, part) : sddmm_out(S, C->dev);
         hipError_t e = launch_sddmm_spmm(S->dtype, chained != 0, view, A->dev, B->dev, out, Y->dev,
                                          K, streams_of(ctx));
         if (e == hipErrorNotSupported) {
@@ -1991,7 +2065,7 @@ int spc3d_sddmm_spmm(spc3d_ctx *ctx, spc3d_plan *S, const spc3d_panel *A, const 
     if (staged)
         HIP_TRY(unstage(S, C));
     else
-        HIP_TRY(unstage_stores(S, C->dev));
+        HIP_TRY(finish_sddmm(S, C->dev));
     return SPC3D_OK;
 }
 

@@ -67,6 +67,14 @@ hipError_t launch_unstage(int dtype, const void *in, const uint32_t *pos, void *
 // out[dst[h]] = stage[src[h]], h < n (dst ascending, mostly consecutive)
 hipError_t launch_unstage_pairs(int dtype, const void *stage, const uint32_t *src,
                                 const uint32_t *dst, void *out, uint64_t n, hipStream_t stream);
+// out[perm[p]] = stage[p] for the permutation whose two-pass tables (TwoPass in plan_device.h,
+// built for tiles of two_pass_tile_elems(dtype) elements) are l1, dst1, l2; `mid` holds n reals
+// in between.  Needs two_pass_lds_bytes() of LDS per workgroup (all 160 KiB of a gfx950 CU).
+uint32_t two_pass_tile_elems(int dtype);
+uint32_t two_pass_lds_bytes();
+hipError_t launch_unpermute_two_pass(int dtype, const void *stage, void *mid, const uint16_t *l1,
+                                     const uint32_t *dst1, const uint16_t *l2, void *out, uint64_t n,
+                                     hipStream_t stream);
 // out[p] = in[perm[p]] (perm == null: copy)
 hipError_t launch_gather_vals(int dtype, const void *in, const uint32_t *perm, void *out,
                               uint64_t n, hipStream_t stream);

@@ -1233,6 +1233,140 @@ unstage_pairs_kernel(const T *__restrict__ stage, const uint32_t *__restrict__ s
         out[dst[h]] = stage[src[h]];
 }
 
+// ---- results of an arbitrary entry order to the caller's positions in two passes ------
+// (see TwoPass in plan_device.h).  One workgroup per tile of kTwoPassBytes of results,
+// held in LDS between its coalesced read and its grouped write.
+constexpr uint32_t kTwoPassBytes = 160u << 10; // all of a CU's LDS
+constexpr int kTwoPassBlock = 1024;
+template <typename T> constexpr uint32_t two_pass_tile() { return kTwoPassBytes / sizeof(T); }
+
+template <typename T>
+__device__ __forceinline__ void tile_to_lds(T *buf, const T *__restrict__ src, uint32_t cnt)
+{
+    using V = typename Vec<T>::type;
+    constexpr uint32_t VN = Vec<T>::N;
+    constexpr uint32_t TILE = two_pass_tile<T>();
+    constexpr uint32_t R = TILE / VN / kTwoPassBlock; // 16-byte loads per lane and tile: 10
+    static_assert(R * VN * kTwoPassBlock == TILE, "a tile is a whole number of rounds");
+    const V *in = reinterpret_cast<const V *>(src); // 16-byte aligned: a whole tile into a library buffer
+    V *to = reinterpret_cast<V *>(buf);
+    if (cnt == TILE) { // every load in flight before the first word is stored
+        V v[R];
+#pragma unroll
+        for (uint32_t r = 0; r < R; ++r)
+            v[r] = nt_load(in + threadIdx.x + r * kTwoPassBlock);
+#pragma unroll
+        for (uint32_t r = 0; r < R; ++r)
+            to[threadIdx.x + r * kTwoPassBlock] = v[r];
+        return;
+    }
+    const uint32_t nvec = cnt / VN;
+    for (uint32_t i = threadIdx.x; i < nvec; i += kTwoPassBlock)
+        to[i] = nt_load(in + i);
+    for (uint32_t i = nvec * VN + threadIdx.x; i < cnt; i += kTwoPassBlock)
+        buf[i] = src[i];
+}
+
+// Pass 1: tile blockIdx.x of `stage` (kernel order), out grouped by bucket of destination.
+template <typename T>
+__global__ void __launch_bounds__(kTwoPassBlock)
+unpermute_pass1_kernel(const T *__restrict__ stage, const uint16_t *__restrict__ l1,
+                       const uint32_t *__restrict__ dst1, T *__restrict__ mid, uint64_t n)
+{
+    constexpr uint32_t TILE = two_pass_tile<T>();
+    __shared__ T buf[TILE];
+    const uint64_t base = (uint64_t)blockIdx.x * TILE;
+    if (base >= n)
+        return;
+    const uint32_t cnt = (uint32_t)(n - base < TILE ? n - base : TILE);
+    constexpr uint32_t U = 10;
+    // the first positions are asked for before the tile is: they do not depend on it
+    uint32_t l[U], d[U];
+    uint32_t s = threadIdx.x;
+    const bool first_full = s + (U - 1) * kTwoPassBlock < cnt;
+    if (first_full) {
+#pragma unroll
+        for (uint32_t u = 0; u < U; ++u) {
+            l[u] = nt_load(l1 + base + s + u * kTwoPassBlock);
+            d[u] = nt_load(dst1 + base + s + u * kTwoPassBlock);
+        }
+    }
+    tile_to_lds(buf, stage + base, cnt);
+    __syncthreads();
+    if (first_full) {
+#pragma unroll
+        for (uint32_t u = 0; u < U; ++u)
+            nt_store(buf[l[u]], mid + d[u]);
+        s += U * kTwoPassBlock;
+    }
+    for (; s + (U - 1) * kTwoPassBlock < cnt; s += U * kTwoPassBlock) {
+#pragma unroll
+        for (uint32_t u = 0; u < U; ++u) {
+            l[u] = nt_load(l1 + base + s + u * kTwoPassBlock);
+            d[u] = nt_load(dst1 + base + s + u * kTwoPassBlock);
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < U; ++u)
+            nt_store(buf[l[u]], mid + d[u]);
+    }
+    for (; s < cnt; s += kTwoPassBlock)
+        nt_store(buf[nt_load(l1 + base + s)], mid + nt_load(dst1 + base + s));
+}
+
+// Pass 2: bucket blockIdx.x of `mid`, out to the caller's positions [base, base + cnt) in order.
+template <typename T>
+__global__ void __launch_bounds__(kTwoPassBlock)
+unpermute_pass2_kernel(const T *__restrict__ mid, const uint16_t *__restrict__ l2,
+                       T *__restrict__ C, uint64_t n)
+{
+    using V = typename Vec<T>::type;
+    constexpr uint32_t VN = Vec<T>::N;
+    constexpr uint32_t TILE = two_pass_tile<T>();
+    __shared__ T buf[TILE];
+    const uint64_t base = (uint64_t)blockIdx.x * TILE;
+    if (base >= n)
+        return;
+    const uint32_t cnt = (uint32_t)(n - base < TILE ? n - base : TILE);
+    typedef uint16_t Idx __attribute__((ext_vector_type(VN)));
+    constexpr uint32_t R = TILE / VN / kTwoPassBlock; // 16-byte stores per lane and tile: 10
+    T *out = C + base;
+    const bool fast = cnt == TILE && (reinterpret_cast<uintptr_t>(out) & 15u) == 0;
+    Idx li[R];
+    if (fast) { // the positions do not depend on the tile: asked for first
+#pragma unroll
+        for (uint32_t r = 0; r < R; ++r)
+            li[r] = nt_load(reinterpret_cast<const Idx *>(l2 + base) + threadIdx.x + r * kTwoPassBlock);
+    }
+    tile_to_lds(buf, mid + base, cnt);
+    __syncthreads();
+    if (fast) {
+#pragma unroll
+        for (uint32_t r = 0; r < R; ++r) {
+            V v;
+#pragma unroll
+            for (uint32_t e = 0; e < VN; ++e)
+                v[e] = buf[li[r][e]];
+            nt_store(v, reinterpret_cast<V *>(out) + threadIdx.x + r * kTwoPassBlock);
+        }
+        return;
+    }
+    uint32_t done = 0;
+    if ((reinterpret_cast<uintptr_t>(out) & 15u) == 0) { // the caller's C may be a wrapped vector
+        const uint32_t nvec = cnt / VN;
+        for (uint32_t i = threadIdx.x; i < nvec; i += kTwoPassBlock) {
+            const Idx l = nt_load(reinterpret_cast<const Idx *>(l2 + base) + i);
+            V v;
+#pragma unroll
+            for (uint32_t e = 0; e < VN; ++e)
+                v[e] = buf[l[e]];
+            nt_store(v, reinterpret_cast<V *>(out) + i);
+        }
+        done = nvec * VN;
+    }
+    for (uint32_t j = done + threadIdx.x; j < cnt; j += kTwoPassBlock)
+        out[j] = buf[l2[base + j]];
+}
+
 template <typename T>
 __global__ void __launch_bounds__(kBlock) fill_kernel(T *__restrict__ p, uint64_t n, T value)
 {
@@ -1668,6 +1802,35 @@ hipError_t launch_unstage_pairs(int dtype, const void *stage, const uint32_t *sr
     else
         hipLaunchKernelGGL((unstage_pairs_kernel<float>), dim3(grid), dim3(kBlock), 0, stream,
                            (const float *)stage, src, dst, (float *)out, n);
+    return hipGetLastError();
+}
+
+uint32_t two_pass_lds_bytes() { return kTwoPassBytes; }
+
+uint32_t two_pass_tile_elems(int dtype)
+{
+    return dtype == 1 ? two_pass_tile<double>() : two_pass_tile<float>();
+}
+
+hipError_t launch_unpermute_two_pass(int dtype, const void *stage, void *mid, const uint16_t *l1,
+                                     const uint32_t *dst1, const uint16_t *l2, void *out, uint64_t n,
+                                     hipStream_t stream)
+{
+    if (n == 0)
+        return hipSuccess;
+    const uint64_t T = two_pass_tile_elems(dtype);
+    const uint32_t grid = (uint32_t)((n + T - 1) / T);
+    if (dtype == 1) {
+        hipLaunchKernelGGL((unpermute_pass1_kernel<double>), dim3(grid), dim3(kTwoPassBlock), 0,
+                           stream, (const double *)stage, l1, dst1, (double *)mid, n);
+        hipLaunchKernelGGL((unpermute_pass2_kernel<double>), dim3(grid), dim3(kTwoPassBlock), 0,
+                           stream, (const double *)mid, l2, (double *)out, n);
+    } else {
+        hipLaunchKernelGGL((unpermute_pass1_kernel<float>), dim3(grid), dim3(kTwoPassBlock), 0,
+                           stream, (const float *)stage, l1, dst1, (float *)mid, n);
+        hipLaunchKernelGGL((unpermute_pass2_kernel<float>), dim3(grid), dim3(kTwoPassBlock), 0,
+                           stream, (const float *)mid, l2, (float *)out, n);
+    }
     return hipGetLastError();
 }
 

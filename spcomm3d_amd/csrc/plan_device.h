@@ -93,6 +93,32 @@ struct StoreStaging {
 int build_store_staging(hipStream_t stream, const Seg *d_segs, uint32_t nseg, const uint32_t *d_perm,
                         uint64_t nnz, StoreStaging &out, std::string &err);
 
+// ---- SDDMM results of an arbitrary entry order, brought home in two passes -------------
+// C[perm[p]] = r[p] for all p, with r in kernel order, is one store (or one load) per result
+// into a line of its own however it is turned.  Any permutation of n elements is two passes
+// of tile-local moves when tile^2 >= n: with T elements per tile (what fits LDS),
+//   pass 1, tile t of r (kernel positions [tT, tT + T)): the tile is read into LDS and written
+//           out grouped by bucket of destination (bucket b = caller's positions [bT, bT + T)),
+//           into an intermediate vector laid out bucket by bucket, inside a bucket tile by
+//           tile: runs of about T^2 / n elements;
+//   pass 2, bucket b of the intermediate vector: read into LDS, written to C in order.
+// Everything is fixed by `perm`, so the plan holds, per element,
+//   l1[s]   = which element of its tile goes to slot s of the tile's output order  (uint16)
+//   dst1[s] = where slot s goes in the intermediate vector                         (uint32)
+//   l2[q]   = which element of its bucket (as the intermediate vector holds it) is the
+//             result for caller's position q                                      (uint16)
+// T <= 65536.  n == 0: not built (n < 2 tiles, or the tile pairs do not fit a 32-bit sort key).
+// The arrays belong to the receiver (hipFree).  Synchronous.
+struct TwoPass {
+    uint16_t *l1 = nullptr;  // [n]
+    uint32_t *dst1 = nullptr; // [n]
+    uint16_t *l2 = nullptr;  // [n]
+    uint32_t tile = 0;       // T
+    uint64_t n = 0;
+};
+int build_two_pass(hipStream_t stream, const uint32_t *d_perm, uint64_t nnz, uint32_t tile,
+                   TwoPass &out, std::string &err);
+
 // *out = d[0] <= d[1] <= ... <= d[n - 1] (device array); synchronous.
 int is_nondecreasing_device(hipStream_t stream, const uint32_t *d, uint64_t n, bool *out,
                             std::string &err);

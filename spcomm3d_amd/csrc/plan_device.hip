@@ -1387,6 +1387,87 @@ int build_store_staging(hipStream_t st, const Seg *d_segs, uint32_t nseg, const 
     return SPC3D_OK;
 }
 
+// key1 = tile of the kernel position, then bucket of the caller's position; key2 the other
+// way round
+__global__ void two_pass_keys_k(const uint32_t *__restrict__ perm, uint64_t n, uint32_t T,
+                                uint32_t ntiles, uint32_t *key1, uint32_t *key2)
+{
+    GRID_STRIDE(p, n)
+    {
+        const uint32_t t = (uint32_t)(p / T), b = perm[p] / T;
+        key1[p] = t * ntiles + b;
+        key2[p] = b * ntiles + t;
+    }
+}
+
+__global__ void two_pass_mid_k(const uint32_t *__restrict__ sp2, const uint32_t *__restrict__ perm,
+                               uint64_t n, uint32_t T, uint32_t *mid_of, uint16_t *l2)
+{
+    GRID_STRIDE(m, n)
+    {
+        const uint32_t p = sp2[m];
+        mid_of[p] = (uint32_t)m;
+        l2[perm[p]] = (uint16_t)(m % T);
+    }
+}
+
+__global__ void two_pass_slots_k(const uint32_t *__restrict__ sp1,
+                                 const uint32_t *__restrict__ mid_of, uint64_t n, uint32_t T,
+                                 uint16_t *l1, uint32_t *dst1)
+{
+    GRID_STRIDE(s, n)
+    {
+        const uint32_t p = sp1[s];
+        l1[s] = (uint16_t)(p - (uint32_t)(s / T) * T); // the sort kept every tile in its place
+        dst1[s] = mid_of[p];
+    }
+}
+
+int build_two_pass(hipStream_t st, const uint32_t *d_perm, uint64_t nnz, uint32_t T, TwoPass &out,
+                   std::string &err)
+{
+    out = TwoPass();
+    if (!d_perm || T == 0 || T > 65536 || nnz >= (1ull << 32) || nnz < 2ull * T)
+        return SPC3D_OK;
+    const uint64_t ntiles64 = (nnz + T - 1) / T;
+    if (ntiles64 * ntiles64 >= (1ull << 32))
+        return SPC3D_OK;
+    const uint32_t ntiles = (uint32_t)ntiles64;
+    Arena arena;
+    HIP_OK(arena.reserve((size_t)nnz * 24 + ((size_t)8 << 20)));
+    Temp tmp(arena);
+    SBuf<uint32_t> key1, key2, idx, key_out, sp1, sp2, mid_of;
+    HIP_OK(key1.alloc(arena, nnz));
+    HIP_OK(key2.alloc(arena, nnz));
+    HIP_OK(idx.alloc(arena, nnz));
+    HIP_OK(key_out.alloc(arena, nnz));
+    HIP_OK(sp1.alloc(arena, nnz));
+    HIP_OK(sp2.alloc(arena, nnz));
+    LAUNCH(two_pass_keys_k, nnz, d_perm, nnz, T, ntiles, key1.p, key2.p);
+    LAUNCH(iota_k, nnz, idx.p, nnz);
+    const int bits = bits_for(ntiles64 * ntiles64 - 1);
+    TRY(sort_pairs<uint32_t>(tmp, key1.p, key_out.p, idx.p, sp1.p, (uint32_t)nnz, bits, false, st,
+                             err));
+    TRY(sort_pairs<uint32_t>(tmp, key2.p, key_out.p, idx.p, sp2.p, (uint32_t)nnz, bits, false, st,
+                             err));
+    mid_of.p = key1.p; // the keys are no longer needed
+    DBuf<uint16_t> l1, l2;
+    DBuf<uint32_t> dst1;
+    HIP_OK(l1.alloc(nnz));
+    HIP_OK(l2.alloc(nnz));
+    HIP_OK(dst1.alloc(nnz));
+    LAUNCH(two_pass_mid_k, nnz, sp2.p, d_perm, nnz, T, mid_of.p, l2.p);
+    LAUNCH(two_pass_slots_k, nnz, sp1.p, mid_of.p, nnz, T, l1.p, dst1.p);
+    HIP_OK(hipGetLastError());
+    HIP_OK(hipStreamSynchronize(st));
+    out.l1 = l1.release();
+    out.l2 = l2.release();
+    out.dst1 = dst1.release();
+    out.tile = T;
+    out.n = nnz;
+    return SPC3D_OK;
+}
+
 __global__ void descents_k(const uint32_t *__restrict__ d, uint64_t n, unsigned long long *acc)
 {
     unsigned long long c = 0;

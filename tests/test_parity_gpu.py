@@ -11,6 +11,7 @@ import numpy as np
 import pytest
 
 from spcomm3d_amd import _capi as capi
+from spcomm3d_amd import device
 from spcomm3d_amd import workloads as W
 from tests import _oracle as oracle
 
@@ -580,6 +581,62 @@ def test_column_sorted_input_runs_sddmm_through_the_exchanged_plan(ctx, dtype, k
     ctx.sddmm(S2, dA2, dB2, dC2)
     check_sddmm(A2, B2, ii2, jj2, vv3, dC2.download())
     for h in (S, S2, dA, dB, dY, dC, dv, dA2, dB2, dC2):
+        h.close()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_arbitrary_order_brings_results_home_in_two_passes(ctx, dtype, monkeypatch):
+    """An arbitrary entry order: the kernels write in kernel order, two passes of tile-local
+    moves bring the results to the caller's positions (plan info two_pass_results; from 2^22
+    entries on by default, here from the smallest size the scheme takes).  Bit for bit what the
+    plain plan stores, through spc3d_sddmm and both one-pass forms, wide rows included, and
+    into a wrapped value vector."""
+    w = W.rmat(14, 16, 64).shuffled()
+    A, B, Y0, vv = w.panel_A(dtype), w.panel_B(dtype), w.panel_Y0(dtype), w.values(dtype)
+    monkeypatch.setenv("SPC3D_TWO_PASS", "0")
+    plain = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, vv)
+    monkeypatch.delenv("SPC3D_TWO_PASS")
+    monkeypatch.setenv("SPC3D_TWO_PASS_MIN", "1")
+    S = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, vv)
+    tiny = ctx.plan(w.nrows, w.ncols, w.ii[:1000], w.jj[:1000], vv[:1000])  # under two tiles
+    monkeypatch.delenv("SPC3D_TWO_PASS_MIN")
+    assert plain.info.two_pass_results == 0 and tiny.info.two_pass_results == 0
+    assert S.info.two_pass_results == 1 and S.info.staged_entries == 0
+    dA, dB, dY, dC = ctx.panel_from(A), ctx.panel_from(B), ctx.panel_from(Y0), ctx.vals(w.nnz, dtype)
+    ctx.sddmm(plain, dA, dB, dC)
+    want = dC.download()
+    check_sddmm(A, B, w.ii, w.jj, vv, want)
+    for _ in range(2):
+        dC.fill(np.nan)
+        ctx.sddmm(S, dA, dB, dC)
+        assert np.array_equal(dC.download(), want)
+    for chained in (False, True):
+        dC.fill(np.nan)
+        dY.upload(Y0)
+        ctx.sddmm_spmm(S, dA, dB, dC, dY, chained=chained)
+        assert np.array_equal(dC.download(), want)
+        check_spmm(B, w.ii, w.jj, want if chained else vv, Y0, dY.download())
+    lead = 16 // np.dtype(dtype).itemsize  # C some way into a vector the caller owns
+    big = ctx.vals(w.nnz + 3 * lead, dtype)
+    big.fill(np.nan)
+    inner = device.Vals(ctx, w.nnz, dtype, dev=big.device_ptr() + 3 * 16)
+    ctx.sddmm(S, dA, dB, inner)
+    assert np.array_equal(big.download()[3 * lead:], want)
+    inner.close()
+    big.close()
+    # SpMM and the plan's own arrays know nothing of it
+    dY.upload(Y0)
+    ctx.spmm(S, dB, dY)
+    check_spmm(B, w.ii, w.jj, vv, Y0, dY.download())
+    assert np.array_equal(S.download()["perm"], plain.download()["perm"])
+    # rows over 4 KiB: several launches that accumulate in the staging vector
+    wk = W.rmat(14, 16, 1030).shuffled()
+    Ak, Bk = wk.panel_A(dtype), wk.panel_B(dtype)
+    dAk, dBk = ctx.panel_from(Ak), ctx.panel_from(Bk)
+    dC.fill(np.nan)
+    ctx.sddmm(S, dAk, dBk, dC)
+    check_sddmm(Ak, Bk, w.ii, w.jj, vv, dC.download())
+    for h in (S, plain, tiny, dA, dB, dY, dC, dAk, dBk):
         h.close()
 
 
