@@ -28,7 +28,12 @@
 //          are DPP moves, those across rows the gfx950 row swaps
 //          (v_permlane16_swap, v_permlane32_swap).  The lane that ends up
 //          with entry u's dot product scales it by S.vv and stores it at the
-//          caller's position.
+//          caller's position: read per entry, or once per segment where a
+//          segment's positions are consecutive; segments for which they are
+//          not store in kernel order to a staging vector instead
+//          (unstage_pairs_kernel brings those home), and for an arbitrary
+//          entry order everything is stored in kernel order and brought home
+//          by two tile-local passes through LDS (unpermute_pass1/2_kernel).
 //   spmm : lane = slice of K, no cross-lane reduction; the group accumulates
 //          a * X[c,:] in registers and does one read-modify-write of the Y
 //          row slice.  Rows cut into several segments write partial sums that
