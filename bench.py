@@ -365,7 +365,7 @@ def main():
     ap.add_argument("--config", default="rmat20", help="workload name (spcomm3d_amd.workloads)")
     ap.add_argument("--dtype", default="f64", choices=["f32", "f64"],
                     help="real type of the headline value (the reference's is f64)")
-    ap.add_argument("--order", default="sorted", choices=["sorted", "shuffled"],
+    ap.add_argument("--order", default="sorted", choices=["sorted", "shuffled", "column-major"],
                     help="order in which the COO entries are handed to the library")
     ap.add_argument("--seg-max", type=int, default=None)
     ap.add_argument("--calibration-copies", type=int, default=0,
@@ -388,6 +388,8 @@ def main():
     w = W.make(args.config)
     if args.order == "shuffled":
         w = w.shuffled()
+    elif args.order == "column-major":
+        w = w.column_major()
     log(f"workload {w.name}: {w.nrows}x{w.ncols} nnz={w.nnz} K={w.k} order={w.order} "
         f"(generated in {time.perf_counter() - t0:.1f}s)")
 

@@ -199,9 +199,10 @@ struct spc3d_plan {
     // spc3d_sddmm runs it with A and B exchanged (the same products summed in the same
     // order: the same bits).  SpMM and the one-pass call run this plan.
     spc3d_plan *by_col = nullptr;
-    // An arbitrary entry order (neither of the above applies): the kernels write their results
-    // in kernel order into c_stage, and two tile-local passes through c_mid bring them to the
-    // caller's positions (TwoPass in plan_device.h).
+    // An arbitrary entry order (no runs to store in this plan's kernel order): the kernels
+    // write their results in kernel order into c_stage, and two tile-local passes through
+    // c_mid bring them to the caller's positions (TwoPass in plan_device.h).  With `by_col`
+    // this serves the one-pass call only.
     TwoPass two;
     void *c_mid = nullptr; // [nnz] reals
     void *c_stage = nullptr;       // [nnz] reals (column blocks, two passes), [store.n] (staged segments)
@@ -1165,8 +1166,7 @@ static int add_two_pass(spc3d_plan *p)
     uint64_t least = 1ull << 22;
     if (const char *e = std::getenv("SPC3D_TWO_PASS_MIN")) // for tests on small patterns
         least = std::strtoull(e, nullptr, 10);
-    if (off || !p->perm || p->store.consecutive || p->by_col || !p->blocks.empty() ||
-        p->info.nnz < least)
+    if (off || !p->perm || p->store.consecutive || !p->blocks.empty() || p->info.nnz < least)
         return SPC3D_OK;
     int lds = 0;
     if (hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerBlock, p->ctx->device) !=
