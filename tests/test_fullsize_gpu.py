@@ -17,9 +17,11 @@ from tests import _oracle as oracle
 pytestmark = pytest.mark.gpu
 
 
-def _check_sampled(ctx, w, dtype, n_entries=200_000, n_rows=3000, seed=9, col_blocks=None):
+def _check_sampled(ctx, w, dtype, n_entries=200_000, n_rows=3000, seed=9, col_blocks=None,
+                   how=None):
     """col_blocks: None = a plan with every option at its default; "auto" = the plan must
-    have chosen column blocks by itself (k_hint given, as bench.py does)."""
+    have chosen column blocks by itself (k_hint given, as bench.py does).  how: the entry
+    order, where the plan must have chosen the matching way of storing SDDMM's results."""
     tol = oracle.TOL[np.dtype(W.np_dtype(dtype))]
     rng = np.random.default_rng(seed)
     A, B, Y0, vv = w.panel_A(dtype), w.panel_B(dtype), w.panel_Y0(dtype), w.values(dtype)
@@ -30,6 +32,14 @@ def _check_sampled(ctx, w, dtype, n_entries=200_000, n_rows=3000, seed=9, col_bl
         S = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, vv)
     info = S.info
     assert info.nnz == w.nnz and info.nsegments >= info.rows_touched
+    if how == "sorted":
+        assert info.staged_entries > 0 and info.positions_by_segment == 1
+        assert info.two_pass_results == 0 and info.sddmm_by_column == 0
+    elif how == "shuffled":
+        assert info.two_pass_results == 1 and info.staged_entries == 0
+        assert info.sddmm_by_column == 0
+    elif how == "column-major":
+        assert info.sddmm_by_column == 1 and info.two_pass_results == 1
     dA, dB, dY = ctx.panel_from(A), ctx.panel_from(B), ctx.panel_from(Y0)
     dC = ctx.vals(w.nnz, dtype)
     dC.fill(float("nan"))
@@ -73,13 +83,15 @@ def _check_sampled(ctx, w, dtype, n_entries=200_000, n_rows=3000, seed=9, col_bl
 
 
 @pytest.mark.parametrize("dtype", ["f32", "f64"])
-@pytest.mark.parametrize("order", ["sorted", "shuffled"])
+@pytest.mark.parametrize("order", ["sorted", "shuffled", "column-major"])
 def test_config2_rmat20_full(ctx, dtype, order):
     w = W.rmat(20, 16, 64)
     assert w.nnz == 16_086_740  # the realised nnz of the seeded generator after dedup
     if order == "shuffled":
         w = w.shuffled()
-    _check_sampled(ctx, w, dtype)
+    elif order == "column-major":
+        w = w.column_major()
+    _check_sampled(ctx, w, dtype, how=order)
 
 
 def test_config3_rmat24_block_full(ctx):
