@@ -105,7 +105,7 @@ typedef struct {
                                   so A and B) exchanged, whose kernel order is the caller's:
                                   the same bits, stored in runs instead of one by one; the
                                   plan then holds its arrays twice (GPU builder only) */
-    uint32_t two_pass_results; /* 1: an arbitrary entry order of 2^22 entries or more: the
+    uint32_t two_pass_results; /* 1: an arbitrary entry order of 1.5 M entries or more: the
                                   SDDMM kernels write their results in kernel order to a
                                   vector of the plan, and two passes of tile-local moves
                                   through LDS bring them to the caller's positions (24 more

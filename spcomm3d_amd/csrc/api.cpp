@@ -1157,13 +1157,13 @@ static hipError_t finish_sddmm(const spc3d_plan *S, void *C)
 }
 
 // The two-pass tables of a finished single plan whose results would each be a store of its
-// own (an arbitrary entry order), from 2^22 entries on (SPC3D_TWO_PASS_MIN in the environment
+// own (an arbitrary entry order), from 1.5 M entries on (SPC3D_TWO_PASS_MIN in the environment
 // gives another bound): below that the scattered stores mostly meet in the L2s.
 // SPC3D_TWO_PASS=0 in the environment switches it off.
 static int add_two_pass(spc3d_plan *p)
 {
     const bool off = env_off("SPC3D_TWO_PASS");
-    uint64_t least = 1ull << 22;
+    uint64_t least = 3ull << 19; // measured on R-MAT patterns: slower at 0.95 M entries, faster at 1.9 M
     if (const char *e = std::getenv("SPC3D_TWO_PASS_MIN")) // for tests on small patterns
         least = std::strtoull(e, nullptr, 10);
     if (off || !p->perm || p->store.consecutive || !p->blocks.empty() || p->info.nnz < least)

@@ -587,7 +587,7 @@ def test_column_sorted_input_runs_sddmm_through_the_exchanged_plan(ctx, dtype, k
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_arbitrary_order_brings_results_home_in_two_passes(ctx, dtype, monkeypatch):
     """An arbitrary entry order: the kernels write in kernel order, two passes of tile-local
-    moves bring the results to the caller's positions (plan info two_pass_results; from 2^22
+    moves bring the results to the caller's positions (plan info two_pass_results; from 1.5 M
     entries on by default, here from the smallest size the scheme takes).  Bit for bit what the
     plain plan stores, through spc3d_sddmm and both one-pass forms, wide rows included, and
     into a wrapped value vector."""
