@@ -82,7 +82,7 @@ def ensure_built():
         __graft_entry__.build()
 
 
-def run_gpu(w, dtype, steps, warmup, seg_max=None, max_timed=1300, copies=0, vendor=True):
+def run_gpu(w, dtype, steps, warmup, seg_max=None, max_timed=1300, copies=0):
     """Times `steps` SDDMM+SpMM passes on resident operands; returns a dict."""
     from spcomm3d_amd import device, roofline
     from spcomm3d_amd import workloads as W
@@ -183,15 +183,6 @@ def run_gpu(w, dtype, steps, warmup, seg_max=None, max_timed=1300, copies=0, ven
         ctx.mark(4004)
         copy_gbs = 2 * w.nrows * w.k * wbytes / (ctx.elapsed_ms(4003, 4004) / steps) / 1e6
         dT.close()
-        # The vendor's library on the same resident operands, last (it overwrites Y).
-        vendor_out = None
-        if vendor and w.order == "sorted":
-            try:
-                import vendor_baseline
-
-                vendor_out = vendor_baseline.time_rocsparse(ctx, w, dtype, dA, dB, dY)
-            except Exception as e:  # a measurement aid: never fails the bench
-                log(f"vendor baseline skipped: {type(e).__name__}: {e}")
         for h in (S, dA, dB, dY, dC):
             h.close()
 
@@ -208,12 +199,6 @@ def run_gpu(w, dtype, steps, warmup, seg_max=None, max_timed=1300, copies=0, ven
                          "strict_frac": fb / (fused_wall / steps) / 1e9 / roofline.HBM_PEAK_GBS}
     out["row_copies"] = rows
     out["device_copy_gbs"] = copy_gbs
-    if vendor_out:
-        sd_ms, sp_ms = float(sd.mean()), float(sp.mean())
-        vendor_out["sddmm_ratio"] = vendor_out["sddmm_us"] / (sd_ms * 1e3)
-        if "spmm_best" in vendor_out:
-            vendor_out["spmm_ratio"] = vendor_out["spmm_best"]["us"] / (sp_ms * 1e3)
-        out["vendor_baseline"] = vendor_out
     for name, ms, strict, gather in (
             ("sddmm", sd,
              roofline.sddmm_bytes(w.nrows, w.nnz, w.k, wbytes, m_t, n_t, with_perm),
@@ -373,8 +358,6 @@ def main():
                          "(a known-size dispatch for counter calibration)")
     ap.add_argument("--only", action="store_true", help="skip the other real type")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--no-vendor", action="store_true",
-                    help="skip the rocSPARSE timings on the same operands")
     ap.add_argument("--no-configs", action="store_true",
                     help="skip the shuffled-order runs and the rows of the other configurations")
     args = ap.parse_args()
@@ -394,13 +377,12 @@ def main():
         f"(generated in {time.perf_counter() - t0:.1f}s)")
 
     main_r = run_gpu(w, args.dtype, args.steps, args.warmup, args.seg_max,
-                     copies=args.calibration_copies, vendor=not args.no_vendor)
+                     copies=args.calibration_copies)
     log(json.dumps(main_r))
     also = {}
     if not args.only:
         other = "f32" if args.dtype == "f64" else "f64"
-        also[other] = run_gpu(w, other, args.steps, args.warmup, args.seg_max,
-                              vendor=not args.no_vendor)
+        also[other] = run_gpu(w, other, args.steps, args.warmup, args.seg_max)
         log(json.dumps(also[other]))
     if not (args.only or args.no_configs):
         ws = w.shuffled() if w.order == "sorted" else None
@@ -466,7 +448,6 @@ def main():
         "kernels": main_r["kernels"],
         "fused_step": main_r["fused_step"],
         "row_copies": main_r["row_copies"],
-        "vendor_baseline": main_r.get("vendor_baseline"),
         "plan": {k: main_r[k] for k in ("plan_build_s", "upload_s", "nsegments", "nsplit_rows",
                                         "seg_max")},
         "also": also,

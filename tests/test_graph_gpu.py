@@ -119,7 +119,7 @@ def test_a_recording_survives_a_later_call_with_wider_rows(ctx):
     g.close()
 
 
-def test_replay_of_a_short_step_costs_less_than_its_eager_calls(ctx):
+def test_replay_of_a_short_step_gives_the_eager_bits(ctx):
     w = W.erdos_renyi(16384, 16, 32)
     S, dA, dB = operands(ctx, w, np.float64)
     dY, dC = ctx.panel_from(w.panel_Y0("f64")), ctx.vals(w.nnz, np.float64)
@@ -147,5 +147,18 @@ def test_replay_of_a_short_step_costs_less_than_its_eager_calls(ctx):
     eager = timed(lambda: [step() for _ in range(10)], 50)
     replay = timed(g.launch, 50)
     print(f"ER 16384 K=32 fp64, 10 steps: eager {eager * 1e6:.1f} us, one replay {replay * 1e6:.1f} us")
-    assert replay < eager * 1.5  # never a regression worth the name; usually well below
+    # the two times are printed, never asserted on (wall-clock comparisons flake); what
+    # is asserted is that the replay leaves the bits of the ten eager steps
+    Y0 = w.panel_Y0("f64")
+    dY.upload(Y0)
+    for _ in range(10):
+        step()
+    ctx.sync()
+    eager_C, eager_Y = dC.download(), dY.download()
+    dY.upload(Y0)
+    dC.fill(0.0)
+    g.launch()
+    ctx.sync()
+    assert np.array_equal(dC.download(), eager_C)
+    assert np.array_equal(dY.download(), eager_Y)
     g.close()
