@@ -216,6 +216,44 @@ def run_gpu(w, dtype, steps, warmup, seg_max=None, max_timed=1300, copies=0):
     return out
 
 
+def run_floors(w, dtype, steps, warmup, seg_max=None):
+    """The two floors of the same launches: the plan of `w` as the timed runs build it, with
+    its columns rewritten on the device (spc3d_plan_probe_columns) so that every gathered
+    dense row is found in the L2 (a table of 1 MiB per L2), then so that nearly none is
+    (uniform random columns).  Segments, queues, streams and instruction stream are those
+    of the real plan; only the gather addresses differ."""
+    from spcomm3d_amd import device
+    from spcomm3d_amd import workloads as W
+
+    wbytes = np.dtype(W.np_dtype(dtype)).itemsize
+    modulus = max(64, (1 << 20) // (w.k * wbytes))
+    out = {"dtype": dtype, "all_hit_table_rows": modulus, "steps": steps}
+    with device.Context(0) as ctx:
+        hint = {} if w.k == 64 else {"k_hint": w.k}
+        S = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, w.values(dtype), seg_max=seg_max, **hint)
+        dA, dB = ctx.panel_from(w.panel_A(dtype)), ctx.panel_from(w.panel_B(dtype))
+        dY = ctx.panel_from(w.panel_Y0(dtype))
+        dC = ctx.vals(w.nnz, dtype)
+        for mode in ("all_hit", "all_miss"):
+            S.probe_columns(mode, modulus)
+            for _ in range(warmup):
+                ctx.sddmm(S, dA, dB, dC)
+                ctx.spmm(S, dB, dY)
+            ctx.sync()
+            ctx.mark(0)
+            for _ in range(steps):
+                ctx.sddmm(S, dA, dB, dC)
+            ctx.mark(1)
+            for _ in range(steps):
+                ctx.spmm(S, dB, dY)
+            ctx.mark(2)
+            out[mode] = {"sddmm_ms": ctx.elapsed_ms(0, 1) / steps,
+                         "spmm_ms": ctx.elapsed_ms(1, 2) / steps}
+        for h in (S, dA, dB, dY, dC):
+            h.close()
+    return out
+
+
 def run_compact(w, dtype, steps, warmup):
     """One compact row for a workload: mean time per kernel over `steps` passes on
     resident operands, strict-model fraction of the HBM peak."""
@@ -356,6 +394,10 @@ def main():
     ap.add_argument("--calibration-copies", type=int, default=0,
                     help="also launch this many plain device copies of an m x K panel "
                          "(a known-size dispatch for counter calibration)")
+    ap.add_argument("--floors", action="store_true",
+                    help="only the all-hit / all-miss floors of the workload's launches "
+                         "(they are part of the default run as well)")
+    ap.add_argument("--no-floors", action="store_true", help="skip the floors")
     ap.add_argument("--only", action="store_true", help="skip the other real type")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-configs", action="store_true",
@@ -376,6 +418,13 @@ def main():
     log(f"workload {w.name}: {w.nrows}x{w.ncols} nnz={w.nnz} K={w.k} order={w.order} "
         f"(generated in {time.perf_counter() - t0:.1f}s)")
 
+    if args.floors:
+        fl = {dt: run_floors(w, dt, max(5, args.steps // 2), args.warmup, args.seg_max)
+              for dt in (("f64", "f32") if not args.only else (args.dtype,))}
+        print(json.dumps({"workload": f"{w.name} K={w.k} ({w.order} COO)", "floors": fl}),
+              flush=True)
+        return
+
     main_r = run_gpu(w, args.dtype, args.steps, args.warmup, args.seg_max,
                      copies=args.calibration_copies)
     log(json.dumps(main_r))
@@ -384,6 +433,11 @@ def main():
         other = "f32" if args.dtype == "f64" else "f64"
         also[other] = run_gpu(w, other, args.steps, args.warmup, args.seg_max)
         log(json.dumps(also[other]))
+    floors = None
+    if not args.no_floors:
+        floors = {dt: run_floors(w, dt, max(5, args.steps // 2), args.warmup, args.seg_max)
+                  for dt in ((args.dtype,) if args.only else ("f64", "f32"))}
+        log(json.dumps(floors))
     if not (args.only or args.no_configs):
         ws = w.shuffled() if w.order == "sorted" else None
         if ws is not None:
@@ -442,6 +496,11 @@ def main():
                      "frac_of_device_copy": kd["strict_gbs"] / main_r["device_copy_gbs"],
                      "traffic_frac_of_device_copy": None if traffic is None else
                      traffic / kd["ms_avg"] / 1e6 / main_r["device_copy_gbs"],
+                     "floor_all_hit_ms": None if floors is None else
+                     floors[args.dtype]["all_hit"][dom + "_ms"],
+                     "floor_all_miss_ms": None if floors is None else
+                     floors[args.dtype]["all_miss"][dom + "_ms"],
+                     "floors": floors,
                      "bytes_per_launch": kd["strict_bytes"],
                      "ms_per_launch": kd["ms_avg"], "model": "strict (each operand once)"},
         "cpu_baseline": cpu,

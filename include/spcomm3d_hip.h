@@ -298,6 +298,17 @@ SPC3D_API int spc3d_plan_destroy(spc3d_plan *plan);
 SPC3D_API int spc3d_plan_set_values(spc3d_plan *plan, const void *vv_host);       /* caller's COO order */
 SPC3D_API int spc3d_plan_set_values_device(spc3d_plan *plan, const spc3d_vals *vv); /* caller's COO order */
 SPC3D_API int spc3d_plan_get_info(const spc3d_plan *plan, spc3d_plan_info *info);
+/* Measurement aid, for the floors a benchmark quotes beside its timings; has no counterpart
+ * in the reference.  Rewrites the columns of a plan's entries in place on the device, so
+ * that the same launches over the same segments, queues and streams find every gathered
+ * dense row in the L2 (SPC3D_PROBE_ALL_HIT: column c becomes c % modulus, inside its own
+ * block of columns for a plan kept in column blocks; choose modulus * K * sizeof(real) well
+ * under one 4 MiB L2) or nearly none of them (SPC3D_PROBE_ALL_MISS: a hash of the entry's
+ * position, uniform over all columns; modulus is ignored).  The plan afterwards computes
+ * another pattern than the caller's: time it, then destroy it.  Synchronous. */
+#define SPC3D_PROBE_ALL_HIT 1
+#define SPC3D_PROBE_ALL_MISS 2
+SPC3D_API int spc3d_plan_probe_columns(spc3d_plan *plan, int mode, uint32_t modulus);
 
 /* ---- the hot path -------------------------------------------------------
  * spc3d_sddmm  = SpKernels::sddmm (src/core_ops.cpp:5-22):

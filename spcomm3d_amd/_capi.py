@@ -91,6 +91,7 @@ SIGNATURES = {
     "spc3d_plan_set_values": (c_int, [c_vp, c_vp]),
     "spc3d_plan_set_values_device": (c_int, [c_vp, c_vp]),
     "spc3d_plan_get_info": (c_int, [c_vp, P(PlanInfo)]),
+    "spc3d_plan_probe_columns": (c_int, [c_vp, c_int, c_u32]),
     "spc3d_sddmm": (c_int, [c_vp, c_vp, c_vp, c_vp, c_vp]),
     "spc3d_spmm": (c_int, [c_vp, c_vp, c_vp, c_vp]),
     "spc3d_spmm_noalloc": (c_int, [c_vp, c_vp, c_vp, c_vp]),

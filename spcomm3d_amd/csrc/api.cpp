@@ -209,6 +209,7 @@ struct spc3d_plan {
     uint32_t *stage_pos = nullptr; // [nnz] caller's position -> staging position
     uint32_t *stage_of = nullptr;  // [nnz]
     uint64_t stage_off = 0;
+    uint32_t col_base = 0; // a block of a plan kept in column blocks: its first column
 };
 
 // A cached plan answers for a pattern when the keys of every block of ii and jj, the
@@ -1441,6 +1442,7 @@ static int build_from_device(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t
         if (child->perm) (void)hipFree(child->perm);
         child->perm = gperm;
         child->stage_off = first[b];
+        child->col_base = b * ((ncols + nb - 1) / nb);
         child->info.order_is_identity = 0;
         total.nsegments += child->info.nsegments;
         total.nsegments_padded += child->info.nsegments_padded;
@@ -1828,6 +1830,45 @@ int spc3d_plan_set_values_device(spc3d_plan *plan, const spc3d_vals *vv)
         plan->by_col->has_values = true;
     }
     plan->has_values = true;
+    return SPC3D_OK;
+}
+
+// One plan's columns rewritten in place, and its table of first columns with them.
+static int probe_columns_of(spc3d_plan *p, int mode, uint32_t modulus)
+{
+    HIP_TRY(launch_probe_cols(p->col, p->info.nnz, (uint32_t)mode, p->col_base, modulus,
+                              p->info.ncols, p->ctx->stream));
+    const uint32_t nshort = p->info.nsegments_padded - p->info.nsegments_long;
+    HIP_TRY(launch_first_cols(p->segs + p->info.nsegments_long, nshort, p->col, p->first_cols,
+                              p->ctx->stream));
+    return SPC3D_OK;
+}
+
+int spc3d_plan_probe_columns(spc3d_plan *plan, int mode, uint32_t modulus)
+{
+    if (!live(plan))
+        return fail(SPC3D_ERR_INVALID_ARG, "plan is NULL or destroyed");
+    if (mode != SPC3D_PROBE_ALL_HIT && mode != SPC3D_PROBE_ALL_MISS)
+        return fail(SPC3D_ERR_INVALID_ARG, "unknown probe mode");
+    if (mode == SPC3D_PROBE_ALL_HIT && modulus == 0)
+        return fail(SPC3D_ERR_INVALID_ARG, "modulus is 0");
+    if (plan->info.nnz == 0)
+        return SPC3D_OK;
+    int rc = use_device(plan->ctx);
+    if (rc)
+        return rc;
+    std::vector<spc3d_plan *> self;
+    for (spc3d_plan *part : parts_of(plan, self)) {
+        rc = probe_columns_of(part, mode, modulus);
+        if (rc)
+            return rc;
+    }
+    if (plan->by_col) { // its columns are the pattern's rows
+        rc = probe_columns_of(plan->by_col, mode, modulus);
+        if (rc)
+            return rc;
+    }
+    HIP_TRY(hipStreamSynchronize(plan->ctx->stream));
     return SPC3D_OK;
 }
 

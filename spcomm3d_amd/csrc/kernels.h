@@ -92,6 +92,11 @@ hipError_t launch_rows(int op, int dtype, void *panel, const RowMapView &M, uint
                        hipStream_t stream);
 // out[b] = id of the XCD workgroup b of an nblocks-wide grid ran on
 hipError_t launch_xcc_probe(uint32_t *out, uint32_t nblocks, hipStream_t stream);
+// Measurement aid: col[i] = base + (col[i] - base) % modulus (mode 1: every gather then hits
+// a table of `modulus` dense rows) or a hash of i, uniform over [0, ncols) (mode 2: nearly
+// every gather misses); the plan then computes another pattern with the same segments.
+hipError_t launch_probe_cols(uint32_t *col, uint64_t n, uint32_t mode, uint32_t base,
+                             uint32_t modulus, uint32_t ncols, hipStream_t stream);
 // dst[0..bytes) = src[0..bytes); both 16-byte aligned, non-overlapping
 hipError_t launch_copy(void *dst, const void *src, uint64_t bytes, hipStream_t stream);
 hipError_t launch_fill(int dtype, void *p, uint64_t n, double value, hipStream_t stream);

@@ -1172,6 +1172,29 @@ __global__ void __launch_bounds__(64) xcc_probe_kernel(uint32_t *__restrict__ ou
 }
 
 // ------------------------------------------------------------- utilities ----
+// Measurement aid (launch_probe_cols): the column of every kernel-order entry replaced so
+// that the launches keep their instruction stream, segments and queues while every gather
+// hits (mode 1: base + (c - base) % modulus, a table of `modulus` dense rows) or nearly
+// every gather misses (mode 2: a hash of the entry's position, uniform over ncols).
+__global__ void __launch_bounds__(kBlock)
+probe_cols_kernel(uint32_t *__restrict__ col, uint64_t n, uint32_t mode, uint32_t base,
+                  uint32_t modulus, uint32_t ncols)
+{
+    const uint64_t stride = (uint64_t)gridDim.x * kBlock;
+    for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) {
+        if (mode == 1) {
+            const uint32_t c = col[i];
+            col[i] = c >= base ? base + (c - base) % modulus : c % modulus;
+        } else {
+            uint64_t x = (i + 1) * 0x9E3779B97F4A7C15ull; // splitmix64 finaliser
+            x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+            x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
+            x ^= x >> 31;
+            col[i] = (uint32_t)(x % ncols);
+        }
+    }
+}
+
 template <typename T>
 __global__ void __launch_bounds__(kBlock)
 gather_kernel(const T *__restrict__ in, const uint32_t *__restrict__ perm, T *__restrict__ out,
@@ -1897,6 +1920,16 @@ hipError_t launch_xcc_probe(uint32_t *out, uint32_t nblocks, hipStream_t stream)
     if (nblocks == 0)
         return hipSuccess;
     hipLaunchKernelGGL(xcc_probe_kernel, dim3(nblocks), dim3(64), 0, stream, out);
+    return hipGetLastError();
+}
+
+hipError_t launch_probe_cols(uint32_t *col, uint64_t n, uint32_t mode, uint32_t base,
+                             uint32_t modulus, uint32_t ncols, hipStream_t stream)
+{
+    if (n == 0)
+        return hipSuccess;
+    hipLaunchKernelGGL(probe_cols_kernel, dim3(stream_grid(n)), dim3(kBlock), 0, stream, col, n,
+                       mode, base, modulus, ncols);
     return hipGetLastError();
 }
 

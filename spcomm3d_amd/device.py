@@ -360,6 +360,14 @@ class Plan:
         check(self.ctx._lib.spc3d_plan_set_values_device(self._h, vv._h),
               "spc3d_plan_set_values_device")
 
+    def probe_columns(self, mode: str, modulus: int = 0):
+        """Measurement aid: rewrites the plan's columns in place so that every gather hits
+        the L2 ("all_hit": c % modulus) or nearly none does ("all_miss"); the plan then
+        computes another pattern and is good for timing only."""
+        code = {"all_hit": 1, "all_miss": 2}[mode]
+        check(self.ctx._lib.spc3d_plan_probe_columns(self._h, code, int(modulus)),
+              "spc3d_plan_probe_columns")
+
     @property
     def info(self) -> PlanInfo:
         info = PlanInfo()

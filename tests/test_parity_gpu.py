@@ -732,3 +732,33 @@ def test_panel_copy_on_device(ctx, shape):
     assert np.array_equal(dst.download(), a)
     with pytest.raises(capi.Spc3dError):
         ctx.panel(shape[0], shape[1] + 1, np.float32).copy_from(src)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("col_blocks", [None, 3])
+def test_probe_columns_keeps_the_launches_and_moves_the_gathers(ctx, dtype, col_blocks):
+    """spc3d_plan_probe_columns (a measurement aid): after the all-hit rewrite the plan
+    computes the pattern (ii, c % modulus inside the entry's block of columns), entry by
+    entry at the caller's positions; after the all-miss one every column is in range."""
+    w = W.rmat(12, 16, 32).shuffled()
+    vv, A, B, Y0 = w.values(dtype), w.panel_A(dtype), w.panel_B(dtype), w.panel_Y0(dtype)
+    S = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, vv, k_hint=w.k, col_blocks=col_blocks)
+    dA, dB, dY, dC = ctx.panel_from(A), ctx.panel_from(B), ctx.panel_from(Y0), ctx.vals(w.nnz, dtype)
+    modulus = 61
+    S.probe_columns("all_hit", modulus)
+    nb = S.info.ncol_blocks if col_blocks else 1
+    bc = (w.ncols + nb - 1) // nb if nb > 1 else w.ncols
+    base = (w.jj // bc) * bc
+    jj2 = (base + (w.jj - base) % modulus).astype(np.uint32)
+    ctx.sddmm(S, dA, dB, dC)
+    ctx.spmm(S, dB, dY)
+    check_sddmm(A, B, w.ii, jj2, vv, dC.download())
+    check_spmm(B, w.ii, jj2, vv, Y0, dY.download())
+    S.probe_columns("all_miss")
+    dY.upload(Y0)
+    ctx.sddmm(S, dA, dB, dC)
+    ctx.spmm(S, dB, dY)
+    ctx.sync()  # every gather stayed inside B: nothing to fault on, finite results
+    assert np.isfinite(dC.download()).all() and np.isfinite(dY.download()).all()
+    for h in (S, dA, dB, dY, dC):
+        h.close()
