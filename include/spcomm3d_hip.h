@@ -110,7 +110,11 @@ typedef struct {
                                   vector of the plan, and two passes of tile-local moves
                                   through LDS bring them to the caller's positions (24 more
                                   bytes per entry in fp64, 16 in fp32) */
-    uint32_t reserved1;
+    uint32_t entries_by_column; /* 1: the rows arrived unsorted, and the plan orders the entries
+                                  of every row by column (spc3d_spmm then adds a row's entries
+                                  in that order); 0: the caller's order inside every row */
+    uint64_t device_bytes;     /* device memory the plan holds: its arrays, values, partial-sum
+                                  rows, result staging, a companion plan, every column block */
 } spc3d_plan_info;
 
 /* Plan tuning; a zero field selects the default.  Only speed depends on these. */
@@ -138,8 +142,24 @@ typedef struct {
                               16 times the block count); 1: never; n > 1: in n blocks (at
                               most 4096).  Built on the GPU only; results are those of the
                               whole plan up to summation order (SpMM adds block after block) */
-    uint32_t reserved[1];  /* must be 0 */
+    uint32_t flags;        /* SPC3D_PLAN_* bits, 0: defaults */
+    uint32_t two_pass_min; /* entries from which the results of an arbitrary entry order go home
+                              in two tile-local passes (default 1,572,864: measured slower
+                              under 1 M entries, faster from 1.9 M on) */
+    uint32_t reserved[3];  /* must be 0 */
 } spc3d_plan_opts;
+/* spc3d_plan_opts.flags.  The first three keep spc3d_sddmm's plain stores where the plan
+ * would otherwise stage the results of regrouped segments, run a column-sorted pattern
+ * through a second plan with rows and columns exchanged, or bring an arbitrary order home in
+ * two passes (spc3d_plan_info: staged_entries, sddmm_by_column, two_pass_results): the same
+ * bits either way, for comparisons and for callers short of device memory.  The fourth keeps
+ * the caller's order inside every row also when the rows arrive unsorted (by default such
+ * rows are ordered by column, which is what the gathers of a sorted pattern see). */
+#define SPC3D_PLAN_NO_STAGED_STORES 1u
+#define SPC3D_PLAN_NO_SDDMM_BY_COLUMN 2u
+#define SPC3D_PLAN_NO_TWO_PASS 4u
+#define SPC3D_PLAN_KEEP_ENTRY_ORDER 8u
+#define SPC3D_PLAN_ALL_FLAGS 15u
 
 /* ---- library / errors ------------------------------------------------- */
 SPC3D_API const char *spc3d_version(void);
@@ -236,9 +256,10 @@ SPC3D_API int spc3d_coo_validate(uint32_t nrows, uint32_t ncols, uint64_t nnz,
  * SPC3D_PLAN_BUILDER=host in the environment (spc3d_plan_create only) selects
  * the single-threaded host builder instead.  How spc3d_sddmm brings its results to
  * the caller's positions is settled here as well (spc3d_plan_info: staged_entries,
- * positions_by_segment, sddmm_by_column, two_pass_results; the environment variables
- * SPC3D_STAGE_STORES=0, SPC3D_SDDMM_BY_COLUMN=0 and SPC3D_TWO_PASS=0 keep the plain form,
- * for comparisons).  `vv` (nnz reals of
+ * positions_by_segment, sddmm_by_column, two_pass_results; spc3d_plan_opts.flags keeps the
+ * plain form, and for spc3d_plan_create and the one-shot host calls, which take no options,
+ * so do SPC3D_STAGE_STORES=0, SPC3D_SDDMM_BY_COLUMN=0 and SPC3D_TWO_PASS=0 in the
+ * environment, read once per plan).  `vv` (nnz reals of
  * `dtype`, caller's order) may be NULL and set later.  The pattern is copied:
  * the caller's arrays are not referenced afterwards.  Replaces nothing in the
  * reference (it walks the unsorted COO directly, core_ops.cpp:7-10); it is the

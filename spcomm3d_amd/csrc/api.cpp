@@ -172,6 +172,7 @@ struct spc3d_plan {
     // until the plan is destroyed: a sequence recorded earlier (spc3d_capture_*) keeps
     // the block's address in its kernel arguments and goes on using it.
     std::vector<void *> retired_partial;
+    uint64_t retired_bytes = 0;
     // A pattern kept in column blocks: one complete plan per block of columns, each over
     // the entries of its block with `perm` giving the caller's positions; this plan then
     // holds no arrays of its own, only `info` for the whole pattern.  The calls run the
@@ -342,6 +343,7 @@ void plan_free_device(spc3d_plan *p)
     for (void *old : p->retired_partial)
         (void)hipFree(old);
     p->retired_partial.clear();
+    p->retired_bytes = 0;
     p->segs = nullptr;
     p->col = p->perm = nullptr;
     p->sval = p->partial = nullptr;
@@ -1014,7 +1016,8 @@ static void fill_info(spc3d_plan_info &info, const HostPlan &H)
     info.positions_by_segment = 0;
     info.sddmm_by_column = 0;
     info.two_pass_results = 0;
-    info.reserved1 = 0;
+    info.entries_by_column = H.by_column_in_rows ? 1 : 0;
+    info.device_bytes = 0;
 }
 
 // Library defaults, overridable field by field.  With XCD slicing, 2 MiB of
@@ -1025,8 +1028,10 @@ static int resolve_opts(int dtype, const spc3d_plan_opts *o, PlanOpts &out)
     std::memset(&z, 0, sizeof z);
     if (o)
         z = *o;
-    if (z.reserved[0])
+    if (z.reserved[0] || z.reserved[1] || z.reserved[2])
         return fail(SPC3D_ERR_INVALID_ARG, "spc3d_plan_opts.reserved must be 0");
+    if (z.flags & ~(uint32_t)SPC3D_PLAN_ALL_FLAGS)
+        return fail(SPC3D_ERR_INVALID_ARG, "spc3d_plan_opts.flags has unknown bits set");
     if (z.col_blocks > kMaxColBlocks)
         return fail(SPC3D_ERR_INVALID_ARG, "spc3d_plan_opts.col_blocks must be at most 4096");
     if (z.col_blocks > 1 && z.builder == 1)
@@ -1037,6 +1042,7 @@ static int resolve_opts(int dtype, const spc3d_plan_opts *o, PlanOpts &out)
     if (z.xcd_slices != 0 && z.xcd_slices != 1 && z.xcd_slices != 8)
         return fail(SPC3D_ERR_INVALID_ARG, "xcd_slices must be 0, 1 or 8");
     out.seg_max = z.seg_max;
+    out.keep_entry_order = (z.flags & SPC3D_PLAN_KEEP_ENTRY_ORDER) != 0;
     out.hub_min = z.hub_min;
     out.xcd_slices = z.xcd_slices;
     const uint64_t k = z.k_hint ? z.k_hint : 64;
@@ -1098,27 +1104,50 @@ static int finish_plan(spc3d_plan *p, uint32_t k0)
     return ensure_partial(p, k0);
 }
 
-// A switch in the environment, read at every plan creation: set to 0 it keeps the plain form.
-static bool env_off(const char *name)
+// How a plan may bring SDDMM results to the caller's positions (spc3d_plan_opts.flags,
+// two_pass_min): each of the three forms can be switched off, which keeps the plain stores.
+struct StoreOpts {
+    bool stage = true, by_column = true, two_pass = true;
+    // measured on R-MAT patterns: two passes are slower at 0.95 M entries, faster at 1.9 M
+    uint64_t two_pass_min = 3ull << 19;
+};
+static StoreOpts store_opts_of(const spc3d_plan_opts *o)
 {
-    const char *e = std::getenv(name);
-    return e && *e && std::atoi(e) == 0;
+    StoreOpts so;
+    if (o) {
+        so.stage = !(o->flags & SPC3D_PLAN_NO_STAGED_STORES);
+        so.by_column = !(o->flags & SPC3D_PLAN_NO_SDDMM_BY_COLUMN);
+        so.two_pass = !(o->flags & SPC3D_PLAN_NO_TWO_PASS);
+        if (o->two_pass_min)
+            so.two_pass_min = o->two_pass_min;
+    }
+    return so;
+}
+
+// The result paths below are optional: when one of them cannot get its memory the plan
+// goes on without it (plain stores), what it had allocated is freed by its builder, and the
+// HIP error state is cleared.  Any other failure fails the plan.
+static int optional_path(int rc)
+{
+    if (rc != SPC3D_ERR_ALLOC)
+        return rc;
+    (void)hipGetLastError();
+    return SPC3D_OK;
 }
 
 // A finished single plan (not a block of a plan kept in column blocks) whose kernel order
 // regroups entries inside rows gets the staging of its SDDMM results (see StoreStaging).
-// SPC3D_STAGE_STORES=0 in the environment keeps every result on its way straight to C.
-static int add_store_staging(spc3d_plan *p)
+// SPC3D_PLAN_NO_STAGED_STORES keeps every result on its way straight to C.
+static int add_store_staging(spc3d_plan *p, const StoreOpts &so)
 {
-    const bool off = env_off("SPC3D_STAGE_STORES");
-    if (off || !p->perm || !p->blocks.empty())
+    if (!so.stage || !p->perm || !p->blocks.empty())
         return SPC3D_OK;
     std::string err;
     StoreStaging st;
     int rc = build_store_staging(p->ctx->stream, p->segs, p->info.nsegments_padded, p->perm,
                                  p->info.nnz, st, err);
     if (rc)
-        return fail(rc, err);
+        return optional_path(fail(rc, err));
     p->store.consecutive = st.consecutive;
     p->info.positions_by_segment = st.consecutive ? 1 : 0;
     if (!st.n)
@@ -1130,7 +1159,7 @@ static int add_store_staging(spc3d_plan *p)
         (void)hipFree(st.src);
         p->store = StoreStaging();
         p->info.positions_by_segment = 0;
-        return rc;
+        return optional_path(rc);
     }
     p->store = st;
     p->info.staged_entries = st.n;
@@ -1158,16 +1187,12 @@ static hipError_t finish_sddmm(const spc3d_plan *S, void *C)
 }
 
 // The two-pass tables of a finished single plan whose results would each be a store of its
-// own (an arbitrary entry order), from 1.5 M entries on (SPC3D_TWO_PASS_MIN in the environment
-// gives another bound): below that the scattered stores mostly meet in the L2s.
-// SPC3D_TWO_PASS=0 in the environment switches it off.
-static int add_two_pass(spc3d_plan *p)
+// own (an arbitrary entry order), from StoreOpts::two_pass_min entries on: below that the
+// scattered stores mostly meet in the L2s.  SPC3D_PLAN_NO_TWO_PASS switches it off.
+static int add_two_pass(spc3d_plan *p, const StoreOpts &so)
 {
-    const bool off = env_off("SPC3D_TWO_PASS");
-    uint64_t least = 3ull << 19; // measured on R-MAT patterns: slower at 0.95 M entries, faster at 1.9 M
-    if (const char *e = std::getenv("SPC3D_TWO_PASS_MIN")) // for tests on small patterns
-        least = std::strtoull(e, nullptr, 10);
-    if (off || !p->perm || p->store.consecutive || !p->blocks.empty() || p->info.nnz < least)
+    if (!so.two_pass || !p->perm || p->store.consecutive || !p->blocks.empty() ||
+        p->info.nnz < so.two_pass_min)
         return SPC3D_OK;
     int lds = 0;
     if (hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerBlock, p->ctx->device) !=
@@ -1179,7 +1204,7 @@ static int add_two_pass(spc3d_plan *p)
     int rc = build_two_pass(p->ctx->stream, p->perm, p->info.nnz, two_pass_tile_elems(p->dtype), tp,
                             err);
     if (rc)
-        return fail(rc, err);
+        return optional_path(fail(rc, err));
     if (!tp.n)
         return SPC3D_OK;
     const size_t bytes = (size_t)p->info.nnz * elem_size(p->dtype);
@@ -1191,7 +1216,7 @@ static int add_two_pass(spc3d_plan *p)
         (void)hipFree(tp.l2);
         if (p->c_stage) (void)hipFree(p->c_stage);
         p->c_stage = nullptr;
-        return rc;
+        return optional_path(rc);
     }
     p->two = tp;
     p->info.two_pass_results = 1;
@@ -1297,12 +1322,12 @@ static int choose_col_blocks(spc3d_plan *p, const spc3d_plan_opts *opts, uint32_
 
 // The companion plan for SDDMM (spc3d_plan::by_col) of a finished single plan whose results
 // would be stored one by one, when the pattern is sorted by column and the exchanged plan
-// does store in runs.  SPC3D_SDDMM_BY_COLUMN=0 in the environment switches it off.
+// does store in runs.  SPC3D_PLAN_NO_SDDMM_BY_COLUMN switches it off.
 static int add_sddmm_companion(spc3d_plan *p, uint32_t nrows, uint32_t ncols, uint64_t nnz,
-                               const uint32_t *d_ii, const uint32_t *d_jj, const PlanOpts &po)
+                               const uint32_t *d_ii, const uint32_t *d_jj, const PlanOpts &po,
+                               const StoreOpts &so)
 {
-    const bool off = env_off("SPC3D_SDDMM_BY_COLUMN");
-    if (off || nnz < 2 || !p->perm || p->store.consecutive || !p->blocks.empty())
+    if (!so.by_column || nnz < 2 || !p->perm || p->store.consecutive || !p->blocks.empty())
         return SPC3D_OK;
     std::string err;
     bool sorted = false;
@@ -1315,11 +1340,11 @@ static int add_sddmm_companion(spc3d_plan *p, uint32_t nrows, uint32_t ncols, ui
     DevPlanArrays arr;
     rc = build_device_plan(p->ctx->stream, ncols, nrows, nnz, d_jj, d_ii, po, meta, arr, err);
     if (rc)
-        return fail(rc, err);
+        return optional_path(fail(rc, err));
     spc3d_plan *q = nullptr;
     rc = adopt_device_plan(p->ctx, p->dtype, meta, arr, 0 /* never runs SpMM */, &q);
     if (!rc)
-        rc = add_store_staging(q);
+        rc = add_store_staging(q, so);
     if (rc || (q->perm && !q->store.consecutive)) { // no better than what there is
         if (q) {
             const std::string keep = g_err;
@@ -1327,9 +1352,9 @@ static int add_sddmm_companion(spc3d_plan *p, uint32_t nrows, uint32_t ncols, ui
             q->magic = 0;
             delete q;
             if (rc)
-                return fail(rc, keep);
+                return optional_path(fail(rc, keep));
         }
-        return rc;
+        return optional_path(rc);
     }
     p->by_col = q;
     p->info.sddmm_by_column = 1;
@@ -1354,13 +1379,14 @@ static int build_from_device(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t
     if (rc)
         return rc;
     uint32_t nb = 1;
+    const StoreOpts so = store_opts_of(opts);
     rc = choose_col_blocks(p, opts, &nb);
     if (!rc && nb <= 1)
-        rc = add_store_staging(p);
+        rc = add_store_staging(p, so);
     if (!rc && nb <= 1)
-        rc = add_sddmm_companion(p, nrows, ncols, nnz, d_ii, d_jj, po);
+        rc = add_sddmm_companion(p, nrows, ncols, nnz, d_ii, d_jj, po, so);
     if (!rc && nb <= 1)
-        rc = add_two_pass(p);
+        rc = add_two_pass(p, so);
     if (rc || nb <= 1) {
         if (rc) {
             const std::string keep = g_err;
@@ -1580,9 +1606,9 @@ int spc3d_plan_create_ex(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t nco
         if (!rc)
             rc = finish_plan(p, planned_k(opts));
         if (!rc)
-            rc = add_store_staging(p);
+            rc = add_store_staging(p, store_opts_of(opts));
         if (!rc)
-            rc = add_two_pass(p);
+            rc = add_two_pass(p, store_opts_of(opts));
         if (rc) {
             plan_free_device(p);
             delete p;
@@ -1678,7 +1704,25 @@ int spc3d_plan_download(spc3d_plan *plan, uint32_t *col, uint32_t *perm, uint32_
     return rc;
 }
 
-// Library defaults, each overridable from the environment for tuning runs.
+// A whole non-negative decimal number in the environment; anything else is ignored.
+static bool env_number(const char *name, unsigned long long *out)
+{
+    const char *s = std::getenv(name);
+    if (!s || !*s)
+        return false;
+    unsigned long long v = 0;
+    for (const char *c = s; *c; ++c) {
+        if (*c < '0' || *c > '9' || v > (~0ull - 9) / 10)
+            return false;
+        v = v * 10 + (unsigned)(*c - '0');
+    }
+    *out = v;
+    return true;
+}
+
+// The defaults of spc3d_plan_create and of the one-shot host calls: the library's, each
+// overridable from the environment for tuning runs and A/B comparisons (read here, once
+// per plan, and nowhere else; spc3d_plan_create_ex takes what its caller passes).
 static spc3d_plan_opts opts_from_env()
 {
     spc3d_plan_opts o;
@@ -1691,13 +1735,23 @@ static spc3d_plan_opts opts_from_env()
                {"SPC3D_L2_HOT_BYTES", &o.l2_hot_bytes},
                {"SPC3D_HUB_MIN", &o.hub_min},
                {"SPC3D_XCD_SLICES", &o.xcd_slices},
-               {"SPC3D_COL_BLOCKS", &o.col_blocks}};
+               {"SPC3D_COL_BLOCKS", &o.col_blocks},
+               {"SPC3D_TWO_PASS_MIN", &o.two_pass_min}};
+    unsigned long long v = 0;
     for (auto &e : env)
-        if (const char *s = std::getenv(e.name)) {
-            const long long v = std::atoll(s);
-            if (v > 0 && v <= 0xFFFFFFFFll)
-                *e.field = (uint32_t)v;
-        }
+        if (env_number(e.name, &v) && v > 0 && v <= 0xFFFFFFFFull)
+            *e.field = (uint32_t)v;
+    struct {
+        const char *name;
+        uint32_t off_flag;
+    } sw[] = {{"SPC3D_STAGE_STORES", SPC3D_PLAN_NO_STAGED_STORES},
+              {"SPC3D_SDDMM_BY_COLUMN", SPC3D_PLAN_NO_SDDMM_BY_COLUMN},
+              {"SPC3D_TWO_PASS", SPC3D_PLAN_NO_TWO_PASS}};
+    for (auto &e : sw)
+        if (env_number(e.name, &v) && v == 0)
+            o.flags |= e.off_flag;
+    if (env_number("SPC3D_KEEP_ENTRY_ORDER", &v) && v != 0)
+        o.flags |= SPC3D_PLAN_KEEP_ENTRY_ORDER;
     if (const char *b = std::getenv("SPC3D_PLAN_BUILDER"))
         o.builder = std::strcmp(b, "host") == 0 ? 1u : 2u;
     return o;
@@ -1872,11 +1926,38 @@ int spc3d_plan_probe_columns(spc3d_plan *plan, int mode, uint32_t modulus)
     return SPC3D_OK;
 }
 
+// Device memory one plan object holds (its blocks and companion are added by the caller).
+static uint64_t own_device_bytes(const spc3d_plan *p)
+{
+    const uint64_t w = elem_size(p->dtype), nnz = p->info.nnz;
+    uint64_t b = 0;
+    if (p->segs) b += (uint64_t)p->info.nsegments_padded * sizeof(Seg);
+    if (p->col) b += nnz * 4;
+    if (p->perm) b += nnz * 4;
+    if (p->sval) b += nnz * w;
+    if (p->splits) b += (uint64_t)p->info.nsplit_rows * sizeof(SplitRow);
+    if (p->first_cols)
+        b += (uint64_t)(p->info.nsegments_padded - p->info.nsegments_long) * kFirstCols * 4;
+    if (p->partial) b += (uint64_t)p->info.npartial_slots * p->partial_k * w;
+    b += p->retired_bytes;
+    if (p->store.perm2) b += nnz * 4;
+    if (p->store.n) b += (uint64_t)p->store.n * (8 + w); // dst, src, staged results
+    if (p->two.n) b += nnz * (2 + 4 + 2) + 2 * nnz * w;  // l1, dst1, l2; c_stage, c_mid
+    if (!p->blocks.empty()) b += nnz * (w + 8);          // c_stage, stage_pos, stage_of
+    return b;
+}
+
 int spc3d_plan_get_info(const spc3d_plan *plan, spc3d_plan_info *info)
 {
     if (!live(plan) || !info)
         return fail(SPC3D_ERR_INVALID_ARG, "plan or info is NULL");
     *info = plan->info;
+    uint64_t b = own_device_bytes(plan);
+    for (const spc3d_plan *blk : plan->blocks)
+        b += own_device_bytes(blk);
+    if (plan->by_col)
+        b += own_device_bytes(plan->by_col);
+    info->device_bytes = b;
     return SPC3D_OK;
 }
 
@@ -1898,6 +1979,7 @@ static int ensure_partial(spc3d_plan *p, uint32_t K)
     if (p->partial) {
         try {
             p->retired_partial.push_back(p->partial);
+            p->retired_bytes += (uint64_t)p->info.npartial_slots * p->partial_k * elem_size(p->dtype);
         } catch (const std::bad_alloc &) {
             (void)hipFree(grown);
             return fail(SPC3D_ERR_ALLOC, "host allocation failed");

@@ -364,19 +364,23 @@ __global__ void hubcount_k(const uint32_t *__restrict__ ii, const uint32_t *__re
 }
 
 // Sort key of entry e: its row, then (hub rows of the sliced layout) its group.
+// `visit` (may be null): the keys are laid out in that order of the entries, key[v] = key of
+// entry visit[v].
 template <typename KeyT>
 __global__ void keys_k(const uint32_t *__restrict__ ii, const uint32_t *__restrict__ jj,
                        uint64_t nnz, bool slices, const uint32_t *__restrict__ hubflag,
-                       const uint8_t *__restrict__ cls, KeyT *key)
+                       const uint8_t *__restrict__ cls, const uint32_t *__restrict__ visit,
+                       KeyT *key)
 {
-    GRID_STRIDE(e, nnz)
+    GRID_STRIDE(v, nnz)
     {
+        const uint64_t e = visit ? visit[v] : v;
         const uint32_t r = ii[e];
         if (!slices) {
-            key[e] = (KeyT)r;
+            key[v] = (KeyT)r;
         } else {
             const uint32_t g = hubflag[r] ? hub_group(r, cls[jj[e]]) : 0u;
-            key[e] = (KeyT)(((KeyT)r << 4) | (KeyT)g);
+            key[v] = (KeyT)(((KeyT)r << 4) | (KeyT)g);
         }
     }
 }
@@ -748,18 +752,29 @@ int fetch(hipStream_t st, void *host, const void *dev, size_t bytes, std::string
 
 // Sorts the entries into kernel order: perm (kernel position -> caller's
 // position) and col.  KeyT is wide enough for (row << 4 | group).
+// by_column: the entries are first brought into ascending column order (stable), so that
+// every row ends up ordered by column (col_bits: bits of the largest column id).
 template <typename KeyT>
 int order_entries(Arena &arena, Temp &tmp, hipStream_t st, uint64_t nnz, int key_bits, bool slices,
-                  const uint32_t *d_ii, const uint32_t *d_jj, const uint32_t *hubflag,
-                  const uint8_t *cls, uint32_t *perm, uint32_t *col, Counters *C, std::string &err)
+                  bool by_column, int col_bits, const uint32_t *d_ii, const uint32_t *d_jj,
+                  const uint32_t *hubflag, const uint8_t *cls, uint32_t *perm, uint32_t *col,
+                  Counters *C, std::string &err)
 {
     SBuf<KeyT> key, key_out;
     SBuf<uint32_t> ident;
     HIP_OK(key.alloc(arena, nnz));
     HIP_OK(key_out.alloc(arena, nnz));
     HIP_OK(ident.alloc(arena, nnz));
-    LAUNCH((keys_k<KeyT>), nnz, d_ii, d_jj, nnz, slices, hubflag, cls, key.p);
     LAUNCH(iota_k, nnz, ident.p, nnz);
+    const uint32_t *visit = nullptr;
+    if (by_column) {
+        // col and perm are free until the end: sorted columns (unused) and the visiting order
+        TRY(sort_pairs<uint32_t>(tmp, d_jj, col, ident.p, perm, (uint32_t)nnz, col_bits, false, st,
+                                 err));
+        HIP_OK(hipMemcpyAsync(ident.p, perm, nnz * sizeof(uint32_t), hipMemcpyDeviceToDevice, st));
+        visit = ident.p;
+    }
+    LAUNCH((keys_k<KeyT>), nnz, d_ii, d_jj, nnz, slices, hubflag, cls, visit, key.p);
     TRY(sort_pairs<KeyT>(tmp, key.p, key_out.p, ident.p, perm, (uint32_t)nnz, key_bits, false, st,
                          err));
     LAUNCH(gather_cols_k, nnz, d_jj, perm, nnz, col, C);
@@ -889,10 +904,12 @@ int build_device_plan(hipStream_t st, uint32_t nrows, uint32_t ncols, uint64_t n
         err = buf;
         return SPC3D_ERR_BAD_INDEX;
     }
+    bool rows_unsorted = false;
     {
         SBuf<uint32_t> sorted, start;
         HIP_OK(sorted.alloc(arena, nnz));
         HIP_OK(start.alloc(arena, std::max<size_t>(ncols, nrows)));
+        rows_unsorted = hC.rows_unsorted != 0;
         if (hC.rows_unsorted) {
             TRY(sort_keys(tmp, d_ii, sorted.p, (uint32_t)nnz, bits_for(nrows ? nrows - 1 : 0), st,
                           err));
@@ -970,12 +987,16 @@ int build_device_plan(hipStream_t st, uint32_t nrows, uint32_t ncols, uint64_t n
     {
         const int row_bits = bits_for(nrows ? nrows - 1 : 0);
         const int key_bits = row_bits + (slices ? 4 : 0);
+        const bool by_column = rows_unsorted && !opts.keep_entry_order;
+        const int col_bits = bits_for(ncols ? ncols - 1 : 0);
+        P.by_column_in_rows = by_column;
         if (key_bits <= 32)
-            TRY(order_entries<uint32_t>(arena, tmp, st, nnz, key_bits, slices, d_ii, d_jj, hubflag.p,
-                                        cls.p, perm.p, col.p, dC.p, err));
+            TRY(order_entries<uint32_t>(arena, tmp, st, nnz, key_bits, slices, by_column, col_bits,
+                                        d_ii, d_jj, hubflag.p, cls.p, perm.p, col.p, dC.p, err));
         else
-            TRY(order_entries<unsigned long long>(arena, tmp, st, nnz, key_bits, slices, d_ii, d_jj,
-                                                  hubflag.p, cls.p, perm.p, col.p, dC.p, err));
+            TRY(order_entries<unsigned long long>(arena, tmp, st, nnz, key_bits, slices, by_column,
+                                                  col_bits, d_ii, d_jj, hubflag.p, cls.p, perm.p,
+                                                  col.p, dC.p, err));
     }
 
     // ---- segments --------------------------------------------------------------------

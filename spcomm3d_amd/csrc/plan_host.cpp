@@ -181,6 +181,23 @@ int build_host_plan(uint32_t nrows, uint32_t ncols, uint64_t nnz, const uint32_t
         }
 
         // ---- stable scatter into kernel order ------------------------------
+        // Rows that arrive unsorted: the entries are visited in ascending column order
+        // (a stable counting sort), so that every row ends up ordered by column.
+        std::vector<uint32_t> visit;
+        {
+            bool down = false;
+            for (uint64_t e = 1; e < nnz && !down; ++e)
+                down = ii[e - 1] > ii[e];
+            if (down && !opts.keep_entry_order) {
+                std::vector<uint32_t> at((size_t)ncols + 1, 0);
+                for (uint32_t c = 0; c < ncols; ++c)
+                    at[(size_t)c + 1] = at[c] + coldeg[c];
+                visit.resize(nnz);
+                for (uint64_t e = 0; e < nnz; ++e)
+                    visit[at[jj[e]]++] = (uint32_t)e;
+                P.by_column_in_rows = true;
+            }
+        }
         P.col.resize(nnz);
         P.perm.resize(nnz);
         {
@@ -196,7 +213,8 @@ int build_host_plan(uint32_t nrows, uint32_t ncols, uint64_t nnz, const uint32_t
                 }
             }
             uint32_t notid = 0;
-            for (uint64_t e = 0; e < nnz; ++e) {
+            for (uint64_t v = 0; v < nnz; ++v) {
+                const uint64_t e = visit.empty() ? v : visit[v];
                 const uint32_t r = ii[e];
                 const uint32_t p = (slices && hubidx[r] >= 0)
                                        ? cur_h[(size_t)hubidx[r] * 9 + group_of(r, jj[e])]++

@@ -44,6 +44,11 @@ struct PlanOpts {
     uint32_t xcd_slices = 0; // 8 (default): hot columns are dealt to the 8 XCD L2s; 1: off
     uint32_t hot_cols = 0;   // slicing: dense rows one L2 is expected to keep
     uint32_t hub_min = 0;    // slicing: rows with at least this many entries are cut by slice (default 128)
+    // A pattern whose rows arrive unsorted (ii steps down somewhere) has no order inside
+    // its rows worth keeping for the gathers: its entries are then ordered by column inside
+    // every row (equal columns in the caller's order), which is what a row-sorted
+    // pattern's entries usually are.  true: always keep the caller's order inside a row.
+    bool keep_entry_order = false;
 };
 
 struct HostPlan {
@@ -61,6 +66,7 @@ struct HostPlan {
     uint64_t hot_entries = 0;      // entries in those columns
     uint32_t hub_rows = 0;         // rows cut by column slice
     bool identity = true;          // perm[p] == p for all p
+    bool by_column_in_rows = false; // unsorted rows: entries ordered by column inside each row
     std::vector<uint32_t> col;     // [nnz] column of kernel-order entry p
     std::vector<uint32_t> perm;    // [nnz] caller's position of kernel-order entry p
     std::vector<Seg> segs;         // chunked: chunk v (64 segments) belongs to queue v % nqueues
@@ -173,7 +179,8 @@ int validate_coo(uint32_t nrows, uint32_t ncols, uint64_t nnz, const uint32_t *i
                  const uint32_t *jj, std::string &err);
 
 // Validates, then builds.  Entries are grouped by row, the caller's order kept
-// inside a row (the order the reference accumulates in, core_ops.cpp:26-34).
+// inside a row (the order the reference accumulates in, core_ops.cpp:26-34) when the
+// rows arrive sorted or PlanOpts::keep_entry_order is set, else ascending by column.
 // With XCD slicing, the entries of a hub row are further grouped by the slice
 // of their column, the caller's order kept inside each group.
 int build_host_plan(uint32_t nrows, uint32_t ncols, uint64_t nnz, const uint32_t *ii,

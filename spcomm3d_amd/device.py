@@ -32,10 +32,20 @@ _BUILDERS = {None: 0, "device": 2, "host": 1}
 
 
 def make_opts(seg_max=None, k_hint=None, l2_hot_bytes=None, hub_min=None,
-              xcd_slices=None, builder=None, col_blocks=None) -> PlanOpts:
+              xcd_slices=None, builder=None, col_blocks=None, staged_stores=None,
+              sddmm_by_column=None, two_pass=None, two_pass_min=None,
+              keep_entry_order=None) -> PlanOpts:
     """``spc3d_plan_opts``; ``None`` keeps the library default.  ``builder``:
-    ``"device"`` or ``"host"`` (where ``spc3d_plan_create_ex`` builds the plan)."""
+    ``"device"`` or ``"host"`` (where ``spc3d_plan_create_ex`` builds the plan).
+    ``staged_stores`` / ``sddmm_by_column`` / ``two_pass`` = False keep the plain stores
+    of SDDMM results; ``keep_entry_order`` = True keeps the caller's order inside rows
+    that arrive unsorted."""
     o = PlanOpts()
+    o.flags = ((capi.PLAN_NO_STAGED_STORES if staged_stores is False else 0) |
+               (capi.PLAN_NO_SDDMM_BY_COLUMN if sddmm_by_column is False else 0) |
+               (capi.PLAN_NO_TWO_PASS if two_pass is False else 0) |
+               (capi.PLAN_KEEP_ENTRY_ORDER if keep_entry_order else 0))
+    o.two_pass_min = int(two_pass_min or 0)
     o.builder = _BUILDERS[builder]
     o.seg_max = int(seg_max or 0)
     o.k_hint = int(k_hint or 0)

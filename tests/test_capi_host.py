@@ -93,9 +93,17 @@ def _check_plan(nrows, ncols, ii, jj, **opts):
     assert np.array_equal(col, jj[perm])
     rows_k = ii[perm]
     assert np.all(np.diff(rows_k.astype(np.int64)) >= 0)
-    if info.nqueues == 1:  # no slicing: the caller's order survives inside every row
+    unsorted = bool(np.any(np.diff(ii.astype(np.int64)) < 0)) and not opts.get("keep_entry_order")
+    assert info.entries_by_column == int(unsorted)
+    if info.nqueues == 1:
         same = rows_k[1:] == rows_k[:-1]
-        assert np.all(perm[1:][same] > perm[:-1][same])
+        if not unsorted:  # no slicing: the caller's order survives inside every row
+            assert np.all(perm[1:][same] > perm[:-1][same])
+        else:  # rows that arrive unsorted: by column inside a row, equal columns in caller's order
+            c = col.astype(np.int64)
+            assert np.all((c[1:] >= c[:-1])[same])
+            tie = same & (c[1:] == c[:-1])
+            assert np.all(perm[1:][tie] > perm[:-1][tie])
     assert bool(info.order_is_identity) == bool(np.array_equal(perm, np.arange(nnz)))
     assert info.rows_touched == np.unique(ii).size and info.cols_touched == np.unique(jj).size
     assert info.max_row_nnz == (np.bincount(ii).max() if nnz else 0)
@@ -155,6 +163,7 @@ def test_plan_random_unsorted_with_duplicates(seg_max):
     ii[:300] = 7  # a hub row
     o = rng.permutation(900)
     _check_plan(50, 70, ii[o], jj[o], seg_max=seg_max)
+    _check_plan(50, 70, ii[o], jj[o], seg_max=seg_max, keep_entry_order=True)
 
 
 def test_plan_default_seg_max_follows_nnz():
@@ -206,10 +215,17 @@ def test_plan_xcd_slicing_on_skewed_pattern():
     chunk = np.arange(segs.shape[0]) // 64
     load = np.array([segs[(chunk % 8) == q][:, 2].sum() for q in range(8)], dtype=np.int64)
     assert load.max() - load.min() <= 0.02 * load.mean() + 256
-    # inside a hub row the caller's order survives within each piece
-    perm, rows_k = P["perm"], w.ii[P["perm"]]
+    # the rows arrive unsorted: inside each piece the entries are ordered by column
+    # (R-MAT patterns hold no duplicates), and with keep_entry_order in the caller's order
+    perm, rows_k, col = P["perm"], w.ii[P["perm"]], P["col"]
+    assert info.entries_by_column == 1
     for row, start, ln, slot in segs[segs[:, 2] > 1][:200]:
-        assert np.all(np.diff(perm[start:start + ln].astype(np.int64)) > 0)
+        assert np.all(np.diff(col[start:start + ln].astype(np.int64)) > 0)
+    K = _check_plan(w.nrows, w.ncols, w.ii, w.jj, xcd_slices=8, l2_hot_bytes=64 * 1024,
+                    hub_min=32, seg_max=256, keep_entry_order=True)
+    assert K["info"].entries_by_column == 0
+    for row, start, ln, slot in K["segs"][K["segs"][:, 2] > 1][:200]:
+        assert np.all(np.diff(K["perm"][start:start + ln].astype(np.int64)) > 0)
     # every entry of one hub piece with a slice column sits in that slice's queue:
     # same column -> same queue, wherever it appears in hub rows
     counts = np.bincount(w.ii, minlength=w.nrows)

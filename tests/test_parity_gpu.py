@@ -585,7 +585,7 @@ def test_column_sorted_input_runs_sddmm_through_the_exchanged_plan(ctx, dtype, k
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_arbitrary_order_brings_results_home_in_two_passes(ctx, dtype, monkeypatch):
+def test_arbitrary_order_brings_results_home_in_two_passes(ctx, dtype):
     """An arbitrary entry order: the kernels write in kernel order, two passes of tile-local
     moves bring the results to the caller's positions (plan info two_pass_results; from 1.5 M
     entries on by default, here from the smallest size the scheme takes).  Bit for bit what the
@@ -593,13 +593,10 @@ def test_arbitrary_order_brings_results_home_in_two_passes(ctx, dtype, monkeypat
     into a wrapped value vector."""
     w = W.rmat(14, 16, 64).shuffled()
     A, B, Y0, vv = w.panel_A(dtype), w.panel_B(dtype), w.panel_Y0(dtype), w.values(dtype)
-    monkeypatch.setenv("SPC3D_TWO_PASS", "0")
-    plain = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, vv)
-    monkeypatch.delenv("SPC3D_TWO_PASS")
-    monkeypatch.setenv("SPC3D_TWO_PASS_MIN", "1")
-    S = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, vv)
-    tiny = ctx.plan(w.nrows, w.ncols, w.ii[:1000], w.jj[:1000], vv[:1000])  # under two tiles
-    monkeypatch.delenv("SPC3D_TWO_PASS_MIN")
+    plain = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, vv, two_pass=False, two_pass_min=1)
+    S = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, vv, two_pass_min=1)
+    tiny = ctx.plan(w.nrows, w.ncols, w.ii[:1000], w.jj[:1000], vv[:1000],
+                    two_pass_min=1)  # under two tiles
     assert plain.info.two_pass_results == 0 and tiny.info.two_pass_results == 0
     assert S.info.two_pass_results == 1 and S.info.staged_entries == 0
     dA, dB, dY, dC = ctx.panel_from(A), ctx.panel_from(B), ctx.panel_from(Y0), ctx.vals(w.nnz, dtype)
