@@ -254,6 +254,36 @@ def run_floors(w, dtype, steps, warmup, seg_max=None):
     return out
 
 
+def run_dist_step(w, dtype, reps):
+    """One step of the reference's distributed wrappers over device-resident operands
+    (dist_sddmm_spcomm, dist_spmm_spcomm; src/distributed_comp.cpp:141-193,17-76): the
+    host C++ program spcomm3d_amd/lib/dist_step_<real> reads the workload from a .bin file
+    (the reference's format, tools/read_convert_mm.cpp:81-94) written here, and reports the
+    wall-clock time per wrapper call beside the device time of the kernel inside it.  None
+    when the program is not built."""
+    import subprocess
+    import tempfile
+
+    exe = os.path.join(ROOT, "spcomm3d_amd", "lib", f"dist_step_{dtype}")
+    if not os.path.exists(exe):
+        return None
+    rec = np.empty(w.nnz, dtype=np.dtype([("r", "<u4"), ("c", "<u4"), ("v", "<f8")]))
+    rec["r"], rec["c"], rec["v"] = w.ii, w.jj, w.values("f64")
+    with tempfile.TemporaryDirectory(dir="/dev/shm" if os.path.isdir("/dev/shm") else None) as d:
+        path = os.path.join(d, "workload.bin")
+        with open(path, "wb") as f:
+            f.write(np.array([w.nrows, w.ncols], dtype="<u4").tobytes())
+            f.write(np.array([w.nnz], dtype="<u8").tobytes())
+            rec.tofile(f)
+        del rec
+        r = subprocess.run([exe, path, str(w.k), str(reps)], capture_output=True, text=True,
+                           timeout=600)
+    if r.returncode != 0:
+        log(f"dist_step failed: {r.stderr[-500:]}")
+        return None
+    return json.loads(r.stdout.strip().splitlines()[-1])
+
+
 def run_compact(w, dtype, steps, warmup):
     """One compact row for a workload: mean time per kernel over `steps` passes on
     resident operands, strict-model fraction of the HBM peak."""
@@ -398,6 +428,8 @@ def main():
                     help="only the all-hit / all-miss floors of the workload's launches "
                          "(they are part of the default run as well)")
     ap.add_argument("--no-floors", action="store_true", help="skip the floors")
+    ap.add_argument("--no-dist", action="store_true",
+                    help="skip the step through the device-resident dist_* wrappers")
     ap.add_argument("--only", action="store_true", help="skip the other real type")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-configs", action="store_true",
@@ -438,6 +470,10 @@ def main():
         floors = {dt: run_floors(w, dt, max(5, args.steps // 2), args.warmup, args.seg_max)
                   for dt in ((args.dtype,) if args.only else ("f64", "f32"))}
         log(json.dumps(floors))
+    dist_step = None
+    if not args.no_dist:
+        dist_step = run_dist_step(w, args.dtype, max(5, args.steps // 2))
+        log(json.dumps(dist_step))
     if not (args.only or args.no_configs):
         ws = w.shuffled() if w.order == "sorted" else None
         if ws is not None:
@@ -506,6 +542,7 @@ def main():
         "cpu_baseline": cpu,
         "kernels": main_r["kernels"],
         "fused_step": main_r["fused_step"],
+        "dist_step": dist_step,
         "row_copies": main_r["row_copies"],
         "plan": {k: main_r[k] for k in ("plan_build_s", "upload_s", "nsegments", "nsplit_rows",
                                         "seg_max")},

@@ -241,6 +241,13 @@ SPC3D_API int spc3d_vals_upload(spc3d_vals *v, const void *host);
 SPC3D_API int spc3d_vals_download(spc3d_vals *v, void *host);
 SPC3D_API int spc3d_vals_fill(spc3d_vals *v, double value);
 SPC3D_API int spc3d_vals_device_ptr(spc3d_vals *v, void **dev);
+/* dst[dst_off .. dst_off + n) = src[src_off .. src_off + n) on the device (same dtype, ranges
+ * that do not overlap): what a message a rank addresses to itself amounts to, sendBuff +
+ * sendDisp to recvBuff + recvDisp (src/comm.hpp:113-130), and the Z reduction of SDDMM over
+ * one rank, C.vv to C.ownedVals (src/denseComm.hpp:39).  Asynchronous on the context's
+ * stream; may be recorded. */
+SPC3D_API int spc3d_vals_copy(spc3d_vals *dst, uint64_t dst_off, const spc3d_vals *src,
+                    uint64_t src_off, uint64_t n);
 
 /* ---- plan: the sparse operand ------------------------------------------ */
 /* Host-only check of a COO pattern; needs no GPU.  Mirrors the bounds checks

@@ -79,6 +79,7 @@ SIGNATURES = {
     "spc3d_vals_download": (c_int, [c_vp, c_vp]),
     "spc3d_vals_fill": (c_int, [c_vp, c_double]),
     "spc3d_vals_device_ptr": (c_int, [c_vp, P(c_vp)]),
+    "spc3d_vals_copy": (c_int, [c_vp, c_u64, c_vp, c_u64, c_u64]),
     "spc3d_coo_validate": (c_int, [c_u32, c_u32, c_u64, c_vp, c_vp]),
     "spc3d_plan_create": (c_int, [c_vp, c_int, c_u32, c_u32, c_u64, c_vp, c_vp, c_vp, P(c_vp)]),
     "spc3d_plan_create_ex": (c_int, [c_vp, c_int, c_u32, c_u32, c_u64, c_vp, c_vp, c_vp,

@@ -983,6 +983,36 @@ int spc3d_vals_device_ptr(spc3d_vals *v, void **dev)
     return SPC3D_OK;
 }
 
+static bool ranges_overlap(const void *a, size_t abytes, const void *b, size_t bbytes);
+
+int spc3d_vals_copy(spc3d_vals *dst, uint64_t dst_off, const spc3d_vals *src, uint64_t src_off,
+                    uint64_t n)
+{
+    if (!live(dst) || !live(src))
+        return fail(SPC3D_ERR_INVALID_ARG, "a value vector is NULL or destroyed");
+    if (dst->ctx != src->ctx)
+        return fail(SPC3D_ERR_INVALID_ARG, "operands belong to different contexts");
+    if (dst->dtype != src->dtype)
+        return fail(SPC3D_ERR_SIZE_MISMATCH, "value vectors of different types");
+    if (dst_off > dst->n || n > dst->n - dst_off || src_off > src->n || n > src->n - src_off)
+        return fail(SPC3D_ERR_SIZE_MISMATCH, "the range leaves a value vector");
+    if (n == 0)
+        return SPC3D_OK;
+    int rc = use_device(dst->ctx, true);
+    if (rc)
+        return rc;
+    const size_t w = elem_size(dst->dtype);
+    char *d = static_cast<char *>(dst->dev) + dst_off * w;
+    const char *s = static_cast<const char *>(src->dev) + src_off * w;
+    if (ranges_overlap(d, n * w, s, n * w))
+        return fail(SPC3D_ERR_INVALID_ARG, "source and destination ranges overlap");
+    if ((((uintptr_t)d | (uintptr_t)s) & 15u) == 0)
+        HIP_TRY(launch_copy(d, s, n * w, dst->ctx->stream));
+    else
+        HIP_TRY(hipMemcpyAsync(d, s, n * w, hipMemcpyDeviceToDevice, dst->ctx->stream));
+    return SPC3D_OK;
+}
+
 /* ---- plan ---------------------------------------------------------------- */
 int spc3d_coo_validate(uint32_t nrows, uint32_t ncols, uint64_t nnz, const uint32_t *ii,
                        const uint32_t *jj)

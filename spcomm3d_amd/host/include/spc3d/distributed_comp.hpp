@@ -36,9 +36,13 @@ struct Mesh {
     int X = 1, Y = 1, Z = 1;
 };
 
-// Sparse point-to-point plan of one rank (src/comm.hpp:33-52): who sends what
-// to whom.  On one rank there is nobody to talk to; a plan that says otherwise
-// cannot be executed here.
+// Sparse point-to-point plan of one rank (src/comm.hpp:33-52): who sends what to
+// whom.  On one rank the only possible peer is the rank itself: a plan may hold
+// messages addressed to rank 0 (what MPI delivers when a rank sends to itself), which
+// exercises the copies either side of an exchange (src/comm.hpp:90-103,166-189)
+// exactly as the reference runs them; a plan that names any other rank cannot be
+// executed here.  Counts and displacements are in reals, as in the reference; send i is
+// matched with receive i (one source, one tag: MPI matches them in order).
 template <typename T> class SparseComm {
   public:
     int inDegree = 0, outDegree = 0;
@@ -52,20 +56,71 @@ template <typename T> class SparseComm {
     SparseComm() = default;
     explicit SparseComm(idx_t unitSize) : dataUnitSize(unitSize) {}
 
-    void issue_Irecvs() { require_single(); }
-    void issue_Sends(bool = false) { require_single(); }
-    void issue_Waitall() { require_single(); }
-    void copy_to_sendbuff() { require_single(); }
-    void copy_from_recvbuff() { require_single(); }
-    void SUM_from_recvbuff() { require_single(); }
-    void perform_sparse_comm(bool = true, bool = true) { require_single(); }
+    void issue_Irecvs() { require_self(); }
+    // with_DT: the reference sends straight out of the dense panel through derived
+    // datatypes (src/comm.hpp:113-118); no self-addressed form of that is kept here.
+    void issue_Sends(bool with_DT = false)
+    {
+        require_self();
+        if (with_DT && outDegree != 0)
+            throw std::runtime_error("SparseComm: datatype sends have no single-rank form");
+        for (int i = 0; i < outDegree; ++i) {
+            if (sendCount.at(i) != recvCount.at(i))
+                throw std::runtime_error("SparseComm: a self-addressed message must be received "
+                                         "with the length it is sent with");
+            for (int k = 0; k < sendCount[i]; ++k)
+                recvBuff.at((size_t)recvDisp.at(i) + k) = sendBuff.at((size_t)sendDisp.at(i) + k);
+        }
+    }
+    void issue_Waitall() { require_self(); }
+    void copy_to_sendbuff() // src/comm.hpp:90-103
+    {
+        require_self();
+        size_t idx = 0;
+        for (size_t i = 0; i < sendptr.size(); ++i)
+            for (size_t j = 0; j < dataUnitSize; ++j)
+                sendBuff.at(idx++) = sendptr[i][j];
+    }
+    void copy_from_recvbuff() // src/comm.hpp:166-177
+    {
+        require_self();
+        size_t idx = 0;
+        for (size_t i = 0; i < recvptr.size(); ++i)
+            for (size_t j = 0; j < dataUnitSize; ++j)
+                recvptr[i][j] = recvBuff.at(idx++);
+    }
+    void SUM_from_recvbuff() // src/comm.hpp:178-189
+    {
+        require_self();
+        size_t idx = 0;
+        for (size_t i = 0; i < recvptr.size(); ++i)
+            for (size_t j = 0; j < dataUnitSize; ++j)
+                recvptr[i][j] += recvBuff.at(idx++);
+    }
+    void perform_sparse_comm(bool sendcopyflag = true, bool recvcopyflag = true)
+    {
+        issue_Irecvs();
+        if (sendcopyflag)
+            copy_to_sendbuff();
+        issue_Sends();
+        issue_Waitall();
+        if (recvcopyflag)
+            copy_from_recvbuff();
+    }
 
   private:
-    void require_single() const
+    void require_self() const
     {
-        if (inDegree != 0 || outDegree != 0)
+        bool ok = inDegree == outDegree && (size_t)inDegree == inSet.size() &&
+                  (size_t)outDegree == outSet.size();
+        for (int r : inSet)
+            ok = ok && r == 0;
+        for (int r : outSet)
+            ok = ok && r == 0;
+        if (!ok)
             throw std::runtime_error("SparseComm: exchanges between ranks are outside this "
-                                     "single-GPU library");
+                                     "single-GPU library (only messages a rank addresses to "
+                                     "itself can be carried out)");
     }
 };
 
@@ -143,9 +198,12 @@ void dist_set_stats_stream(std::FILE *f);
 // Phase times of the last dist_* call on this thread: the reference's five
 // millisecond counters, and the compute phase again as the device measured it, in
 // microseconds (a GPU kernel lasts well under the reference's 1 ms resolution).
+// The device-resident wrappers (distributed_comp_device.hpp) fill every microsecond field
+// from device events; the host-memory wrappers fill compTimeUs only.
 struct distTiming {
     SpKernels::parallelTiming pt;
     SpKernels::idx_large_t compTimeUs = 0;
+    SpKernels::idx_large_t comm1TimeUs = 0, comm2TimeUs = 0, commcpyTimeUs = 0, totalTimeUs = 0;
 };
 const distTiming &dist_last_timing();
 

@@ -9,6 +9,8 @@
 
 #include "spc3d/core_ops.hpp"
 
+#include "dist_internal.hpp"
+
 using namespace SpKernels;
 using DComm::DenseComm;
 
@@ -18,82 +20,40 @@ std::FILE *g_stats = stdout;
 thread_local distTiming g_last;
 
 using clk = std::chrono::high_resolution_clock;
+using spc3d_dist::print_line;
+using spc3d_dist::require_single;
+using spc3d_dist::stats_sparse;
+using spc3d_dist::stats_sparse2;
 
 idx_t ms_since(clk::time_point t0)
 {
     return (idx_t)std::chrono::duration_cast<std::chrono::milliseconds>(clk::now() - t0).count();
 }
 
-void require_single(const Mesh &mesh)
+spc3d_dist::DenseShape shape_of(const DenseComm &d)
 {
-    if (mesh.X != 1 || mesh.Y != 1 || mesh.Z != 1)
-        throw std::runtime_error("dist_*: this library runs one rank on one GPU; the mesh must be "
-                                 "1 x 1 x 1");
+    spc3d_dist::DenseShape s;
+    s.reduce_scatter = d.OP == 1 && d.commXflag && d.commYflag;
+    s.x = d.commXflag;
+    s.y = d.commYflag;
+    if (!d.bcastXcnt.empty()) {
+        s.cnt0 = d.bcastXcnt[0];
+        s.last_end = (d.bcastXdisp.empty() ? 0 : d.bcastXdisp.back()) + d.bcastXcnt.back();
+        s.x0 = d.bcastXcnt[0];
+    }
+    if (!d.bcastYcnt.empty())
+        s.y0 = d.bcastYcnt[0];
+    s.all_x = (idx_large_t)std::accumulate(d.bcastXcnt.begin(), d.bcastXcnt.end(), 0.0);
+    s.all_y = (idx_large_t)std::accumulate(d.bcastYcnt.begin(), d.bcastYcnt.end(), 0.0);
+    s.outDegreeX = d.outDegreeX;
+    s.outDegreeY = d.outDegreeY;
+    return s;
 }
 
-// "mtx alg P Kloc Z avgSendMsg avgSendVol avgRecvMsg avgRecvVol maxSendMsg
-//  maxSendVol maxRecvMsg maxRecvVol comm1 comm2 commcpy comp total"
-// (src/comm_stats.cpp:33-36,53,71-73) with P = 1: averages equal maxima.
-void print_line(const std::string &mtx, const char *alg, idx_t f, const Mesh &mesh,
-                idx_large_t sendMsg, idx_large_t sendVol, idx_large_t recvMsg,
-                idx_large_t recvVol, const parallelTiming &pt)
-{
-    if (!g_stats)
-        return;
-    std::fprintf(g_stats, "%s %s %d %u %d %.2f %.2f %.2f %.2f %lu %lu %lu %lu %u %u %u %u %u\n",
-                 mtx.c_str(), alg, 1, f, mesh.Z, (float)sendMsg, (float)sendVol, (float)recvMsg,
-                 (float)recvVol, (unsigned long)sendMsg, (unsigned long)sendVol,
-                 (unsigned long)recvMsg, (unsigned long)recvVol, pt.comm1Time, pt.comm2Time,
-                 pt.commcpyTime, pt.compTime, pt.totalTime);
-}
-
-// src/comm_stats.cpp:59-73
-void stats_sparse(const std::string &mtx, const char *alg, const SparseComm<real_t> &c, idx_t f,
-                  const parallelTiming &pt, const Mesh &mesh)
-{
-    const idx_large_t sv = (idx_large_t)std::accumulate(c.sendCount.begin(), c.sendCount.end(), 0.0);
-    const idx_large_t rv = (idx_large_t)std::accumulate(c.recvCount.begin(), c.recvCount.end(), 0.0);
-    print_line(mtx, alg, f, mesh, (idx_large_t)c.outDegree, sv, (idx_large_t)c.inDegree, rv, pt);
-}
-
-// src/comm_stats.cpp:74-92
-void stats_sparse2(const std::string &mtx, const char *alg, const SparseComm<real_t> &a,
-                   const SparseComm<real_t> &b, idx_t f, const parallelTiming &pt,
-                   const Mesh &mesh)
-{
-    const idx_large_t sv =
-        (idx_large_t)(std::accumulate(a.sendCount.begin(), a.sendCount.end(), 0.0) +
-                      std::accumulate(b.sendCount.begin(), b.sendCount.end(), 0.0));
-    const idx_large_t rv =
-        (idx_large_t)(std::accumulate(a.recvCount.begin(), a.recvCount.end(), 0.0) +
-                      std::accumulate(b.recvCount.begin(), b.recvCount.end(), 0.0));
-    print_line(mtx, alg, f, mesh, (idx_large_t)(a.outDegree + b.outDegree), sv,
-               (idx_large_t)(a.inDegree + b.inDegree), rv, pt);
-}
-
-// src/comm_stats.cpp:93-129, with this rank being rank 0 of every sub-communicator
 void stats_dense(const std::string &mtx, const char *alg, const DenseComm &d, idx_t f,
                  const parallelTiming &pt, const Mesh &mesh)
 {
-    idx_large_t sendVol = 0, recvVol = 0, sendMsg = 1, recvMsg = 0;
-    if (d.OP == 1 && d.commXflag && d.commYflag) {
-        if (!d.bcastXcnt.empty()) {
-            sendVol = (d.bcastXdisp.empty() ? 0 : d.bcastXdisp.back()) + d.bcastXcnt.back();
-            recvVol = d.bcastXcnt[0];
-        }
-        recvMsg = 1;
-    } else {
-        idx_large_t all = 0;
-        if (d.commXflag)
-            all += (idx_large_t)std::accumulate(d.bcastXcnt.begin(), d.bcastXcnt.end(), 0.0);
-        if (d.commYflag)
-            all += (idx_large_t)std::accumulate(d.bcastYcnt.begin(), d.bcastYcnt.end(), 0.0);
-        sendVol = (d.commXflag && !d.bcastXcnt.empty() ? d.bcastXcnt[0] : 0) +
-                  (d.commYflag && !d.bcastYcnt.empty() ? d.bcastYcnt[0] : 0);
-        recvVol = all - sendVol;
-        recvMsg = (d.commXflag ? d.outDegreeX : 0) + (d.commYflag ? d.outDegreeY : 0);
-    }
-    print_line(mtx, alg, f, mesh, sendMsg, sendVol, recvMsg, recvVol, pt);
+    spc3d_dist::stats_dense(mtx, alg, shape_of(d), f, pt, mesh);
 }
 
 // Times fn with the wall clock (integer ms, as the reference) and takes the
@@ -107,6 +67,9 @@ template <typename F> void timed_kernel(parallelTiming &pt, F fn)
 }
 
 } // namespace
+
+std::FILE *&spc3d_dist::stats_stream() { return g_stats; }
+distTiming &spc3d_dist::last_timing() { return g_last; }
 
 void dist_set_stats_stream(std::FILE *f) { g_stats = f; }
 

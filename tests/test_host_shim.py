@@ -56,6 +56,16 @@ def test_shim_on_gpu(name):
     _run(name)
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["test_dist_resident_f64", "test_dist_resident_f32"])
+def test_dist_wrappers_over_device_resident_operands(name):
+    # the six wrappers over panels, plan, values and exchange buffers that stay on the device,
+    # with self-addressed exchanges so that the pack / unpack / sum-unpack kernels run
+    # (src/distributed_comp.cpp:17-76,141-236, src/comm.hpp:90-103,166-189): bit-equal to
+    # the host-memory wrappers, both against the oracle
+    _run(name)
+
+
 def _mpi_env():
     """Environment in which a program linked with the image's MPI library starts: the
     system's libstdc++ ahead of the MPI library's own directory."""
