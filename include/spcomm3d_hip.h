@@ -176,7 +176,27 @@ SPC3D_API const char *spc3d_status_name(int status);
 SPC3D_API int spc3d_device_count(int *count);
 
 /* ---- context ----------------------------------------------------------- */
+/* A context is one device, one stream (plus an auxiliary one of the same priority on which
+ * the short-segment launch of a call runs beside the long-segment one) and what the one-shot
+ * host calls keep between calls.  One caller thread per context, as the reference runs one
+ * thread per MPI rank (MPI_Init in miniapp/bench_both.cpp:124): host_threads is how many host
+ * threads a one-shot call over host memory (spc3d_*_host) may use, the caller's included, for
+ * reading operands and moving Y; the default, 1, starts none, so that several ranks per node
+ * do not oversubscribe it (SPC3D_HOST_THREADS in the environment gives spc3d_ctx_create
+ * another default; 8 is what one rank per node can use).  Everything else in the library
+ * runs on the caller's thread. */
+typedef struct {
+    uint32_t host_threads; /* 0: default (1); at most 256 */
+    uint32_t flags;        /* SPC3D_CTX_* bits */
+    uint32_t reserved[6];  /* must be 0 */
+} spc3d_ctx_opts;
+#define SPC3D_CTX_NO_AUX_STREAM 1u /* every launch on the one stream */
+#define SPC3D_CTX_NO_HOST_CACHE 2u /* one-shot host calls: plan, upload, run, download, free, every call */
+/* spc3d_ctx_create takes its options from the environment (SPC3D_HOST_THREADS=n,
+ * SPC3D_AUX_STREAM=0, SPC3D_HOST_CACHE=0; read here and nowhere else), spc3d_ctx_create_ex
+ * from its argument (NULL: the library defaults). */
 SPC3D_API int spc3d_ctx_create(int device, spc3d_ctx **out);
+SPC3D_API int spc3d_ctx_create_ex(int device, const spc3d_ctx_opts *opts, spc3d_ctx **out);
 SPC3D_API int spc3d_ctx_destroy(spc3d_ctx *ctx);
 SPC3D_API int spc3d_ctx_sync(spc3d_ctx *ctx);                 /* wait for the context's stream */
 SPC3D_API int spc3d_ctx_stream(spc3d_ctx *ctx, void **hip_stream); /* the hipStream_t, for callers that share it */
@@ -430,8 +450,9 @@ SPC3D_API int spc3d_rows_unpack_sum(spc3d_ctx *ctx, spc3d_panel *P, const spc3d_
  *   - the result vector of SDDMM.
  * Reading an unchanged operand for its keys (several threads) takes about half the time
  * of sending it.  The cache holds device memory until spc3d_host_cache_clear or
- * spc3d_ctx_destroy; SPC3D_HOST_CACHE=0 in the environment gives plan, upload, run,
- * download, free on every call instead.  One-shot calls on one context run one at a time
+ * spc3d_ctx_destroy; a context created with SPC3D_CTX_NO_HOST_CACHE does plan, upload, run,
+ * download, free on every call instead.  The reading and the Y transfers use the context's
+ * host_threads (spc3d_ctx_opts): with the default, 1, everything runs on the caller's thread.  One-shot calls on one context run one at a time
  * (they take a lock).  The kernels of the last one-shot call lie between the timer slots
  * SPC3D_TIMER_HOST_CALL_BEGIN and _END. */
 #define SPC3D_TIMER_HOST_CALL_BEGIN 4094

@@ -36,6 +36,13 @@ class PlanInfo(ctypes.Structure):
                 ("entries_by_column", c_u32), ("device_bytes", c_u64)]
 
 
+class CtxOpts(ctypes.Structure):
+    _fields_ = [("host_threads", c_u32), ("flags", c_u32), ("reserved", c_u32 * 6)]
+
+
+CTX_NO_AUX_STREAM, CTX_NO_HOST_CACHE = 1, 2
+
+
 class PlanOpts(ctypes.Structure):
     _fields_ = [("seg_max", c_u32), ("k_hint", c_u32), ("l2_hot_bytes", c_u32),
                 ("hub_min", c_u32), ("xcd_slices", c_u32), ("builder", c_u32),
@@ -53,6 +60,7 @@ SIGNATURES = {
     "spc3d_status_name": (ctypes.c_char_p, [c_int]),
     "spc3d_device_count": (c_int, [P(c_int)]),
     "spc3d_ctx_create": (c_int, [c_int, P(c_vp)]),
+    "spc3d_ctx_create_ex": (c_int, [c_int, P(CtxOpts), P(c_vp)]),
     "spc3d_ctx_destroy": (c_int, [c_vp]),
     "spc3d_ctx_sync": (c_int, [c_vp]),
     "spc3d_ctx_stream": (c_int, [c_vp, P(c_vp)]),

@@ -9,6 +9,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <atomic>
+#include <condition_variable>
 #include <cstring>
 #include <functional>
 #include <memory>
@@ -117,6 +118,8 @@ struct spc3d_ctx {
     hipEvent_t timers[kTimerSlots];
     bool timer_set[kTimerSlots];
     HostCallCache *host_cache; // made by the first spc3d_*_host call
+    bool use_host_cache;       // false: the one-shot calls keep nothing between calls
+    unsigned host_threads;     // host threads a one-shot call may use, the caller's included
     std::mutex host_mutex;     // the one-shot calls of a context run one at a time
 };
 
@@ -434,8 +437,40 @@ int spc3d_device_count(int *count)
 }
 
 /* ---- context ------------------------------------------------------------- */
+static bool env_number(const char *name, unsigned long long *out);
+
+// The defaults of spc3d_ctx_create: the library's, each overridable from the environment.
+static spc3d_ctx_opts ctx_opts_from_env()
+{
+    spc3d_ctx_opts o;
+    std::memset(&o, 0, sizeof o);
+    unsigned long long v = 0;
+    if (env_number("SPC3D_HOST_THREADS", &v) && v >= 1 && v <= 256)
+        o.host_threads = (uint32_t)v;
+    if (env_number("SPC3D_AUX_STREAM", &v) && v == 0)
+        o.flags |= SPC3D_CTX_NO_AUX_STREAM;
+    if (env_number("SPC3D_HOST_CACHE", &v) && v == 0)
+        o.flags |= SPC3D_CTX_NO_HOST_CACHE;
+    return o;
+}
+
 int spc3d_ctx_create(int device, spc3d_ctx **out)
 {
+    const spc3d_ctx_opts o = ctx_opts_from_env();
+    return spc3d_ctx_create_ex(device, &o, out);
+}
+
+int spc3d_ctx_create_ex(int device, const spc3d_ctx_opts *opts, spc3d_ctx **out)
+{
+    spc3d_ctx_opts o;
+    std::memset(&o, 0, sizeof o);
+    if (opts)
+        o = *opts;
+    if ((o.flags & ~(uint32_t)(SPC3D_CTX_NO_AUX_STREAM | SPC3D_CTX_NO_HOST_CACHE)) || o.reserved[0] ||
+        o.reserved[1] || o.reserved[2] || o.reserved[3] || o.reserved[4] || o.reserved[5])
+        return fail(SPC3D_ERR_INVALID_ARG, "spc3d_ctx_opts has unknown flags or reserved words set");
+    if (o.host_threads > 256)
+        return fail(SPC3D_ERR_INVALID_ARG, "spc3d_ctx_opts.host_threads must be at most 256");
     if (!out)
         return fail(SPC3D_ERR_INVALID_ARG, "out is NULL");
     *out = nullptr;
@@ -460,12 +495,13 @@ int spc3d_ctx_create(int device, spc3d_ctx **out)
         delete c;
         return fail_hip(e, "hipStreamCreateWithFlags");
     }
-    // Same (default) priority as the main stream.  SPC3D_AUX_STREAM=0 keeps every
+    // Same (default) priority as the main stream.  SPC3D_CTX_NO_AUX_STREAM keeps every
     // launch on the main stream.
     c->aux_stream = nullptr;
     c->fork_event = c->join_event = nullptr;
-    const char *aux = std::getenv("SPC3D_AUX_STREAM");
-    if (!aux || std::atoi(aux) != 0) {
+    c->use_host_cache = !(o.flags & SPC3D_CTX_NO_HOST_CACHE);
+    c->host_threads = o.host_threads ? o.host_threads : 1;
+    if (!(o.flags & SPC3D_CTX_NO_AUX_STREAM)) {
         e = hipStreamCreateWithFlags(&c->aux_stream, hipStreamNonBlocking);
         if (e == hipSuccess)
             e = hipEventCreateWithFlags(&c->fork_event, hipEventDisableTiming);
@@ -2359,11 +2395,7 @@ int spc3d_rows_unpack_sum(spc3d_ctx *ctx, spc3d_panel *P, const spc3d_rowmap *ma
 
 namespace {
 
-bool host_cache_enabled()
-{
-    const char *e = std::getenv("SPC3D_HOST_CACHE");
-    return !e || std::atoi(e) != 0;
-}
+bool host_cache_enabled(const spc3d_ctx *ctx) { return ctx->use_host_cache; }
 
 HostCallCache *cache_of(spc3d_ctx *ctx)
 {
@@ -2395,8 +2427,8 @@ int host_plan(spc3d_ctx *ctx, HostCallCache *hc, int dtype, uint32_t nrows, uint
         return fail(SPC3D_ERR_INVALID_ARG, "ii or jj is NULL");
     std::vector<BlockKey> kii, kjj;
     std::vector<uint32_t> sample;
-    keys_of(ii, (size_t)nnz * 4, kii);
-    keys_of(jj, (size_t)nnz * 4, kjj);
+    keys_of(ii, (size_t)nnz * 4, kii, ctx->host_threads);
+    keys_of(jj, (size_t)nnz * 4, kjj, ctx->host_threads);
     sample_indices(ii, jj, nnz, sample);
     ++hc->clock;
     for (CachedHostPlan &e : hc->plans) {
@@ -2576,7 +2608,7 @@ int host_input(spc3d_ctx *ctx, HostCallCache *hc, int dtype, uint32_t m, uint32_
     if (bytes && !host)
         return fail(SPC3D_ERR_INVALID_ARG, "a dense operand is NULL");
     std::vector<BlockKey> keys;
-    keys_of(host, bytes, keys);
+    keys_of(host, bytes, keys, ctx->host_threads);
     CachedHostPanel *slot = nullptr;
     int rc = pick_panel(ctx, hc, dtype, m, n, keys, false, host, stamp, &slot);
     if (rc)
@@ -2601,8 +2633,8 @@ void send_output_operand(spc3d_ctx *ctx, CachedHostPanel *slot, const void *host
     std::vector<BlockKey> keys;
     const bool read_first = !slot->keys.empty() && slot->skip == 0;
     try { // runs as a thread's function: nothing may leave it
-        if (read_first)
-            keys_of(host, bytes, keys, 4);
+        if (read_first) // beside the thread that reads X: half of the context's threads each
+            keys_of(host, bytes, keys, std::max(1u, ctx->host_threads / 2));
         else if (slot->skip)
             --slot->skip;
     } catch (const std::exception &) {
@@ -2627,34 +2659,49 @@ int fetch_output_operand(spc3d_ctx *ctx, CachedHostPanel *slot, void *host)
     const size_t bytes = (size_t)P->m * P->n * elem_size(P->dtype);
     const size_t nblocks = (bytes + kKeyBlockBytes - 1) / kKeyBlockBytes;
     std::vector<BlockKey> keys(nblocks);
-    std::atomic<size_t> ready{0}, next{0};
+    // `ready` blocks have arrived; the workers sleep on the condition until theirs has.
+    std::mutex mu;
+    std::condition_variable cv;
+    size_t ready = 0;
+    std::atomic<size_t> next{0};
     char *dst = static_cast<char *>(host);
+    auto publish = [&](size_t upto) {
+        {
+            std::lock_guard<std::mutex> lock(mu);
+            ready = upto;
+        }
+        cv.notify_all();
+    };
     auto work = [&]() {
         for (;;) {
             const size_t b = next.fetch_add(1, std::memory_order_relaxed);
             if (b >= nblocks)
                 return;
-            while (ready.load(std::memory_order_acquire) <= b)
-                std::this_thread::yield();
+            {
+                std::unique_lock<std::mutex> lock(mu);
+                cv.wait(lock, [&] { return ready > b; });
+            }
             const size_t off = b * kKeyBlockBytes;
             keys[b] = key_of_block(dst + off, std::min(kKeyBlockBytes, bytes - off));
         }
     };
-    const unsigned hw = std::thread::hardware_concurrency();
-    const unsigned nthreads = (unsigned)std::min<size_t>(std::min(4u, hw ? hw : 1u), nblocks);
+    // Workers beside the copying thread: what the context allows, at most 4 (a 16 MiB piece is
+    // keyed faster than the next one arrives).  None: this thread keys everything at the end.
+    const unsigned nthreads =
+        (unsigned)std::min<size_t>(std::min(4u, ctx->host_threads > 1 ? ctx->host_threads - 1 : 0u),
+                                   nblocks);
     // Joined on every way out, after the workers have been let run out.
     struct Pool {
         std::vector<std::thread> threads;
-        std::atomic<size_t> &ready;
-        size_t nblocks;
+        std::function<void()> release;
         ~Pool()
         {
-            ready.store(nblocks, std::memory_order_release);
+            release();
             for (std::thread &t : threads)
                 if (t.joinable())
                     t.join();
         }
-    } workers{{}, ready, nblocks};
+    } workers{{}, [&] { publish(nblocks); }};
     std::vector<std::thread> &pool = workers.threads;
     try {
         pool.reserve(nthreads);
@@ -2673,9 +2720,9 @@ int fetch_output_operand(spc3d_ctx *ctx, CachedHostPanel *slot, void *host)
         if (err == hipSuccess)
             err = hipStreamSynchronize(ctx->stream);
         if (err == hipSuccess)
-            ready.store(std::min(nblocks, b + kPiece), std::memory_order_release);
+            publish(std::min(nblocks, b + kPiece));
     }
-    ready.store(nblocks, std::memory_order_release); // lets the workers run out also after a failure
+    publish(nblocks); // lets the workers run out also after a failure
     work(); // whatever no worker has taken
     for (std::thread &t : pool)
         t.join();
@@ -2776,7 +2823,9 @@ static int sddmm_host_call(spc3d_ctx *ctx, int dtype, uint32_t m, uint32_t n, ui
     if (!live(ctx) || !dtype_ok(dtype)) // reported as plan creation reports it (bad pattern first)
         return sddmm_host_uncached(ctx, dtype, m, n, k, A, B, nnz, ii, jj, svv, cvv);
     std::lock_guard<std::mutex> lock(ctx->host_mutex);
-    if (!host_cache_enabled())
+    if (!live(ctx))
+        return fail(SPC3D_ERR_INVALID_ARG, "context is NULL or destroyed");
+    if (!host_cache_enabled(ctx))
         return sddmm_host_uncached(ctx, dtype, m, n, k, A, B, nnz, ii, jj, svv, cvv);
     HostCallCache *hc = nullptr;
     int rc = host_call_begin(ctx, &hc);
@@ -2846,7 +2895,9 @@ static int spmm_host_call(spc3d_ctx *ctx, int dtype, uint32_t ncols, uint32_t nr
     if (!live(ctx) || !dtype_ok(dtype))
         return spmm_host_uncached(ctx, dtype, ncols, nrows, k, X, nnz, ii, jj, avv, Y);
     std::lock_guard<std::mutex> lock(ctx->host_mutex);
-    if (!host_cache_enabled())
+    if (!live(ctx))
+        return fail(SPC3D_ERR_INVALID_ARG, "context is NULL or destroyed");
+    if (!host_cache_enabled(ctx))
         return spmm_host_uncached(ctx, dtype, ncols, nrows, k, X, nnz, ii, jj, avv, Y);
     HostCallCache *hc = nullptr;
     int rc = host_call_begin(ctx, &hc);
@@ -2885,10 +2936,14 @@ static int spmm_host_call(spc3d_ctx *ctx, int dtype, uint32_t ncols, uint32_t nr
                 t.join();
         }
     } joined{ythread};
-    try {
-        ythread = std::thread(send_output_operand, ctx, yslot, (const void *)Y, std::ref(ymv));
-    } catch (const std::system_error &) {
-        send_output_operand(ctx, yslot, Y, ymv); // no thread to be had: one after the other
+    if (ctx->host_threads < 2) {
+        send_output_operand(ctx, yslot, Y, ymv); // one thread: one after the other
+    } else {
+        try {
+            ythread = std::thread(send_output_operand, ctx, yslot, (const void *)Y, std::ref(ymv));
+        } catch (const std::system_error &) {
+            send_output_operand(ctx, yslot, Y, ymv); // no thread to be had: one after the other
+        }
     }
     rc = host_input(ctx, hc, dtype, ncols, k, X, stamp, &x);
     if (ythread.joinable())

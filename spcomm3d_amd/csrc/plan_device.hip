@@ -5,7 +5,10 @@
 #include "plan_device.h"
 
 #include <hip/hip_runtime.h>
-#include <hipcub/hipcub.hpp>
+#include <cstring>
+
+#include <rocprim/device/device_radix_sort.hpp>
+#include <rocprim/device/device_scan.hpp>
 
 #include <algorithm>
 #include <cstdio>
@@ -691,9 +694,9 @@ template <typename T>
 int exclusive_sum(Temp &tmp, const T *in, T *out, size_t n, hipStream_t st, std::string &err)
 {
     size_t bytes = 0;
-    HIP_OK(hipcub::DeviceScan::ExclusiveSum(nullptr, bytes, in, out, n, st));
+    HIP_OK(rocprim::exclusive_scan(nullptr, bytes, in, out, T(0), n, rocprim::plus<T>(), st));
     HIP_OK(tmp.need(bytes));
-    HIP_OK(hipcub::DeviceScan::ExclusiveSum(tmp.p, bytes, in, out, n, st));
+    HIP_OK(rocprim::exclusive_scan(tmp.p, bytes, in, out, T(0), n, rocprim::plus<T>(), st));
     return SPC3D_OK;
 }
 
@@ -704,17 +707,17 @@ int sort_pairs(Temp &tmp, const KeyT *kin, KeyT *kout, const uint32_t *vin, uint
 {
     size_t bytes = 0;
     if (descending) {
-        HIP_OK(hipcub::DeviceRadixSort::SortPairsDescending(nullptr, bytes, kin, kout, vin, vout,
-                                                            n, 0, bits, st));
+        HIP_OK(rocprim::radix_sort_pairs_desc(nullptr, bytes, kin, kout, vin, vout, (size_t)n, 0u,
+                                              (unsigned)bits, st));
         HIP_OK(tmp.need(bytes));
-        HIP_OK(hipcub::DeviceRadixSort::SortPairsDescending(tmp.p, bytes, kin, kout, vin,
-                                                            vout, n, 0, bits, st));
+        HIP_OK(rocprim::radix_sort_pairs_desc(tmp.p, bytes, kin, kout, vin, vout, (size_t)n, 0u,
+                                              (unsigned)bits, st));
     } else {
-        HIP_OK(hipcub::DeviceRadixSort::SortPairs(nullptr, bytes, kin, kout, vin, vout, n, 0,
-                                                  bits, st));
+        HIP_OK(rocprim::radix_sort_pairs(nullptr, bytes, kin, kout, vin, vout, (size_t)n, 0u,
+                                         (unsigned)bits, st));
         HIP_OK(tmp.need(bytes));
-        HIP_OK(hipcub::DeviceRadixSort::SortPairs(tmp.p, bytes, kin, kout, vin, vout, n, 0,
-                                                  bits, st));
+        HIP_OK(rocprim::radix_sort_pairs(tmp.p, bytes, kin, kout, vin, vout, (size_t)n, 0u,
+                                         (unsigned)bits, st));
     }
     return SPC3D_OK;
 }
@@ -724,9 +727,9 @@ int sort_keys(Temp &tmp, const uint32_t *kin, uint32_t *kout, uint32_t n, int bi
               hipStream_t st, std::string &err)
 {
     size_t bytes = 0;
-    HIP_OK(hipcub::DeviceRadixSort::SortKeys(nullptr, bytes, kin, kout, n, 0, bits, st));
+    HIP_OK(rocprim::radix_sort_keys(nullptr, bytes, kin, kout, (size_t)n, 0u, (unsigned)bits, st));
     HIP_OK(tmp.need(bytes));
-    HIP_OK(hipcub::DeviceRadixSort::SortKeys(tmp.p, bytes, kin, kout, n, 0, bits, st));
+    HIP_OK(rocprim::radix_sort_keys(tmp.p, bytes, kin, kout, (size_t)n, 0u, (unsigned)bits, st));
     return SPC3D_OK;
 }
 

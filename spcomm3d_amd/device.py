@@ -68,10 +68,21 @@ def _as_idx(a, name: str) -> np.ndarray:
 class Context:
     """One device and one stream (``spc3d_ctx``)."""
 
-    def __init__(self, device: int = 0):
+    def __init__(self, device: int = 0, host_threads: int | None = None,
+                 aux_stream: bool | None = None, host_cache: bool | None = None):
+        """No option given: ``spc3d_ctx_create`` (defaults, environment overrides); else
+        ``spc3d_ctx_create_ex`` with ``spc3d_ctx_opts`` (``None`` fields keep the default)."""
         self._lib = capi.load()
         h = ctypes.c_void_p()
-        check(self._lib.spc3d_ctx_create(device, ctypes.byref(h)), "spc3d_ctx_create")
+        if host_threads is None and aux_stream is None and host_cache is None:
+            check(self._lib.spc3d_ctx_create(device, ctypes.byref(h)), "spc3d_ctx_create")
+        else:
+            o = capi.CtxOpts()
+            o.host_threads = int(host_threads or 0)
+            o.flags = ((capi.CTX_NO_AUX_STREAM if aux_stream is False else 0) |
+                       (capi.CTX_NO_HOST_CACHE if host_cache is False else 0))
+            check(self._lib.spc3d_ctx_create_ex(device, ctypes.byref(o), ctypes.byref(h)),
+                  "spc3d_ctx_create_ex")
         self._h = h
         self.device = device
 

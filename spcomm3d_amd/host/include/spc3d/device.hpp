@@ -36,6 +36,11 @@ template <typename T> constexpr int dtype_of()
 class Context {
   public:
     explicit Context(int device = 0) { check(spc3d_ctx_create(device, &h_), "spc3d_ctx_create"); }
+    // With explicit options (host threads of the one-shot calls, auxiliary stream, host cache).
+    Context(int device, const spc3d_ctx_opts &opts)
+    {
+        check(spc3d_ctx_create_ex(device, &opts, &h_), "spc3d_ctx_create_ex");
+    }
     ~Context()
     {
         if (h_)

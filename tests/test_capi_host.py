@@ -268,6 +268,21 @@ def test_plan_build_host_rejects_bad_arguments():
     assert rc == capi.ERR_INVALID_ARG
 
 
+def test_context_options_are_validated_before_any_device_is_touched():
+    lib = capi.load()
+    h = ctypes.c_void_p()
+    o = capi.CtxOpts()
+    o.flags = 4  # unknown bit
+    assert lib.spc3d_ctx_create_ex(0, ctypes.byref(o), ctypes.byref(h)) == capi.ERR_INVALID_ARG
+    o = capi.CtxOpts()
+    o.reserved[2] = 1
+    assert lib.spc3d_ctx_create_ex(0, ctypes.byref(o), ctypes.byref(h)) == capi.ERR_INVALID_ARG
+    o = capi.CtxOpts()
+    o.host_threads = 1000
+    assert lib.spc3d_ctx_create_ex(0, ctypes.byref(o), ctypes.byref(h)) == capi.ERR_INVALID_ARG
+    assert not h.value
+
+
 def test_kernel_variant_for_every_kind_of_row_width():
     lib = capi.load()
     def v(dtype, k):

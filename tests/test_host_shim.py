@@ -109,11 +109,19 @@ def test_files_through_this_builds_readers_onto_the_gpu(name, k):
 
 
 @pytest.mark.gpu
-def test_one_shot_host_calls_reuse_only_what_still_holds():
+@pytest.mark.parametrize("threads", [None, "8"])
+def test_one_shot_host_calls_reuse_only_what_still_holds(threads):
     # spc3d_sddmm_host / spc3d_spmm_host called five times over one pattern as the reference's
     # drivers call the kernels (miniapp/bench_both.cpp:202-203), then with every operand
     # changed in the smallest way: plan and panels are reused by content, results against the oracle
-    r = subprocess.run([_binary("test_host_calls")], capture_output=True, text=True, timeout=600)
+    # once on the caller's thread alone (the default: one thread per rank, as the reference's
+    # ranks run), once with eight host threads reading the operands and moving Y
+    env = dict(os.environ)
+    env.pop("SPC3D_HOST_THREADS", None)
+    if threads:
+        env["SPC3D_HOST_THREADS"] = threads
+    r = subprocess.run([_binary("test_host_calls")], capture_output=True, text=True, timeout=600,
+                       env=env)
     assert r.returncode == 0 and "PASSED" in r.stdout, r.stdout[-3000:] + r.stderr[-3000:]
     print("\n".join(ln for ln in r.stdout.splitlines() if ln.startswith("TIMING")))
 

@@ -39,6 +39,20 @@ def test_two_calls_in_a_row_the_second_smaller(ctx):
     both_ways(ctx, W.rmat(16, 16, 64), np.float64)
 
 
+def test_column_blocks_and_wide_rows_share_the_array(ctx):
+    # a plan kept in column blocks: the blocks use the array one after the other, each
+    # block's fix-up ordered before the next block's launches
+    both_ways(ctx, W.rmat(14, 16, 64).shuffled(), np.float64, seg_max=32, col_blocks=4)
+    both_ways(ctx, W.rmat(13, 16, 32), np.float32, seg_max=32, col_blocks=3, k_hint=32)
+    # dense rows over 4 KiB run as column slices, every slice through the same partial rows
+    w = W.rmat(11, 16, 1024)
+    S = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, w.values(np.float64), k_hint=w.k)
+    need = S.info.npartial_slots * w.k * 8
+    S.close()
+    assert 0 < need <= 32 << 20  # few cut rows: fits the array at 8 KiB per partial row
+    both_ways(ctx, w, np.float64, k_hint=w.k)
+
+
 def test_a_plan_beyond_the_array_is_refused_and_nothing_runs(ctx):
     w = W.rmat(14, 16, 1024).shuffled()
     vv = w.values(np.float64)
