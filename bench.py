@@ -190,6 +190,7 @@ def run_gpu(w, dtype, steps, warmup, seg_max=None, max_timed=1300, copies=0):
     with_perm = not info.order_is_identity
     fl = roofline.flops(w.nnz, w.k)
     out = {"dtype": dtype, "ms_per_step": wall / steps * 1e3, "plan_build_s": plan_s,
+           "plan_device_bytes": int(info.device_bytes),
            "upload_s": upload_s, "nsegments": info.nsegments, "nsplit_rows": info.nsplit_rows,
            "seg_max": info.seg_max, "rows_touched": m_t, "cols_touched": n_t,
            "gflops": 2 * fl / (wall / steps) / 1e9, "kernels": {}}
@@ -286,7 +287,8 @@ def run_dist_step(w, dtype, reps):
 
 def run_compact(w, dtype, steps, warmup):
     """One compact row for a workload: mean time per kernel over `steps` passes on
-    resident operands, strict-model fraction of the HBM peak."""
+    resident operands, strict-model fraction of the HBM peak, the rows and columns that
+    hold entries, and the device memory the plan takes."""
     from spcomm3d_amd import device, roofline
     from spcomm3d_amd import workloads as W
 
@@ -328,6 +330,9 @@ def run_compact(w, dtype, steps, warmup):
             "sddmm_ms": sd_ms, "spmm_ms": sp_ms,
             "sddmm_frac": sd_b / sd_ms / 1e6 / roofline.HBM_PEAK_GBS,
             "spmm_frac": sp_b / sp_ms / 1e6 / roofline.HBM_PEAK_GBS,
+            "sddmm_strict_bytes": int(sd_b), "spmm_strict_bytes": int(sp_b),
+            "rows_touched": m_t, "cols_touched": n_t,
+            "plan_device_bytes": int(info.device_bytes), "col_blocks": int(info.ncol_blocks),
             "gflops": 2 * fl / (sd_ms + sp_ms) / 1e6, "plan_build_s": plan_s}
 
 
@@ -479,6 +484,16 @@ def main():
         if ws is not None:
             also["shuffled"] = {dt: run_compact(ws, dt, max(5, args.steps // 2), args.warmup)
                                 for dt in ("f64", "f32")}
+            # unsorted COO is what the reference's kernels are handed (src/core_ops.cpp:7-10):
+            # the same roofline object as the headline's, for that order
+            r = also["shuffled"][args.dtype]
+            sdom = "sddmm" if r["sddmm_ms"] >= r["spmm_ms"] else "spmm"
+            also["shuffled"]["roofline"] = {
+                "bound": "hbm", "kernel": sdom, "dtype": args.dtype,
+                "achieved": r[sdom + "_strict_bytes"] / r[sdom + "_ms"] / 1e6,
+                "peak": 8000.0, "unit": "GB/s", "frac": r[sdom + "_frac"],
+                "bytes_per_launch": r[sdom + "_strict_bytes"], "ms_per_launch": r[sdom + "_ms"],
+                "model": "strict (each operand once)"}
             log(json.dumps(also["shuffled"]))
             del ws
             wc = w.column_major()
@@ -498,6 +513,18 @@ def main():
                 rows.append(row)
                 log(json.dumps(row))
                 t0 = time.perf_counter()
+            if name == "rmat24_block":
+                # the same block at the shape a rank of the reference runs it on: local
+                # indices in first-appearance order, panels of the touched rows / columns only
+                # (src/SparseMatrix.hpp:69-99, miniapp/bench_both.cpp:158,189-190)
+                wl = wo.localized()
+                for dt in dtypes:
+                    row = run_compact(wl, dt, steps, 2)
+                    row["wall_s"] = time.perf_counter() - t0
+                    rows.append(row)
+                    log(json.dumps(row))
+                    t0 = time.perf_counter()
+                del wl
             del wo
         also["configs"] = rows
     cpu = None
@@ -545,7 +572,7 @@ def main():
         "dist_step": dist_step,
         "row_copies": main_r["row_copies"],
         "plan": {k: main_r[k] for k in ("plan_build_s", "upload_s", "nsegments", "nsplit_rows",
-                                        "seg_max")},
+                                        "seg_max", "plan_device_bytes")},
         "also": also,
     }
     print(json.dumps(line), flush=True)

@@ -115,6 +115,11 @@ typedef struct {
                                   in that order); 0: the caller's order inside every row */
     uint64_t device_bytes;     /* device memory the plan holds: its arrays, values, partial-sum
                                   rows, result staging, a companion plan, every column block */
+    uint64_t sweep_entries;    /* entries kept as row tiles x column blocks (spc3d_plan_opts.sweep);
+                                  0: none.  The segment counts above are then those of the plan
+                                  of the other entries */
+    uint32_t sweep_tiles;      /* tiles of rows of that layout */
+    uint32_t sweep_k;          /* the K it is laid out for (k_hint): calls at another K are refused */
 } spc3d_plan_info;
 
 /* Plan tuning; a zero field selects the default.  Only speed depends on these. */
@@ -146,7 +151,20 @@ typedef struct {
     uint32_t two_pass_min; /* entries from which the results of an arbitrary entry order go home
                               in two tile-local passes (default 1,572,864: measured slower
                               under 1 M entries, faster from 1.9 M on) */
-    uint32_t reserved[3];  /* must be 0 */
+    uint32_t sweep;        /* row tiles x column blocks.  Where column blocks would be chosen
+                              (col_blocks above) and k_hint is given with dense rows of 256,
+                              512 or 1024 bytes, the rows of at least sweep_min_row entries are
+                              not cut at block boundaries: tiles of rows (128 KiB of A rows, or
+                              of Y accumulators) stay in LDS while their workgroups walk the
+                              column blocks in step, one workgroup per CU; the other rows form
+                              an ordinary plan.  Such a plan runs at K = k_hint only (other
+                              calls return SPC3D_ERR_INVALID_ARG), spc3d_spmm adds a row's
+                              entries block after block, and runs give the same bits.
+                              0 (default): as described; 1: never; 2: whenever k_hint has such
+                              a width, whatever the pattern (col_blocks, if given, is the
+                              number of blocks) */
+    uint32_t sweep_min_row; /* shortest row kept in the tiles (default 64) */
+    uint32_t reserved[1];  /* must be 0 */
 } spc3d_plan_opts;
 /* spc3d_plan_opts.flags.  The first three keep spc3d_sddmm's plain stores where the plan
  * would otherwise stage the results of regrouped segments, run a column-sorted pattern

@@ -33,7 +33,8 @@ class PlanInfo(ctypes.Structure):
                 ("nsegments_long", c_u32), ("ncol_blocks", c_u32),
                 ("staged_entries", c_u64), ("positions_by_segment", c_u32),
                 ("sddmm_by_column", c_u32), ("two_pass_results", c_u32),
-                ("entries_by_column", c_u32), ("device_bytes", c_u64)]
+                ("entries_by_column", c_u32), ("device_bytes", c_u64),
+                ("sweep_entries", c_u64), ("sweep_tiles", c_u32), ("sweep_k", c_u32)]
 
 
 class CtxOpts(ctypes.Structure):
@@ -47,7 +48,7 @@ class PlanOpts(ctypes.Structure):
     _fields_ = [("seg_max", c_u32), ("k_hint", c_u32), ("l2_hot_bytes", c_u32),
                 ("hub_min", c_u32), ("xcd_slices", c_u32), ("builder", c_u32),
                 ("col_blocks", c_u32), ("flags", c_u32), ("two_pass_min", c_u32),
-                ("reserved", c_u32 * 3)]
+                ("sweep", c_u32), ("sweep_min_row", c_u32), ("reserved", c_u32 * 1)]
 
 PLAN_NO_STAGED_STORES, PLAN_NO_SDDMM_BY_COLUMN, PLAN_NO_TWO_PASS, PLAN_KEEP_ENTRY_ORDER = 1, 2, 4, 8
 

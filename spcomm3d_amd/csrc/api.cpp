@@ -146,6 +146,12 @@ int spc3d_ctx_create_ex(int device, const spc3d_ctx_opts *opts, spc3d_ctx **out)
     c->fork_event = c->join_event = nullptr;
     c->use_host_cache = !(o.flags & SPC3D_CTX_NO_HOST_CACHE);
     c->host_threads = o.host_threads ? o.host_threads : 1;
+    c->cu_count = 0;
+    if (hipDeviceGetAttribute(&c->cu_count, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess ||
+        c->cu_count < 1) {
+        (void)hipGetLastError();
+        c->cu_count = 256;
+    }
     if (!(o.flags & SPC3D_CTX_NO_AUX_STREAM)) {
         e = hipStreamCreateWithFlags(&c->aux_stream, hipStreamNonBlocking);
         if (e == hipSuccess)
@@ -711,7 +717,8 @@ static hipError_t finish_sddmm(const spc3d_plan *S, void *C)
 static DevPlanView staged_view(const spc3d_plan *parent, const spc3d_plan *block)
 {
     DevPlanView v = view_of(block);
-    v.perm = parent->stage_of + block->stage_off;
+    // beside a sweep: the plan of the rest, its results in its own kernel order
+    v.perm = parent->sweep.n ? nullptr : parent->stage_of + block->stage_off;
     v.stream_c = true;
     return v;
 }
@@ -727,7 +734,20 @@ static hipError_t unstage(const spc3d_plan *S, spc3d_vals *C)
 }
 static void *staged_out(const spc3d_plan *parent, const spc3d_plan *)
 {
-    return parent->c_stage;
+    return static_cast<char *>(parent->c_stage) + parent->rest_off * elem_size(parent->dtype);
+}
+
+// A plan kept as row tiles x column blocks runs at the K it was laid out for.
+static int sweep_check(const spc3d_plan *S, uint32_t K)
+{
+    if (!S->sweep.n || K == S->sweep_k)
+        return SPC3D_OK;
+    char msg[224];
+    std::snprintf(msg, sizeof msg,
+                  "the plan is laid out as row tiles for K = %u (spc3d_plan_info.sweep_k) and the "
+                  "panels have K = %u: create it with k_hint = K, or with spc3d_plan_opts.sweep = 1",
+                  S->sweep_k, K);
+    return fail(SPC3D_ERR_INVALID_ARG, msg);
 }
 
 
@@ -768,15 +788,21 @@ int spc3d_sddmm(spc3d_ctx *ctx, spc3d_plan *S, const spc3d_panel *A, const spc3d
         HIP_TRY(unstage_stores(T, C->dev));
         return SPC3D_OK;
     }
-    if (S->blocks.empty()) {
+    if (S->blocks.empty() && !S->sweep.n) {
         HIP_TRY(launch_sddmm(S->dtype, view_of(S), A->dev, B->dev, sddmm_out(S, C->dev), K,
                              streams_of(ctx)));
         HIP_TRY(finish_sddmm(S, C->dev));
         return SPC3D_OK;
     }
+    rc = sweep_check(S, K);
+    if (rc)
+        return rc;
     for (spc3d_plan *part : S->blocks)
         HIP_TRY(launch_sddmm(S->dtype, staged_view(S, part), A->dev, B->dev, staged_out(S, part), K,
                              streams_of(ctx)));
+    if (S->sweep.n)
+        HIP_TRY(launch_sweep_sddmm(S->dtype, sweep_view_of(S), A->dev, B->dev, S->c_stage,
+                                   ctx->stream));
     HIP_TRY(unstage(S, C));
     return SPC3D_OK;
 }
@@ -813,6 +839,9 @@ int spc3d_spmm(spc3d_ctx *ctx, spc3d_plan *Ap, const spc3d_panel *X, spc3d_panel
     int rc = spmm_check(ctx, Ap, X, Y, &K);
     if (rc || K == 0)
         return rc;
+    rc = sweep_check(Ap, K);
+    if (rc)
+        return rc;
     rc = use_device(ctx, true);
     if (rc)
         return rc;
@@ -825,6 +854,8 @@ int spc3d_spmm(spc3d_ctx *ctx, spc3d_plan *Ap, const spc3d_panel *X, spc3d_panel
     // The blocks add into Y one after the other on the stream: a fixed order.
     for (spc3d_plan *part : parts_of(Ap, self))
         HIP_TRY(launch_spmm(Ap->dtype, view_of(part), X->dev, Y->dev, K, streams_of(ctx)));
+    if (Ap->sweep.n) // rows of their own: none of them is in the plan of the rest
+        HIP_TRY(launch_sweep_spmm(Ap->dtype, sweep_view_of(Ap), X->dev, Y->dev, ctx->stream));
     return SPC3D_OK;
 }
 
@@ -843,6 +874,9 @@ int spc3d_spmm_noalloc(spc3d_ctx *ctx, spc3d_plan *Ap, const spc3d_panel *X, spc
                       (unsigned long long)need, K, (unsigned long long)kStaticScratchBytes);
         return fail(SPC3D_ERR_TOO_LARGE, msg);
     }
+    rc = sweep_check(Ap, K);
+    if (rc)
+        return rc;
     rc = use_device(ctx, true);
     if (rc)
         return rc;
@@ -850,12 +884,15 @@ int spc3d_spmm_noalloc(spc3d_ctx *ctx, spc3d_plan *Ap, const spc3d_panel *X, spc
     // call first, so what an earlier call left in the array needs no clearing.  (The
     // blocks of a plan kept in column blocks use the array one after the other;
     // npartial_slots is the largest block's.)
-    const size_t nparts = Ap->blocks.empty() ? 1 : Ap->blocks.size(); // no container: no host heap either
+    // no container: no host heap either
+    const size_t nparts = Ap->blocks.empty() ? (Ap->sweep.n ? 0 : 1) : Ap->blocks.size();
     for (size_t i = 0; i < nparts; ++i) {
         DevPlanView view = view_of(Ap->blocks.empty() ? Ap : Ap->blocks[i]);
         view.partial = ctx->scratch;
         HIP_TRY(launch_spmm(Ap->dtype, view, X->dev, Y->dev, K, streams_of(ctx)));
     }
+    if (Ap->sweep.n) // the tiles' sums live in LDS: nothing to allocate either
+        HIP_TRY(launch_sweep_spmm(Ap->dtype, sweep_view_of(Ap), X->dev, Y->dev, ctx->stream));
     return SPC3D_OK;
 }
 
@@ -890,13 +927,16 @@ int spc3d_sddmm_spmm(spc3d_ctx *ctx, spc3d_plan *S, const spc3d_panel *A, const 
         HIP_TRY(launch_fill(C->dtype, C->dev, S->info.nnz, 0.0, ctx->stream));
         return SPC3D_OK;
     }
+    rc = sweep_check(S, K);
+    if (rc)
+        return rc;
     std::vector<spc3d_plan *> self;
     for (spc3d_plan *part : parts_of(S, self)) {
         rc = ensure_partial(part, K);
         if (rc)
             return rc;
     }
-    const bool staged = !S->blocks.empty();
+    const bool staged = !S->blocks.empty() || S->sweep.n;
     for (spc3d_plan *part : parts_of(S, self)) {
         const DevPlanView view = staged ? staged_view(S, part) : view_of(part);
         void *out = staged ? staged_out(S, part) : sddmm_out(S, C->dev);
@@ -914,6 +954,14 @@ int spc3d_sddmm_spmm(spc3d_ctx *ctx, spc3d_plan *S, const spc3d_panel *A, const 
             continue;
         }
         HIP_TRY(e);
+    }
+    if (S->sweep.n) { // the tiles: SDDMM, then SpMM over the same entries (with the results
+                      // just written as its values when chained)
+        SweepView v = sweep_view_of(S);
+        HIP_TRY(launch_sweep_sddmm(S->dtype, v, A->dev, B->dev, S->c_stage, ctx->stream));
+        if (chained)
+            v.sval = S->c_stage;
+        HIP_TRY(launch_sweep_spmm(S->dtype, v, B->dev, Y->dev, ctx->stream));
     }
     if (staged)
         HIP_TRY(unstage(S, C));

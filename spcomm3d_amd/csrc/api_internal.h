@@ -79,6 +79,7 @@ struct spc3d_ctx {
     hipStream_t aux_stream; // short-segment launches run here, beside the long-segment ones
     hipEvent_t fork_event, join_event;
     uint32_t aux_rot; // (XCD of workgroup 0 on aux - XCD of workgroup 0 on main) mod 8
+    int cu_count;     // compute units of the device
     void *scratch;    // this device's copy of the static scratch array (spc3d_spmm_noalloc)
     bool capturing;   // between spc3d_capture_begin and spc3d_capture_end
     hipEvent_t timers[kTimerSlots];
@@ -180,7 +181,32 @@ struct spc3d_plan {
     uint32_t *stage_of = nullptr;  // [nnz]
     uint64_t stage_off = 0;
     uint32_t col_base = 0; // a block of a plan kept in column blocks: its first column
+    // Row tiles x column blocks (SweepPlan in plan_device.h, the sweep kernels in kernels.h):
+    // the long rows of a pattern over unskewed columns, laid out for dense rows of sweep_k
+    // reals.  `blocks` then holds at most one ordinary plan, over the entries of the other
+    // rows ("rest").  SDDMM results: the sweep's in kernel order at c_stage[0 .. sweep.n),
+    // the rest's in its kernel order from c_stage[rest_off]; stage_pos brings both home.
+    SweepPlan sweep;
+    void *sweep_sval = nullptr; // [sweep.n] values in sweep order
+    uint32_t sweep_k = 0;
+    uint64_t rest_off = 0;
 };
+
+inline SweepView sweep_view_of(const spc3d_plan *p)
+{
+    SweepView v;
+    v.ptr = p->sweep.ptr;
+    v.tile_rows = p->sweep.tile_rows;
+    v.col = p->sweep.col;
+    v.lrow = p->sweep.lrow;
+    v.sval = p->sweep_sval;
+    v.ntiles = p->sweep.ntiles;
+    v.nblocks = p->sweep.nblocks;
+    v.rows_per_tile = p->sweep.rows_per_tile;
+    v.lanes = p->sweep.lanes;
+    v.per_launch = p->sweep.per_launch;
+    return v;
+}
 
 // A cached plan answers for a pattern when the keys of every block of ii and jj, the
 // sizes, the type and the row width agree, and a sample of the indices read back equal.
@@ -393,12 +419,15 @@ inline size_t panel_bytes(const spc3d_panel *p)
     return (size_t)p->m * p->n * elem_size(p->dtype);
 }
 
-// The parts a call works on: the plan itself, or its column blocks.
+// The ordinary parts a call works on: the plan itself, or its column blocks (beside a
+// sweep: the plan of the rest, if there is one).
 inline std::vector<spc3d_plan *> &parts_of(spc3d_plan *plan, std::vector<spc3d_plan *> &self)
 {
     if (!plan->blocks.empty())
         return plan->blocks;
-    self.assign(1, plan);
+    self.clear();
+    if (!plan->sweep.n) // a plan that is all sweep has no ordinary part
+        self.push_back(plan);
     return self;
 }
 

@@ -39,6 +39,9 @@ static void fill_info(spc3d_plan_info &info, const HostPlan &H)
     info.two_pass_results = 0;
     info.entries_by_column = H.by_column_in_rows ? 1 : 0;
     info.device_bytes = 0;
+    info.sweep_entries = 0;
+    info.sweep_tiles = 0;
+    info.sweep_k = 0;
 }
 
 // Library defaults, overridable field by field.  With XCD slicing, 2 MiB of
@@ -49,8 +52,13 @@ static int resolve_opts(int dtype, const spc3d_plan_opts *o, PlanOpts &out)
     std::memset(&z, 0, sizeof z);
     if (o)
         z = *o;
-    if (z.reserved[0] || z.reserved[1] || z.reserved[2])
+    if (z.reserved[0])
         return fail(SPC3D_ERR_INVALID_ARG, "spc3d_plan_opts.reserved must be 0");
+    if (z.sweep > 2)
+        return fail(SPC3D_ERR_INVALID_ARG, "spc3d_plan_opts.sweep must be 0, 1 or 2");
+    if (z.sweep == 2 && z.builder == 1)
+        return fail(SPC3D_ERR_INVALID_ARG,
+                    "row tiles are built on the GPU: builder must be 0 or 2 with sweep = 2");
     if (z.flags & ~(uint32_t)SPC3D_PLAN_ALL_FLAGS)
         return fail(SPC3D_ERR_INVALID_ARG, "spc3d_plan_opts.flags has unknown bits set");
     if (z.col_blocks > kMaxColBlocks)
@@ -281,6 +289,14 @@ static void destroy_blocks(spc3d_plan *p)
     if (p->stage_of) (void)hipFree(p->stage_of);
     p->c_stage = nullptr;
     p->stage_pos = p->stage_of = nullptr;
+    if (p->sweep.perm) (void)hipFree(p->sweep.perm);
+    if (p->sweep.col) (void)hipFree(p->sweep.col);
+    if (p->sweep.lrow) (void)hipFree(p->sweep.lrow);
+    if (p->sweep.ptr) (void)hipFree(p->sweep.ptr);
+    if (p->sweep.tile_rows) (void)hipFree(p->sweep.tile_rows);
+    if (p->sweep_sval) (void)hipFree(p->sweep_sval);
+    p->sweep = SweepPlan();
+    p->sweep_sval = nullptr;
 }
 
 // How many column blocks a finished single plan should be rebuilt in (1: keep it).
@@ -363,6 +379,162 @@ static int add_sddmm_companion(spc3d_plan *p, uint32_t nrows, uint32_t ncols, ui
     return SPC3D_OK;
 }
 
+// Whether the pattern of a finished single plan goes into row tiles x column blocks
+// (spc3d_plan_opts.sweep), for how many lanes per dense row and in how many blocks;
+// *lanes = 0: no.  `nb_blocks` is what choose_col_blocks said.
+static void choose_sweep(const spc3d_plan *p, const spc3d_plan_opts *opts, uint32_t nb_blocks,
+                         uint32_t *lanes, uint32_t *nblocks)
+{
+    *lanes = *nblocks = 0;
+    if (!opts || opts->sweep == 1 || !opts->k_hint || opts->builder == 1)
+        return;
+    const uint32_t l = sweep_lanes(p->dtype, opts->k_hint);
+    if (!l || p->info.nnz == 0)
+        return;
+    const bool forced = opts->sweep == 2;
+    if (!forced && (nb_blocks <= 1 || opts->col_blocks > 1))
+        return; // a caller's own block count means blocks
+    uint64_t nb = forced && opts->col_blocks > 1 ? opts->col_blocks : 0;
+    if (!nb) {
+        // 2.5 MiB of dense rows per block: of 96, 128 and 192 blocks over a 244 MiB panel, 96
+        // were the fastest (5.2 / 5.1 ms against 5.4 / 5.8 ms at 192 on a 143 M-entry pattern)
+        const uint64_t panel = (uint64_t)p->info.cols_touched * opts->k_hint * elem_size(p->dtype);
+        nb = std::max<uint64_t>(1, (panel + ((uint64_t)5 << 19) - 1) / ((uint64_t)5 << 19));
+    }
+    nb = std::min<uint64_t>(nb, std::min<uint32_t>(sweep_max_blocks(l), p->info.ncols));
+    *lanes = l;
+    *nblocks = (uint32_t)std::max<uint64_t>(1, nb);
+}
+
+// Rebuilds a finished single plan `p` as row tiles x column blocks plus an ordinary plan of
+// the rows too short for the tiles.  *taken = false (and p untouched) when no row qualifies
+// or the device memory does not reach; any other failure is returned.
+static int rebuild_as_sweep(spc3d_plan *p, uint32_t nrows, uint32_t ncols, uint64_t nnz,
+                            const uint32_t *d_ii, const uint32_t *d_jj, const PlanOpts &po,
+                            const spc3d_plan_opts *opts, uint32_t lanes, uint32_t nb, bool *taken)
+{
+    *taken = false;
+    spc3d_ctx *ctx = p->ctx;
+    const size_t w = elem_size(p->dtype);
+    const uint32_t min_row = opts->sweep_min_row ? opts->sweep_min_row : 64;
+    const uint32_t per_launch = (uint32_t)std::max(1, ctx->cu_count);
+    std::string err;
+    SweepPlan sw;
+    int rc = build_sweep(ctx->stream, nrows, ncols, nnz, d_ii, d_jj, lanes,
+                         sweep_rows_per_tile(lanes), nb, min_row, per_launch, sw, err);
+    if (rc)
+        return optional_path(fail(rc, err));
+    if (sw.n == 0)
+        return SPC3D_OK;
+    const uint64_t nrest = nnz - sw.n;
+    const uint64_t rest_off = (sw.n + 63) / 64 * 64; // the rest's results start on a line of their own
+    spc3d_plan *child = nullptr;
+    uint32_t *r_ii = nullptr, *r_jj = nullptr, *gperm = nullptr, *stage_pos = nullptr;
+    void *c_stage = nullptr, *sval = nullptr;
+    if (nrest) {
+        rc = dev_alloc(&r_ii, (size_t)nrest);
+        if (!rc) rc = dev_alloc(&r_jj, (size_t)nrest);
+        if (!rc) rc = dev_alloc(&gperm, (size_t)nrest);
+        if (!rc) {
+            rc = gather_u32_device(ctx->stream, d_ii, sw.perm + sw.n, nrest, r_ii, err);
+            if (!rc) rc = gather_u32_device(ctx->stream, d_jj, sw.perm + sw.n, nrest, r_jj, err);
+            HostPlan meta;
+            DevPlanArrays arr;
+            if (!rc) rc = build_device_plan(ctx->stream, nrows, ncols, nrest, r_ii, r_jj, po, meta, arr, err);
+            if (rc)
+                fail(rc, err);
+            else
+                rc = adopt_device_plan(ctx, p->dtype, meta, arr, planned_k(opts), &child);
+        }
+        if (!rc) {
+            // the rest's kernel order -> the caller's positions
+            rc = compose_perm_device(ctx->stream, sw.perm + sw.n, child->perm, nrest, gperm, err);
+            if (rc)
+                fail(rc, err);
+        }
+        if (!rc) {
+            hipError_t e = hipStreamSynchronize(ctx->stream); // child->perm is read until here
+            if (e != hipSuccess)
+                rc = fail_hip(e, "hipStreamSynchronize");
+        }
+        if (!rc) {
+            if (child->perm) (void)hipFree(child->perm);
+            child->perm = gperm;
+            gperm = nullptr;
+            child->info.order_is_identity = 0;
+        }
+    }
+    if (!rc) rc = dev_alloc_bytes(&c_stage, (size_t)(rest_off + nrest) * w);
+    if (!rc) rc = dev_alloc(&stage_pos, (size_t)nnz);
+    if (!rc) rc = dev_alloc_bytes(&sval, (size_t)sw.n * w);
+    if (!rc) {
+        rc = inverse_offsets_device(ctx->stream, sw.perm, sw.n, 0, stage_pos, err);
+        if (!rc && nrest)
+            rc = inverse_offsets_device(ctx->stream, child->perm, nrest, (uint32_t)rest_off, stage_pos, err);
+        if (rc)
+            fail(rc, err);
+    }
+    if (!rc) {
+        hipError_t e = hipStreamSynchronize(ctx->stream);
+        if (e != hipSuccess)
+            rc = fail_hip(e, "hipStreamSynchronize");
+    }
+    if (r_ii) (void)hipFree(r_ii);
+    if (r_jj) (void)hipFree(r_jj);
+    if (gperm) (void)hipFree(gperm);
+    if (rc) {
+        const std::string keep = g_err;
+        if (child) {
+            plan_free_device(child);
+            child->magic = 0;
+            delete child;
+        }
+        if (c_stage) (void)hipFree(c_stage);
+        if (stage_pos) (void)hipFree(stage_pos);
+        if (sval) (void)hipFree(sval);
+        (void)hipFree(sw.perm), (void)hipFree(sw.col), (void)hipFree(sw.lrow), (void)hipFree(sw.ptr),
+            (void)hipFree(sw.tile_rows);
+        return optional_path(fail(rc, keep));
+    }
+    // the whole pattern's arrays give way
+    plan_free_device(p);
+    p->partial_k = 0;
+    spc3d_plan_info &I = p->info;
+    I.nsegments = I.nsegments_padded = I.nsplit_rows = I.npartial_slots = I.nsegments_long = 0;
+    I.order_is_identity = 0;
+    if (child) {
+        try {
+            p->blocks.push_back(child);
+        } catch (const std::bad_alloc &) {
+            plan_free_device(child);
+            child->magic = 0;
+            delete child;
+            (void)hipFree(c_stage), (void)hipFree(stage_pos), (void)hipFree(sval);
+            (void)hipFree(sw.perm), (void)hipFree(sw.col), (void)hipFree(sw.lrow),
+                (void)hipFree(sw.ptr), (void)hipFree(sw.tile_rows);
+            return fail(SPC3D_ERR_ALLOC, "host allocation failed");
+        }
+        I.nsegments = child->info.nsegments;
+        I.nsegments_padded = child->info.nsegments_padded;
+        I.nsegments_long = child->info.nsegments_long;
+        I.nsplit_rows = child->info.nsplit_rows;
+        I.npartial_slots = child->info.npartial_slots;
+        I.nqueues = child->info.nqueues;
+    }
+    p->sweep = sw;
+    p->sweep_sval = sval;
+    p->sweep_k = opts->k_hint;
+    p->rest_off = rest_off;
+    p->c_stage = c_stage;
+    p->stage_pos = stage_pos;
+    I.ncol_blocks = sw.nblocks;
+    I.sweep_entries = sw.n;
+    I.sweep_tiles = sw.ntiles;
+    I.sweep_k = opts->k_hint;
+    *taken = true;
+    return SPC3D_OK;
+}
+
 // Plan of a pattern that lies on the device: the single plan first (validation, the
 // whole pattern's figures), then, where choose_col_blocks says so, one plan per block
 // of columns in its place.
@@ -383,6 +555,24 @@ static int build_from_device(spc3d_ctx *ctx, int dtype, uint32_t nrows, uint32_t
     uint32_t nb = 1;
     const StoreOpts so = store_opts_of(opts);
     rc = choose_col_blocks(p, opts, &nb);
+    if (!rc) {
+        uint32_t sw_lanes = 0, sw_nb = 0;
+        choose_sweep(p, opts, nb, &sw_lanes, &sw_nb);
+        bool taken = false;
+        if (sw_lanes)
+            rc = rebuild_as_sweep(p, nrows, ncols, nnz, d_ii, d_jj, po, opts, sw_lanes, sw_nb, &taken);
+        if (rc) {
+            const std::string keep = g_err;
+            spc3d_plan_destroy(p);
+            return fail(rc, keep);
+        }
+        if (taken) {
+            *out = p;
+            return SPC3D_OK;
+        }
+        if (sw_lanes && opts->sweep == 2 && opts->col_blocks <= 1)
+            nb = 1; // asked for tiles, not for blocks
+    }
     if (!rc && nb <= 1)
         rc = add_store_staging(p, so);
     if (!rc && nb <= 1)
@@ -668,6 +858,10 @@ int spc3d_plan_download(spc3d_plan *plan, uint32_t *col, uint32_t *perm, uint32_
     if (!live(plan))
         return fail(SPC3D_ERR_INVALID_ARG, "plan is NULL or destroyed");
     const spc3d_plan_info &I = plan->info;
+    if (plan->sweep.n)
+        return fail(SPC3D_ERR_INVALID_ARG,
+                    "the plan is kept as row tiles x column blocks "
+                    "(spc3d_plan_info.sweep_entries > 0): there is no single set of arrays");
     if (!plan->blocks.empty())
         return fail(SPC3D_ERR_INVALID_ARG,
                     "the plan is kept in column blocks (spc3d_plan_info.ncol_blocks > 1): there "
@@ -785,7 +979,7 @@ int spc3d_plan_set_values(spc3d_plan *plan, const void *vv_host)
     if (rc)
         return rc;
     const size_t bytes = (size_t)nnz * elem_size(plan->dtype);
-    if (plan->blocks.empty() && !plan->perm && !plan->by_col) {
+    if (plan->blocks.empty() && !plan->perm && !plan->by_col && !plan->sweep.n) {
         rc = copy_h2d(plan->ctx, plan->sval, vv_host, bytes);
     } else {
         void *tmp = nullptr;
@@ -793,6 +987,12 @@ int spc3d_plan_set_values(spc3d_plan *plan, const void *vv_host)
         if (rc)
             return rc;
         rc = copy_h2d(plan->ctx, tmp, vv_host, bytes);
+        if (!rc && plan->sweep.n) {
+            hipError_t e = launch_gather_vals(plan->dtype, tmp, plan->sweep.perm, plan->sweep_sval,
+                                              plan->sweep.n, plan->ctx->stream);
+            if (e != hipSuccess)
+                rc = fail_hip(e, "gather of sparse values");
+        }
         std::vector<spc3d_plan *> self;
         for (spc3d_plan *part : parts_of(plan, self)) {
             if (rc)
@@ -831,6 +1031,9 @@ int spc3d_plan_set_values_device(spc3d_plan *plan, const spc3d_vals *vv)
     int rc = use_device(plan->ctx, true);
     if (rc)
         return rc;
+    if (plan->sweep.n)
+        HIP_TRY(launch_gather_vals(plan->dtype, vv->dev, plan->sweep.perm, plan->sweep_sval,
+                                   plan->sweep.n, plan->ctx->stream));
     std::vector<spc3d_plan *> self;
     for (spc3d_plan *part : parts_of(plan, self))
         HIP_TRY(launch_gather_vals(plan->dtype, vv->dev, part->perm, part->sval, part->info.nnz,
@@ -868,6 +1071,9 @@ int spc3d_plan_probe_columns(spc3d_plan *plan, int mode, uint32_t modulus)
     int rc = use_device(plan->ctx);
     if (rc)
         return rc;
+    if (plan->sweep.n) // one range of columns for every block: all hit, or all miss
+        HIP_TRY(launch_probe_cols(plan->sweep.col, plan->sweep.n, (uint32_t)mode, 0, modulus,
+                                  plan->info.ncols, plan->ctx->stream));
     std::vector<spc3d_plan *> self;
     for (spc3d_plan *part : parts_of(plan, self)) {
         rc = probe_columns_of(part, mode, modulus);
@@ -900,7 +1106,15 @@ static uint64_t own_device_bytes(const spc3d_plan *p)
     if (p->store.perm2) b += nnz * 4;
     if (p->store.n) b += (uint64_t)p->store.n * (8 + w); // dst, src, staged results
     if (p->two.n) b += nnz * (2 + 4 + 2) + 2 * nnz * w;  // l1, dst1, l2; c_stage, c_mid
-    if (!p->blocks.empty()) b += nnz * (w + 8);          // c_stage, stage_pos, stage_of
+    if (p->sweep.n) {
+        const uint64_t n = p->sweep.n, rest = nnz - n;
+        b += n * (4 + 2 + w) + nnz * 4; // col, lrow, values; perm
+        b += ((uint64_t)p->sweep.ntiles * p->sweep.nblocks * p->sweep.groups + 1) * 4;
+        b += (uint64_t)p->sweep.ntiles * p->sweep.rows_per_tile * 4;
+        b += ((n + 63) / 64 * 64 + rest) * w + nnz * 4; // c_stage, stage_pos
+    } else if (!p->blocks.empty()) {
+        b += nnz * (w + 8); // c_stage, stage_pos, stage_of
+    }
     return b;
 }
 

@@ -58,6 +58,32 @@ hipError_t launch_spmm(int dtype, const DevPlanView &P, const void *X, void *Y, 
 // (dense rows over 4096 bytes).
 hipError_t launch_sddmm_spmm(int dtype, int chained, const DevPlanView &P, const void *A,
                              const void *B, void *C, void *Y, uint32_t K, const Streams &streams);
+// ---- row tiles x column blocks ("sweep") -------------------------------------------
+// Device-side view of a sweep plan (SweepPlan in plan_device.h): the entries of rows of at
+// least a minimum length, ordered by tile of rows, column block, lane group, row.
+struct SweepView {
+    const uint32_t *ptr = nullptr;       // [ntiles * nblocks * groups + 1] entry ranges
+    const uint32_t *tile_rows = nullptr; // [ntiles * rows_per_tile] row of each local row, or 0xFFFFFFFF
+    const uint32_t *col = nullptr;       // [n] sweep order
+    const uint16_t *lrow = nullptr;      // [n] local row in the tile
+    const void *sval = nullptr;          // [n] values in sweep order
+    uint32_t ntiles = 0, nblocks = 0, rows_per_tile = 0;
+    uint32_t lanes = 0;                  // lanes per dense row the plan was made for: 16, 32 or 64
+    uint32_t per_launch = 0;             // tiles per generation (the GPU's CU count)
+};
+// Lanes per dense row of K reals when the sweep kernels take that width (dense rows of 256,
+// 512 or 1024 bytes), else 0; lane groups per workgroup, rows of a tile, and the most column
+// blocks a tile's range bounds fit LDS for, for that many lanes.
+uint32_t sweep_lanes(int dtype, uint32_t K);
+uint32_t sweep_groups(uint32_t lanes);
+uint32_t sweep_rows_per_tile(uint32_t lanes);
+uint32_t sweep_max_blocks(uint32_t lanes);
+// SDDMM over the sweep's entries: C[k] = sval[k] * <A[row of k,:], B[col[k],:]> in sweep order
+// (the caller brings them to the caller's positions); SpMM: Y[row,:] += sums.  K = lanes * 16
+// bytes / sizeof(real) exactly.  One launch per generation of per_launch tiles.
+hipError_t launch_sweep_sddmm(int dtype, const SweepView &S, const void *A, const void *B, void *C,
+                              hipStream_t stream);
+hipError_t launch_sweep_spmm(int dtype, const SweepView &S, const void *X, void *Y, hipStream_t stream);
 // first_cols[s * kFirstCols + u] = column of entry min(u, len - 1) of segment segs[s], s < n
 hipError_t launch_first_cols(const Seg *segs, uint32_t n, const uint32_t *col, uint32_t *first_cols,
                              hipStream_t stream);

@@ -1114,6 +1114,218 @@ spmm_fixup_kernel(const SplitRow *__restrict__ splits, uint32_t nsplit,
     }
 }
 
+// ------------------------------------------------- row tiles x column blocks ----
+// Long rows over columns that are not skewed (a hypergraph's incidence matrix: 1024 entries
+// per row, uniform over 500 k columns; 512-byte dense rows): every entry gathers a dense row
+// that no cache holds unless the columns are visited block by block, and cutting a row at
+// every block boundary costs its A row (SDDMM) or its Y row (SpMM) again per piece.  Here a
+// workgroup keeps a TILE of rows in LDS for a whole sweep over the column blocks: kSweepRowBytes
+// of A rows (SDDMM, read-only) or of Y accumulators (SpMM), one workgroup per CU, one launch
+// per "generation" of as many tiles as the GPU has CUs.  The workgroups of a generation start
+// together and meet the same amount of work in every block, so they walk the blocks in step,
+// and a barrier per block keeps the wavefronts of one workgroup in step too (without it the
+// oldest wavefronts run ahead by tens of blocks): at any time one block of dense rows is
+// what an L2 sees, and the gathers hit.
+//
+// The plan (build_sweep in plan_device.h) orders a tile's entries by block, inside a block
+// by lane group (a row belongs to lane group local_row % G for the whole sweep, so that SpMM
+// needs no atomics: its sums are the same bits run to run), inside a group by row.
+// ptr[(tile * nb + b) * G + g] .. [.. + 1) is the range of group g in block b.
+constexpr int kSweepBlock = 1024;
+constexpr uint32_t kSweepRowBytes = 128u << 10; // of LDS for the tile's rows
+constexpr uint32_t kSweepPtrWords = 6148;       // nb * G + 1 range bounds of a tile, in LDS too
+template <typename T, int LPR>
+__device__ __forceinline__ T sweep_dot(const typename Vec<T>::type &a, const typename Vec<T>::type &b)
+{
+    T d = a[0] * b[0];
+#pragma unroll
+    for (int i = 1; i < Vec<T>::N; ++i)
+        d += a[i] * b[i];
+    return d;
+}
+
+// One batch of a lane group: its entries' columns, local rows and (for the lanes that need
+// one) sparse values, asked for one batch ahead.
+template <typename T> struct SweepIdx {
+    uint32_t n = 0, col = 0, row = 0;
+    T val = (T)0;
+};
+
+template <typename T, int LPR, int UB>
+__global__ void __launch_bounds__(kSweepBlock)
+sweep_sddmm_kernel(const uint32_t *__restrict__ ptr, const uint32_t *__restrict__ tile_rows,
+                   const uint32_t *__restrict__ col, const uint16_t *__restrict__ lrow,
+                   const T *__restrict__ sval, const T *__restrict__ A, const T *__restrict__ B,
+                   T *__restrict__ C, uint32_t nb, uint32_t R, uint32_t tile0)
+{
+    using V = typename Vec<T>::type;
+    constexpr uint32_t G = kSweepBlock / LPR;
+    __shared__ V tile_a[kSweepRowBytes / 16];
+    __shared__ uint32_t lptr[kSweepPtrWords];
+    const uint32_t tile = tile0 + blockIdx.x;
+    for (uint32_t i = threadIdx.x; i < R * LPR; i += kSweepBlock) {
+        const uint32_t g = tile_rows[(uint64_t)tile * R + i / LPR];
+        V v{};
+        if (g != 0xFFFFFFFFu)
+            v = nt_load(reinterpret_cast<const V *>(A) + (uint64_t)g * LPR + i % LPR);
+        tile_a[i] = v;
+    }
+    for (uint32_t i = threadIdx.x; i < nb * G + 1; i += kSweepBlock)
+        lptr[i] = ptr[(uint64_t)tile * nb * G + i];
+    __syncthreads();
+    const uint32_t grp = threadIdx.x / LPR, sub = threadIdx.x % LPR;
+    const uint32_t uo = entry_of<LPR, UB>(sub);
+    const bool wlane = is_writer<LPR, UB>(sub);
+    const V *Bv = reinterpret_cast<const V *>(B);
+    auto fetch = [&](uint32_t q, uint32_t qhi) {
+        SweepIdx<T> x;
+        x.n = qhi - q < (uint32_t)UB ? qhi - q : (uint32_t)UB;
+        uint32_t e = sub & (UB - 1);
+        e = e < x.n ? e : x.n - 1;
+        x.col = nt_load(col + q + e);
+        x.row = nt_load(lrow + q + e);
+        x.val = (wlane && uo < x.n) ? nt_load(sval + q + uo) : (T)0;
+        return x;
+    };
+    uint32_t p = lptr[grp], hi = lptr[grp + 1];
+    SweepIdx<T> cur;
+    if (p < hi)
+        cur = fetch(p, hi);
+    for (uint32_t b = 0; b < nb; ++b) {
+        uint32_t p_nb = 0, hi_nb = 0; // the next block's range
+        if (b + 1 < nb) {
+            p_nb = lptr[(b + 1) * G + grp];
+            hi_nb = lptr[(b + 1) * G + grp + 1];
+        }
+        const bool had = p < hi;
+        while (p < hi) {
+            // the next batch's indices (this block's, or the first of the next block) before
+            // this batch's gathers
+            const uint32_t np = p + UB;
+            SweepIdx<T> nxt;
+            if (np < hi)
+                nxt = fetch(np, hi);
+            else if (p_nb < hi_nb)
+                nxt = fetch(p_nb, hi_nb);
+            V bv[UB];
+#pragma unroll
+            for (int u = 0; u < UB; ++u) {
+                const uint32_t c = __shfl(cur.col, u, LPR);
+                bv[u] = Bv[(uint64_t)c * LPR + sub];
+            }
+            __builtin_amdgcn_sched_barrier(0); // all gathers in flight before the first use
+            T part[UB];
+#pragma unroll
+            for (int u = 0; u < UB; ++u) {
+                const uint32_t l = __shfl(cur.row, u, LPR);
+                part[u] = sweep_dot<T, LPR>(tile_a[l * LPR + sub], bv[u]);
+            }
+            group_reduce<T, LPR, UB>(part, sub);
+            if (wlane && uo < cur.n)
+                nt_store(part[0] * cur.val, C + p + uo); // kernel order: whole lines, streaming
+            p = np;
+            cur = nxt;
+        }
+        p = p_nb;
+        hi = hi_nb;
+        if (!had && p < hi) // nothing of this group in block b: the next batch was not asked for
+            cur = fetch(p, hi);
+        __syncthreads(); // every lane group leaves block b before any enters block b + 1
+    }
+}
+
+template <typename T, int LPR, int UB>
+__global__ void __launch_bounds__(kSweepBlock)
+sweep_spmm_kernel(const uint32_t *__restrict__ ptr, const uint32_t *__restrict__ tile_rows,
+                  const uint32_t *__restrict__ col, const uint16_t *__restrict__ lrow,
+                  const T *__restrict__ sval, const T *__restrict__ X, T *__restrict__ Y,
+                  uint32_t nb, uint32_t R, uint32_t tile0)
+{
+    using V = typename Vec<T>::type;
+    constexpr uint32_t G = kSweepBlock / LPR;
+    __shared__ V tile_y[kSweepRowBytes / 16];
+    __shared__ uint32_t lptr[kSweepPtrWords];
+    const uint32_t tile = tile0 + blockIdx.x;
+    for (uint32_t i = threadIdx.x; i < R * LPR; i += kSweepBlock)
+        tile_y[i] = V{};
+    for (uint32_t i = threadIdx.x; i < nb * G + 1; i += kSweepBlock)
+        lptr[i] = ptr[(uint64_t)tile * nb * G + i];
+    __syncthreads();
+    const uint32_t grp = threadIdx.x / LPR, sub = threadIdx.x % LPR;
+    const V *Xv = reinterpret_cast<const V *>(X);
+    auto fetch = [&](uint32_t q, uint32_t qhi) {
+        SweepIdx<T> x;
+        x.n = qhi - q < (uint32_t)UB ? qhi - q : (uint32_t)UB;
+        uint32_t e = sub & (UB - 1);
+        e = e < x.n ? e : x.n - 1;
+        x.col = nt_load(col + q + e);
+        x.row = nt_load(lrow + q + e);
+        x.val = nt_load(sval + q + e);
+        return x;
+    };
+    // The rows of this lane group are its own for the whole sweep: sums of a row's run of
+    // entries are kept in registers and added to the row's accumulator in LDS when the run
+    // ends, in the plan's order: no atomics, the same bits run to run.
+    uint32_t row = 0xFFFFFFFFu;
+    V acc{};
+    uint32_t p = lptr[grp], hi = lptr[grp + 1];
+    SweepIdx<T> cur;
+    if (p < hi)
+        cur = fetch(p, hi);
+    for (uint32_t b = 0; b < nb; ++b) {
+        uint32_t p_nb = 0, hi_nb = 0;
+        if (b + 1 < nb) {
+            p_nb = lptr[(b + 1) * G + grp];
+            hi_nb = lptr[(b + 1) * G + grp + 1];
+        }
+        const bool had = p < hi;
+        while (p < hi) {
+            const uint32_t np = p + UB;
+            SweepIdx<T> nxt;
+            if (np < hi)
+                nxt = fetch(np, hi);
+            else if (p_nb < hi_nb)
+                nxt = fetch(p_nb, hi_nb);
+            V xv[UB];
+#pragma unroll
+            for (int u = 0; u < UB; ++u) {
+                const uint32_t c = __shfl(cur.col, u, LPR);
+                xv[u] = Xv[(uint64_t)c * LPR + sub];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int u = 0; u < UB; ++u) {
+                const uint32_t l = __shfl(cur.row, u, LPR);
+                const T a = (uint32_t)u < cur.n ? __shfl(cur.val, u, LPR) : (T)0;
+                if (l != row) {
+                    if (row != 0xFFFFFFFFu)
+                        tile_y[row * LPR + sub] += acc;
+                    acc = V{};
+                    row = l;
+                }
+                acc += xv[u] * a;
+            }
+            p = np;
+            cur = nxt;
+        }
+        p = p_nb;
+        hi = hi_nb;
+        if (!had && p < hi)
+            cur = fetch(p, hi);
+        __syncthreads();
+    }
+    if (row != 0xFFFFFFFFu)
+        tile_y[row * LPR + sub] += acc;
+    __syncthreads();
+    for (uint32_t i = threadIdx.x; i < R * LPR; i += kSweepBlock) {
+        const uint32_t g = tile_rows[(uint64_t)tile * R + i / LPR];
+        if (g != 0xFFFFFFFFu) {
+            V *y = reinterpret_cast<V *>(Y) + (uint64_t)g * LPR + i % LPR;
+            nt_store(nt_load(y) + tile_y[i], y);
+        }
+    }
+}
+
 // ---------------------------------------------- row pack / unpack (comm buffers) ----
 // The copies either side of the reference's sparse exchanges
 // (SparseComm::copy_to_sendbuff / copy_from_recvbuff / SUM_from_recvbuff,
@@ -1789,6 +2001,68 @@ hipError_t launch_spmm(int dtype, const DevPlanView &P, const void *X, void *Y, 
 {
     return dtype == 1 ? spmm_typed<double>(P, X, Y, K, stream)
                       : spmm_typed<float>(P, X, Y, K, stream);
+}
+
+uint32_t sweep_lanes(int dtype, uint32_t K)
+{
+    const uint64_t bytes = (uint64_t)K * (dtype == 1 ? 8 : 4);
+    return bytes == 256 ? 16u : (bytes == 512 ? 32u : (bytes == 1024 ? 64u : 0u));
+}
+uint32_t sweep_groups(uint32_t lanes) { return lanes ? kSweepBlock / lanes : 0; }
+uint32_t sweep_rows_per_tile(uint32_t lanes) { return lanes ? kSweepRowBytes / (lanes * 16) : 0; }
+uint32_t sweep_max_blocks(uint32_t lanes)
+{
+    return lanes ? (kSweepPtrWords - 1) / (kSweepBlock / lanes) : 0;
+}
+
+namespace {
+template <typename T, int LPR>
+void sweep_launch(bool spmm, const SweepView &S, const T *A, const T *B, T *out, uint32_t tile0,
+                  uint32_t ntiles, hipStream_t stream)
+{
+    if (spmm)
+        hipLaunchKernelGGL((sweep_spmm_kernel<T, LPR, 16>), dim3(ntiles), dim3(kSweepBlock), 0,
+                           stream, S.ptr, S.tile_rows, S.col, S.lrow, (const T *)S.sval, B, out,
+                           S.nblocks, S.rows_per_tile, tile0);
+    else
+        hipLaunchKernelGGL((sweep_sddmm_kernel<T, LPR, 16>), dim3(ntiles), dim3(kSweepBlock), 0,
+                           stream, S.ptr, S.tile_rows, S.col, S.lrow, (const T *)S.sval, A, B, out,
+                           S.nblocks, S.rows_per_tile, tile0);
+}
+template <typename T>
+hipError_t sweep_run(bool spmm, const SweepView &S, const T *A, const T *B, T *out, hipStream_t stream)
+{
+    if (S.ntiles == 0)
+        return hipSuccess;
+    // what the kernels assume of the plan: the tile's rows and range bounds fit their LDS
+    if ((S.lanes != 16 && S.lanes != 32 && S.lanes != 64) || S.per_launch == 0 ||
+        S.rows_per_tile * S.lanes * 16 > kSweepRowBytes ||
+        (uint64_t)S.nblocks * (kSweepBlock / S.lanes) + 1 > kSweepPtrWords)
+        return hipErrorInvalidValue;
+    for (uint32_t t0 = 0; t0 < S.ntiles; t0 += S.per_launch) { // one generation per launch
+        const uint32_t n = S.ntiles - t0 < S.per_launch ? S.ntiles - t0 : S.per_launch;
+        if (S.lanes == 16)
+            sweep_launch<T, 16>(spmm, S, A, B, out, t0, n, stream);
+        else if (S.lanes == 32)
+            sweep_launch<T, 32>(spmm, S, A, B, out, t0, n, stream);
+        else
+            sweep_launch<T, 64>(spmm, S, A, B, out, t0, n, stream);
+    }
+    return hipGetLastError();
+}
+} // namespace
+
+hipError_t launch_sweep_sddmm(int dtype, const SweepView &S, const void *A, const void *B, void *C,
+                              hipStream_t stream)
+{
+    return dtype == 1 ? sweep_run<double>(false, S, (const double *)A, (const double *)B, (double *)C, stream)
+                      : sweep_run<float>(false, S, (const float *)A, (const float *)B, (float *)C, stream);
+}
+
+hipError_t launch_sweep_spmm(int dtype, const SweepView &S, const void *X, void *Y, hipStream_t stream)
+{
+    return dtype == 1 ? sweep_run<double>(true, S, nullptr, (const double *)X, (double *)Y, stream)
+                      : sweep_run<float>(true, S, nullptr, (const float *)X, (float *)Y, stream);
 }
 
 hipError_t launch_first_cols(const Seg *segs, uint32_t n, const uint32_t *col, uint32_t *first_cols,

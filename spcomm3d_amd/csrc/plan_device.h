@@ -93,6 +93,37 @@ struct StoreStaging {
 int build_store_staging(hipStream_t stream, const Seg *d_segs, uint32_t nseg, const uint32_t *d_perm,
                         uint64_t nnz, StoreStaging &out, std::string &err);
 
+// ---- row tiles x column blocks ("sweep") -------------------------------------------------
+// For long rows over columns without skew (see the sweep kernels in kernels.hip).  Rows of at
+// least min_row entries are ranked longest first and dealt to tiles of rows_per_tile rows,
+// the rows of rank j in a generation of per_launch tiles going to tile j % per_launch, so
+// that the tiles of a generation hold the same mix of lengths; local row l of a tile belongs
+// to lane group l % groups.  Their entries are sorted by (tile, column block, lane group,
+// local row), the caller's order kept inside a row's run; the entries of shorter rows follow
+// in the caller's order ("rest"; another plan runs them).
+//   perm[k]      caller's position of entry k of that order                [nnz]
+//   col, lrow    column and local row of sweep entry k                     [n]
+//   ptr          range bounds per (tile, block, group)                     [ntiles*nblocks*groups + 1]
+//   tile_rows    row of local row l of tile t, 0xFFFFFFFF where there is none [ntiles*rows_per_tile]
+// The arrays belong to the receiver (hipFree).  Synchronous.
+struct SweepPlan {
+    uint32_t *perm = nullptr, *col = nullptr, *ptr = nullptr, *tile_rows = nullptr;
+    uint16_t *lrow = nullptr;
+    uint64_t n = 0; // entries in the sweep; the other nnz - n are the rest
+    uint32_t ntiles = 0, nblocks = 0, rows_per_tile = 0, groups = 0, lanes = 0, per_launch = 0;
+    uint32_t nrows_in = 0; // rows in the sweep
+};
+int build_sweep(hipStream_t stream, uint32_t nrows, uint32_t ncols, uint64_t nnz,
+                const uint32_t *d_ii, const uint32_t *d_jj, uint32_t lanes, uint32_t rows_per_tile,
+                uint32_t nblocks, uint32_t min_row, uint32_t per_launch, SweepPlan &out,
+                std::string &err);
+// d_out[d_perm[q]] = base + q, q < n.  Asynchronous on `stream`.
+int inverse_offsets_device(hipStream_t stream, const uint32_t *d_perm, uint64_t n, uint32_t base,
+                           uint32_t *d_out, std::string &err);
+// d_out[q] = d_in[d_idx[q]], q < n.  Asynchronous on `stream`.
+int gather_u32_device(hipStream_t stream, const uint32_t *d_in, const uint32_t *d_idx, uint64_t n,
+                      uint32_t *d_out, std::string &err);
+
 // ---- SDDMM results of an arbitrary entry order, brought home in two passes -------------
 // C[perm[p]] = r[p] for all p, with r in kernel order, is one store (or one load) per result
 // into a line of its own however it is turned.  Any permutation of n elements is two passes

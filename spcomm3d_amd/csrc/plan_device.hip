@@ -1492,6 +1492,204 @@ int build_two_pass(hipStream_t st, const uint32_t *d_perm, uint64_t nnz, uint32_
     return SPC3D_OK;
 }
 
+// ---- row tiles x column blocks ("sweep") ---------------------------------------------
+// Tile and local row of the row of rank j (longest first) among the nin rows of the sweep.
+__global__ void sweep_rows_k(const uint32_t *__restrict__ order, uint32_t nin, uint32_t P,
+                             uint32_t R, uint32_t *row_tile, uint32_t *row_local,
+                             uint32_t *tile_rows)
+{
+    GRID_STRIDE(j, nin)
+    {
+        const uint32_t row = order[j];
+        const uint64_t per_gen = (uint64_t)P * R;
+        const uint32_t gen = (uint32_t)(j / per_gen), jl = (uint32_t)(j % per_gen);
+        const uint32_t t = gen * P + jl % P, l = jl / P;
+        row_tile[row] = t;
+        row_local[row] = l;
+        tile_rows[(uint64_t)t * R + l] = row;
+    }
+}
+
+__global__ void sweep_hist_k(const uint32_t *__restrict__ ii, uint64_t nnz, uint32_t *rowcnt)
+{
+    GRID_STRIDE(e, nnz) atomicAdd(&rowcnt[ii[e]], 1u);
+}
+
+// out[perm[q]] = base + q
+__global__ void inverse_offsets_k(const uint32_t *__restrict__ perm, uint64_t n, uint32_t base,
+                                  uint32_t *out)
+{
+    GRID_STRIDE(q, n) out[perm[q]] = base + (uint32_t)q;
+}
+
+// Sort key of entry e: (tile, block, lane group, local row / groups); one past the largest
+// such key for an entry of a row outside the sweep (they sort last, in the caller's order).
+__global__ void sweep_keys_k(const uint32_t *__restrict__ ii, const uint32_t *__restrict__ jj,
+                             uint64_t nnz, const uint32_t *__restrict__ row_tile,
+                             const uint32_t *__restrict__ row_local, uint32_t block_cols,
+                             uint32_t nb, uint32_t G, uint32_t per_group,
+                             unsigned long long rest_key, unsigned long long *key,
+                             unsigned long long *nin)
+{
+    unsigned long long mine = 0;
+    GRID_STRIDE(e, nnz)
+    {
+        const uint32_t r = ii[e], t = row_tile[r];
+        if (t == 0xFFFFFFFFu) {
+            key[e] = rest_key;
+            continue;
+        }
+        const uint32_t l = row_local[r], b = jj[e] / block_cols;
+        key[e] = (((unsigned long long)t * nb + b) * G + l % G) * per_group + l / G;
+        ++mine;
+    }
+    mine = block_sum(mine);
+    if (threadIdx.x == 0 && mine)
+        atomicAdd(nin, mine);
+}
+
+// Of the sorted sweep entries: column, local row, and the (tile, block, group) bin.
+__global__ void sweep_entries_k(const unsigned long long *__restrict__ skey,
+                                const uint32_t *__restrict__ perm,
+                                const uint32_t *__restrict__ jj, uint64_t n, uint32_t G,
+                                uint32_t per_group, uint32_t *col, uint16_t *lrow, uint32_t *bin)
+{
+    GRID_STRIDE(k, n)
+    {
+        const unsigned long long key = skey[k];
+        const unsigned long long b = key / per_group;
+        bin[k] = (uint32_t)b;
+        lrow[k] = (uint16_t)((uint32_t)(key % per_group) * G + (uint32_t)(b % G));
+        col[k] = jj[perm[k]];
+    }
+}
+
+int build_sweep(hipStream_t st, uint32_t nrows, uint32_t ncols, uint64_t nnz, const uint32_t *d_ii,
+                const uint32_t *d_jj, uint32_t lanes, uint32_t R, uint32_t nb, uint32_t min_row,
+                uint32_t P, SweepPlan &out, std::string &err)
+{
+    out = SweepPlan();
+    if (nnz == 0 || nnz >= (1ull << 32) || lanes == 0 || R == 0 || R > 65536 || nb == 0 || P == 0)
+        return SPC3D_OK;
+    const uint32_t G = 1024 / lanes;
+    if (G == 0 || R % G != 0)
+        return SPC3D_OK;
+    const uint32_t per_group = R / G;
+    const uint32_t block_cols = (ncols + nb - 1) / nb;
+    Arena arena;
+    HIP_OK(arena.reserve(((size_t)nrows + 1) * 28 + (size_t)nnz * 28 + ((size_t)8 << 20)));
+    Temp tmp(arena);
+    // ---- rows by length ----
+    SBuf<uint32_t> rowcnt, rowid, order, cnt_sorted, row_tile, row_local;
+    SBuf<unsigned long long> total;
+    HIP_OK(rowcnt.alloc(arena, (size_t)nrows + 1));
+    HIP_OK(rowid.alloc(arena, nrows));
+    HIP_OK(order.alloc(arena, nrows));
+    HIP_OK(cnt_sorted.alloc(arena, nrows));
+    HIP_OK(row_tile.alloc(arena, nrows));
+    HIP_OK(row_local.alloc(arena, nrows));
+    HIP_OK(total.alloc(arena, 1));
+    HIP_OK(hipMemsetAsync(rowcnt.p, 0, ((size_t)nrows + 1) * sizeof(uint32_t), st));
+    HIP_OK(hipMemsetAsync(total.p, 0, sizeof(unsigned long long), st));
+    LAUNCH(sweep_hist_k, nnz, d_ii, nnz, rowcnt.p);
+    // rows by length, longest first, equal lengths in row order; those of at least min_row
+    // entries come first and are the sweep's
+    LAUNCH(iota_k, nrows, rowid.p, (uint64_t)nrows);
+    TRY(sort_pairs<uint32_t>(tmp, rowcnt.p, cnt_sorted.p, rowid.p, order.p, nrows, 32, true, st, err));
+    std::vector<uint32_t> lens;
+    try {
+        lens.resize(nrows);
+    } catch (const std::bad_alloc &) {
+        err = "host allocation failed";
+        return SPC3D_ERR_ALLOC;
+    }
+    TRY(fetch(st, lens.data(), cnt_sorted.p, (size_t)nrows * sizeof(uint32_t), err));
+    uint32_t nin = 0;
+    while (nin < nrows && lens[nin] >= min_row && lens[nin] > 0)
+        ++nin;
+    if (nin == 0)
+        return SPC3D_OK;
+    const uint64_t per_gen = (uint64_t)P * R;
+    const uint64_t gens = (nin + per_gen - 1) / per_gen;
+    const uint64_t last = nin - (gens - 1) * per_gen; // rows of the last generation
+    const uint64_t ntiles64 = (gens - 1) * P + std::min<uint64_t>(P, last);
+    if (ntiles64 * nb * G + 1 >= (1ull << 32))
+        return SPC3D_OK;
+    const uint32_t ntiles = (uint32_t)ntiles64;
+    DBuf<uint32_t> tile_rows, perm, col, ptr;
+    DBuf<uint16_t> lrow;
+    HIP_OK(tile_rows.alloc((size_t)ntiles * R));
+    HIP_OK(hipMemsetAsync(tile_rows.p, 0xFF, (size_t)ntiles * R * sizeof(uint32_t), st));
+    HIP_OK(hipMemsetAsync(row_tile.p, 0xFF, (size_t)nrows * sizeof(uint32_t), st));
+    LAUNCH(sweep_rows_k, nin, order.p, nin, P, R, row_tile.p, row_local.p, tile_rows.p);
+    // ---- entries ----
+    SBuf<unsigned long long> key, skey;
+    SBuf<uint32_t> ident, bin;
+    HIP_OK(key.alloc(arena, nnz));
+    HIP_OK(skey.alloc(arena, nnz));
+    HIP_OK(ident.alloc(arena, nnz));
+    HIP_OK(perm.alloc(nnz));
+    const unsigned long long rest_key = (unsigned long long)ntiles * nb * G * per_group;
+    LAUNCH_SMALL(sweep_keys_k, nnz, d_ii, d_jj, nnz, row_tile.p, row_local.p, block_cols, nb, G,
+                 per_group, rest_key, key.p, total.p);
+    LAUNCH(iota_k, nnz, ident.p, nnz);
+    TRY(sort_pairs<unsigned long long>(tmp, key.p, skey.p, ident.p, perm.p, (uint32_t)nnz,
+                                       bits_for(rest_key), false, st, err));
+    unsigned long long n = 0;
+    TRY(fetch(st, &n, total.p, sizeof n, err));
+    if (n == 0)
+        return SPC3D_OK;
+    HIP_OK(col.alloc(n));
+    HIP_OK(lrow.alloc(n));
+    HIP_OK(bin.alloc(arena, n));
+    const uint64_t nbins = (uint64_t)ntiles * nb * G;
+    HIP_OK(ptr.alloc(nbins + 1));
+    SBuf<uint32_t> bstart, bcnt;
+    HIP_OK(bstart.alloc(arena, nbins));
+    HIP_OK(bcnt.alloc(arena, nbins + 1));
+    HIP_OK(hipMemsetAsync(bcnt.p, 0, (nbins + 1) * sizeof(uint32_t), st));
+    LAUNCH(sweep_entries_k, n, skey.p, perm.p, d_jj, n, G, per_group, col.p, lrow.p, bin.p);
+    LAUNCH(run_bounds_k, n, bin.p, n, (uint32_t)nbins, bstart.p, bcnt.p);
+    LAUNCH(run_lengths_k, nbins, bstart.p, nbins, bcnt.p);
+    TRY(exclusive_sum(tmp, bcnt.p, ptr.p, (size_t)nbins + 1, st, err));
+    HIP_OK(hipGetLastError());
+    HIP_OK(hipStreamSynchronize(st));
+    out.perm = perm.release();
+    out.col = col.release();
+    out.lrow = lrow.release();
+    out.ptr = ptr.release();
+    out.tile_rows = tile_rows.release();
+    out.n = n;
+    out.ntiles = ntiles;
+    out.nblocks = nb;
+    out.rows_per_tile = R;
+    out.groups = G;
+    out.lanes = lanes;
+    out.per_launch = P;
+    out.nrows_in = nin;
+    return SPC3D_OK;
+}
+
+int inverse_offsets_device(hipStream_t st, const uint32_t *d_perm, uint64_t n, uint32_t base,
+                           uint32_t *d_out, std::string &err)
+{
+    if (n == 0)
+        return SPC3D_OK;
+    LAUNCH(inverse_offsets_k, n, d_perm, n, base, d_out);
+    HIP_OK(hipGetLastError());
+    return SPC3D_OK;
+}
+
+int gather_u32_device(hipStream_t st, const uint32_t *d_in, const uint32_t *d_idx, uint64_t n,
+                      uint32_t *d_out, std::string &err)
+{
+    if (n == 0)
+        return SPC3D_OK;
+    LAUNCH(gather_u32_k, n, d_in, d_idx, n, d_out);
+    HIP_OK(hipGetLastError());
+    return SPC3D_OK;
+}
+
 __global__ void descents_k(const uint32_t *__restrict__ d, uint64_t n, unsigned long long *acc)
 {
     unsigned long long c = 0;

@@ -6,9 +6,11 @@
 // time of the kernel inside it, as JSON on stdout.
 //
 //   dist_step <file.bin> <K> <reps>
+#include <algorithm>
 #include <chrono>
 #include <cstdio>
 #include <cstdlib>
+#include <memory>
 #include <random>
 #include <string>
 #include <vector>
@@ -72,7 +74,65 @@ int main(int argc, char **argv)
         double sc, sk, sp, pc, pk, pp;
         run(true, sc, sk, sp);
         run(false, pc, pk, pp);
-        std::printf("{\"wrappers\": \"dist_sddmm_spcomm, dist_spmm_spcomm (device-resident, one rank)\", "
+        // The reference's loop around its kernels on resident operands (miniapp/bench_both.cpp:
+        // 196-205): ReMapIndices over the pattern, NUM_ITER = 5 calls of the wrapper over the
+        // remapped pattern, ReMapIndices back.  The pattern lives on the device; the plan is made
+        // from it there after the remap (a plan is tied to the indices it was made from).
+        double loop_us = 0, loop_plan_us = 0, loop_calls_us = 0;
+        {
+            std::vector<idx_t> mapA(m), mapB(n), mapAI(m), mapBI(n);
+            for (idx_t i = 0; i < m; ++i) mapA[i] = i;
+            for (idx_t i = 0; i < n; ++i) mapB[i] = i;
+            std::shuffle(mapA.begin(), mapA.end(), g);
+            std::shuffle(mapB.begin(), mapB.end(), g);
+            for (idx_t i = 0; i < m; ++i) mapAI[mapA[i]] = i;
+            for (idx_t i = 0; i < n; ++i) mapBI[mapB[i]] = i;
+            // 32-bit words on the device: index arrays and maps travel as value vectors of floats
+            auto words = [&](const std::vector<idx_t> &v) {
+                auto *d = new spc3d::Vals<float>(ctx, v.size());
+                d->upload(reinterpret_cast<const float *>(v.data()));
+                return std::unique_ptr<spc3d::Vals<float>>(d);
+            };
+            auto dii = words(S.ii), djj = words(S.jj), dA = words(mapA), dB = words(mapB),
+                 dAI = words(mapAI), dBI = words(mapBI);
+            spc3d::Vals<real_t> vv(ctx, S.nnz);
+            vv.upload(S.vv.data());
+            auto remap = [&](spc3d::Vals<float> &idx, spc3d::Vals<float> &map, idx_t len) {
+                spc3d::check(spc3d_remap_device(ctx.get(), S.nnz, idx.device_ptr(), map.device_ptr(), len),
+                             "spc3d_remap_device");
+            };
+            const int loops = 3;
+            for (int it = 0; it < loops + 1; ++it) { // the first pass warms up
+                ctx.sync();
+                const auto t0 = clk::now();
+                remap(*dii, *dA, m);
+                remap(*djj, *dB, n);
+                const auto t1 = clk::now();
+                spc3d::Plan<real_t> Q(spc3d::Plan<real_t>::FromDevice{}, ctx, m, n, S.nnz,
+                                      dii->device_ptr(), djj->device_ptr());
+                Q.set_values(vv);
+                ctx.sync();
+                const auto t2 = clk::now();
+                for (int i = 0; i < 5; ++i)
+                    dist_sddmm_spcomm(ctx, A, B, Q, pre, zred, C, mesh, "bench");
+                const auto t3 = clk::now();
+                remap(*dii, *dAI, m);
+                remap(*djj, *dBI, n);
+                ctx.sync();
+                const auto t4 = clk::now();
+                if (it == 0)
+                    continue;
+                loop_us += std::chrono::duration<double, std::micro>(t4 - t0).count() / loops;
+                loop_plan_us += std::chrono::duration<double, std::micro>(t2 - t1).count() / loops;
+                loop_calls_us += std::chrono::duration<double, std::micro>(t3 - t2).count() / loops;
+            }
+        }
+        std::printf("{\"reference_loop\": {\"what\": \"ReMapIndices, plan from the device, 5 x "
+                    "dist_sddmm_spcomm, ReMapIndices back; all operands resident "
+                    "(miniapp/bench_both.cpp:196-205)\", \"total_us\": %.1f, \"plan_us\": %.1f, "
+                    "\"five_calls_us\": %.1f, \"remaps_us\": %.1f}, ",
+                    loop_us, loop_plan_us, loop_calls_us, loop_us - loop_plan_us - loop_calls_us);
+        std::printf("\"wrappers\": \"dist_sddmm_spcomm, dist_spmm_spcomm (device-resident, one rank)\", "
                     "\"real\": \"%s\", \"nnz\": %llu, \"k\": %u, \"reps\": %d, "
                     "\"sddmm_call_us\": %.1f, \"sddmm_kernel_us\": %.1f, \"sddmm_z_reduce_us\": %.1f, "
                     "\"spmm_call_us\": %.1f, \"spmm_kernel_us\": %.1f, "

@@ -153,6 +153,25 @@ class Workload:
                         np.ascontiguousarray(self.ii[p]), np.ascontiguousarray(self.jj[p]),
                         np.ascontiguousarray(self.vv64[p]), "shuffled", dict(self.notes))
 
+    def localized(self) -> "Workload":
+        """Same entries with the local indices ``COOMatrix::localizeIndices`` gives them
+        (src/SparseMatrix.hpp:69-99): every row (column) that holds an entry gets the next
+        id the first time it appears in the entry stream, and the panels shrink to the
+        touched rows and columns, which is the shape a rank of the reference runs its
+        kernels on (miniapp/bench_both.cpp:158,189-190)."""
+        def first_appearance(idx):
+            u, first, inv = np.unique(idx, return_index=True, return_inverse=True)
+            rank = np.empty(u.size, dtype=np.uint32)
+            rank[np.argsort(first, kind="stable")] = np.arange(u.size, dtype=np.uint32)
+            return np.ascontiguousarray(rank[inv]), int(u.size)
+        li, m = first_appearance(self.ii)
+        lj, n = first_appearance(self.jj)
+        w = Workload(self.name + "_localized", m, n, self.k, li, lj, self.vv64, self.order,
+                     dict(self.notes))
+        w.notes["touched"] = (m, n)
+        w.notes["global_shape"] = (self.nrows, self.ncols)
+        return w
+
     def column_major(self) -> "Workload":
         """Same matrix, entries sorted by column and by row inside a column: the order
         of a MatrixMarket file, which the reference's converter and readers keep

@@ -1,0 +1,164 @@
+"""Row tiles x column blocks (spc3d_plan_opts.sweep): long rows kept in LDS while their
+workgroups walk the column blocks.  Same results as the ordinary plan to the tolerance of
+the parity tests, the same bits run to run, through every entry point."""
+import numpy as np
+import pytest
+
+from spcomm3d_amd import _capi as capi
+from tests import _oracle as oracle
+
+pytestmark = pytest.mark.gpu
+
+TOL = {np.dtype(np.float32): 1e-5, np.dtype(np.float64): 1e-12}
+
+
+def long_rows(seed, m, n, k, dtype, lens):
+    """Rows of the given lengths over uniform columns (repeats allowed), in a shuffled
+    order, with values and panels."""
+    rng = np.random.default_rng(seed)
+    lens = np.asarray(lens, dtype=np.int64)
+    ii = np.repeat(np.arange(m, dtype=np.uint32), lens)
+    jj = rng.integers(0, n, ii.size).astype(np.uint32)
+    o = rng.permutation(ii.size)
+    ii, jj = np.ascontiguousarray(ii[o]), np.ascontiguousarray(jj[o])
+    vv = rng.random(ii.size).astype(dtype)
+    A = rng.uniform(-1, 1, (m, k)).astype(dtype)
+    B = rng.uniform(-1, 1, (n, k)).astype(dtype)
+    Y0 = rng.uniform(-1, 1, (m, k)).astype(dtype)
+    return ii, jj, vv, A, B, Y0
+
+
+def run_all(ctx, m, n, ii, jj, vv, A, B, Y0, **opts):
+    """C of sddmm, Y of spmm (twice: bits), Y of spmm_noalloc, C and Y of the one-pass call
+    plain and chained; and the plan's info."""
+    S = ctx.plan(m, n, ii, jj, vv, **opts)
+    info = S.info
+    dA, dB = ctx.panel_from(A), ctx.panel_from(B)
+    dC = ctx.vals(ii.size, A.dtype)
+    dC.fill(-7.0)
+    ctx.sddmm(S, dA, dB, dC)
+    out = {"C": dC.download()}
+    for name, call in (("Y", ctx.spmm), ("Y_again", ctx.spmm), ("Y_noalloc", ctx.spmm_noalloc)):
+        dY = ctx.panel_from(Y0)
+        call(S, dB, dY)
+        out[name] = dY.download()
+        dY.close()
+    for name, chained in (("one", False), ("chain", True)):
+        dY = ctx.panel_from(Y0)
+        dC.fill(3.0)
+        ctx.sddmm_spmm(S, dA, dB, dC, dY, chained=chained)
+        out["C_" + name], out["Y_" + name] = dC.download(), dY.download()
+        dY.close()
+    for h in (S, dA, dB, dC):
+        h.close()
+    return out, info
+
+
+def check(out, ii, jj, vv, A, B, Y0):
+    tol = TOL[A.dtype]
+    assert oracle.sddmm_rel_err(A, B, ii, jj, vv, out["C"]) <= tol
+    assert oracle.spmm_rel_err(B, ii, jj, vv, Y0, out["Y"]) <= tol
+    assert np.array_equal(out["Y"], out["Y_again"])
+    assert np.array_equal(out["Y"], out["Y_noalloc"])
+    assert np.array_equal(out["C_one"], out["C"]) and np.array_equal(out["C_chain"], out["C"])
+    assert oracle.spmm_rel_err(B, ii, jj, vv, Y0, out["Y_one"]) <= tol
+    assert oracle.spmm_rel_err(B, ii, jj, out["C"], Y0, out["Y_chain"]) <= tol
+
+
+@pytest.mark.parametrize("dtype,k", [(np.float32, 64), (np.float32, 128), (np.float32, 256),
+                                     (np.float64, 32), (np.float64, 64), (np.float64, 128)])
+def test_tiles_and_rest_against_the_oracle(ctx, dtype, k):
+    rng = np.random.default_rng(k)
+    m, n = 700, 3000
+    lens = rng.integers(0, 400, m)
+    lens[::7] = rng.integers(1, 12, lens[::7].size)  # short rows: the plan of the rest
+    lens[5] = 0
+    lens[11] = 5000                                  # more entries than columns
+    case = long_rows(1000 + k, m, n, k, dtype, lens)
+    ii, jj, vv, A, B, Y0 = case
+    out, info = run_all(ctx, m, n, *case, k_hint=k, sweep=True, sweep_min_row=12, col_blocks=7)
+    assert info.sweep_k == k and info.sweep_tiles > 0 and info.ncol_blocks == 7
+    want = int(lens[lens >= 12].sum())
+    assert info.sweep_entries == want and info.nsegments > 0
+    assert info.device_bytes > ii.size * 10
+    check(out, *case)
+    # against the ordinary plan: the same products, another summation order
+    ref, rinfo = run_all(ctx, m, n, *case, k_hint=k, sweep=False)
+    assert rinfo.sweep_entries == 0
+    scale = oracle.sddmm_scale(A, B, ii, jj, vv)
+    assert oracle.rel_err(out["C"], ref["C"], scale) <= TOL[A.dtype]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_every_row_in_the_tiles_and_more_tiles_than_one_launch_takes(ctx, dtype):
+    # 512-byte dense rows: 256 rows per tile, one launch per CU-count tiles; 150 k rows of
+    # a few entries each make more than two launches' worth of tiles, the last one partial
+    k = 128 if dtype == np.float32 else 64
+    m, n = 150_000, 4096
+    rng = np.random.default_rng(5)
+    lens = rng.integers(1, 9, m)
+    case = long_rows(77, m, n, k, dtype, lens)
+    out, info = run_all(ctx, m, n, *case, k_hint=k, sweep=True, sweep_min_row=1, col_blocks=3)
+    assert info.sweep_entries == case[0].size and info.nsegments == 0
+    # a launch deals its rows over as many tiles as there are CUs: two full launches of 256
+    # rows per tile, and the last one's 18,928 rows thinly over its tiles
+    cus = info.sweep_tiles // 3
+    assert info.sweep_tiles == 3 * cus and 2 * cus * 256 < m <= 3 * cus * 256
+    check(out, *case)
+
+
+def test_a_single_block_and_as_many_as_fit(ctx):
+    k, m, n = 128, 300, 5000
+    lens = np.full(m, 200)
+    case = long_rows(3, m, n, k, np.float32, lens)
+    for nb in (1, 192, 4000):  # 4000: cut down to what a tile's range bounds allow
+        out, info = run_all(ctx, m, n, *case, k_hint=k, sweep=True, sweep_min_row=1, col_blocks=nb)
+        assert info.sweep_entries == case[0].size and info.ncol_blocks == min(nb, 192)
+        check(out, *case)
+
+
+def test_another_k_is_refused_and_other_widths_keep_the_ordinary_plan(ctx):
+    k, m, n = 128, 200, 1000
+    case = long_rows(9, m, n, k, np.float32, np.full(m, 100))
+    ii, jj, vv, A, B, Y0 = case
+    S = ctx.plan(m, n, ii, jj, vv, k_hint=k, sweep=True, sweep_min_row=1)
+    assert S.info.sweep_entries == ii.size
+    dA, dB, dY = ctx.panel_from(A[:, :64]), ctx.panel_from(B[:, :64]), ctx.panel_from(Y0[:, :64])
+    dC = ctx.vals(ii.size, np.float32)
+    for call in (lambda: ctx.sddmm(S, dA, dB, dC), lambda: ctx.spmm(S, dB, dY),
+                 lambda: ctx.spmm_noalloc(S, dB, dY), lambda: ctx.sddmm_spmm(S, dA, dB, dC, dY)):
+        with pytest.raises(capi.Spc3dError) as e:
+            call()
+        assert e.value.status == capi.ERR_INVALID_ARG and "k_hint" in str(e.value)
+    ctx.sync()
+    assert np.array_equal(dY.download(), Y0[:, :64])
+    for h in (S, dA, dB, dC, dY):
+        h.close()
+    # a width the tile kernels do not take, or no k_hint: the ordinary plan
+    for opts in ({"k_hint": 100, "sweep": True}, {"sweep": True}):
+        S = ctx.plan(m, n, ii, jj, vv, **opts)
+        assert S.info.sweep_entries == 0 and S.info.nsegments > 0
+        S.close()
+
+
+def test_values_set_later_and_from_the_device(ctx):
+    k, m, n = 64, 400, 2000
+    rng = np.random.default_rng(1)
+    lens = rng.integers(0, 150, m)
+    ii, jj, vv, A, B, Y0 = long_rows(21, m, n, k, np.float64, lens)
+    S = ctx.plan(m, n, ii, jj, None, dtype=np.float64, k_hint=k, sweep=True, sweep_min_row=20,
+                 col_blocks=4)
+    assert 0 < S.info.sweep_entries < ii.size
+    dA, dB = ctx.panel_from(A), ctx.panel_from(B)
+    dC = ctx.vals(ii.size, np.float64)
+    S.set_values(vv)
+    ctx.sddmm(S, dA, dB, dC)
+    first = dC.download()
+    assert oracle.sddmm_rel_err(A, B, ii, jj, vv, first) <= 1e-12
+    dV = ctx.vals(ii.size, np.float64)
+    dV.upload(2 * vv)
+    S.set_values_device(dV)
+    ctx.sddmm(S, dA, dB, dC)
+    assert np.array_equal(dC.download(), 2 * first)
+    for h in (S, dA, dB, dC, dV):
+        h.close()
