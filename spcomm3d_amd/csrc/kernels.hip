@@ -1127,10 +1127,13 @@ spmm_fixup_kernel(const SplitRow *__restrict__ splits, uint32_t nsplit,
 // oldest wavefronts run ahead by tens of blocks): at any time one block of dense rows is
 // what an L2 sees, and the gathers hit.
 //
-// The plan (build_sweep in plan_device.h) orders a tile's entries by block, inside a block
-// by lane group (a row belongs to lane group local_row % G for the whole sweep, so that SpMM
-// needs no atomics: its sums are the same bits run to run), inside a group by row.
-// ptr[(tile * nb + b) * G + g] .. [.. + 1) is the range of group g in block b.
+// The plan (build_sweep in plan_device.h) orders a tile's entries by block, inside a block by
+// row, and cuts every (tile, block) range into G chunks at row boundaries, as equal as those
+// allow: ptr[(tile * nb + b) * G + g] .. [.. + 1) is chunk g of block b.  SpMM gives chunk g
+// to lane group g: within a block a row belongs to one lane group, the barrier separates the
+// blocks, so its sums need no atomics and are the same bits run to run.  SDDMM, where any
+// lane group can take any entry, deals the batches of the whole (tile, block) range to the
+// lane groups in turn, which leaves them within one batch of each other.
 constexpr int kSweepBlock = 1024;
 constexpr uint32_t kSweepRowBytes = 128u << 10; // of LDS for the tile's rows
 constexpr uint32_t kSweepPtrWords = 6148;       // nb * G + 1 range bounds of a tile, in LDS too
@@ -1187,21 +1190,22 @@ sweep_sddmm_kernel(const uint32_t *__restrict__ ptr, const uint32_t *__restrict_
         x.val = (wlane && uo < x.n) ? nt_load(sval + q + uo) : (T)0;
         return x;
     };
-    uint32_t p = lptr[grp], hi = lptr[grp + 1];
+    // batch i of a block's range belongs to lane group i % G
+    uint32_t p = lptr[0] + grp * UB, hi = lptr[G];
     SweepIdx<T> cur;
     if (p < hi)
         cur = fetch(p, hi);
     for (uint32_t b = 0; b < nb; ++b) {
         uint32_t p_nb = 0, hi_nb = 0; // the next block's range
         if (b + 1 < nb) {
-            p_nb = lptr[(b + 1) * G + grp];
-            hi_nb = lptr[(b + 1) * G + grp + 1];
+            p_nb = lptr[(b + 1) * G] + grp * UB;
+            hi_nb = lptr[(b + 2) * G];
         }
         const bool had = p < hi;
         while (p < hi) {
             // the next batch's indices (this block's, or the first of the next block) before
             // this batch's gathers
-            const uint32_t np = p + UB;
+            const uint32_t np = p + G * UB;
             SweepIdx<T> nxt;
             if (np < hi)
                 nxt = fetch(np, hi);
@@ -1263,8 +1267,8 @@ sweep_spmm_kernel(const uint32_t *__restrict__ ptr, const uint32_t *__restrict__
         x.val = nt_load(sval + q + e);
         return x;
     };
-    // The rows of this lane group are its own for the whole sweep: sums of a row's run of
-    // entries are kept in registers and added to the row's accumulator in LDS when the run
+    // Within a block the rows of this lane group's chunk are its own: the sum of a row's run
+    // of entries is kept in registers and added to the row's accumulator in LDS when the run
     // ends, in the plan's order: no atomics, the same bits run to run.
     uint32_t row = 0xFFFFFFFFu;
     V acc{};
@@ -1312,11 +1316,13 @@ sweep_spmm_kernel(const uint32_t *__restrict__ ptr, const uint32_t *__restrict__
         hi = hi_nb;
         if (!had && p < hi)
             cur = fetch(p, hi);
+        if (row != 0xFFFFFFFFu) { // in the next block the row may be another lane group's
+            tile_y[row * LPR + sub] += acc;
+            acc = V{};
+            row = 0xFFFFFFFFu;
+        }
         __syncthreads();
     }
-    if (row != 0xFFFFFFFFu)
-        tile_y[row * LPR + sub] += acc;
-    __syncthreads();
     for (uint32_t i = threadIdx.x; i < R * LPR; i += kSweepBlock) {
         const uint32_t g = tile_rows[(uint64_t)tile * R + i / LPR];
         if (g != 0xFFFFFFFFu) {

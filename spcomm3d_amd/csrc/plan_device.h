@@ -95,15 +95,15 @@ int build_store_staging(hipStream_t stream, const Seg *d_segs, uint32_t nseg, co
 
 // ---- row tiles x column blocks ("sweep") -------------------------------------------------
 // For long rows over columns without skew (see the sweep kernels in kernels.hip).  Rows of at
-// least min_row entries are ranked longest first and dealt to tiles of rows_per_tile rows,
-// the rows of rank j in a generation of per_launch tiles going to tile j % per_launch, so
-// that the tiles of a generation hold the same mix of lengths; local row l of a tile belongs
-// to lane group l % groups.  Their entries are sorted by (tile, column block, lane group,
-// local row), the caller's order kept inside a row's run; the entries of shorter rows follow
-// in the caller's order ("rest"; another plan runs them).
+// least min_row entries are ranked longest first; every per_launch * rows_per_tile of them
+// make a generation (one launch), inside which a tile takes rows_per_tile rows that are
+// consecutive by row number.  Their entries are sorted by (tile, column block, local row),
+// the caller's order kept inside a row's run, and every (tile, block) range is cut into
+// `groups` chunks at row boundaries, as equal as those allow; the entries of shorter rows
+// follow in the caller's order ("rest"; another plan runs them).
 //   perm[k]      caller's position of entry k of that order                [nnz]
 //   col, lrow    column and local row of sweep entry k                     [n]
-//   ptr          range bounds per (tile, block, group)                     [ntiles*nblocks*groups + 1]
+//   ptr          chunk bounds per (tile, block, group)                     [ntiles*nblocks*groups + 1]
 //   tile_rows    row of local row l of tile t, 0xFFFFFFFF where there is none [ntiles*rows_per_tile]
 // The arrays belong to the receiver (hipFree).  Synchronous.
 struct SweepPlan {

@@ -1493,23 +1493,6 @@ int build_two_pass(hipStream_t st, const uint32_t *d_perm, uint64_t nnz, uint32_
 }
 
 // ---- row tiles x column blocks ("sweep") ---------------------------------------------
-// Tile and local row of the row of rank j (longest first) among the nin rows of the sweep.
-__global__ void sweep_rows_k(const uint32_t *__restrict__ order, uint32_t nin, uint32_t P,
-                             uint32_t R, uint32_t *row_tile, uint32_t *row_local,
-                             uint32_t *tile_rows)
-{
-    GRID_STRIDE(j, nin)
-    {
-        const uint32_t row = order[j];
-        const uint64_t per_gen = (uint64_t)P * R;
-        const uint32_t gen = (uint32_t)(j / per_gen), jl = (uint32_t)(j % per_gen);
-        const uint32_t t = gen * P + jl % P, l = jl / P;
-        row_tile[row] = t;
-        row_local[row] = l;
-        tile_rows[(uint64_t)t * R + l] = row;
-    }
-}
-
 __global__ void sweep_hist_k(const uint32_t *__restrict__ ii, uint64_t nnz, uint32_t *rowcnt)
 {
     GRID_STRIDE(e, nnz) atomicAdd(&rowcnt[ii[e]], 1u);
@@ -1522,14 +1505,39 @@ __global__ void inverse_offsets_k(const uint32_t *__restrict__ perm, uint64_t n,
     GRID_STRIDE(q, n) out[perm[q]] = base + (uint32_t)q;
 }
 
-// Sort key of entry e: (tile, block, lane group, local row / groups); one past the largest
-// such key for an entry of a row outside the sweep (they sort last, in the caller's order).
+// key[j] = (generation of rank j) << 32 | row of rank j
+__global__ void sweep_gen_keys_k(const uint32_t *__restrict__ order, uint32_t nin, uint64_t per_gen,
+                                 unsigned long long *key)
+{
+    GRID_STRIDE(j, nin) key[j] = ((unsigned long long)(j / per_gen) << 32) | order[j];
+}
+
+// Tile and local row of the j-th row of the sweep (by generation, inside a generation by row
+// number): rpt consecutive rows make a tile (rpt_last in the last generation).
+__global__ void sweep_rows_k(const unsigned long long *__restrict__ gen_row, uint32_t nin,
+                             uint32_t P, uint32_t R, uint32_t last_gen, uint32_t rpt_last,
+                             uint32_t *row_tile, uint32_t *row_local, uint32_t *tile_rows)
+{
+    GRID_STRIDE(j, nin)
+    {
+        const uint32_t row = (uint32_t)gen_row[j];
+        const uint64_t per_gen = (uint64_t)P * R;
+        const uint32_t gen = (uint32_t)(j / per_gen), jl = (uint32_t)(j % per_gen);
+        const uint32_t rpt = gen == last_gen ? rpt_last : R;
+        const uint32_t t = gen * P + jl / rpt, l = jl % rpt;
+        row_tile[row] = t;
+        row_local[row] = l;
+        tile_rows[(uint64_t)t * R + l] = row;
+    }
+}
+
+// Sort key of entry e: (tile, block, local row); one past the largest such key for an entry
+// of a row outside the sweep (they sort last, in the caller's order).
 __global__ void sweep_keys_k(const uint32_t *__restrict__ ii, const uint32_t *__restrict__ jj,
                              uint64_t nnz, const uint32_t *__restrict__ row_tile,
                              const uint32_t *__restrict__ row_local, uint32_t block_cols,
-                             uint32_t nb, uint32_t G, uint32_t per_group,
-                             unsigned long long rest_key, unsigned long long *key,
-                             unsigned long long *nin)
+                             uint32_t nb, uint32_t R, unsigned long long rest_key,
+                             unsigned long long *key, unsigned long long *nin)
 {
     unsigned long long mine = 0;
     GRID_STRIDE(e, nnz)
@@ -1539,8 +1547,7 @@ __global__ void sweep_keys_k(const uint32_t *__restrict__ ii, const uint32_t *__
             key[e] = rest_key;
             continue;
         }
-        const uint32_t l = row_local[r], b = jj[e] / block_cols;
-        key[e] = (((unsigned long long)t * nb + b) * G + l % G) * per_group + l / G;
+        key[e] = ((unsigned long long)t * nb + jj[e] / block_cols) * R + row_local[r];
         ++mine;
     }
     mine = block_sum(mine);
@@ -1548,19 +1555,38 @@ __global__ void sweep_keys_k(const uint32_t *__restrict__ ii, const uint32_t *__
         atomicAdd(nin, mine);
 }
 
-// Of the sorted sweep entries: column, local row, and the (tile, block, group) bin.
+// Of the sorted sweep entries: column, local row, and the (tile, block) bin.
 __global__ void sweep_entries_k(const unsigned long long *__restrict__ skey,
                                 const uint32_t *__restrict__ perm,
-                                const uint32_t *__restrict__ jj, uint64_t n, uint32_t G,
-                                uint32_t per_group, uint32_t *col, uint16_t *lrow, uint32_t *bin)
+                                const uint32_t *__restrict__ jj, uint64_t n, uint32_t R,
+                                uint32_t *col, uint16_t *lrow, uint32_t *bin)
 {
     GRID_STRIDE(k, n)
     {
         const unsigned long long key = skey[k];
-        const unsigned long long b = key / per_group;
-        bin[k] = (uint32_t)b;
-        lrow[k] = (uint16_t)((uint32_t)(key % per_group) * G + (uint32_t)(b % G));
+        bin[k] = (uint32_t)(key / R);
+        lrow[k] = (uint16_t)(key % R);
         col[k] = jj[perm[k]];
+    }
+}
+
+// Chunk g of a bin starts at the first row boundary at or after the g-th G-th of its range.
+__global__ void sweep_chunks_k(const uint32_t *__restrict__ binptr, uint64_t nbins, uint32_t G,
+                               const uint16_t *__restrict__ lrow, uint32_t *ptr)
+{
+    GRID_STRIDE(i, nbins * G + 1)
+    {
+        if (i == nbins * G) {
+            ptr[i] = binptr[nbins];
+            continue;
+        }
+        const uint64_t bin = i / G;
+        const uint32_t g = (uint32_t)(i % G);
+        const uint32_t s = binptr[bin], e = binptr[bin + 1];
+        uint32_t q = s + (uint32_t)((uint64_t)(e - s) * g / G);
+        while (q > s && q < e && lrow[q] == lrow[q - 1])
+            ++q;
+        ptr[i] = q;
     }
 }
 
@@ -1572,16 +1598,15 @@ int build_sweep(hipStream_t st, uint32_t nrows, uint32_t ncols, uint64_t nnz, co
     if (nnz == 0 || nnz >= (1ull << 32) || lanes == 0 || R == 0 || R > 65536 || nb == 0 || P == 0)
         return SPC3D_OK;
     const uint32_t G = 1024 / lanes;
-    if (G == 0 || R % G != 0)
+    if (G == 0)
         return SPC3D_OK;
-    const uint32_t per_group = R / G;
     const uint32_t block_cols = (ncols + nb - 1) / nb;
     Arena arena;
-    HIP_OK(arena.reserve(((size_t)nrows + 1) * 28 + (size_t)nnz * 28 + ((size_t)8 << 20)));
+    HIP_OK(arena.reserve(((size_t)nrows + 1) * 40 + (size_t)nnz * 36 + ((size_t)8 << 20)));
     Temp tmp(arena);
     // ---- rows by length ----
     SBuf<uint32_t> rowcnt, rowid, order, cnt_sorted, row_tile, row_local;
-    SBuf<unsigned long long> total;
+    SBuf<unsigned long long> total, gkey, gkey_sorted;
     HIP_OK(rowcnt.alloc(arena, (size_t)nrows + 1));
     HIP_OK(rowid.alloc(arena, nrows));
     HIP_OK(order.alloc(arena, nrows));
@@ -1609,19 +1634,33 @@ int build_sweep(hipStream_t st, uint32_t nrows, uint32_t ncols, uint64_t nnz, co
         ++nin;
     if (nin == 0)
         return SPC3D_OK;
+    // A generation: the next P * R rows by length, which one launch of P tiles takes.  Inside
+    // a generation the rows are of similar length, and a tile takes R of them that are
+    // consecutive by row number: the tiles of a launch stay level to about a percent, and
+    // what a tile reads and writes (its rows of A or Y, its SDDMM results on their way to
+    // the caller's order) lies together.  The last generation spreads its rows over the P
+    // tiles.
     const uint64_t per_gen = (uint64_t)P * R;
     const uint64_t gens = (nin + per_gen - 1) / per_gen;
     const uint64_t last = nin - (gens - 1) * per_gen; // rows of the last generation
-    const uint64_t ntiles64 = (gens - 1) * P + std::min<uint64_t>(P, last);
+    const uint32_t rpt_last = (uint32_t)((last + P - 1) / P);
+    const uint64_t ntiles64 = (gens - 1) * P + (last + rpt_last - 1) / rpt_last;
     if (ntiles64 * nb * G + 1 >= (1ull << 32))
         return SPC3D_OK;
     const uint32_t ntiles = (uint32_t)ntiles64;
+    HIP_OK(gkey.alloc(arena, nin));
+    HIP_OK(gkey_sorted.alloc(arena, nin));
+    LAUNCH(sweep_gen_keys_k, nin, order.p, nin, per_gen, gkey.p);
+    // (values unused: cnt_sorted and rowid are free by now)
+    TRY(sort_pairs<unsigned long long>(tmp, gkey.p, gkey_sorted.p, rowid.p, cnt_sorted.p, nin,
+                                       32 + bits_for(gens), false, st, err));
     DBuf<uint32_t> tile_rows, perm, col, ptr;
     DBuf<uint16_t> lrow;
     HIP_OK(tile_rows.alloc((size_t)ntiles * R));
     HIP_OK(hipMemsetAsync(tile_rows.p, 0xFF, (size_t)ntiles * R * sizeof(uint32_t), st));
     HIP_OK(hipMemsetAsync(row_tile.p, 0xFF, (size_t)nrows * sizeof(uint32_t), st));
-    LAUNCH(sweep_rows_k, nin, order.p, nin, P, R, row_tile.p, row_local.p, tile_rows.p);
+    LAUNCH(sweep_rows_k, nin, gkey_sorted.p, nin, P, R, (uint32_t)(gens - 1), rpt_last, row_tile.p,
+           row_local.p, tile_rows.p);
     // ---- entries ----
     SBuf<unsigned long long> key, skey;
     SBuf<uint32_t> ident, bin;
@@ -1629,9 +1668,9 @@ int build_sweep(hipStream_t st, uint32_t nrows, uint32_t ncols, uint64_t nnz, co
     HIP_OK(skey.alloc(arena, nnz));
     HIP_OK(ident.alloc(arena, nnz));
     HIP_OK(perm.alloc(nnz));
-    const unsigned long long rest_key = (unsigned long long)ntiles * nb * G * per_group;
-    LAUNCH_SMALL(sweep_keys_k, nnz, d_ii, d_jj, nnz, row_tile.p, row_local.p, block_cols, nb, G,
-                 per_group, rest_key, key.p, total.p);
+    const unsigned long long rest_key = (unsigned long long)ntiles * nb * R;
+    LAUNCH_SMALL(sweep_keys_k, nnz, d_ii, d_jj, nnz, row_tile.p, row_local.p, block_cols, nb, R,
+                 rest_key, key.p, total.p);
     LAUNCH(iota_k, nnz, ident.p, nnz);
     TRY(sort_pairs<unsigned long long>(tmp, key.p, skey.p, ident.p, perm.p, (uint32_t)nnz,
                                        bits_for(rest_key), false, st, err));
@@ -1642,16 +1681,18 @@ int build_sweep(hipStream_t st, uint32_t nrows, uint32_t ncols, uint64_t nnz, co
     HIP_OK(col.alloc(n));
     HIP_OK(lrow.alloc(n));
     HIP_OK(bin.alloc(arena, n));
-    const uint64_t nbins = (uint64_t)ntiles * nb * G;
-    HIP_OK(ptr.alloc(nbins + 1));
-    SBuf<uint32_t> bstart, bcnt;
+    const uint64_t nbins = (uint64_t)ntiles * nb;
+    HIP_OK(ptr.alloc(nbins * G + 1));
+    SBuf<uint32_t> bstart, bcnt, binptr;
     HIP_OK(bstart.alloc(arena, nbins));
     HIP_OK(bcnt.alloc(arena, nbins + 1));
+    HIP_OK(binptr.alloc(arena, nbins + 1));
     HIP_OK(hipMemsetAsync(bcnt.p, 0, (nbins + 1) * sizeof(uint32_t), st));
-    LAUNCH(sweep_entries_k, n, skey.p, perm.p, d_jj, n, G, per_group, col.p, lrow.p, bin.p);
+    LAUNCH(sweep_entries_k, n, skey.p, perm.p, d_jj, n, R, col.p, lrow.p, bin.p);
     LAUNCH(run_bounds_k, n, bin.p, n, (uint32_t)nbins, bstart.p, bcnt.p);
     LAUNCH(run_lengths_k, nbins, bstart.p, nbins, bcnt.p);
-    TRY(exclusive_sum(tmp, bcnt.p, ptr.p, (size_t)nbins + 1, st, err));
+    TRY(exclusive_sum(tmp, bcnt.p, binptr.p, (size_t)nbins + 1, st, err));
+    LAUNCH(sweep_chunks_k, nbins * G + 1, binptr.p, nbins, G, lrow.p, ptr.p);
     HIP_OK(hipGetLastError());
     HIP_OK(hipStreamSynchronize(st));
     out.perm = perm.release();
