@@ -160,6 +160,10 @@ typedef struct {
                               an ordinary plan.  Such a plan runs at K = k_hint only (other
                               calls return SPC3D_ERR_INVALID_ARG), spc3d_spmm adds a row's
                               entries block after block, and runs give the same bits.
+                              spc3d_sddmm stores the tiles' results straight to the caller's
+                              positions when four in five of them follow their predecessor
+                              there (a row's entries together), else through a staging vector
+                              (spc3d_plan_info.staged_entries).
                               0 (default): as described; 1: never; 2: whenever k_hint has such
                               a width, whatever the pattern (col_blocks, if given, is the
                               number of blocks) */
@@ -177,7 +181,11 @@ typedef struct {
 #define SPC3D_PLAN_NO_SDDMM_BY_COLUMN 2u
 #define SPC3D_PLAN_NO_TWO_PASS 4u
 #define SPC3D_PLAN_KEEP_ENTRY_ORDER 8u
-#define SPC3D_PLAN_ALL_FLAGS 15u
+/* Row tiles (sweep): stage the tiles' SDDMM results in kernel order and bring them home in
+ * one more pass also when the caller's order keeps a row's entries together (by default the
+ * tile kernels then store straight to the caller's positions, and nothing is staged). */
+#define SPC3D_PLAN_SWEEP_STAGED 16u
+#define SPC3D_PLAN_ALL_FLAGS 31u
 
 /* ---- library / errors ------------------------------------------------- */
 SPC3D_API const char *spc3d_version(void);

@@ -797,6 +797,14 @@ int spc3d_sddmm(spc3d_ctx *ctx, spc3d_plan *S, const spc3d_panel *A, const spc3d
     rc = sweep_check(S, K);
     if (rc)
         return rc;
+    if (S->sweep.n && !S->c_stage) { // the tiles and the rest store at the caller's positions
+        for (spc3d_plan *part : S->blocks)
+            HIP_TRY(launch_sddmm(S->dtype, view_of(part), A->dev, B->dev, C->dev, K, streams_of(ctx)));
+        SweepView v = sweep_view_of(S);
+        v.pos = S->sweep.perm;
+        HIP_TRY(launch_sweep_sddmm(S->dtype, v, A->dev, B->dev, C->dev, ctx->stream));
+        return SPC3D_OK;
+    }
     for (spc3d_plan *part : S->blocks)
         HIP_TRY(launch_sddmm(S->dtype, staged_view(S, part), A->dev, B->dev, staged_out(S, part), K,
                              streams_of(ctx)));
@@ -936,7 +944,8 @@ int spc3d_sddmm_spmm(spc3d_ctx *ctx, spc3d_plan *S, const spc3d_panel *A, const 
         if (rc)
             return rc;
     }
-    const bool staged = !S->blocks.empty() || S->sweep.n;
+    const bool direct = S->sweep.n && !S->c_stage; // results straight to the caller's positions
+    const bool staged = (!S->blocks.empty() || S->sweep.n) && !direct;
     for (spc3d_plan *part : parts_of(S, self)) {
         const DevPlanView view = staged ? staged_view(S, part) : view_of(part);
         void *out = staged ? staged_out(S, part) : sddmm_out(S, C->dev);
@@ -958,11 +967,18 @@ int spc3d_sddmm_spmm(spc3d_ctx *ctx, spc3d_plan *S, const spc3d_panel *A, const 
     if (S->sweep.n) { // the tiles: SDDMM, then SpMM over the same entries (with the results
                       // just written as its values when chained)
         SweepView v = sweep_view_of(S);
-        HIP_TRY(launch_sweep_sddmm(S->dtype, v, A->dev, B->dev, S->c_stage, ctx->stream));
+        if (direct)
+            v.pos = S->sweep.perm;
+        HIP_TRY(launch_sweep_sddmm(S->dtype, v, A->dev, B->dev, direct ? C->dev : S->c_stage,
+                                   ctx->stream));
         if (chained)
-            v.sval = S->c_stage;
+            v.sval = direct ? C->dev : S->c_stage; // (through v.pos when direct)
+        else
+            v.pos = nullptr;
         HIP_TRY(launch_sweep_spmm(S->dtype, v, B->dev, Y->dev, ctx->stream));
     }
+    if (direct)
+        return SPC3D_OK;
     if (staged)
         HIP_TRY(unstage(S, C));
     else

@@ -396,10 +396,12 @@ static void choose_sweep(const spc3d_plan *p, const spc3d_plan_opts *opts, uint3
         return; // a caller's own block count means blocks
     uint64_t nb = forced && opts->col_blocks > 1 ? opts->col_blocks : 0;
     if (!nb) {
-        // 2.5 MiB of dense rows per block: of 96, 128 and 192 blocks over a 244 MiB panel, 96
-        // were the fastest (5.2 / 5.1 ms against 5.4 / 5.8 ms at 192 on a 143 M-entry pattern)
+        // 3.25 MiB of dense rows per block: on a 244 MiB panel (572 M entries, 512-byte rows)
+        // 64 to 78 blocks measured level (19.7 .. 20.5 ms SDDMM, 20.2 .. 20.4 ms SpMM), 48 and
+        // 128 half a millisecond to a millisecond slower, 192 three slower in SpMM
+        constexpr uint64_t kBlockBytes = (uint64_t)13 << 18;
         const uint64_t panel = (uint64_t)p->info.cols_touched * opts->k_hint * elem_size(p->dtype);
-        nb = std::max<uint64_t>(1, (panel + ((uint64_t)5 << 19) - 1) / ((uint64_t)5 << 19));
+        nb = std::max<uint64_t>(1, (panel + kBlockBytes - 1) / kBlockBytes);
     }
     nb = std::min<uint64_t>(nb, std::min<uint32_t>(sweep_max_blocks(l), p->info.ncols));
     *lanes = l;
@@ -464,10 +466,22 @@ static int rebuild_as_sweep(spc3d_plan *p, uint32_t nrows, uint32_t ncols, uint6
             child->info.order_is_identity = 0;
         }
     }
-    if (!rc) rc = dev_alloc_bytes(&c_stage, (size_t)(rest_off + nrest) * w);
-    if (!rc) rc = dev_alloc(&stage_pos, (size_t)nnz);
+    // Where the tiles' SDDMM results go: in a tile's kernel order a row's entries of one
+    // block follow each other; when the caller's order keeps them together too, the kernel
+    // stores them straight to their places (pieces of lines that the same workgroup completes
+    // a few blocks later), else in kernel order to a staging vector that one more pass reads.
+    bool staged = (opts->flags & SPC3D_PLAN_SWEEP_STAGED) != 0;
+    if (!rc && !staged) {
+        uint64_t adjacent = 0;
+        rc = count_adjacent_device(ctx->stream, sw.perm, sw.n, &adjacent, err);
+        if (rc)
+            fail(rc, err);
+        staged = adjacent * 5 < sw.n * 4;
+    }
+    if (!rc && staged) rc = dev_alloc_bytes(&c_stage, (size_t)(rest_off + nrest) * w);
+    if (!rc && staged) rc = dev_alloc(&stage_pos, (size_t)nnz);
     if (!rc) rc = dev_alloc_bytes(&sval, (size_t)sw.n * w);
-    if (!rc) {
+    if (!rc && staged) {
         rc = inverse_offsets_device(ctx->stream, sw.perm, sw.n, 0, stage_pos, err);
         if (!rc && nrest)
             rc = inverse_offsets_device(ctx->stream, child->perm, nrest, (uint32_t)rest_off, stage_pos, err);
@@ -528,6 +542,7 @@ static int rebuild_as_sweep(spc3d_plan *p, uint32_t nrows, uint32_t ncols, uint6
     p->c_stage = c_stage;
     p->stage_pos = stage_pos;
     I.ncol_blocks = sw.nblocks;
+    I.staged_entries = staged ? sw.n : 0;
     I.sweep_entries = sw.n;
     I.sweep_tiles = sw.ntiles;
     I.sweep_k = opts->k_hint;
@@ -1111,7 +1126,8 @@ static uint64_t own_device_bytes(const spc3d_plan *p)
         b += n * (4 + 2 + w) + nnz * 4; // col, lrow, values; perm
         b += ((uint64_t)p->sweep.ntiles * p->sweep.nblocks * p->sweep.groups + 1) * 4;
         b += (uint64_t)p->sweep.ntiles * p->sweep.rows_per_tile * 4;
-        b += ((n + 63) / 64 * 64 + rest) * w + nnz * 4; // c_stage, stage_pos
+        if (p->c_stage)
+            b += ((n + 63) / 64 * 64 + rest) * w + nnz * 4; // c_stage, stage_pos
     } else if (!p->blocks.empty()) {
         b += nnz * (w + 8); // c_stage, stage_pos, stage_of
     }

@@ -67,6 +67,9 @@ struct SweepView {
     const uint32_t *col = nullptr;       // [n] sweep order
     const uint16_t *lrow = nullptr;      // [n] local row in the tile
     const void *sval = nullptr;          // [n] values in sweep order
+    // [n] or null.  SDDMM: where result k goes in C (null: C[k]).  SpMM: value k is
+    // sval[pos[k]] (null: sval[k]).
+    const uint32_t *pos = nullptr;
     uint32_t ntiles = 0, nblocks = 0, rows_per_tile = 0;
     uint32_t lanes = 0;                  // lanes per dense row the plan was made for: 16, 32 or 64
     uint32_t per_launch = 0;             // tiles per generation (the GPU's CU count)

@@ -1150,7 +1150,7 @@ __device__ __forceinline__ T sweep_dot(const typename Vec<T>::type &a, const typ
 // One batch of a lane group: its entries' columns, local rows and (for the lanes that need
 // one) sparse values, asked for one batch ahead.
 template <typename T> struct SweepIdx {
-    uint32_t n = 0, col = 0, row = 0;
+    uint32_t n = 0, col = 0, row = 0, pos = 0;
     T val = (T)0;
 };
 
@@ -1158,8 +1158,9 @@ template <typename T, int LPR, int UB>
 __global__ void __launch_bounds__(kSweepBlock)
 sweep_sddmm_kernel(const uint32_t *__restrict__ ptr, const uint32_t *__restrict__ tile_rows,
                    const uint32_t *__restrict__ col, const uint16_t *__restrict__ lrow,
-                   const T *__restrict__ sval, const T *__restrict__ A, const T *__restrict__ B,
-                   T *__restrict__ C, uint32_t nb, uint32_t R, uint32_t tile0)
+                   const T *__restrict__ sval, const uint32_t *__restrict__ pos,
+                   const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C, uint32_t nb,
+                   uint32_t R, uint32_t tile0)
 {
     using V = typename Vec<T>::type;
     constexpr uint32_t G = kSweepBlock / LPR;
@@ -1188,6 +1189,8 @@ sweep_sddmm_kernel(const uint32_t *__restrict__ ptr, const uint32_t *__restrict_
         x.col = nt_load(col + q + e);
         x.row = nt_load(lrow + q + e);
         x.val = (wlane && uo < x.n) ? nt_load(sval + q + uo) : (T)0;
+        if (pos)
+            x.pos = (wlane && uo < x.n) ? nt_load(pos + q + uo) : 0u;
         return x;
     };
     // batch i of a block's range belongs to lane group i % G
@@ -1225,8 +1228,13 @@ sweep_sddmm_kernel(const uint32_t *__restrict__ ptr, const uint32_t *__restrict_
                 part[u] = sweep_dot<T, LPR>(tile_a[l * LPR + sub], bv[u]);
             }
             group_reduce<T, LPR, UB>(part, sub);
-            if (wlane && uo < cur.n)
-                nt_store(part[0] * cur.val, C + p + uo); // kernel order: whole lines, streaming
+            if (wlane && uo < cur.n) {
+                if (pos) // the caller's positions: pieces of lines that this workgroup's next
+                         // blocks complete, so plain stores, which the L2 merges
+                    C[cur.pos] = part[0] * cur.val;
+                else
+                    nt_store(part[0] * cur.val, C + p + uo); // kernel order: whole lines, streaming
+            }
             p = np;
             cur = nxt;
         }
@@ -1242,8 +1250,8 @@ template <typename T, int LPR, int UB>
 __global__ void __launch_bounds__(kSweepBlock)
 sweep_spmm_kernel(const uint32_t *__restrict__ ptr, const uint32_t *__restrict__ tile_rows,
                   const uint32_t *__restrict__ col, const uint16_t *__restrict__ lrow,
-                  const T *__restrict__ sval, const T *__restrict__ X, T *__restrict__ Y,
-                  uint32_t nb, uint32_t R, uint32_t tile0)
+                  const T *__restrict__ sval, const uint32_t *__restrict__ vpos,
+                  const T *__restrict__ X, T *__restrict__ Y, uint32_t nb, uint32_t R, uint32_t tile0)
 {
     using V = typename Vec<T>::type;
     constexpr uint32_t G = kSweepBlock / LPR;
@@ -1264,7 +1272,7 @@ sweep_spmm_kernel(const uint32_t *__restrict__ ptr, const uint32_t *__restrict__
         e = e < x.n ? e : x.n - 1;
         x.col = nt_load(col + q + e);
         x.row = nt_load(lrow + q + e);
-        x.val = nt_load(sval + q + e);
+        x.val = vpos ? sval[nt_load(vpos + q + e)] : nt_load(sval + q + e);
         return x;
     };
     // Within a block the rows of this lane group's chunk are its own: the sum of a row's run
@@ -2028,12 +2036,12 @@ void sweep_launch(bool spmm, const SweepView &S, const T *A, const T *B, T *out,
 {
     if (spmm)
         hipLaunchKernelGGL((sweep_spmm_kernel<T, LPR, 16>), dim3(ntiles), dim3(kSweepBlock), 0,
-                           stream, S.ptr, S.tile_rows, S.col, S.lrow, (const T *)S.sval, B, out,
-                           S.nblocks, S.rows_per_tile, tile0);
+                           stream, S.ptr, S.tile_rows, S.col, S.lrow, (const T *)S.sval, S.pos, B,
+                           out, S.nblocks, S.rows_per_tile, tile0);
     else
         hipLaunchKernelGGL((sweep_sddmm_kernel<T, LPR, 16>), dim3(ntiles), dim3(kSweepBlock), 0,
-                           stream, S.ptr, S.tile_rows, S.col, S.lrow, (const T *)S.sval, A, B, out,
-                           S.nblocks, S.rows_per_tile, tile0);
+                           stream, S.ptr, S.tile_rows, S.col, S.lrow, (const T *)S.sval, S.pos, A,
+                           B, out, S.nblocks, S.rows_per_tile, tile0);
 }
 template <typename T>
 hipError_t sweep_run(bool spmm, const SweepView &S, const T *A, const T *B, T *out, hipStream_t stream)

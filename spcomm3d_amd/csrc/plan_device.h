@@ -117,6 +117,9 @@ int build_sweep(hipStream_t stream, uint32_t nrows, uint32_t ncols, uint64_t nnz
                 const uint32_t *d_ii, const uint32_t *d_jj, uint32_t lanes, uint32_t rows_per_tile,
                 uint32_t nblocks, uint32_t min_row, uint32_t per_launch, SweepPlan &out,
                 std::string &err);
+// *out = how many q < n - 1 have d[q + 1] == d[q] + 1.  Synchronous.
+int count_adjacent_device(hipStream_t stream, const uint32_t *d, uint64_t n, uint64_t *out,
+                          std::string &err);
 // d_out[d_perm[q]] = base + q, q < n.  Asynchronous on `stream`.
 int inverse_offsets_device(hipStream_t stream, const uint32_t *d_perm, uint64_t n, uint32_t base,
                            uint32_t *d_out, std::string &err);

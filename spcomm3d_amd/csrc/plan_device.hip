@@ -1711,6 +1711,22 @@ int build_sweep(hipStream_t st, uint32_t nrows, uint32_t ncols, uint64_t nnz, co
     return SPC3D_OK;
 }
 
+int count_adjacent_device(hipStream_t st, const uint32_t *d, uint64_t n, uint64_t *out,
+                          std::string &err)
+{
+    *out = 0;
+    if (n < 2)
+        return SPC3D_OK;
+    DBuf<unsigned long long> acc;
+    HIP_OK(acc.alloc(1));
+    HIP_OK(hipMemsetAsync(acc.p, 0, sizeof(unsigned long long), st));
+    LAUNCH_SMALL(adjacent_k, n, d, n, acc.p);
+    unsigned long long seen = 0;
+    TRY(fetch(st, &seen, acc.p, sizeof seen, err));
+    *out = seen;
+    return SPC3D_OK;
+}
+
 int inverse_offsets_device(hipStream_t st, const uint32_t *d_perm, uint64_t n, uint32_t base,
                            uint32_t *d_out, std::string &err)
 {

@@ -12,14 +12,14 @@ pytestmark = pytest.mark.gpu
 TOL = {np.dtype(np.float32): 1e-5, np.dtype(np.float64): 1e-12}
 
 
-def long_rows(seed, m, n, k, dtype, lens):
+def long_rows(seed, m, n, k, dtype, lens, shuffle=True):
     """Rows of the given lengths over uniform columns (repeats allowed), in a shuffled
-    order, with values and panels."""
+    order or sorted by row and column, with values and panels."""
     rng = np.random.default_rng(seed)
     lens = np.asarray(lens, dtype=np.int64)
     ii = np.repeat(np.arange(m, dtype=np.uint32), lens)
     jj = rng.integers(0, n, ii.size).astype(np.uint32)
-    o = rng.permutation(ii.size)
+    o = rng.permutation(ii.size) if shuffle else np.lexsort((jj, ii))  # or by row, then column
     ii, jj = np.ascontiguousarray(ii[o]), np.ascontiguousarray(jj[o])
     vv = rng.random(ii.size).astype(dtype)
     A = rng.uniform(-1, 1, (m, k)).astype(dtype)
@@ -65,21 +65,30 @@ def check(out, ii, jj, vv, A, B, Y0):
     assert oracle.spmm_rel_err(B, ii, jj, out["C"], Y0, out["Y_chain"]) <= tol
 
 
+@pytest.mark.parametrize("shuffle", [True, False])
 @pytest.mark.parametrize("dtype,k", [(np.float32, 64), (np.float32, 128), (np.float32, 256),
                                      (np.float64, 32), (np.float64, 64), (np.float64, 128)])
-def test_tiles_and_rest_against_the_oracle(ctx, dtype, k):
+def test_tiles_and_rest_against_the_oracle(ctx, dtype, k, shuffle):
     rng = np.random.default_rng(k)
     m, n = 700, 3000
     lens = rng.integers(0, 400, m)
     lens[::7] = rng.integers(1, 12, lens[::7].size)  # short rows: the plan of the rest
     lens[5] = 0
     lens[11] = 5000                                  # more entries than columns
-    case = long_rows(1000 + k, m, n, k, dtype, lens)
+    case = long_rows(1000 + k, m, n, k, dtype, lens, shuffle)
     ii, jj, vv, A, B, Y0 = case
     out, info = run_all(ctx, m, n, *case, k_hint=k, sweep=True, sweep_min_row=12, col_blocks=7)
     assert info.sweep_k == k and info.sweep_tiles > 0 and info.ncol_blocks == 7
     want = int(lens[lens >= 12].sum())
     assert info.sweep_entries == want and info.nsegments > 0
+    # sorted, the tiles store straight to the caller's positions; shuffled, they stage
+    assert info.staged_entries == (want if shuffle else 0)
+    if not shuffle:
+        forced, finfo = run_all(ctx, m, n, *case, k_hint=k, sweep=True, sweep_min_row=12,
+                                col_blocks=7, sweep_staged=True)
+        assert finfo.staged_entries == want
+        for name in out:
+            assert np.array_equal(out[name], forced[name]), name
     assert info.device_bytes > ii.size * 10
     check(out, *case)
     # against the ordinary plan: the same products, another summation order
