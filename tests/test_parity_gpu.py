@@ -692,8 +692,12 @@ def test_column_blocks_are_chosen_for_long_rows_over_a_wide_unskewed_panel(ctx):
     # mean: the rule picks blocks; R-MAT (skewed columns) and short rows stay whole
     w = W.hypergraph_zipf(3000, 140_000, 128)
     vv = w.values("f32")
-    S = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, vv, k_hint=w.k)
+    S = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, vv, k_hint=w.k, sweep=False)
     assert 12 <= S.info.ncol_blocks <= 14 and S.info.nqueues == 1, S.info.ncol_blocks
+    # 512-byte rows are a width the row-tile kernels take: by default the long rows go there
+    T = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, vv, k_hint=w.k)
+    assert T.info.sweep_entries > w.nnz // 2 and 20 <= T.info.ncol_blocks <= 22
+    T.close()
     whole = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, vv, k_hint=w.k, col_blocks=1)
     assert whole.info.ncol_blocks == 1
     A, B, Y0 = w.panel_A("f32"), w.panel_B("f32"), w.panel_Y0("f32")
@@ -732,14 +736,23 @@ def test_panel_copy_on_device(ctx, shape):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("col_blocks", [None, 3])
+@pytest.mark.parametrize("col_blocks", [None, 3, "tiles"])
 def test_probe_columns_keeps_the_launches_and_moves_the_gathers(ctx, dtype, col_blocks):
     """spc3d_plan_probe_columns (a measurement aid): after the all-hit rewrite the plan
     computes the pattern (ii, c % modulus inside the entry's block of columns), entry by
     entry at the caller's positions; after the all-miss one every column is in range."""
     w = W.rmat(12, 16, 32).shuffled()
     vv, A, B, Y0 = w.values(dtype), w.panel_A(dtype), w.panel_B(dtype), w.panel_Y0(dtype)
-    S = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, vv, k_hint=w.k, col_blocks=col_blocks)
+    if col_blocks == "tiles":  # row tiles for the rows of 8 entries and more, in 3 blocks:
+        # one range of columns for every block, in the tiles and in the plan of the rest
+        w = W.rmat(12, 16, 64).shuffled()
+        vv, A, B, Y0 = w.values(dtype), w.panel_A(dtype), w.panel_B(dtype), w.panel_Y0(dtype)
+        S = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, vv, k_hint=w.k, sweep=True, sweep_min_row=8,
+                     col_blocks=3)
+        assert 0 < S.info.sweep_entries < w.nnz
+        col_blocks = None
+    else:
+        S = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, vv, k_hint=w.k, col_blocks=col_blocks)
     dA, dB, dY, dC = ctx.panel_from(A), ctx.panel_from(B), ctx.panel_from(Y0), ctx.vals(w.nnz, dtype)
     modulus = 61
     S.probe_columns("all_hit", modulus)
