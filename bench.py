@@ -54,6 +54,14 @@ TRAFFIC_LEVEL = "l2_fabric (FETCH_SIZE x 2 + WRITE_SIZE: fills and write-backs o
 TRAFFIC_WORKLOAD = ("rmat20_ef16", 64, "sorted")
 
 
+def traffic_is_current(path=TRAFFIC_PROFILE):
+    """True when the traffic profile was recorded on the device code that is in the tree
+    now (the digest in its header against the sources')."""
+    from spcomm3d_amd import provenance
+
+    return provenance.recorded_hash(path) == provenance.source_hash()
+
+
 def measured_traffic(path=TRAFFIC_PROFILE):
     """{(dtype, call): bytes} from the 'Per call' table of the traffic profile."""
     import re
@@ -74,6 +82,19 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
+# Plan options of the main workload's plans beside k_hint (--col-blocks, --sweep): for the
+# comparisons the profile summaries hold; the default run passes none.
+PLAN_OPTS: dict = {}
+
+
+def plan_opts(w):
+    """k_hint when the workload's K is not the library's default of 64 (the plan sizes its
+    L2-resident set, and chooses column blocks / row tiles, for the width it is told), an
+    explicit one whenever other options are given."""
+    hint = {} if w.k == 64 and not PLAN_OPTS else {"k_hint": w.k}
+    return dict(hint, **PLAN_OPTS)
+
+
 def ensure_built():
     need = ["spcomm3d_amd/lib/libspcomm3d_hip.so", "spcomm3d_amd/gen/libspc3d_gen.so"]
     if not all(os.path.exists(os.path.join(ROOT, p)) for p in need):
@@ -91,9 +112,7 @@ def run_gpu(w, dtype, steps, warmup, seg_max=None, max_timed=1300, copies=0):
     A, B, Y0, vv = w.panel_A(dtype), w.panel_B(dtype), w.panel_Y0(dtype), w.values(dtype)
     with device.Context(0) as ctx:
         t0 = time.perf_counter()
-        # the plan sizes its L2-resident set for K = 64 unless told the width it will run with
-        hint = {} if w.k == 64 else {"k_hint": w.k}
-        S = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, vv, seg_max=seg_max, **hint)
+        S = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, vv, seg_max=seg_max, **plan_opts(w))
         ctx.sync()
         plan_s = time.perf_counter() - t0
         info = S.info
@@ -190,7 +209,9 @@ def run_gpu(w, dtype, steps, warmup, seg_max=None, max_timed=1300, copies=0):
     with_perm = not info.order_is_identity
     fl = roofline.flops(w.nnz, w.k)
     out = {"dtype": dtype, "ms_per_step": wall / steps * 1e3, "plan_build_s": plan_s,
-           "plan_device_bytes": int(info.device_bytes),
+           "plan_device_bytes": int(info.device_bytes), "col_blocks": int(info.ncol_blocks),
+           "sweep_entries": int(info.sweep_entries), "sweep_tiles": int(info.sweep_tiles),
+           "staged_entries": int(info.staged_entries),
            "upload_s": upload_s, "nsegments": info.nsegments, "nsplit_rows": info.nsplit_rows,
            "seg_max": info.seg_max, "rows_touched": m_t, "cols_touched": n_t,
            "gflops": 2 * fl / (wall / steps) / 1e9, "kernels": {}}
@@ -230,8 +251,8 @@ def run_floors(w, dtype, steps, warmup, seg_max=None):
     modulus = max(64, (1 << 20) // (w.k * wbytes))
     out = {"dtype": dtype, "all_hit_table_rows": modulus, "steps": steps}
     with device.Context(0) as ctx:
-        hint = {} if w.k == 64 else {"k_hint": w.k}
-        S = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, w.values(dtype), seg_max=seg_max, **hint)
+        S = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, w.values(dtype), seg_max=seg_max,
+                     **plan_opts(w))
         dA, dB = ctx.panel_from(w.panel_A(dtype)), ctx.panel_from(w.panel_B(dtype))
         dY = ctx.panel_from(w.panel_Y0(dtype))
         dC = ctx.vals(w.nnz, dtype)
@@ -333,6 +354,7 @@ def run_compact(w, dtype, steps, warmup):
             "sddmm_strict_bytes": int(sd_b), "spmm_strict_bytes": int(sp_b),
             "rows_touched": m_t, "cols_touched": n_t,
             "plan_device_bytes": int(info.device_bytes), "col_blocks": int(info.ncol_blocks),
+            "sweep_entries": int(info.sweep_entries),
             "gflops": 2 * fl / (sd_ms + sp_ms) / 1e6, "plan_build_s": plan_s}
 
 
@@ -426,6 +448,14 @@ def main():
     ap.add_argument("--order", default="sorted", choices=["sorted", "shuffled", "column-major"],
                     help="order in which the COO entries are handed to the library")
     ap.add_argument("--seg-max", type=int, default=None)
+    ap.add_argument("--localized", action="store_true",
+                    help="the workload at the shape a rank of the reference runs it on: local "
+                         "indices in first-appearance order, panels of the touched rows / "
+                         "columns only")
+    ap.add_argument("--col-blocks", type=int, default=None,
+                    help="spc3d_plan_opts.col_blocks of the main workload's plan")
+    ap.add_argument("--sweep", default=None, choices=["off", "on"],
+                    help="spc3d_plan_opts.sweep of the main workload's plan (row tiles)")
     ap.add_argument("--calibration-copies", type=int, default=0,
                     help="also launch this many plain device copies of an m x K panel "
                          "(a known-size dispatch for counter calibration)")
@@ -452,6 +482,12 @@ def main():
         w = w.shuffled()
     elif args.order == "column-major":
         w = w.column_major()
+    if args.localized:
+        w = w.localized()
+    if args.col_blocks is not None:
+        PLAN_OPTS["col_blocks"] = args.col_blocks
+    if args.sweep is not None:
+        PLAN_OPTS["sweep"] = args.sweep == "on"
     log(f"workload {w.name}: {w.nrows}x{w.ncols} nnz={w.nnz} K={w.k} order={w.order} "
         f"(generated in {time.perf_counter() - t0:.1f}s)")
 
@@ -538,9 +574,14 @@ def main():
     from spcomm3d_amd import roofline
 
     traffic = None
-    if (args.seg_max is None and not any(k.startswith("SPC3D_") for k in os.environ)
+    traffic_stale = False
+    if (args.seg_max is None and not PLAN_OPTS
+            and not any(k.startswith("SPC3D_") for k in os.environ)
             and (w.name, w.k, w.order) == TRAFFIC_WORKLOAD):
-        traffic = measured_traffic().get((args.dtype, dom))
+        if traffic_is_current():
+            traffic = measured_traffic().get((args.dtype, dom))
+        else:  # recorded on other device code than this: not this code's traffic
+            traffic_stale = True
 
     line = {
         "metric": METRIC, "value": main_r["gflops"], "unit": "GFLOP/s", "n_gpus": 1,
@@ -552,7 +593,8 @@ def main():
                    "rows_touched": main_r["rows_touched"], "cols_touched": main_r["cols_touched"]},
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": kd["strict_gbs"],
                      "peak": roofline.HBM_PEAK_GBS, "unit": "GB/s", "frac": kd["strict_frac"],
-                     "traffic": traffic, "traffic_level": TRAFFIC_LEVEL,
+                     "traffic": traffic, "traffic_stale": traffic_stale,
+                     "traffic_level": TRAFFIC_LEVEL,
                      "traffic_source": os.path.relpath(TRAFFIC_PROFILE, ROOT),
                      "traffic_gbs": None if traffic is None else traffic / kd["ms_avg"] / 1e6,
                      "device_copy_gbs": main_r["device_copy_gbs"],
@@ -572,7 +614,8 @@ def main():
         "dist_step": dist_step,
         "row_copies": main_r["row_copies"],
         "plan": {k: main_r[k] for k in ("plan_build_s", "upload_s", "nsegments", "nsplit_rows",
-                                        "seg_max", "plan_device_bytes")},
+                                        "seg_max", "plan_device_bytes", "col_blocks",
+                                        "sweep_entries", "sweep_tiles", "staged_entries")},
         "also": also,
     }
     print(json.dumps(line), flush=True)

@@ -79,6 +79,37 @@ def test_traffic_in_the_bench_line_is_what_the_profile_summary_holds():
     assert "l2_fabric" in bench.TRAFFIC_LEVEL
 
 
+def test_profiles_were_recorded_on_the_device_code_in_the_tree():
+    """Every summary under profiles/ names the digest of the device sources it was recorded
+    on; a change to those sources makes the summaries stale, this test fail and bench.py
+    report `traffic: null, traffic_stale: true` until they are recorded again."""
+    sys.path.insert(0, ROOT)
+    import bench
+    from spcomm3d_amd import provenance
+
+    now = provenance.source_hash()
+    names = sorted(n for n in os.listdir(os.path.join(ROOT, "profiles")) if n.endswith(".md"))
+    assert names
+    stale = [n for n in names
+             if provenance.recorded_hash(os.path.join(ROOT, "profiles", n)) != now]
+    assert not stale, f"recorded on other sources than {now}: {stale}"
+    assert bench.traffic_is_current()
+
+
+def test_a_stale_profile_is_not_quoted(tmp_path):
+    sys.path.insert(0, ROOT)
+    import bench
+
+    text = open(bench.TRAFFIC_PROFILE).read()
+    old = tmp_path / "traffic.md"
+    old.write_text(text.replace("Source hash: `", "Source hash: `0"))
+    assert bench.measured_traffic(str(old))  # the table still parses
+    assert not bench.traffic_is_current(str(old))
+    none = tmp_path / "none.md"
+    none.write_text("# no digest in here\n")
+    assert not bench.traffic_is_current(str(none))
+
+
 @pytest.mark.gpu
 def test_bench_line_has_the_contract_fields():
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--config", "er16k",
@@ -95,8 +126,8 @@ def test_bench_line_has_the_contract_fields():
         assert k in d, k
     assert d["n_gpus"] == 1 and d["steps"] == 5 and d["vs_baseline"] is None
     assert d["dtype"] == "f64" and "workload" in d["config"]
-    assert set(("bound", "achieved", "peak", "unit", "frac", "traffic", "traffic_level")) <= \
-        set(d["roofline"])
+    assert set(("bound", "achieved", "peak", "unit", "frac", "traffic", "traffic_stale",
+                "traffic_level")) <= set(d["roofline"])
     assert d["roofline"]["bound"] == "hbm" and d["roofline"]["peak"] == 8000.0
     assert abs(d["roofline"]["frac"] - d["roofline"]["achieved"] / 8000.0) < 1e-12
     assert set(("value", "unit", "cores", "kind", "sample")) <= set(d["cpu_baseline"])
