@@ -1124,7 +1124,7 @@ static uint64_t own_device_bytes(const spc3d_plan *p)
     if (p->sweep.n) {
         const uint64_t n = p->sweep.n, rest = nnz - n;
         b += n * (4 + 2 + w) + nnz * 4; // col, lrow, values; perm
-        b += ((uint64_t)p->sweep.ntiles * p->sweep.nblocks * p->sweep.groups + 1) * 4;
+        b += ((uint64_t)p->sweep.ntiles * p->sweep.nblocks + 1) * 4;
         b += (uint64_t)p->sweep.ntiles * p->sweep.rows_per_tile * 4;
         if (p->c_stage)
             b += ((n + 63) / 64 * 64 + rest) * w + nnz * 4; // c_stage, stage_pos

@@ -60,9 +60,9 @@ hipError_t launch_sddmm_spmm(int dtype, int chained, const DevPlanView &P, const
                              const void *B, void *C, void *Y, uint32_t K, const Streams &streams);
 // ---- row tiles x column blocks ("sweep") -------------------------------------------
 // Device-side view of a sweep plan (SweepPlan in plan_device.h): the entries of rows of at
-// least a minimum length, ordered by tile of rows, column block, lane group, row.
+// least a minimum length, ordered by tile of rows, column block, row.
 struct SweepView {
-    const uint32_t *ptr = nullptr;       // [ntiles * nblocks * groups + 1] entry ranges
+    const uint32_t *ptr = nullptr;       // [ntiles * nblocks + 1] entry range of every (tile, block)
     const uint32_t *tile_rows = nullptr; // [ntiles * rows_per_tile] row of each local row, or 0xFFFFFFFF
     const uint32_t *col = nullptr;       // [n] sweep order
     const uint16_t *lrow = nullptr;      // [n] local row in the tile

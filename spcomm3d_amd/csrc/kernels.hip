@@ -1128,15 +1128,22 @@ spmm_fixup_kernel(const SplitRow *__restrict__ splits, uint32_t nsplit,
 // what an L2 sees, and the gathers hit.
 //
 // The plan (build_sweep in plan_device.h) orders a tile's entries by block, inside a block by
-// row, and cuts every (tile, block) range into G chunks at row boundaries, as equal as those
-// allow: ptr[(tile * nb + b) * G + g] .. [.. + 1) is chunk g of block b.  SpMM gives chunk g
-// to lane group g: within a block a row belongs to one lane group, the barrier separates the
-// blocks, so its sums need no atomics and are the same bits run to run.  SDDMM, where any
-// lane group can take any entry, deals the batches of the whole (tile, block) range to the
-// lane groups in turn, which leaves them within one batch of each other.
+// row; ptr[tile * nb + b] .. [.. + 1) is the range of block b.  Both kernels cut that range
+// into batches of UB entries and deal them to the G lane groups of the workgroup, which
+// leaves the lane groups within one batch of each other in every block.
+// SDDMM, where any lane group can take any entry: batch i to lane group i % G.
+// SpMM: lane group g takes the contiguous batches [g per, (g + 1) per), per = ceil(nbat / G).  The sum of
+// a row's run of entries is kept in registers and added to the row's accumulator in LDS when
+// the run ends.  A row's entries are contiguous, so a row is shared between lane groups only
+// where a boundary between two chunks falls inside it: its first part then ends a chunk (and
+// is added to the accumulator by that lane group), the later parts each BEGIN a chunk.  The
+// first run of every chunk therefore goes to an edge slot of its lane group instead, and
+// after the block's barrier the edge slots are added to their rows in lane-group order, one
+// lane group per row (the first of those that hold it); a second barrier ends the block.
+// No atomics, one fixed order of additions: the same bits run to run.
 constexpr int kSweepBlock = 1024;
 constexpr uint32_t kSweepRowBytes = 128u << 10; // of LDS for the tile's rows
-constexpr uint32_t kSweepPtrWords = 6148;       // nb * G + 1 range bounds of a tile, in LDS too
+constexpr uint32_t kSweepPtrWords = 1028;       // nb + 1 range bounds of a tile, in LDS too
 template <typename T, int LPR>
 __device__ __forceinline__ T sweep_dot(const typename Vec<T>::type &a, const typename Vec<T>::type &b)
 {
@@ -1174,8 +1181,8 @@ sweep_sddmm_kernel(const uint32_t *__restrict__ ptr, const uint32_t *__restrict_
             v = nt_load(reinterpret_cast<const V *>(A) + (uint64_t)g * LPR + i % LPR);
         tile_a[i] = v;
     }
-    for (uint32_t i = threadIdx.x; i < nb * G + 1; i += kSweepBlock)
-        lptr[i] = ptr[(uint64_t)tile * nb * G + i];
+    for (uint32_t i = threadIdx.x; i < nb + 1; i += kSweepBlock)
+        lptr[i] = ptr[(uint64_t)tile * nb + i];
     __syncthreads();
     const uint32_t grp = threadIdx.x / LPR, sub = threadIdx.x % LPR;
     const uint32_t uo = entry_of<LPR, UB>(sub);
@@ -1194,15 +1201,15 @@ sweep_sddmm_kernel(const uint32_t *__restrict__ ptr, const uint32_t *__restrict_
         return x;
     };
     // batch i of a block's range belongs to lane group i % G
-    uint32_t p = lptr[0] + grp * UB, hi = lptr[G];
+    uint32_t p = lptr[0] + grp * UB, hi = lptr[1];
     SweepIdx<T> cur;
     if (p < hi)
         cur = fetch(p, hi);
     for (uint32_t b = 0; b < nb; ++b) {
         uint32_t p_nb = 0, hi_nb = 0; // the next block's range
         if (b + 1 < nb) {
-            p_nb = lptr[(b + 1) * G] + grp * UB;
-            hi_nb = lptr[(b + 2) * G];
+            p_nb = lptr[b + 1] + grp * UB;
+            hi_nb = lptr[b + 2];
         }
         const bool had = p < hi;
         while (p < hi) {
@@ -1255,13 +1262,16 @@ sweep_spmm_kernel(const uint32_t *__restrict__ ptr, const uint32_t *__restrict__
 {
     using V = typename Vec<T>::type;
     constexpr uint32_t G = kSweepBlock / LPR;
+    constexpr uint32_t kNone = 0xFFFFFFFFu;
     __shared__ V tile_y[kSweepRowBytes / 16];
+    __shared__ V edge[kSweepBlock];   // the sum of the first run of every lane group's chunk
+    __shared__ uint32_t edge_row[G];  // and its row (kNone: the chunk is empty)
     __shared__ uint32_t lptr[kSweepPtrWords];
     const uint32_t tile = tile0 + blockIdx.x;
     for (uint32_t i = threadIdx.x; i < R * LPR; i += kSweepBlock)
         tile_y[i] = V{};
-    for (uint32_t i = threadIdx.x; i < nb * G + 1; i += kSweepBlock)
-        lptr[i] = ptr[(uint64_t)tile * nb * G + i];
+    for (uint32_t i = threadIdx.x; i < nb + 1; i += kSweepBlock)
+        lptr[i] = ptr[(uint64_t)tile * nb + i];
     __syncthreads();
     const uint32_t grp = threadIdx.x / LPR, sub = threadIdx.x % LPR;
     const V *Xv = reinterpret_cast<const V *>(X);
@@ -1275,22 +1285,40 @@ sweep_spmm_kernel(const uint32_t *__restrict__ ptr, const uint32_t *__restrict__
         x.val = vpos ? sval[nt_load(vpos + q + e)] : nt_load(sval + q + e);
         return x;
     };
-    // Within a block the rows of this lane group's chunk are its own: the sum of a row's run
-    // of entries is kept in registers and added to the row's accumulator in LDS when the run
-    // ends, in the plan's order: no atomics, the same bits run to run.
-    uint32_t row = 0xFFFFFFFFu;
-    V acc{};
-    uint32_t p = lptr[grp], hi = lptr[grp + 1];
+    // this lane group's chunk of block b: ceil(nbat / G) batches each, from lane group 0 on, so
+    // that the lane groups with entries are the first ones and those that share a row are
+    // neighbours
+    auto chunk = [&](uint32_t b, uint32_t &lo, uint32_t &up) {
+        const uint32_t s = lptr[b], e = lptr[b + 1];
+        const uint32_t nbat = (e - s + UB - 1) / UB;
+        const uint32_t per = (nbat + G - 1) / G;
+        const uint64_t first = (uint64_t)grp * per, last = first + per;
+        lo = first < nbat ? s + (uint32_t)first * UB : e;
+        up = last < nbat ? s + (uint32_t)last * UB : e;
+    };
+    uint32_t p, hi;
+    chunk(0, p, hi);
     SweepIdx<T> cur;
     if (p < hi)
         cur = fetch(p, hi);
     for (uint32_t b = 0; b < nb; ++b) {
         uint32_t p_nb = 0, hi_nb = 0;
-        if (b + 1 < nb) {
-            p_nb = lptr[(b + 1) * G + grp];
-            hi_nb = lptr[(b + 1) * G + grp + 1];
-        }
+        if (b + 1 < nb)
+            chunk(b + 1, p_nb, hi_nb);
         const bool had = p < hi;
+        uint32_t row = kNone;
+        bool first = true; // the run in `acc` is the chunk's first
+        V acc{};
+        // (The accumulator is read, added to and written back: LDS additions that return
+        // nothing, which need no wait, were measured 2.6 times slower for the whole call.)
+        auto flush = [&]() {
+            if (first)
+                edge[threadIdx.x] = acc;
+            else
+                tile_y[row * LPR + sub] += acc;
+        };
+        if (sub == 0)
+            edge_row[grp] = had ? cur.row : kNone; // lane 0 holds the chunk's first entry
         while (p < hi) {
             const uint32_t np = p + UB;
             SweepIdx<T> nxt;
@@ -1310,8 +1338,10 @@ sweep_spmm_kernel(const uint32_t *__restrict__ ptr, const uint32_t *__restrict__
                 const uint32_t l = __shfl(cur.row, u, LPR);
                 const T a = (uint32_t)u < cur.n ? __shfl(cur.val, u, LPR) : (T)0;
                 if (l != row) {
-                    if (row != 0xFFFFFFFFu)
-                        tile_y[row * LPR + sub] += acc;
+                    if (row != kNone) {
+                        flush();
+                        first = false;
+                    }
                     acc = V{};
                     row = l;
                 }
@@ -1320,16 +1350,23 @@ sweep_spmm_kernel(const uint32_t *__restrict__ ptr, const uint32_t *__restrict__
             p = np;
             cur = nxt;
         }
+        if (row != kNone)
+            flush();
         p = p_nb;
         hi = hi_nb;
         if (!had && p < hi)
             cur = fetch(p, hi);
-        if (row != 0xFFFFFFFFu) { // in the next block the row may be another lane group's
-            tile_y[row * LPR + sub] += acc;
-            acc = V{};
-            row = 0xFFFFFFFFu;
+        __syncthreads(); // the edge slots of block b are written, its direct additions done
+        // one lane group per row among the edge slots: the first that holds it adds them all,
+        // in lane-group order
+        const uint32_t er = edge_row[grp];
+        if (er != kNone && (grp == 0 || edge_row[grp - 1] != er)) {
+            V sum = tile_y[er * LPR + sub];
+            for (uint32_t h = grp; h < G && edge_row[h] == er; ++h)
+                sum += edge[h * LPR + sub];
+            tile_y[er * LPR + sub] = sum;
         }
-        __syncthreads();
+        __syncthreads(); // before block b + 1 writes edge slots and accumulators again
     }
     for (uint32_t i = threadIdx.x; i < R * LPR; i += kSweepBlock) {
         const uint32_t g = tile_rows[(uint64_t)tile * R + i / LPR];
@@ -1441,7 +1478,13 @@ gather4_kernel(const T *__restrict__ in, const uint32_t *__restrict__ pos, T *__
 {
     const uint64_t stride = (uint64_t)gridDim.x * kBlock * 4;
     const uint64_t nfull = n / 4 * 4;
-    for (uint64_t i = ((uint64_t)blockIdx.x * kBlock + threadIdx.x) * 4; i < nfull; i += stride) {
+    // Workgroups are dealt to the XCDs in turn: workgroup b takes the chunk that gives every
+    // XCD a contiguous eighth of each round of chunks, so that neighbours in `out`, whose
+    // reads tend to share lines of `in`, meet in one L2.
+    uint32_t chunk = blockIdx.x;
+    if (gridDim.x % 8 == 0)
+        chunk = (blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8;
+    for (uint64_t i = ((uint64_t)chunk * kBlock + threadIdx.x) * 4; i < nfull; i += stride) {
         const u32x4 p = nt_load(reinterpret_cast<const u32x4 *>(pos + i));
         using V = typename Vec<T>::type; // 16 bytes: 4 floats or 2 doubles
         V v[4 / Vec<T>::N];
@@ -2024,10 +2067,7 @@ uint32_t sweep_lanes(int dtype, uint32_t K)
 }
 uint32_t sweep_groups(uint32_t lanes) { return lanes ? kSweepBlock / lanes : 0; }
 uint32_t sweep_rows_per_tile(uint32_t lanes) { return lanes ? kSweepRowBytes / (lanes * 16) : 0; }
-uint32_t sweep_max_blocks(uint32_t lanes)
-{
-    return lanes ? (kSweepPtrWords - 1) / (kSweepBlock / lanes) : 0;
-}
+uint32_t sweep_max_blocks(uint32_t lanes) { return lanes ? kSweepPtrWords - 1 : 0; }
 
 namespace {
 template <typename T, int LPR>
@@ -2051,7 +2091,7 @@ hipError_t sweep_run(bool spmm, const SweepView &S, const T *A, const T *B, T *o
     // what the kernels assume of the plan: the tile's rows and range bounds fit their LDS
     if ((S.lanes != 16 && S.lanes != 32 && S.lanes != 64) || S.per_launch == 0 ||
         S.rows_per_tile * S.lanes * 16 > kSweepRowBytes ||
-        (uint64_t)S.nblocks * (kSweepBlock / S.lanes) + 1 > kSweepPtrWords)
+        (uint64_t)S.nblocks + 1 > kSweepPtrWords)
         return hipErrorInvalidValue;
     for (uint32_t t0 = 0; t0 < S.ntiles; t0 += S.per_launch) { // one generation per launch
         const uint32_t n = S.ntiles - t0 < S.per_launch ? S.ntiles - t0 : S.per_launch;

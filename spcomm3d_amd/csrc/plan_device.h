@@ -98,12 +98,11 @@ int build_store_staging(hipStream_t stream, const Seg *d_segs, uint32_t nseg, co
 // least min_row entries are ranked longest first; every per_launch * rows_per_tile of them
 // make a generation (one launch), inside which a tile takes rows_per_tile rows that are
 // consecutive by row number.  Their entries are sorted by (tile, column block, local row),
-// the caller's order kept inside a row's run, and every (tile, block) range is cut into
-// `groups` chunks at row boundaries, as equal as those allow; the entries of shorter rows
-// follow in the caller's order ("rest"; another plan runs them).
+// the caller's order kept inside a row's run; the entries of shorter rows follow in the
+// caller's order ("rest"; another plan runs them).
 //   perm[k]      caller's position of entry k of that order                [nnz]
 //   col, lrow    column and local row of sweep entry k                     [n]
-//   ptr          chunk bounds per (tile, block, group)                     [ntiles*nblocks*groups + 1]
+//   ptr          range bounds per (tile, block)                            [ntiles*nblocks + 1]
 //   tile_rows    row of local row l of tile t, 0xFFFFFFFF where there is none [ntiles*rows_per_tile]
 // The arrays belong to the receiver (hipFree).  Synchronous.
 struct SweepPlan {

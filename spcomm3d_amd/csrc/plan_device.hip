@@ -1570,26 +1570,6 @@ __global__ void sweep_entries_k(const unsigned long long *__restrict__ skey,
     }
 }
 
-// Chunk g of a bin starts at the first row boundary at or after the g-th G-th of its range.
-__global__ void sweep_chunks_k(const uint32_t *__restrict__ binptr, uint64_t nbins, uint32_t G,
-                               const uint16_t *__restrict__ lrow, uint32_t *ptr)
-{
-    GRID_STRIDE(i, nbins * G + 1)
-    {
-        if (i == nbins * G) {
-            ptr[i] = binptr[nbins];
-            continue;
-        }
-        const uint64_t bin = i / G;
-        const uint32_t g = (uint32_t)(i % G);
-        const uint32_t s = binptr[bin], e = binptr[bin + 1];
-        uint32_t q = s + (uint32_t)((uint64_t)(e - s) * g / G);
-        while (q > s && q < e && lrow[q] == lrow[q - 1])
-            ++q;
-        ptr[i] = q;
-    }
-}
-
 int build_sweep(hipStream_t st, uint32_t nrows, uint32_t ncols, uint64_t nnz, const uint32_t *d_ii,
                 const uint32_t *d_jj, uint32_t lanes, uint32_t R, uint32_t nb, uint32_t min_row,
                 uint32_t P, SweepPlan &out, std::string &err)
@@ -1645,7 +1625,7 @@ int build_sweep(hipStream_t st, uint32_t nrows, uint32_t ncols, uint64_t nnz, co
     const uint64_t last = nin - (gens - 1) * per_gen; // rows of the last generation
     const uint32_t rpt_last = (uint32_t)((last + P - 1) / P);
     const uint64_t ntiles64 = (gens - 1) * P + (last + rpt_last - 1) / rpt_last;
-    if (ntiles64 * nb * G + 1 >= (1ull << 32))
+    if (ntiles64 * nb + 1 >= (1ull << 32))
         return SPC3D_OK;
     const uint32_t ntiles = (uint32_t)ntiles64;
     HIP_OK(gkey.alloc(arena, nin));
@@ -1682,17 +1662,15 @@ int build_sweep(hipStream_t st, uint32_t nrows, uint32_t ncols, uint64_t nnz, co
     HIP_OK(lrow.alloc(n));
     HIP_OK(bin.alloc(arena, n));
     const uint64_t nbins = (uint64_t)ntiles * nb;
-    HIP_OK(ptr.alloc(nbins * G + 1));
-    SBuf<uint32_t> bstart, bcnt, binptr;
+    HIP_OK(ptr.alloc(nbins + 1));
+    SBuf<uint32_t> bstart, bcnt;
     HIP_OK(bstart.alloc(arena, nbins));
     HIP_OK(bcnt.alloc(arena, nbins + 1));
-    HIP_OK(binptr.alloc(arena, nbins + 1));
     HIP_OK(hipMemsetAsync(bcnt.p, 0, (nbins + 1) * sizeof(uint32_t), st));
     LAUNCH(sweep_entries_k, n, skey.p, perm.p, d_jj, n, R, col.p, lrow.p, bin.p);
     LAUNCH(run_bounds_k, n, bin.p, n, (uint32_t)nbins, bstart.p, bcnt.p);
     LAUNCH(run_lengths_k, nbins, bstart.p, nbins, bcnt.p);
-    TRY(exclusive_sum(tmp, bcnt.p, binptr.p, (size_t)nbins + 1, st, err));
-    LAUNCH(sweep_chunks_k, nbins * G + 1, binptr.p, nbins, G, lrow.p, ptr.p);
+    TRY(exclusive_sum(tmp, bcnt.p, ptr.p, (size_t)nbins + 1, st, err));
     HIP_OK(hipGetLastError());
     HIP_OK(hipStreamSynchronize(st));
     out.perm = perm.release();

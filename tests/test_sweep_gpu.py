@@ -122,7 +122,7 @@ def test_a_single_block_and_as_many_as_fit(ctx):
     case = long_rows(3, m, n, k, np.float32, lens)
     for nb in (1, 192, 4000):  # 4000: cut down to what a tile's range bounds allow
         out, info = run_all(ctx, m, n, *case, k_hint=k, sweep=True, sweep_min_row=1, col_blocks=nb)
-        assert info.sweep_entries == case[0].size and info.ncol_blocks == min(nb, 192)
+        assert info.sweep_entries == case[0].size and info.ncol_blocks == min(nb, 1027)
         check(out, *case)
 
 
