@@ -119,7 +119,8 @@ typedef struct {
                                   0: none.  The segment counts above are then those of the plan
                                   of the other entries */
     uint32_t sweep_tiles;      /* tiles of rows of that layout */
-    uint32_t sweep_k;          /* the K it is laid out for (k_hint): calls at another K are refused */
+    uint32_t sweep_k;          /* the K it is laid out for (k_hint); calls at another K run an
+                                  ordinary plan of the same pattern, made on first use */
 } spc3d_plan_info;
 
 /* Plan tuning; a zero field selects the default.  Only speed depends on these. */
@@ -157,9 +158,15 @@ typedef struct {
                               not cut at block boundaries: tiles of rows (128 KiB of A rows, or
                               of Y accumulators) stay in LDS while their workgroups walk the
                               column blocks in step, one workgroup per CU; the other rows form
-                              an ordinary plan.  Such a plan runs at K = k_hint only (other
-                              calls return SPC3D_ERR_INVALID_ARG), spc3d_spmm adds a row's
-                              entries block after block, and runs give the same bits.
+                              an ordinary plan.  The tiles run at K = k_hint; the first
+                              spc3d_sddmm, spc3d_spmm or spc3d_sddmm_spmm at another K makes an
+                              ordinary plan of the same pattern out of this plan's own arrays
+                              (it allocates and waits, so not while recording, and not in
+                              spc3d_spmm_noalloc, which return SPC3D_ERR_INVALID_ARG until
+                              another call has made it) and later calls at other widths run
+                              that one; spc3d_plan_info.device_bytes then counts both.
+                              spc3d_spmm adds a row's entries block after block, and runs
+                              give the same bits.
                               spc3d_sddmm stores the tiles' results straight to the caller's
                               positions when four in five of them follow their predecessor
                               there (a row's entries together), else through a staging vector

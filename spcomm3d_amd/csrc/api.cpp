@@ -737,20 +737,6 @@ static void *staged_out(const spc3d_plan *parent, const spc3d_plan *)
     return static_cast<char *>(parent->c_stage) + parent->rest_off * elem_size(parent->dtype);
 }
 
-// A plan kept as row tiles x column blocks runs at the K it was laid out for.
-static int sweep_check(const spc3d_plan *S, uint32_t K)
-{
-    if (!S->sweep.n || K == S->sweep_k)
-        return SPC3D_OK;
-    char msg[224];
-    std::snprintf(msg, sizeof msg,
-                  "the plan is laid out as row tiles for K = %u (spc3d_plan_info.sweep_k) and the "
-                  "panels have K = %u: create it with k_hint = K, or with spc3d_plan_opts.sweep = 1",
-                  S->sweep_k, K);
-    return fail(SPC3D_ERR_INVALID_ARG, msg);
-}
-
-
 /* ---- hot path ------------------------------------------------------------ */
 int spc3d_sddmm(spc3d_ctx *ctx, spc3d_plan *S, const spc3d_panel *A, const spc3d_panel *B,
                 spc3d_vals *C)
@@ -782,6 +768,9 @@ int spc3d_sddmm(spc3d_ctx *ctx, spc3d_plan *S, const spc3d_panel *A, const spc3d
     int rc = use_device(ctx, true);
     if (rc)
         return rc;
+    rc = plan_for_k(S, K, true, &S); // a plan in row tiles at another K: its ordinary twin
+    if (rc)
+        return rc;
     if (S->by_col) { // the same entries with rows and columns, and so A and B, exchanged
         const spc3d_plan *T = S->by_col;
         HIP_TRY(launch_sddmm(S->dtype, view_of(T), B->dev, A->dev, C->dev, K, streams_of(ctx)));
@@ -794,9 +783,6 @@ int spc3d_sddmm(spc3d_ctx *ctx, spc3d_plan *S, const spc3d_panel *A, const spc3d
         HIP_TRY(finish_sddmm(S, C->dev));
         return SPC3D_OK;
     }
-    rc = sweep_check(S, K);
-    if (rc)
-        return rc;
     if (S->sweep.n && !S->c_stage) { // the tiles and the rest store at the caller's positions
         for (spc3d_plan *part : S->blocks)
             HIP_TRY(launch_sddmm(S->dtype, view_of(part), A->dev, B->dev, C->dev, K, streams_of(ctx)));
@@ -847,10 +833,10 @@ int spc3d_spmm(spc3d_ctx *ctx, spc3d_plan *Ap, const spc3d_panel *X, spc3d_panel
     int rc = spmm_check(ctx, Ap, X, Y, &K);
     if (rc || K == 0)
         return rc;
-    rc = sweep_check(Ap, K);
+    rc = use_device(ctx, true);
     if (rc)
         return rc;
-    rc = use_device(ctx, true);
+    rc = plan_for_k(Ap, K, true, &Ap);
     if (rc)
         return rc;
     std::vector<spc3d_plan *> self;
@@ -873,6 +859,9 @@ int spc3d_spmm_noalloc(spc3d_ctx *ctx, spc3d_plan *Ap, const spc3d_panel *X, spc
     int rc = spmm_check(ctx, Ap, X, Y, &K);
     if (rc || K == 0)
         return rc;
+    rc = plan_for_k(Ap, K, false, &Ap); // (this call builds nothing)
+    if (rc)
+        return rc;
     const uint64_t need = (uint64_t)Ap->info.npartial_slots * K * elem_size(Ap->dtype);
     if (need > kStaticScratchBytes) {
         char msg[200];
@@ -882,9 +871,6 @@ int spc3d_spmm_noalloc(spc3d_ctx *ctx, spc3d_plan *Ap, const spc3d_panel *X, spc
                       (unsigned long long)need, K, (unsigned long long)kStaticScratchBytes);
         return fail(SPC3D_ERR_TOO_LARGE, msg);
     }
-    rc = sweep_check(Ap, K);
-    if (rc)
-        return rc;
     rc = use_device(ctx, true);
     if (rc)
         return rc;
@@ -935,7 +921,7 @@ int spc3d_sddmm_spmm(spc3d_ctx *ctx, spc3d_plan *S, const spc3d_panel *A, const 
         HIP_TRY(launch_fill(C->dtype, C->dev, S->info.nnz, 0.0, ctx->stream));
         return SPC3D_OK;
     }
-    rc = sweep_check(S, K);
+    rc = plan_for_k(S, K, true, &S);
     if (rc)
         return rc;
     std::vector<spc3d_plan *> self;

@@ -190,6 +190,10 @@ struct spc3d_plan {
     void *sweep_sval = nullptr; // [sweep.n] values in sweep order
     uint32_t sweep_k = 0;
     uint64_t rest_off = 0;
+    // The tiles are laid out for dense rows of sweep_k reals.  A call at another K runs
+    // `other_k`: an ordinary plan of the same pattern, made from this plan's own arrays by the
+    // first such call (plan_for_k) and kept, with this plan's values.
+    spc3d_plan *other_k = nullptr;
 };
 
 inline SweepView sweep_view_of(const spc3d_plan *p)
@@ -435,6 +439,10 @@ inline std::vector<spc3d_plan *> &parts_of(spc3d_plan *plan, std::vector<spc3d_p
 // library is built with hidden visibility and only SPC3D_API symbols are visible).
 // Partial-sum rows of cut rows wide enough for K columns (allocates a larger block when needed).
 extern "C" int ensure_partial(spc3d_plan *p, uint32_t K);
+// The plan a call at K columns runs: `plan` itself, or for a plan in row tiles at another K
+// than it was laid out for, its ordinary twin (built on first use unless may_build is false;
+// never while the context records).
+extern "C" int plan_for_k(spc3d_plan *plan, uint32_t K, bool may_build, spc3d_plan **out);
 // The defaults of spc3d_plan_create and of the one-shot host calls: the library's, each
 // overridable from the environment.
 extern "C" spc3d_plan_opts opts_from_env();

@@ -969,6 +969,11 @@ int spc3d_plan_destroy(spc3d_plan *plan)
     (void)hipSetDevice(plan->ctx->device);
     (void)hipStreamSynchronize(plan->ctx->stream);
     destroy_blocks(plan);
+    if (plan->other_k) {
+        spc3d_plan *o = plan->other_k;
+        plan->other_k = nullptr;
+        (void)spc3d_plan_destroy(o);
+    }
     if (plan->by_col) {
         plan_free_device(plan->by_col);
         plan->by_col->magic = 0;
@@ -1033,6 +1038,8 @@ int spc3d_plan_set_values(spc3d_plan *plan, const void *vv_host)
     }
     if (!rc)
         plan->has_values = true;
+    if (!rc && plan->other_k)
+        rc = spc3d_plan_set_values(plan->other_k, vv_host);
     return rc;
 }
 
@@ -1059,6 +1066,8 @@ int spc3d_plan_set_values_device(spc3d_plan *plan, const spc3d_vals *vv)
         plan->by_col->has_values = true;
     }
     plan->has_values = true;
+    if (plan->other_k)
+        return spc3d_plan_set_values_device(plan->other_k, vv);
     return SPC3D_OK;
 }
 
@@ -1134,6 +1143,110 @@ static uint64_t own_device_bytes(const spc3d_plan *p)
     return b;
 }
 
+// The ordinary twin of a plan in row tiles (spc3d_plan::other_k): the pattern is read back
+// from the plan's own arrays (the tiles' entries and the plan of the rest, each with its
+// caller's positions), planned again without tiles for K columns, and given the values the
+// plan holds.
+static int build_other_k(spc3d_plan *S, uint32_t K)
+{
+    spc3d_ctx *ctx = S->ctx;
+    const uint64_t nnz = S->info.nnz;
+    const size_t w = elem_size(S->dtype);
+    spc3d_plan_opts o;
+    std::memset(&o, 0, sizeof o);
+    o.k_hint = K;
+    o.sweep = 1;
+    PlanOpts po;
+    int rc = resolve_opts(S->dtype, &o, po);
+    if (rc)
+        return rc;
+    uint32_t *d_ii = nullptr, *d_jj = nullptr;
+    void *vals = nullptr;
+    spc3d_plan *q = nullptr;
+    std::string err;
+    rc = dev_alloc(&d_ii, (size_t)nnz);
+    if (!rc) rc = dev_alloc(&d_jj, (size_t)nnz);
+    if (!rc) {
+        rc = sweep_coords_device(ctx->stream, S->sweep, d_ii, d_jj, err);
+        for (spc3d_plan *part : S->blocks)
+            if (!rc)
+                rc = seg_coords_device(ctx->stream, part->segs, part->info.nsegments_padded,
+                                       part->col, part->perm, d_ii, d_jj, err);
+        if (rc)
+            fail(rc, err);
+    }
+    if (!rc)
+        rc = build_from_device(ctx, S->dtype, S->info.nrows, S->info.ncols, nnz, d_ii, d_jj, po, &o, &q);
+    if (!rc && S->has_values) {
+        rc = dev_alloc_bytes(&vals, (size_t)nnz * w);
+        if (!rc) {
+            hipError_t e = launch_scatter_vals(S->dtype, S->sweep_sval, S->sweep.perm, vals,
+                                               S->sweep.n, ctx->stream);
+            for (spc3d_plan *part : S->blocks)
+                if (e == hipSuccess)
+                    e = launch_scatter_vals(S->dtype, part->sval, part->perm, vals, part->info.nnz,
+                                            ctx->stream);
+            std::vector<spc3d_plan *> self;
+            for (spc3d_plan *part : parts_of(q, self))
+                if (e == hipSuccess)
+                    e = launch_gather_vals(S->dtype, vals, part->perm, part->sval, part->info.nnz,
+                                           ctx->stream);
+            if (e == hipSuccess && q->by_col) {
+                e = launch_gather_vals(S->dtype, vals, q->by_col->perm, q->by_col->sval, nnz,
+                                       ctx->stream);
+                q->by_col->has_values = true;
+            }
+            if (e == hipSuccess)
+                e = hipStreamSynchronize(ctx->stream);
+            if (e != hipSuccess)
+                rc = fail_hip(e, "values of the plan for another K");
+            else
+                q->has_values = true;
+        }
+    }
+    if (!rc) {
+        hipError_t e = hipStreamSynchronize(ctx->stream);
+        if (e != hipSuccess)
+            rc = fail_hip(e, "hipStreamSynchronize");
+    }
+    if (d_ii) (void)hipFree(d_ii);
+    if (d_jj) (void)hipFree(d_jj);
+    if (vals) (void)hipFree(vals);
+    if (rc) {
+        const std::string keep = g_err;
+        if (q)
+            (void)spc3d_plan_destroy(q);
+        return fail(rc, keep);
+    }
+    S->other_k = q;
+    return SPC3D_OK;
+}
+
+int plan_for_k(spc3d_plan *plan, uint32_t K, bool may_build, spc3d_plan **out)
+{
+    *out = plan;
+    if (!plan->sweep.n || K == plan->sweep_k)
+        return SPC3D_OK;
+    if (!plan->other_k) {
+        char msg[256];
+        if (!may_build || plan->ctx->capturing) {
+            std::snprintf(msg, sizeof msg,
+                          "the plan is laid out as row tiles for K = %u (spc3d_plan_info.sweep_k); "
+                          "the plan it runs at another K (here %u) is made by the first spc3d_sddmm, "
+                          "spc3d_spmm or spc3d_sddmm_spmm at such a K outside a recording: run one first",
+                          plan->sweep_k, K);
+            return fail(SPC3D_ERR_INVALID_ARG, msg);
+        }
+        int rc = use_device(plan->ctx);
+        if (!rc)
+            rc = build_other_k(plan, K);
+        if (rc)
+            return rc;
+    }
+    *out = plan->other_k;
+    return SPC3D_OK;
+}
+
 int spc3d_plan_get_info(const spc3d_plan *plan, spc3d_plan_info *info)
 {
     if (!live(plan) || !info)
@@ -1144,6 +1257,11 @@ int spc3d_plan_get_info(const spc3d_plan *plan, spc3d_plan_info *info)
         b += own_device_bytes(blk);
     if (plan->by_col)
         b += own_device_bytes(plan->by_col);
+    if (plan->other_k) {
+        spc3d_plan_info twin;
+        if (spc3d_plan_get_info(plan->other_k, &twin) == SPC3D_OK)
+            b += twin.device_bytes;
+    }
     info->device_bytes = b;
     return SPC3D_OK;
 }

@@ -105,6 +105,9 @@ hipError_t launch_unpermute_two_pass(int dtype, const void *stage, void *mid, co
                                      const uint32_t *dst1, const uint16_t *l2, void *out, uint64_t n,
                                      hipStream_t stream);
 // out[p] = in[perm[p]] (perm == null: copy)
+// out[perm[i]] = in[i], i < n (perm null: a copy).
+hipError_t launch_scatter_vals(int dtype, const void *in, const uint32_t *perm, void *out,
+                               uint64_t n, hipStream_t stream);
 hipError_t launch_gather_vals(int dtype, const void *in, const uint32_t *perm, void *out,
                               uint64_t n, hipStream_t stream);
 // Device-side view of a row map (buffer slot i <-> dense row rows[i]).

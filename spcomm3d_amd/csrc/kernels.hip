@@ -1468,6 +1468,17 @@ gather_kernel(const T *__restrict__ in, const uint32_t *__restrict__ perm, T *__
         out[i] = perm ? in[perm[i]] : in[i];
 }
 
+// out[perm[i]] = in[i] (perm null: out[i] = in[i])
+template <typename T>
+__global__ void __launch_bounds__(kBlock)
+scatter_kernel(const T *__restrict__ in, const uint32_t *__restrict__ perm, T *__restrict__ out,
+               uint64_t n)
+{
+    const uint64_t stride = (uint64_t)gridDim.x * kBlock;
+    for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride)
+        out[perm ? perm[i] : i] = in[i];
+}
+
 // out[i] = in[pos[i]], four results per lane: positions and results move as 16-byte
 // vectors, streaming; the reads in between are whatever `pos` makes them (runs, for the
 // staged results of a plan kept in column blocks).
@@ -2187,6 +2198,20 @@ hipError_t launch_unpermute_two_pass(int dtype, const void *stage, void *mid, co
         hipLaunchKernelGGL((unpermute_pass2_kernel<float>), dim3(grid), dim3(kTwoPassBlock), 0,
                            stream, (const float *)mid, l2, (float *)out, n);
     }
+    return hipGetLastError();
+}
+
+hipError_t launch_scatter_vals(int dtype, const void *in, const uint32_t *perm, void *out,
+                               uint64_t n, hipStream_t stream)
+{
+    if (n == 0)
+        return hipSuccess;
+    if (dtype == 1)
+        hipLaunchKernelGGL((scatter_kernel<double>), dim3(stream_grid(n)), dim3(kBlock), 0, stream,
+                           (const double *)in, perm, (double *)out, n);
+    else
+        hipLaunchKernelGGL((scatter_kernel<float>), dim3(stream_grid(n)), dim3(kBlock), 0, stream,
+                           (const float *)in, perm, (float *)out, n);
     return hipGetLastError();
 }
 

@@ -116,6 +116,13 @@ int build_sweep(hipStream_t stream, uint32_t nrows, uint32_t ncols, uint64_t nnz
                 const uint32_t *d_ii, const uint32_t *d_jj, uint32_t lanes, uint32_t rows_per_tile,
                 uint32_t nblocks, uint32_t min_row, uint32_t per_launch, SweepPlan &out,
                 std::string &err);
+// The pattern back from a plan: d_ii / d_jj at the caller's positions of the entries of a
+// sweep, and of a plan in segments (d_perm null: its kernel order is the caller's).
+// Asynchronous on `stream`.
+int sweep_coords_device(hipStream_t stream, const SweepPlan &sw, uint32_t *d_ii, uint32_t *d_jj,
+                        std::string &err);
+int seg_coords_device(hipStream_t stream, const Seg *d_segs, uint64_t nseg, const uint32_t *d_col,
+                      const uint32_t *d_perm, uint32_t *d_ii, uint32_t *d_jj, std::string &err);
 // *out = how many q < n - 1 have d[q + 1] == d[q] + 1.  Synchronous.
 int count_adjacent_device(hipStream_t stream, const uint32_t *d, uint64_t n, uint64_t *out,
                           std::string &err);

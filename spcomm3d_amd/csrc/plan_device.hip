@@ -1493,11 +1493,6 @@ int build_two_pass(hipStream_t st, const uint32_t *d_perm, uint64_t nnz, uint32_
 }
 
 // ---- row tiles x column blocks ("sweep") ---------------------------------------------
-__global__ void sweep_hist_k(const uint32_t *__restrict__ ii, uint64_t nnz, uint32_t *rowcnt)
-{
-    GRID_STRIDE(e, nnz) atomicAdd(&rowcnt[ii[e]], 1u);
-}
-
 // out[perm[q]] = base + q
 __global__ void inverse_offsets_k(const uint32_t *__restrict__ perm, uint64_t n, uint32_t base,
                                   uint32_t *out)
@@ -1596,7 +1591,9 @@ int build_sweep(hipStream_t st, uint32_t nrows, uint32_t ncols, uint64_t nnz, co
     HIP_OK(total.alloc(arena, 1));
     HIP_OK(hipMemsetAsync(rowcnt.p, 0, ((size_t)nrows + 1) * sizeof(uint32_t), st));
     HIP_OK(hipMemsetAsync(total.p, 0, sizeof(unsigned long long), st));
-    LAUNCH(sweep_hist_k, nnz, d_ii, nnz, rowcnt.p);
+    // one addition per run of equal row numbers inside a wavefront: few for rows that arrive
+    // together, one per entry at worst
+    LAUNCH(hist_sorted_k, nnz, d_ii, nnz, rowcnt.p);
     // rows by length, longest first, equal lengths in row order; those of at least min_row
     // entries come first and are the sweep's
     LAUNCH(iota_k, nrows, rowid.p, (uint64_t)nrows);
@@ -1686,6 +1683,67 @@ int build_sweep(hipStream_t st, uint32_t nrows, uint32_t ncols, uint64_t nnz, co
     out.lanes = lanes;
     out.per_launch = P;
     out.nrows_in = nin;
+    return SPC3D_OK;
+}
+
+// ii[perm[k]], jj[perm[k]] = row and column of sweep entry k: its tile by bisection over the
+// tiles' first bounds, its row from the tile's row list.
+__global__ void sweep_coords_k(const uint32_t *__restrict__ ptr, uint32_t ntiles, uint32_t nb,
+                               const uint32_t *__restrict__ tile_rows, uint32_t R,
+                               const uint16_t *__restrict__ lrow, const uint32_t *__restrict__ col,
+                               const uint32_t *__restrict__ perm, uint64_t n, uint32_t *ii,
+                               uint32_t *jj)
+{
+    GRID_STRIDE(k, n)
+    {
+        uint32_t lo = 0, hi = ntiles; // ptr[lo * nb] <= k < ptr[hi * nb]
+        while (hi - lo > 1) {
+            const uint32_t mid = lo + (hi - lo) / 2;
+            if (ptr[(uint64_t)mid * nb] <= k)
+                lo = mid;
+            else
+                hi = mid;
+        }
+        const uint32_t at = perm[k];
+        ii[at] = tile_rows[(uint64_t)lo * R + lrow[k]];
+        jj[at] = col[k];
+    }
+}
+
+// The same for the entries of a plan in segments (perm null: kernel order is the caller's).
+__global__ void seg_coords_k(const Seg *__restrict__ segs, uint64_t nseg,
+                             const uint32_t *__restrict__ col, const uint32_t *__restrict__ perm,
+                             uint32_t *ii, uint32_t *jj)
+{
+    GRID_STRIDE(sg, nseg)
+    {
+        const Seg g = segs[sg];
+        for (uint32_t q = g.start; q < g.start + g.len; ++q) {
+            const uint32_t at = perm ? perm[q] : q;
+            ii[at] = g.row;
+            jj[at] = col[q];
+        }
+    }
+}
+
+int sweep_coords_device(hipStream_t st, const SweepPlan &sw, uint32_t *d_ii, uint32_t *d_jj,
+                        std::string &err)
+{
+    if (sw.n == 0)
+        return SPC3D_OK;
+    LAUNCH(sweep_coords_k, sw.n, sw.ptr, sw.ntiles, sw.nblocks, sw.tile_rows, sw.rows_per_tile,
+           sw.lrow, sw.col, sw.perm, sw.n, d_ii, d_jj);
+    HIP_OK(hipGetLastError());
+    return SPC3D_OK;
+}
+
+int seg_coords_device(hipStream_t st, const Seg *d_segs, uint64_t nseg, const uint32_t *d_col,
+                      const uint32_t *d_perm, uint32_t *d_ii, uint32_t *d_jj, std::string &err)
+{
+    if (nseg == 0)
+        return SPC3D_OK;
+    LAUNCH(seg_coords_k, nseg, d_segs, nseg, d_col, d_perm, d_ii, d_jj);
+    HIP_OK(hipGetLastError());
     return SPC3D_OK;
 }
 

@@ -12,9 +12,16 @@ from spcomm3d_amd import workloads as W
 pytestmark = pytest.mark.gpu
 
 
+def in_tiles(w):
+    w.notes["tiles"] = dict(sweep=True, sweep_min_row=8, col_blocks=5)
+    return w
+
+
 def operands(ctx, w, dtype):
     vv = w.values(dtype)
-    S = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, vv, k_hint=w.k)
+    tiles = w.notes.get("tiles", {})  # plan options of the row-tile case below
+    S = ctx.plan(w.nrows, w.ncols, w.ii, w.jj, vv, k_hint=w.k, **tiles)
+    assert bool(S.info.sweep_entries) == bool(tiles)
     dA, dB = ctx.panel_from(w.panel_A(dtype)), ctx.panel_from(w.panel_B(dtype))
     return S, dA, dB
 
@@ -26,6 +33,9 @@ def operands(ctx, w, dtype):
     (lambda: W.rmat(15, 16, 50).shuffled(), np.float32),         # rows that end inside a vector
     (lambda: W.rmat(13, 16, 1030).shuffled(), np.float64),       # rows over 4 KiB: three slices,
                                                                  # SDDMM slices accumulate into C
+    (lambda: in_tiles(W.rmat(14, 16, 64).shuffled()), np.float64),  # row tiles, staged results,
+                                                                    # and the plan of the rest
+    (lambda: in_tiles(W.rmat(14, 16, 128)), np.float32),         # row tiles, results straight to C
 ])
 def test_replays_equal_eager_runs(ctx, maker, dtype):
     w = maker()

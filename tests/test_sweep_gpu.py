@@ -126,24 +126,58 @@ def test_a_single_block_and_as_many_as_fit(ctx):
         check(out, *case)
 
 
-def test_another_k_is_refused_and_other_widths_keep_the_ordinary_plan(ctx):
-    k, m, n = 128, 200, 1000
-    case = long_rows(9, m, n, k, np.float32, np.full(m, 100))
+def test_another_k_runs_an_ordinary_plan_made_on_first_use(ctx):
+    k, m, n = 128, 300, 1000
+    rng = np.random.default_rng(4)
+    lens = rng.integers(0, 200, m)
+    case = long_rows(9, m, n, k, np.float32, lens)
     ii, jj, vv, A, B, Y0 = case
-    S = ctx.plan(m, n, ii, jj, vv, k_hint=k, sweep=True, sweep_min_row=1)
-    assert S.info.sweep_entries == ii.size
-    dA, dB, dY = ctx.panel_from(A[:, :64]), ctx.panel_from(B[:, :64]), ctx.panel_from(Y0[:, :64])
+    S = ctx.plan(m, n, ii, jj, vv, k_hint=k, sweep=True, sweep_min_row=16, col_blocks=3)
+    assert 0 < S.info.sweep_entries < ii.size
+    before = S.info.device_bytes
+    k2 = 48
+    A2, B2, Y2 = (np.ascontiguousarray(x[:, :k2]) for x in (A, B, Y0))
+    dA, dB, dY = ctx.panel_from(A2), ctx.panel_from(B2), ctx.panel_from(Y2)
     dC = ctx.vals(ii.size, np.float32)
-    for call in (lambda: ctx.sddmm(S, dA, dB, dC), lambda: ctx.spmm(S, dB, dY),
-                 lambda: ctx.spmm_noalloc(S, dB, dY), lambda: ctx.sddmm_spmm(S, dA, dB, dC, dY)):
-        with pytest.raises(capi.Spc3dError) as e:
-            call()
-        assert e.value.status == capi.ERR_INVALID_ARG and "k_hint" in str(e.value)
+    # the call that allocates nothing cannot make that plan, and says who can
+    with pytest.raises(capi.Spc3dError) as e:
+        ctx.spmm_noalloc(S, dB, dY)
+    assert e.value.status == capi.ERR_INVALID_ARG and "spc3d_spmm" in str(e.value)
+    # nor can a call that is being recorded
+    ctx.capture_begin()
+    with pytest.raises(capi.Spc3dError):
+        ctx.sddmm(S, dA, dB, dC)
+    ctx.capture_end().close()
     ctx.sync()
-    assert np.array_equal(dY.download(), Y0[:, :64])
-    for h in (S, dA, dB, dC, dY):
+    assert np.array_equal(dY.download(), Y2) and S.info.device_bytes == before
+    # the first ordinary call makes it; every entry point then runs at that K, and at a third
+    ctx.sddmm(S, dA, dB, dC)
+    assert S.info.device_bytes > before and S.info.sweep_entries > 0
+    assert oracle.sddmm_rel_err(A2, B2, ii, jj, vv, dC.download()) <= 1e-5
+    ctx.spmm(S, dB, dY)
+    Y_spmm = dY.download()
+    assert oracle.spmm_rel_err(B2, ii, jj, vv, Y2, Y_spmm) <= 1e-5
+    dY.upload(Y2)
+    ctx.spmm_noalloc(S, dB, dY)
+    assert np.array_equal(dY.download(), Y_spmm)
+    dY.upload(Y2)
+    ctx.sddmm_spmm(S, dA, dB, dC, dY, chained=True)
+    C = dC.download()
+    assert oracle.spmm_rel_err(B2, ii, jj, C, Y2, dY.download()) <= 1e-5
+    A3, B3 = np.ascontiguousarray(A[:, :7]), np.ascontiguousarray(B[:, :7])
+    dA3, dB3 = ctx.panel_from(A3), ctx.panel_from(B3)
+    ctx.sddmm(S, dA3, dB3, dC)
+    assert oracle.sddmm_rel_err(A3, B3, ii, jj, vv, dC.download()) <= 1e-5
+    # new values reach both forms of the plan
+    S.set_values(2 * vv)
+    ctx.sddmm(S, dA, dB, dC)
+    assert np.array_equal(dC.download(), 2 * C)
+    dA4, dB4 = ctx.panel_from(A), ctx.panel_from(B)
+    ctx.sddmm(S, dA4, dB4, dC)  # and the tiles still run at their own K
+    assert oracle.sddmm_rel_err(A, B, ii, jj, 2 * vv, dC.download()) <= 1e-5
+    for h in (S, dA, dB, dY, dC, dA3, dB3, dA4, dB4):
         h.close()
-    # a width the tile kernels do not take, or no k_hint: the ordinary plan
+    # a width the tile kernels do not take, or no k_hint: the ordinary plan from the start
     for opts in ({"k_hint": 100, "sweep": True}, {"sweep": True}):
         S = ctx.plan(m, n, ii, jj, vv, **opts)
         assert S.info.sweep_entries == 0 and S.info.nsegments > 0
