@@ -2,6 +2,7 @@
 symbol, validates patterns on the host, builds correct plans, and fails loudly
 (no fallback) when there is no GPU.  No kernel is launched here."""
 import ctypes
+import os
 
 import numpy as np
 import pytest
@@ -266,6 +267,54 @@ def test_plan_build_host_rejects_bad_arguments():
     rc = lib.spc3d_plan_build_host(capi.F32, 2, 6, 3, vp(ii), vp(jj), ctypes.byref(o),
                                    ctypes.byref(info), None, None, None, 0, None, 0)
     assert rc == capi.ERR_INVALID_ARG
+    # row tiles: 0, 1, 2 are the modes; the host builder makes none, so asking it for them is an error
+    for field, value in (("sweep", 3), ("flags", 32)):
+        o = capi.PlanOpts()
+        setattr(o, field, value)
+        rc = lib.spc3d_plan_build_host(capi.F32, 2, 6, 3, vp(ii), vp(jj), ctypes.byref(o),
+                                       ctypes.byref(info), None, None, None, 0, None, 0)
+        assert rc == capi.ERR_INVALID_ARG, field
+    o = capi.PlanOpts()
+    o.sweep, o.builder = 2, 1
+    rc = lib.spc3d_plan_build_host(capi.F32, 2, 6, 3, vp(ii), vp(jj), ctypes.byref(o),
+                                   ctypes.byref(info), None, None, None, 0, None, 0)
+    assert rc == capi.ERR_INVALID_ARG
+    o = capi.PlanOpts()
+    o.sweep, o.sweep_min_row, o.flags = 1, 5, capi.PLAN_SWEEP_STAGED  # valid, and without effect here
+    rc = lib.spc3d_plan_build_host(capi.F32, 2, 6, 3, vp(ii), vp(jj), ctypes.byref(o),
+                                   ctypes.byref(info), None, None, None, 0, None, 0)
+    assert rc == capi.OK and info.sweep_entries == 0 and info.sweep_tiles == 0
+
+
+def test_the_python_mirrors_of_the_structs_have_the_headers_layout():
+    """sizeof and the offsets of the last fields, against a C program compiled from the header."""
+    import subprocess
+    import tempfile
+
+    src = r"""
+#include <stdio.h>
+#include <stddef.h>
+#include "spcomm3d_hip.h"
+int main(void) {
+    printf("%zu %zu %zu %zu %zu %zu\n", sizeof(spc3d_plan_opts), offsetof(spc3d_plan_opts, sweep_min_row),
+           sizeof(spc3d_plan_info), offsetof(spc3d_plan_info, sweep_k), sizeof(spc3d_ctx_opts),
+           offsetof(spc3d_plan_info, device_bytes));
+    return 0;
+}
+"""
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    with tempfile.TemporaryDirectory() as d:
+        c = os.path.join(d, "layout.c")
+        with open(c, "w") as f:
+            f.write(src)
+        exe = os.path.join(d, "layout")
+        subprocess.run(["gcc", "-I", os.path.join(root, "include"), "-o", exe, c], check=True)
+        got = [int(x) for x in subprocess.run([exe], capture_output=True, text=True,
+                                              check=True).stdout.split()]
+    want = [ctypes.sizeof(capi.PlanOpts), capi.PlanOpts.sweep_min_row.offset,
+            ctypes.sizeof(capi.PlanInfo), capi.PlanInfo.sweep_k.offset,
+            ctypes.sizeof(capi.CtxOpts), capi.PlanInfo.device_bytes.offset]
+    assert got == want
 
 
 def test_context_options_are_validated_before_any_device_is_touched():
