@@ -192,7 +192,13 @@ typedef struct {
  * one more pass also when the caller's order keeps a row's entries together (by default the
  * tile kernels then store straight to the caller's positions, and nothing is staged). */
 #define SPC3D_PLAN_SWEEP_STAGED 16u
-#define SPC3D_PLAN_ALL_FLAGS 31u
+/* XCD slicing: deal the segments that have no slice of their own (rows under hub_min, the cold
+ * parts of hub rows) by their rank alone.  By default such a segment goes to the queue of the
+ * slice most of its entries in sliced columns belong to, while that queue has room: on R-MAT 20
+ * a third instead of an eighth of those entries then gather on the XCD that keeps their dense
+ * rows (SDDMM / SpMM 2 to 4 % faster). */
+#define SPC3D_PLAN_NO_SLICE_AFFINITY 32u
+#define SPC3D_PLAN_ALL_FLAGS 63u
 
 /* ---- library / errors ------------------------------------------------- */
 SPC3D_API const char *spc3d_version(void);

@@ -51,7 +51,7 @@ class PlanOpts(ctypes.Structure):
                 ("sweep", c_u32), ("sweep_min_row", c_u32), ("reserved", c_u32 * 1)]
 
 PLAN_NO_STAGED_STORES, PLAN_NO_SDDMM_BY_COLUMN, PLAN_NO_TWO_PASS, PLAN_KEEP_ENTRY_ORDER = 1, 2, 4, 8
-PLAN_SWEEP_STAGED = 16
+PLAN_SWEEP_STAGED, PLAN_NO_SLICE_AFFINITY = 16, 32
 
 
 # name -> (restype, argtypes); one entry for every function the header declares.

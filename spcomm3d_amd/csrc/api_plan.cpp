@@ -72,6 +72,7 @@ static int resolve_opts(int dtype, const spc3d_plan_opts *o, PlanOpts &out)
         return fail(SPC3D_ERR_INVALID_ARG, "xcd_slices must be 0, 1 or 8");
     out.seg_max = z.seg_max;
     out.keep_entry_order = (z.flags & SPC3D_PLAN_KEEP_ENTRY_ORDER) != 0;
+    out.slice_affinity = !(z.flags & SPC3D_PLAN_NO_SLICE_AFFINITY);
     out.hub_min = z.hub_min;
     out.xcd_slices = z.xcd_slices;
     const uint64_t k = z.k_hint ? z.k_hint : 64;
@@ -948,6 +949,8 @@ spc3d_plan_opts opts_from_env()
             o.flags |= e.off_flag;
     if (env_number("SPC3D_KEEP_ENTRY_ORDER", &v) && v != 0)
         o.flags |= SPC3D_PLAN_KEEP_ENTRY_ORDER;
+    if (env_number("SPC3D_SLICE_AFFINITY", &v) && v == 0)
+        o.flags |= SPC3D_PLAN_NO_SLICE_AFFINITY;
     if (const char *b = std::getenv("SPC3D_PLAN_BUILDER"))
         o.builder = std::strcmp(b, "host") == 0 ? 1u : 2u;
     return o;

@@ -30,6 +30,7 @@ struct Counters { // one device-resident block, zeroed (first_bad: all ones) bef
     unsigned long long covered;
     unsigned long long load[kSlices];
     unsigned long long any_load;
+    unsigned long long pref_load[kSlices];
 };
 
 // Owning device buffer; freed on scope exit unless released.
@@ -528,6 +529,58 @@ __global__ void any_flags_k(const Seg *__restrict__ pseg, const uint8_t *__restr
     }
 }
 
+// Step 1b: the slice a free piece prefers (the one most of its sliced entries belong to;
+// kNoPref without any), and the free work that prefers each slice.
+__global__ void pref_k(const Seg *__restrict__ pseg, const uint8_t *__restrict__ pqueue, uint64_t n,
+                       const uint32_t *__restrict__ col, const uint8_t *__restrict__ cls,
+                       uint8_t *pref, Counters *C)
+{
+    unsigned long long w[kSlices] = {0};
+    GRID_STRIDE(i, n)
+    {
+        uint8_t p = kNoPref;
+        if (pqueue[i] == kAnyQueue) {
+            const Seg g = pseg[i];
+            uint32_t cnt[kSlices] = {0};
+            for (uint32_t q = g.start; q < g.start + g.len; ++q) {
+                const uint8_t c = cls[col[q]];
+#pragma unroll
+                for (uint32_t k = 0; k < kSlices; ++k)
+                    cnt[k] += c == k;
+            }
+            // ties go to the first slice from a start that the row's hash picks
+            const uint32_t first = rep_slice(g.row);
+            uint32_t best = first, most = 0;
+#pragma unroll
+            for (uint32_t k = 0; k < kSlices; ++k)
+                most = k == first ? cnt[k] : most;
+            for (uint32_t k = 1; k < kSlices; ++k) {
+                const uint32_t q = (first + k) % kSlices;
+                uint32_t c = 0;
+#pragma unroll
+                for (uint32_t j = 0; j < kSlices; ++j)
+                    c = j == q ? cnt[j] : c;
+                if (c > most) {
+                    most = c;
+                    best = q;
+                }
+            }
+            if (most)
+                p = (uint8_t)best;
+#pragma unroll
+            for (uint32_t k = 0; k < kSlices; ++k)
+                w[k] += (most && best == k) ? (unsigned long long)g.len + kSegCost : 0ull;
+        }
+        pref[i] = p;
+    }
+#pragma unroll
+    for (uint32_t k = 0; k < kSlices; ++k) {
+        const unsigned long long t = block_sum(w[k]);
+        if (threadIdx.x == 0 && t)
+            atomicAdd(&C->pref_load[k], t);
+    }
+}
+
 // Step 2: the free pieces, compacted in piece order, with their length keys.
 __global__ void compact_any_k(const Seg *__restrict__ pseg, const uint32_t *__restrict__ anyflag,
                               const uint32_t *__restrict__ anypos, uint64_t n, uint32_t seg_max,
@@ -540,18 +593,16 @@ __global__ void compact_any_k(const Seg *__restrict__ pseg, const uint32_t *__re
     }
 }
 
-struct Upto {
-    uint32_t v[kDealQueues];
-};
 
 // Step 3: every piece gets its queue.  The combined list is [bound pieces in piece
 // order | free pieces longest first]; its key is (queue, seg_max - len).
 __global__ void combine_k(const Seg *__restrict__ pseg, const uint8_t *__restrict__ pqueue,
                           const uint32_t *__restrict__ anyflag,
                           const uint32_t *__restrict__ anypos,
-                          const uint32_t *__restrict__ any_sorted, uint64_t npieces,
-                          uint64_t nany, uint32_t seg_max, Upto upto, uint32_t *comb_idx,
-                          uint32_t *comb_key, Counters *C)
+                          const uint32_t *__restrict__ any_sorted,
+                          const uint8_t *__restrict__ pref, uint64_t npieces, uint64_t nany,
+                          uint32_t seg_max, DealPlan deal, uint32_t *comb_idx, uint32_t *comb_key,
+                          Counters *C)
 {
     const uint64_t nbound = npieces - nany;
     uint32_t cnt[kSlices] = {0}, lng[kSlices] = {0};
@@ -568,7 +619,7 @@ __global__ void combine_k(const Seg *__restrict__ pseg, const uint8_t *__restric
         } else { // the free piece of rank j
             const uint64_t j = t - npieces;
             piece = any_sorted[j];
-            q = deal_queue((uint32_t)j, upto.v);
+            q = deal_queue_pref((uint32_t)j, pref[piece], deal);
             at = nbound + j;
         }
         const uint32_t l = pseg[piece].len;
@@ -1057,10 +1108,14 @@ int build_device_plan(hipStream_t st, uint32_t nrows, uint32_t ncols, uint64_t n
         P.nseg_long = hC.nlong / kChunk * kChunk;
     } else {
         SBuf<uint32_t> anyflag, anypos;
+        SBuf<uint8_t> pref;
         HIP_OK(anyflag.alloc(arena, (size_t)np_total + 1));
         HIP_OK(anypos.alloc(arena, (size_t)np_total + 1));
+        HIP_OK(pref.alloc(arena, np_total));
         LAUNCH_SMALL(any_flags_k, (uint64_t)np_total + 1, pseg.p, pqueue.p, (uint64_t)np_total,
                anyflag.p, dC.p);
+        LAUNCH_SMALL(pref_k, np_total, pseg.p, pqueue.p, (uint64_t)np_total, col.p, cls.p, pref.p,
+                     dC.p);
         TRY(exclusive_sum(tmp, anyflag.p, anypos.p, (size_t)np_total + 1, st, err));
         uint32_t nany = 0;
         TRY(fetch(st, &nany, anypos.p + np_total, sizeof nany, err));
@@ -1077,11 +1132,13 @@ int build_device_plan(hipStream_t st, uint32_t nrows, uint32_t ncols, uint64_t n
             TRY(sort_pairs<uint32_t>(tmp, any_key.p, any_key_out.p, any_idx.p, any_sorted.p, nany,
                                      len_bits, false, st, err));
         }
-        uint64_t load[kDealQueues];
-        for (uint32_t q = 0; q < kDealQueues; ++q)
+        uint64_t load[kDealQueues], pref_load[kDealQueues];
+        for (uint32_t q = 0; q < kDealQueues; ++q) {
             load[q] = hC.load[q];
-        Upto upto;
-        deal_thresholds(load, hC.any_load, upto.v);
+            pref_load[q] = hC.pref_load[q];
+        }
+        DealPlan deal;
+        deal_plan(load, pref_load, hC.any_load, opts.slice_affinity, deal);
 
         SBuf<uint32_t> comb_idx, comb_key, comb_idx_out, comb_key_out;
         HIP_OK(comb_idx.alloc(arena, np_total));
@@ -1089,7 +1146,7 @@ int build_device_plan(hipStream_t st, uint32_t nrows, uint32_t ncols, uint64_t n
         HIP_OK(comb_idx_out.alloc(arena, np_total));
         HIP_OK(comb_key_out.alloc(arena, np_total));
         LAUNCH_SMALL(combine_k, (uint64_t)np_total + nany, pseg.p, pqueue.p, anyflag.p, anypos.p,
-               any_sorted.p, (uint64_t)np_total, (uint64_t)nany, seg_max, upto, comb_idx.p,
+               any_sorted.p, pref.p, (uint64_t)np_total, (uint64_t)nany, seg_max, deal, comb_idx.p,
                comb_key.p, dC.p);
         const int comb_bits = bits_for((uint64_t)kSlices * ((uint64_t)seg_max + 1) - 1);
         TRY(sort_pairs<uint32_t>(tmp, comb_key.p, comb_key_out.p, comb_idx.p, comb_idx_out.p,

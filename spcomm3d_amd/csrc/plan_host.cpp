@@ -47,6 +47,7 @@ constexpr uint8_t kRep = kClsRep, kCold = kClsCold;
 struct Piece {
     Seg seg;
     uint8_t queue;
+    uint8_t pref = kNoPref; // a free piece: the slice most of its sliced entries belong to
 };
 
 inline uint32_t seg_len(const Seg &s) { return s.len; }
@@ -280,8 +281,10 @@ int build_host_plan(uint32_t nrows, uint32_t ncols, uint64_t nnz, const uint32_t
             for (size_t i = 0; i < pieces.size(); ++i)
                 P.segs[i] = pieces[i].seg;
         } else {
-            // Hub pieces go to the queue of their column slice.  The rest, longest
-            // first, fill every queue up to the same total: piece i of that order
+            // Hub pieces go to the queue of their column slice.  Of the rest, longest
+            // first, a piece with entries in sliced columns goes to the queue of the
+            // slice that holds most of them while that queue has room (deal_plan);
+            // the others fill every queue up to the same total: piece i of that order
             // goes to the queue whose share of the unit interval holds the i-th
             // point of a low-discrepancy sequence, shares being proportional to
             // what each queue still lacks.  Any window of consecutive (hence
@@ -290,9 +293,27 @@ int build_host_plan(uint32_t nrows, uint32_t ncols, uint64_t nnz, const uint32_t
             // builder deals identically.
             P.nqueues = kSlices;
             std::vector<Piece> queue[kSlices], any;
-            uint64_t load[kSlices] = {0}, any_load = 0;
-            for (const Piece &p : pieces) {
+            uint64_t load[kSlices] = {0}, pref_load[kSlices] = {0}, any_load = 0;
+            for (Piece &p : pieces) {
                 if (p.queue == kAnyQueue) {
+                    // the slice most of its sliced entries belong to (see deal_plan)
+                    uint32_t cnt[kSlices] = {0};
+                    for (uint32_t q = p.seg.start; q < p.seg.start + seg_len(p.seg); ++q) {
+                        const uint8_t c = cls[P.col[q]];
+                        if (c < kSlices)
+                            ++cnt[c];
+                    }
+                    // (ties go to the first slice from a start that the row's hash picks, so
+                    // that no slice collects the short pieces)
+                    uint32_t best = rep_slice(p.seg.row);
+                    for (uint32_t k = 1; k < kSlices; ++k) {
+                        const uint32_t q = (rep_slice(p.seg.row) + k) % kSlices;
+                        if (cnt[q] > cnt[best])
+                            best = q;
+                    }
+                    p.pref = cnt[best] ? (uint8_t)best : kNoPref;
+                    if (p.pref < kNoPref)
+                        pref_load[p.pref] += seg_len(p.seg) + kSegCost;
                     any.push_back(p);
                     any_load += seg_len(p.seg) + kSegCost;
                 } else {
@@ -301,10 +322,10 @@ int build_host_plan(uint32_t nrows, uint32_t ncols, uint64_t nnz, const uint32_t
                 }
             }
             sort_longest_first(any, seg_max);
-            uint32_t upto[kSlices];
-            deal_thresholds(load, any_load, upto);
+            DealPlan deal;
+            deal_plan(load, pref_load, any_load, opts.slice_affinity, deal);
             for (size_t i = 0; i < any.size(); ++i)
-                queue[deal_queue((uint32_t)i, upto)].push_back(any[i]);
+                queue[deal_queue_pref((uint32_t)i, any[i].pref, deal)].push_back(any[i]);
             size_t nchunks = 0;
             for (uint32_t q = 0; q < kSlices; ++q) {
                 sort_longest_first(queue[q], seg_max);

@@ -49,6 +49,9 @@ struct PlanOpts {
     // every row (equal columns in the caller's order), which is what a row-sorted
     // pattern's entries usually are.  true: always keep the caller's order inside a row.
     bool keep_entry_order = false;
+    // slicing: false keeps the free segments dealt by rank alone (no affinity to the slice of
+    // their entries, see deal_plan)
+    bool slice_affinity = true;
 };
 
 struct HostPlan {
@@ -158,6 +161,56 @@ SPC3D_HD inline uint32_t deal_queue(uint32_t i, const uint32_t (&upto)[kDealQueu
     while (q + 1 < kDealQueues && x > upto[q])
         ++q;
     return q;
+}
+
+// ---- affinity of free segments to a slice ------------------------------------
+// A free segment (a row under the hub threshold, or the cold part of a hub row) has no
+// queue of its own, but its entries in sliced columns hit only in the L2 of their slice:
+// one in eight by chance.  Such a segment PREFERS the slice most of its sliced entries
+// belong to (on ties the first from a start picked by the row's hash; kNoPref without any), and is queued there while that queue
+// has room below the common level; the others are dealt as before.  R-MAT 20: 32 % instead
+// of 12.5 % of the sliced entries of free segments then gather in their slice's XCD.
+constexpr uint8_t kNoPref = 8;
+
+struct DealPlan {
+    uint32_t keep[kDealQueues]; // a free segment of rank i that prefers q stays with q when
+                                // i * 0x85EBCA6B mod 2^32 <= keep[q]
+    uint32_t upto[kDealQueues]; // deal_queue() shares for the others
+};
+
+// load[q]: work bound to queue q; pref_load[q]: free work that prefers q; free_load: all
+// free work (the preferring part included).  Every queue accepts of its preferrers what
+// fits under the common level (total / 8), a hashed share of them when they are too many.
+inline void deal_plan(const uint64_t (&load)[kDealQueues], const uint64_t (&pref_load)[kDealQueues],
+                      uint64_t free_load, bool affinity, DealPlan &out)
+{
+    uint64_t total = free_load, with_pref[kDealQueues], left = free_load;
+    for (uint32_t q = 0; q < kDealQueues; ++q)
+        total += load[q];
+    const uint64_t level = total / kDealQueues;
+    for (uint32_t q = 0; q < kDealQueues; ++q) {
+        const uint64_t room = level > load[q] ? level - load[q] : 0;
+        const uint64_t want = affinity ? pref_load[q] : 0;
+        const uint64_t take = want < room ? want : room;
+        // take / want of 2^32 (loads are < 2^40: 24 fractional bits, then 8 more)
+        uint64_t k = 0;
+        if (want != 0 && take == want)
+            k = 0xFFFFFFFFull;
+        else if (want != 0)
+            k = ((take << 24) / want) << 8;
+        out.keep[q] = (uint32_t)(k > 0xFFFFFFFFull ? 0xFFFFFFFFull : k);
+        with_pref[q] = load[q] + take;
+        left -= take;
+    }
+    deal_thresholds(with_pref, left, out.upto);
+}
+
+// Queue of the free segment of rank i (longest first) with preference `pref`.
+SPC3D_HD inline uint32_t deal_queue_pref(uint32_t i, uint8_t pref, const DealPlan &d)
+{
+    if (pref < kNoPref && i * 0x85EBCA6Bu <= d.keep[pref])
+        return pref;
+    return deal_queue(i, d.upto);
 }
 
 // Default longest segment: long enough that few rows are cut (each cut costs a

@@ -35,14 +35,15 @@ def make_opts(seg_max=None, k_hint=None, l2_hot_bytes=None, hub_min=None,
               xcd_slices=None, builder=None, col_blocks=None, staged_stores=None,
               sddmm_by_column=None, two_pass=None, two_pass_min=None,
               keep_entry_order=None, sweep=None, sweep_min_row=None,
-              sweep_staged=None) -> PlanOpts:
+              sweep_staged=None, slice_affinity=None) -> PlanOpts:
     """``spc3d_plan_opts``; ``None`` keeps the library default.  ``builder``:
     ``"device"`` or ``"host"`` (where ``spc3d_plan_create_ex`` builds the plan).
     ``staged_stores`` / ``sddmm_by_column`` / ``two_pass`` = False keep the plain stores
     of SDDMM results; ``keep_entry_order`` = True keeps the caller's order inside rows
     that arrive unsorted.  ``sweep``: ``None`` (the library decides), ``False`` (never) or
     ``True`` (row tiles x column blocks whenever ``k_hint`` has a width the kernels take);
-    ``sweep_staged`` = True stages the tiles' SDDMM results whatever the entry order."""
+    ``sweep_staged`` = True stages the tiles' SDDMM results whatever the entry order;
+    ``slice_affinity`` = False deals the free segments of a sliced plan by rank alone."""
     o = PlanOpts()
     o.sweep = 0 if sweep is None else (2 if sweep else 1)
     o.sweep_min_row = int(sweep_min_row or 0)
@@ -50,7 +51,8 @@ def make_opts(seg_max=None, k_hint=None, l2_hot_bytes=None, hub_min=None,
                (capi.PLAN_NO_SDDMM_BY_COLUMN if sddmm_by_column is False else 0) |
                (capi.PLAN_NO_TWO_PASS if two_pass is False else 0) |
                (capi.PLAN_KEEP_ENTRY_ORDER if keep_entry_order else 0) |
-               (capi.PLAN_SWEEP_STAGED if sweep_staged else 0))
+               (capi.PLAN_SWEEP_STAGED if sweep_staged else 0) |
+               (capi.PLAN_NO_SLICE_AFFINITY if slice_affinity is False else 0))
     o.two_pass_min = int(two_pass_min or 0)
     o.builder = _BUILDERS[builder]
     o.seg_max = int(seg_max or 0)

@@ -240,6 +240,31 @@ def test_plan_xcd_slicing_on_skewed_pattern():
             qcol.setdefault(int(c), set()).add(int(q))
     sliced = [c for c, qs in qcol.items() if len(qs) == 1]
     assert len(sliced) > 0.3 * len(qcol)
+    # rows under the hub threshold go, where there is room, to the queue of the slice most of
+    # their sliced entries belong to: of their entries in columns with a queue of their own,
+    # far more than the eighth that chance gives sit in that queue, and none of that without
+    own = np.full(w.ncols, -1, dtype=np.int64)
+    for c in sliced:
+        own[c] = next(iter(qcol[c]))
+
+    def at_home(plan):
+        sg, cols = plan["segs"], plan["col"]
+        home = total = 0
+        for idx in np.flatnonzero(sg[:, 2] > 0):
+            row, start, ln, slot = sg[idx]
+            if counts[row] >= 32:
+                continue
+            o = own[cols[start:start + ln]]
+            total += int((o >= 0).sum())
+            home += int((o == (idx // 64) % 8).sum())
+        return home / max(total, 1)
+
+    F = _check_plan(w.nrows, w.ncols, w.ii, w.jj, xcd_slices=8, l2_hot_bytes=64 * 1024,
+                    hub_min=32, seg_max=256, slice_affinity=False)
+    assert at_home(P) > 0.25 and at_home(F) < 0.16
+    fl = np.array([F["segs"][(np.arange(F["segs"].shape[0]) // 64 % 8) == q][:, 2].sum()
+                   for q in range(8)], dtype=np.int64)
+    assert fl.max() - fl.min() <= 0.02 * fl.mean() + 256
 
 
 def test_plan_slicing_stays_off_for_uniform_columns():
@@ -268,7 +293,7 @@ def test_plan_build_host_rejects_bad_arguments():
                                    ctypes.byref(info), None, None, None, 0, None, 0)
     assert rc == capi.ERR_INVALID_ARG
     # row tiles: 0, 1, 2 are the modes; the host builder makes none, so asking it for them is an error
-    for field, value in (("sweep", 3), ("flags", 32)):
+    for field, value in (("sweep", 3), ("flags", 64)):
         o = capi.PlanOpts()
         setattr(o, field, value)
         rc = lib.spc3d_plan_build_host(capi.F32, 2, 6, 3, vp(ii), vp(jj), ctypes.byref(o),

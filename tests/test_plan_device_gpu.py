@@ -89,6 +89,10 @@ def test_sliced_layout_on_skewed_pattern(ctx, shuffled):
     P = both(ctx, w.nrows, w.ncols, w.ii, w.jj, xcd_slices=8, l2_hot_bytes=64 * 1024, hub_min=32,
              seg_max=256)
     assert P["info"].nqueues == 8 and P["info"].hub_rows > 0 and P["info"].nsplit_rows > 0
+    # free segments dealt by rank alone
+    Q = both(ctx, w.nrows, w.ncols, w.ii, w.jj, xcd_slices=8, l2_hot_bytes=64 * 1024, hub_min=32,
+             seg_max=256, slice_affinity=False)
+    assert Q["info"].nqueues == 8 and not np.array_equal(Q["segs"], P["segs"])
     # the same pattern with slicing switched off
     P = both(ctx, w.nrows, w.ncols, w.ii, w.jj, xcd_slices=1, seg_max=256)
     assert P["info"].nqueues == 1
@@ -132,7 +136,8 @@ def test_random_patterns_and_options_differential(ctx):
                     hub_min=int(rng.choice([1, 2, 8, 32, 128])),
                     l2_hot_bytes=int(rng.choice([64, 256, 1024, 4096])),
                     k_hint=int(rng.choice([1, 16, 64])),
-                    xcd_slices=int(rng.choice([0, 8, 8, 1])))
+                    xcd_slices=int(rng.choice([0, 8, 8, 1])),
+                    slice_affinity=bool(rng.random() < 0.7))
         P = both(ctx, m, n, ii, jj, **opts)
         sliced += P["info"].nqueues == 8
     assert sliced >= 10  # the sliced layout was exercised, not only the plain one
