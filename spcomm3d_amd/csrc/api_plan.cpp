@@ -417,6 +417,8 @@ static int rebuild_as_sweep(spc3d_plan *p, uint32_t nrows, uint32_t ncols, uint6
                             const spc3d_plan_opts *opts, uint32_t lanes, uint32_t nb, bool *taken)
 {
     *taken = false;
+    if (nnz + 64 >= (1ull << 32)) // staging places are 32-bit, the rest's start rounded up to 64
+        return SPC3D_OK;
     spc3d_ctx *ctx = p->ctx;
     const size_t w = elem_size(p->dtype);
     const uint32_t min_row = opts->sweep_min_row ? opts->sweep_min_row : 64;
