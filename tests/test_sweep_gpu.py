@@ -205,3 +205,38 @@ def test_values_set_later_and_from_the_device(ctx):
     assert np.array_equal(dC.download(), 2 * first)
     for h in (S, dA, dB, dC, dV):
         h.close()
+
+
+def test_random_shapes_differential(ctx):
+    """Seeded random patterns, tile and block counts: few rows per tile, blocks without entries,
+    rows longer than a block's share of the lane groups, single-entry rows, every row width."""
+    rng = np.random.default_rng(2024)
+    widths = [(np.float32, 64), (np.float32, 128), (np.float32, 256),
+              (np.float64, 32), (np.float64, 64), (np.float64, 128)]
+    for case_no in range(24):
+        dtype, k = widths[case_no % len(widths)]
+        m = int(rng.choice([1, 3, 40, 300, 1500]))
+        n = int(rng.choice([1, 7, 100, 5000]))
+        shape = rng.choice(["short", "mixed", "long", "one_huge"])
+        if shape == "short":
+            lens = rng.integers(0, 4, m)
+        elif shape == "mixed":
+            lens = rng.integers(0, 60, m)
+        elif shape == "long":
+            lens = rng.integers(100, 400, m) if m <= 300 else rng.integers(0, 80, m)
+        else:
+            lens = rng.integers(0, 3, m)
+            lens[rng.integers(0, m)] = 20000
+        if lens.sum() == 0:
+            lens[0] = 1
+        case = long_rows(int(rng.integers(1 << 30)), m, n, k, dtype, lens,
+                         shuffle=bool(rng.random() < 0.5))
+        nb = int(rng.choice([1, 2, 5, 33, 1000]))
+        min_row = int(rng.choice([1, 1, 2, 10, 50]))
+        out, info = run_all(ctx, m, n, *case, k_hint=k, sweep=True, sweep_min_row=min_row,
+                            col_blocks=nb, sweep_staged=bool(rng.random() < 0.3))
+        want = int(lens[lens >= min_row].sum())
+        assert info.sweep_entries == want, (case_no, shape, m, n, nb, min_row)
+        if want and nb > 1:  # (1 leaves the number of blocks to the rule)
+            assert info.ncol_blocks == min(nb, n)
+        check(out, *case)
